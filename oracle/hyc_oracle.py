@@ -1,0 +1,395 @@
+"""CPU oracle for the HyC-LoRA hybrid activation-compression hot path.
+
+THIS IS TEST INFRASTRUCTURE, NOT PRODUCT CODE.  Only tests, the smoke check and
+the benchmark's cpu-baseline leg may import it; the product package never does.
+
+Everything here is a restatement, on CPU PyTorch tensors, of the arithmetic the
+reference performs (same op order, same dtypes, hence the same bf16 roundings).
+Each function cites the reference lines it follows.  Two families:
+
+* ``ref_*``  - the scheme the reference snapshot implements: element-threshold
+  outliers kept as a COO sparse tensor, a static scale (per-tensor / per-channel
+  / per-token), an optional rank-r base ``L @ R``.
+* ``hyc_*``  - the channel-structured variant: the k channels with the largest
+  per-channel abs-max are kept verbatim as a dense ``[M, k]`` side tensor, the
+  rest is quantised with a scale per (token, group of G channels).  The reference
+  holds no implementation of the channel selection rule; the functions below are
+  composed from the reference's primitives (zero-out, divide, round, clamp,
+  offset, half-split packing).  PARITY UNPINNED BY THE REFERENCE for the selection
+  rule and for the group-scale granularity; pinned for quantise / pack / unpack /
+  dequantise, which are shared with the ``ref_*`` family.
+
+Pinning status (see tests/test_oracle_*.py):
+* pack / unpack                - brute force over all byte values, pure Python loops
+* quantise                     - all 65536 bf16 patterns x scales vs exact rationals
+* ref_compress / ref_decompress / get_statistics / softmax helpers / SiLU, GELU,
+  Hadamard, softmax backward / calibration protocol
+                               - golden vectors written by importing the reference
+* rmsnorm_fwd / rmsnorm_bwd    - closed form + torch.autograd (reference kernels are
+                                 Triton and cannot run without a GPU)
+* linear_bwd                   - torch.matmul in fp32
+* hyc_select_channels / hyc group scales - parity unpinned (no reference code)
+"""
+import math
+
+import torch
+
+BF16 = torch.bfloat16
+
+
+# --------------------------------------------------------------------------------------
+# shape helpers                                  operators/compress_function.py:4-12
+# --------------------------------------------------------------------------------------
+def hidden_to_head_shape(x, num_heads):
+    b, s, h = x.shape
+    return x.reshape(b, s, num_heads, h // num_heads).transpose(1, 2)
+
+
+def head_to_hidden_shape(x):
+    b, nh, s, hd = x.shape
+    return x.transpose(1, 2).reshape(b, s, nh * hd)
+
+
+def pad_cut_L(src_L, tgt_L):
+    """Zero-pad or cut the rows of src_L to the row count of tgt_L.
+    operators/compress_function.py:350-360"""
+    have, r = src_L.shape
+    want = tgt_L.shape[0]
+    if have < want:
+        pad = torch.zeros(want - have, r, dtype=src_L.dtype, device=src_L.device)
+        src_L = torch.cat((src_L, pad), dim=0)
+    elif have > want:
+        src_L = src_L[:want, :]
+    return src_L.contiguous()
+
+
+# --------------------------------------------------------------------------------------
+# bit packing                                     operators/compress_function.py:175-197, 218-255
+# --------------------------------------------------------------------------------------
+def pack_codes(codes_u8, bits):
+    """codes_u8 [..., H] uint8 in [0, 2^bits) -> [..., H*bits/8] uint8.
+
+    Segment layout: the last dim is cut into n = 8/bits equal segments; byte j holds
+    segment i's element j in bit field [i*bits, (i+1)*bits).  (bits == 8 is not packed
+    by the reference - it stores int8 - and is not handled here.)"""
+    assert bits in (1, 2, 4)
+    n = 8 // bits
+    H = codes_u8.shape[-1]
+    seg = H // n
+    out = None
+    # the reference adds the highest segment first; uint8 addition is commutative and
+    # the fields are disjoint, so the order is immaterial.
+    for i in range(n):
+        part = codes_u8[..., i * seg:(i + 1) * seg] * (2 ** (i * bits))
+        out = part if out is None else out + part
+    return out
+
+
+def unpack_codes(packed_u8, bits):
+    """Inverse of pack_codes using the reference's %, -, // chain (:222-252)."""
+    assert bits in (1, 2, 4)
+    n = 8 // bits
+    base = 2 ** bits
+    rest = packed_u8
+    parts = []
+    for i in range(n):
+        if i < n - 1:
+            low = rest % base
+            rest = (rest - low) // base
+            parts.append(low)
+        else:
+            parts.append(rest)
+    return torch.cat(parts, dim=-1)
+
+
+# --------------------------------------------------------------------------------------
+# quantise / dequantise primitives              operators/compress_function.py:170, 221-255
+# --------------------------------------------------------------------------------------
+def quantize_q(x, scale, bits, guard_zero_scale=False):
+    """q = clamp(round(x / scale), -2^(b-1), 2^(b-1)-1); x, scale bf16 (broadcastable).
+
+    The division result is a bf16 tensor (fp32 divide rounded to nearest even), round is
+    half-to-even, then the clamp.  With guard_zero_scale, positions whose scale is 0
+    give q = 0 instead of the reference's undefined NaN -> integer cast."""
+    off = 2 ** (bits - 1)
+    q = torch.clamp(torch.round(x / scale), min=-off, max=off - 1)
+    if guard_zero_scale:
+        q = torch.where((scale == 0).expand_as(q), torch.zeros_like(q), q)
+    return q
+
+
+def encode_q(q, bits):
+    """q (bf16 integers) -> stored tensor: int8 for 8 bits, packed uint8 otherwise."""
+    if bits == 8:
+        return q.to(torch.int8)
+    off = 2 ** (bits - 1)
+    return pack_codes((q + off).to(torch.uint8), bits)
+
+
+def decode_stored(stored, bits, scale, dtype=BF16):
+    """stored -> dequantised bf16 ((code - off) * scale, each op rounding to bf16)."""
+    if bits == 8:
+        return stored.to(dtype) * scale
+    off = 2 ** (bits - 1)
+    return (unpack_codes(stored, bits).to(dtype) - off) * scale
+
+
+# --------------------------------------------------------------------------------------
+# calibration                                    operators/compress_function.py:292-347
+# --------------------------------------------------------------------------------------
+@torch.no_grad()
+def get_statistics(x, iteration, outlier_ratio, sub_outlier_ratio, sub_outlier_bit=8,
+                   sub_outlier_quantize_method='per-tensor', svd_rank=16):
+    """Threshold, rank-r base and static scale from batch element 0.
+    Returns (thr f32 0-d, L bf16 [S,r], R bf16 [r,H], scale bf16)."""
+    if x.dim() == 4:
+        b, nh, s, hd = x.shape
+        x = x.permute(0, 2, 1, 3).reshape(b, s, nh * hd)
+    if svd_rank > 0:
+        U, S, V = torch.svd_lowrank(x[0].to(torch.float32), q=svd_rank, niter=16)
+        L = U.contiguous()
+        R = (torch.diag(S) @ V.T).contiguous()
+        x = x - L @ R                       # promotes x to fp32 from here on
+    else:
+        L = torch.zeros((x.shape[-2], 16), dtype=x.dtype, device=x.device)
+        R = torch.zeros((16, x.shape[-1]), dtype=x.dtype, device=x.device)
+
+    first = x[0]
+    kth = int(first.numel() * (1 - outlier_ratio))
+    thr = torch.kthvalue(first.flatten().to(torch.float32), kth).values     # signed quantile
+    big = (first * (first.abs() > thr)).to(BF16)
+    x = x - big                             # batch 0's outliers, broadcast over the batch
+
+    if sub_outlier_ratio > 0 and sub_outlier_bit != 16:
+        z = x[0]
+        levels = 2 ** sub_outlier_bit - 1
+        if sub_outlier_quantize_method == 'per-tensor':
+            scale = (z.max() - z.min()) / levels
+        elif sub_outlier_quantize_method == 'per-channel':
+            scale = (z.max(dim=-2, keepdim=True).values - z.min(dim=-2, keepdim=True).values) / levels
+        elif sub_outlier_quantize_method == 'per-token':
+            scale = (z.max(dim=-1, keepdim=True).values - z.min(dim=-1, keepdim=True).values) / levels
+        else:
+            raise ValueError("Unsupport Quantize Method")
+    else:
+        scale = torch.tensor(1., device=x.device)
+    return thr, L.to(BF16), R.to(BF16), scale.to(BF16)
+
+
+@torch.no_grad()
+def get_statistics_softmax(y, iteration, outlier_ratio):
+    """operators/compress_function.py:343-347"""
+    first = y[0]
+    return torch.kthvalue(first.float().flatten(), int(first.numel() * (1 - outlier_ratio))).values
+
+
+def running_mean_update(static, fresh, iteration):
+    """One step of the modules' calibration average, e.g. operators/efficient_silu.py:86-111.
+    static / fresh are [thr, L, scale, R] lists (note the order)."""
+    if iteration >= 2:
+        return static
+    out = list(static)
+    for slot in range(4):
+        new = fresh[slot]
+        if static[slot] is None:
+            out[slot] = new
+        else:
+            if slot == 1:
+                new = pad_cut_L(new, static[slot])
+            out[slot] = (iteration * static[slot] + new) / (iteration + 1)
+    return out
+
+
+# --------------------------------------------------------------------------------------
+# ref-mode compress / decompress                 operators/compress_function.py:136-261
+# --------------------------------------------------------------------------------------
+@torch.no_grad()
+def ref_compress(x, thr, scale, bits=8, sub_outlier_ratio=1., L=None, R=None):
+    """-> (coo sparse bf16 of the outliers, stored codes, scale).  x is [B,S,H] or [B,nh,S,hd]."""
+    if x.dim() == 4:
+        x = head_to_hidden_shape(x)
+    S = x.shape[-2]
+    base = pad_cut_L(L, torch.zeros((S, L.shape[-1]))) @ R          # bf16 matmul -> bf16
+    x = x - base
+    hot = x.abs() > thr                                             # thr rounds to x's dtype
+    big = x * hot
+    x = x - big                                                     # exact zeros at hot positions
+    if torch.sum(scale) != 1.:
+        big_c = big.to(BF16).to_sparse()
+    else:
+        big_c = big
+    assert sub_outlier_ratio != 0., "the no-quantisation branch is not part of the path"
+    assert bits in (1, 2, 4, 8), "bits must be 1, 2, 4 or 8 on this path"
+    q = quantize_q(x, scale, bits)
+    return big_c, encode_q(q, bits), scale
+
+
+@torch.no_grad()
+def ref_decompress(big_c, stored, bits, scale, is_head=False, num_heads=1, L=None, R=None):
+    big = big_c.to_dense() if big_c.is_sparse else big_c
+    S = big.shape[-2]
+    x = (pad_cut_L(L, torch.zeros((S, L.shape[-1]))) @ R).to(BF16)
+    x = x + big
+    if torch.sum(scale) != 1.:
+        x = x + decode_stored(stored, bits, scale, big.dtype)
+    if is_head:
+        x = hidden_to_head_shape(x, num_heads)
+    return x
+
+
+# --------------------------------------------------------------------------------------
+# softmax sparsification                          operators/compress_function.py:264-281
+# --------------------------------------------------------------------------------------
+def prune_softmax(y, thr):
+    return y * (y > thr)
+
+
+@torch.no_grad()
+def true_compress_softmax(y, thr):
+    return prune_softmax(y, thr).to_sparse()
+
+
+@torch.no_grad()
+def true_decompress_softmax(y_sparse):
+    return y_sparse.to_dense()
+
+
+# --------------------------------------------------------------------------------------
+# low-rank helpers                                operators/fused_compression.py:5-67, 102-171
+# --------------------------------------------------------------------------------------
+def low_rank_extraction(l, r, x):
+    """x[b] - l@r accumulated in fp32 from the bf16 operands, one rounding to bf16."""
+    return (x.float() - (l.float() @ r.float())[None]).to(BF16)
+
+
+def low_rank_addition(l, r, x):
+    return (x.float() + (l.float() @ r.float())[None]).to(BF16)
+
+
+# --------------------------------------------------------------------------------------
+# hyc mode: channel outliers + per-(token, group) scales
+# --------------------------------------------------------------------------------------
+def hyc_num_outlier_channels(H, ratio):
+    return int(math.floor(ratio * H + 0.5))
+
+
+def hyc_channel_scores(x):
+    """max over all tokens of |x[..., c]| - exact in bf16; returned as fp32 [H]."""
+    return x.reshape(-1, x.shape[-1]).abs().amax(dim=0).float()
+
+
+def hyc_select_channels(scores, k):
+    """k largest scores, ties to the lower channel index, returned ascending (int32)."""
+    order = torch.sort(scores, descending=True, stable=True).indices[:k]
+    return torch.sort(order).values.to(torch.int32)
+
+
+@torch.no_grad()
+def hyc_compress(x, idx, bits, group):
+    """x [M,H] bf16, idx [k] ascending -> (vals [M,k] bf16, stored, scales [M,H/G] bf16).
+
+    Composition of the reference steps (:149-151 zero-out, :170 quantise, :175-197 pack) with
+    the channel mask in place of the threshold mask, and the reference scale formula
+    (max - min) / (2^b - 1) (:328-334) evaluated per token and group of G channels.
+    A group whose scale is 0 (constant group) is given code = offset (q = 0)."""
+    M, H = x.shape
+    idx = idx.long()
+    hot = torch.zeros(H, dtype=torch.bool)
+    hot[idx] = True
+    big = x * hot
+    vals = big[:, idx].contiguous()
+    rest = x - big
+    g = rest.reshape(M, H // group, group)
+    scales = (g.amax(dim=-1) - g.amin(dim=-1)) / (2 ** bits - 1)
+    q = quantize_q(g, scales[..., None], bits, guard_zero_scale=True).reshape(M, H)
+    return vals, encode_q(q, bits), scales
+
+
+@torch.no_grad()
+def hyc_decompress(vals, stored, idx, scales, bits, group):
+    """-> x_hat [M,H] bf16 = (0 + scatter(vals)) + dequant (the order of :205-256)."""
+    M = stored.shape[0]
+    H = stored.shape[1] * (8 // bits)
+    big = torch.zeros(M, H, dtype=BF16)
+    big[:, idx.long()] = vals
+    x = torch.zeros(M, H, dtype=BF16) + big
+    sc = scales[..., None].expand(M, H // group, group).reshape(M, H)
+    return x + decode_stored(stored, bits, sc)
+
+
+# --------------------------------------------------------------------------------------
+# RMSNorm                                         operators/efficient_rmsnorm.py:15-143
+# --------------------------------------------------------------------------------------
+def rmsnorm_fwd(x, w, eps):
+    """fp32 math, one rounding: y = bf16((x * rstd) * w); rstd = 1/sqrt(mean(x^2) + eps).
+    Returns (y in x's dtype, rstd fp32 [M])."""
+    H = x.shape[-1]
+    xf = x.reshape(-1, H).float()
+    var = (xf * xf).sum(dim=-1) / H
+    rstd = 1 / torch.sqrt(var + eps)
+    y = ((xf * rstd[:, None]) * w.float()[None, :]).to(x.dtype)
+    return y.reshape(x.shape), rstd
+
+
+def rmsnorm_bwd(dy, x_hat, w, rstd, c2_quirk=True):
+    """dx = (w*dy - (xn*c1 + c2)) * rstd with xn = x_hat*rstd, c1 = mean(xn*w*dy),
+    c2 = mean(w*dy) (the reference keeps this LayerNorm term, :102-104; c2_quirk=False drops
+    it, which is the true RMSNorm gradient).  dw = sum_rows dy*xn, accumulated in fp32 (the
+    reference accumulates partials in a bf16 buffer in lock order, :107-119, so its dw is a
+    noisier evaluation of the same sum).  Returns (dx bf16, dw in w's dtype)."""
+    H = x_hat.shape[-1]
+    xf = x_hat.reshape(-1, H).float()
+    g = dy.reshape(-1, H).to(BF16).float()
+    xn = xf * rstd[:, None]
+    wdy = w.float()[None, :] * g
+    c1 = (xn * wdy).sum(dim=-1, keepdim=True) / H
+    c2 = wdy.sum(dim=-1, keepdim=True) / H if c2_quirk else 0.
+    dx = ((wdy - (xn * c1 + c2)) * rstd[:, None]).to(BF16).reshape(dy.shape)
+    dw = (g * xn).sum(dim=0).to(w.dtype)
+    return dx, dw
+
+
+# --------------------------------------------------------------------------------------
+# activation / elementwise backward (bf16 op-by-op, as torch evaluates the expressions)
+# --------------------------------------------------------------------------------------
+def silu_bwd(x_hat, g):
+    """operators/efficient_silu.py:50-51"""
+    s = torch.sigmoid(x_hat)
+    return s * (1 + x_hat - x_hat * s) * g
+
+
+def gelu_bwd(x_hat, g):
+    """tanh-form derivative, operators/efficient_gelu.py:49-62"""
+    gamma = math.sqrt(2 / math.pi)
+    kappa = 0.044715
+    inner = gamma * (x_hat + kappa * x_hat ** 3)
+    t = torch.tanh(inner)
+    return 0.5 * ((1 + t) + x_hat * ((1 - t ** 2) * gamma * (1 + 3 * kappa * x_hat ** 2))) * g
+
+
+def hadamard_bwd(x1_hat, x2_hat, g):
+    """operators/efficient_hadamard.py:62-66"""
+    return g * x2_hat, x1_hat * g
+
+
+def softmax_bwd(y_hat, g):
+    """operators/efficient_softmax.py:37-45"""
+    return (g - (g * y_hat).sum(dim=-1, keepdims=True)) * y_hat
+
+
+# --------------------------------------------------------------------------------------
+# linear                                          operators/efficient_linear.py:56-83
+# --------------------------------------------------------------------------------------
+def linear_bwd(dy, x_hat, w, use_bias=False):
+    """dX = dY @ W; dW = sum_b dY[b]^T @ x_hat[b] (the reference forms [B,out,in] in bf16 and
+    autograd sum-reduces it over B); db = sum over every leading dim of dY.
+    Returns (dX bf16, dW_literal bf16, dW_fp32 (single rounding-free reference), db or None)."""
+    g = dy.to(w.dtype)
+    dX = g @ w
+    g2 = g.to(x_hat.dtype)
+    per_batch = g2.transpose(-2, -1) @ x_hat
+    dW_lit = per_batch.sum(0) if per_batch.dim() == 3 else per_batch
+    out_f = dy.shape[-1]
+    dW_f32 = g2.reshape(-1, out_f).float().t() @ x_hat.reshape(-1, x_hat.shape[-1]).float()
+    db = g2.reshape(-1, out_f).float().sum(0).to(w.dtype) if use_bias else None
+    return dX, dW_lit, dW_f32, db

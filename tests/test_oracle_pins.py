@@ -1,0 +1,274 @@
+"""Independent pins for the CPU oracle: brute force, exact arithmetic, closed forms and torch.autograd.
+None of these re-type the oracle's own formula with the same library calls."""
+from fractions import Fraction
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import bf16_ulp_diff, bits_equal
+from oracle import hyc_oracle as O
+
+
+# ------------------------------------------------------------------ pack / unpack
+@pytest.mark.parametrize("bits", [1, 2, 4])
+@pytest.mark.parametrize("H", [8, 16, 64])
+def test_pack_layout_bruteforce(bits, H):
+    n = 8 // bits
+    seg = H // n
+    rng = np.random.default_rng(bits * 100 + H)
+    codes = rng.integers(0, 2 ** bits, size=(5, H), dtype=np.uint8)
+    packed = O.pack_codes(torch.from_numpy(codes), bits).numpy()
+    assert packed.shape == (5, seg) and packed.dtype == np.uint8
+    for r in range(5):
+        for j in range(seg):
+            want = 0
+            for i in range(n):
+                want |= int(codes[r, j + i * seg]) << (i * bits)
+            assert packed[r, j] == want
+    back = O.unpack_codes(torch.from_numpy(packed), bits).numpy()
+    assert np.array_equal(back, codes)
+
+
+@pytest.mark.parametrize("bits", [1, 2, 4])
+def test_unpack_every_byte(bits):
+    n = 8 // bits
+    allb = torch.arange(256, dtype=torch.uint8)[None, :]
+    u = O.unpack_codes(allb, bits).numpy()[0]
+    for v in range(256):
+        for i in range(n):
+            assert u[i * 256 + v] == (v >> (i * bits)) & (2 ** bits - 1)
+
+
+# ------------------------------------------------------------------ quantise
+def _all_finite_bf16():
+    pat = np.arange(65536, dtype=np.uint32)
+    exp = (pat >> 7) & 0xFF
+    pat = pat[exp != 0xFF]
+    return pat
+
+
+def _bf16_to_f32(pat):
+    return (pat.astype(np.uint32) << 16).view(np.float32)
+
+
+def _f32_to_bf16_rne(f):
+    b = f.view(np.uint32).astype(np.uint64)
+    b = (b + 0x7FFF + ((b >> 16) & 1)) >> 16
+    return b.astype(np.uint32)
+
+
+@pytest.mark.parametrize("bits", [1, 2, 4, 8])
+def test_quantize_exhaustive_numpy(bits):
+    """every finite bf16 x against a handful of scales; model = IEEE fp32 divide (numpy), RNE to bf16
+    by integer arithmetic, rint half-even, clip."""
+    pat = _all_finite_bf16()
+    x = _bf16_to_f32(pat)
+    off = 2 ** (bits - 1)
+    for s_pat in (0x3F80, 0x3E1A, 0x3DCD, 0x4049, 0x3C03, 0x0080, 0x7F00):
+        s = _bf16_to_f32(np.array([s_pat], dtype=np.uint32))
+        with np.errstate(over="ignore"):
+            q32 = (x / s).astype(np.float32)
+        qb = _bf16_to_f32(_f32_to_bf16_rne(q32))
+        want = np.clip(np.rint(qb), -off, off - 1)
+        xt = torch.from_numpy(pat.astype(np.uint16).view(np.int16).copy()).view(torch.bfloat16)
+        st = torch.from_numpy(np.array([s_pat], dtype=np.uint16).view(np.int16).copy()).view(torch.bfloat16)
+        got = O.quantize_q(xt, st, bits).float().numpy()
+        assert np.array_equal(got, want), hex(s_pat)
+
+
+def test_quantize_exact_rationals():
+    """a random subset against exact rational arithmetic (two roundings: to fp32, then to bf16)."""
+    rng = np.random.default_rng(7)
+    pat = _all_finite_bf16()
+    pick = rng.choice(pat, size=1500, replace=False)
+    s_pats = [0x3E1A, 0x3DCD, 0x3F00, 0x3E99]
+
+    def rne(fr, mant_bits):
+        if fr == 0:
+            return Fraction(0)
+        sign = -1 if fr < 0 else 1
+        a = abs(fr)
+        e = 0
+        while a >= 2:
+            a /= 2; e += 1
+        while a < 1:
+            a *= 2; e -= 1
+        scaled = a * (1 << mant_bits)
+        fl = scaled.numerator // scaled.denominator
+        rem = scaled - fl
+        if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and fl % 2 == 1):
+            fl += 1
+        return sign * Fraction(fl, 1 << mant_bits) * (Fraction(2) ** e)
+
+    for sp in s_pats:
+        s = Fraction(float(_bf16_to_f32(np.array([sp], dtype=np.uint32))[0]))
+        for p in pick:
+            xv = float(_bf16_to_f32(np.array([p], dtype=np.uint32))[0])
+            if abs(xv) < 1e-30 and xv != 0:
+                continue                                   # keep clear of the subnormal range of the model
+            q = rne(rne(Fraction(xv) / s, 23), 7)
+            fl = q.numerator // q.denominator
+            rem = q - fl
+            r = fl + 1 if (rem > Fraction(1, 2) or (rem == Fraction(1, 2) and fl % 2 == 1)) else fl
+            want = max(-8, min(7, r))
+            xt = torch.tensor([xv]).bfloat16()
+            st = torch.tensor([float(s)]).bfloat16()
+            assert float(O.quantize_q(xt, st, 4)[0]) == want
+
+
+def test_threshold_is_rounded_to_bf16():
+    """the strict compare happens in bf16: an element equal to bf16(thr) is not an outlier."""
+    thr = torch.tensor(0.7123)
+    x = torch.tensor([[[0.7109375, 0.71484375, -0.71484375, 0.1]]]).bfloat16()
+    L, R = torch.zeros(1, 16).bfloat16(), torch.zeros(16, 4).bfloat16()
+    coo, stored, _ = O.ref_compress(x, thr, torch.tensor(0.25).bfloat16(), 4, 1.0, L, R)
+    assert coo.coalesce().indices()[2].tolist() == [1, 2]
+
+
+# ------------------------------------------------------------------ hyc mode
+def test_select_channels_bruteforce():
+    rng = np.random.default_rng(3)
+    scores = rng.integers(0, 6, size=40).astype(np.float32)         # many ties
+    for k in (0, 1, 5, 17, 40):
+        got = O.hyc_select_channels(torch.from_numpy(scores), k).tolist()
+        order = sorted(range(40), key=lambda c: (-scores[c], c))[:k]
+        assert got == sorted(order)
+
+
+@pytest.mark.parametrize("bits,group", [(4, 128), (2, 64), (8, 32), (1, 64)])
+def test_hyc_invariants(bits, group):
+    gen = torch.Generator().manual_seed(bits)
+    M, H = 24, 512
+    x = torch.randn(M, H, generator=gen)
+    hot = torch.randperm(H, generator=gen)[:5]
+    x[:, hot] *= 40
+    x = x.bfloat16()
+    k = O.hyc_num_outlier_channels(H, 0.01)
+    idx = O.hyc_select_channels(O.hyc_channel_scores(x), k)
+    assert sorted(idx.tolist()) == sorted(hot.tolist())
+    vals, stored, scales = O.hyc_compress(x, idx, bits, group)
+    assert bits_equal(vals, x[:, idx.long()])
+    xh = O.hyc_decompress(vals, stored, idx, scales, bits, group)
+    # outlier channels come back verbatim
+    assert bits_equal(xh[:, idx.long()], x[:, idx.long()])
+    # everything else: within half a step unless clamped at the top code
+    keep = torch.ones(H, dtype=torch.bool); keep[idx.long()] = False
+    sc = scales[..., None].expand(M, H // group, group).reshape(M, H).float()
+    off = 2 ** (bits - 1)
+    err = (xh.float() - x.float()).abs()
+    q_unclamped = torch.round(x.float() / sc)
+    ok = (q_unclamped >= -off) & (q_unclamped <= off - 1) & keep[None, :]
+    # half a step, plus the bf16 roundings of x/scale and of code*scale (each <= |q| * 2^-8 steps)
+    assert torch.all(err[ok] <= sc[ok] * (0.5 + off * 2 ** -7) + 1e-30)
+
+
+def test_ref_static_scale_idempotent():
+    """with a static scale, compressing a decompressed tensor reproduces the same codes."""
+    gen = torch.Generator().manual_seed(11)
+    x = torch.randn(1, 16, 64, generator=gen).bfloat16()
+    L, R = torch.zeros(16, 16).bfloat16(), torch.zeros(16, 64).bfloat16()
+    thr = torch.tensor(2.5)
+    for bits in (2, 4, 8):
+        scale = torch.tensor(6.0 / (2 ** bits - 1)).bfloat16()
+        coo, stored, _ = O.ref_compress(x, thr, scale, bits, 1.0, L, R)
+        xh = O.ref_decompress(coo, stored, bits, scale, L=L, R=R)
+        coo2, stored2, _ = O.ref_compress(xh, thr, scale, bits, 1.0, L, R)
+        assert torch.equal(stored, stored2)
+        assert torch.equal(coo.coalesce().indices(), coo2.coalesce().indices())
+
+
+def test_hyc_constant_group_is_defined():
+    x = torch.zeros(2, 256).bfloat16()
+    x[0, :128] = 3.0
+    idx = torch.tensor([], dtype=torch.int32)
+    vals, stored, scales = O.hyc_compress(x, idx, 4, 128)
+    assert torch.all(scales == 0)
+    assert torch.all(O.unpack_codes(stored, 4) == 8)
+    assert torch.all(O.hyc_decompress(vals, stored, idx, scales, 4, 128) == 0)
+
+
+# ------------------------------------------------------------------ RMSNorm
+def test_rmsnorm_fwd_closed_form():
+    gen = torch.Generator().manual_seed(0)
+    x = torch.randn(6, 256, generator=gen).bfloat16()
+    w = (1 + 0.1 * torch.randn(256, generator=gen))
+    y, rstd = O.rmsnorm_fwd(x, w, 1e-6)
+    xd = x.double()
+    want_rstd = 1 / torch.sqrt((xd ** 2).mean(-1) + 1e-6)
+    assert torch.allclose(rstd.double(), want_rstd, rtol=1e-6)
+    want = (xd * want_rstd[:, None] * w.double()).bfloat16()
+    assert bf16_ulp_diff(y, want).max() <= 1
+    # constant row: y = sign * w / sqrt(1 + eps/c^2)
+    xc = torch.full((1, 64), 2.0).bfloat16()
+    yc, rc = O.rmsnorm_fwd(xc, torch.ones(64), 0.0)
+    assert torch.all(yc == 1) and abs(float(rc[0]) - 0.5) < 1e-7
+
+
+@pytest.mark.parametrize("quirk", [True, False])
+def test_rmsnorm_bwd_autograd(quirk):
+    gen = torch.Generator().manual_seed(1)
+    M, H = 8, 128
+    xh = torch.randn(M, H, generator=gen).bfloat16()
+    w = (1 + 0.1 * torch.randn(H, generator=gen))
+    dy = (0.02 * torch.randn(M, H, generator=gen)).bfloat16()
+    _, rstd = O.rmsnorm_fwd(xh, w, 1e-6)
+    dx, dw = O.rmsnorm_bwd(dy, xh, w, rstd, c2_quirk=quirk)
+    xa = xh.double().requires_grad_(True)
+    wa = w.double().requires_grad_(True)
+    ya = xa * torch.rsqrt((xa ** 2).mean(-1, keepdim=True) + 1e-6) * wa
+    ya.backward(dy.double())
+    want_dx = xa.grad
+    if quirk:   # the reference's extra LayerNorm term: - mean(w*dy) * rstd
+        want_dx = want_dx - (wa.detach() * dy.double()).mean(-1, keepdim=True) * rstd.double()[:, None]
+    assert torch.allclose(dx.double(), want_dx, rtol=1e-2, atol=1e-5)
+    assert torch.allclose(dw.double(), wa.grad, rtol=1e-4, atol=1e-6)
+
+
+# ------------------------------------------------------------------ activation backward
+def _grad_of(fn, x, g):
+    xa = x.double().requires_grad_(True)
+    fn(xa).backward(g.double())
+    return xa.grad
+
+
+def test_silu_gelu_softmax_hadamard_bwd_identities():
+    gen = torch.Generator().manual_seed(2)
+    x = (2 * torch.randn(64, 128, generator=gen)).bfloat16()
+    g = (0.1 * torch.randn(64, 128, generator=gen)).bfloat16()
+    F = torch.nn.functional
+    assert torch.allclose(O.silu_bwd(x, g).double(), _grad_of(F.silu, x, g), rtol=3e-2, atol=2e-3)
+    assert torch.allclose(O.gelu_bwd(x, g).double(), _grad_of(lambda t: F.gelu(t, approximate="tanh"), x, g),
+                          rtol=5e-2, atol=3e-3)
+    y = torch.softmax(x.float(), -1).bfloat16()
+    ya = x.double().requires_grad_(True)
+    torch.softmax(ya, -1).backward(g.double())
+    assert torch.allclose(O.softmax_bwd(y, g).double(), ya.grad, rtol=5e-2, atol=2e-4)
+    d1, d2 = O.hadamard_bwd(x, y, g)
+    assert bits_equal(d1, g * y) and bits_equal(d2, x * g)
+
+
+def test_linear_bwd_autograd():
+    gen = torch.Generator().manual_seed(4)
+    xh = torch.randn(2, 16, 64, generator=gen).bfloat16()
+    w = (0.05 * torch.randn(8, 64, generator=gen)).bfloat16()
+    dy = (0.1 * torch.randn(2, 16, 8, generator=gen)).bfloat16()
+    dX, dW_lit, dW_f32, db = O.linear_bwd(dy, xh, w, use_bias=True)
+    xa, wa = xh.double().requires_grad_(True), w.double().requires_grad_(True)
+    ba = torch.zeros(8, dtype=torch.double, requires_grad=True)
+    torch.nn.functional.linear(xa, wa, ba).backward(dy.double())
+    assert torch.allclose(dX.double(), xa.grad, rtol=2e-2, atol=1e-3)
+    assert torch.allclose(dW_f32.double(), wa.grad, rtol=1e-5, atol=1e-6)
+    assert torch.allclose(dW_lit.double(), wa.grad, rtol=2e-2, atol=2e-2)
+    assert torch.allclose(db.double(), ba.grad, rtol=1e-2, atol=1e-2)
+
+
+def test_low_rank_helpers():
+    gen = torch.Generator().manual_seed(5)
+    x = torch.randn(2, 32, 64, generator=gen).bfloat16()
+    l = torch.randn(32, 4, generator=gen).bfloat16()
+    r = torch.randn(4, 64, generator=gen).bfloat16()
+    want = (x.double() - (l.double() @ r.double())[None])
+    assert bf16_ulp_diff(O.low_rank_extraction(l, r, x), want.bfloat16()).max() <= 1
+    want = (x.double() + (l.double() @ r.double())[None])
+    assert bf16_ulp_diff(O.low_rank_addition(l, r, x), want.bfloat16()).max() <= 1
