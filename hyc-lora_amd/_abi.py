@@ -1,0 +1,94 @@
+"""ctypes binding of the C ABI declared in include/hyc_abi.h.
+
+The library is built in-tree by build.py (hipcc, gfx950).  There is no CPU fallback: if the shared
+library is missing, loading fails with an error that says how to build it.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libhyc_gfx950.so")
+
+MODE_CHANNEL, MODE_THRESHOLD, MODE_DENSE = 0, 1, 2
+DTYPE_BF16, DTYPE_F32 = 0, 1
+ACT_SILU, ACT_GELU_TANH = 0, 1
+EINVAL, EFAULT, ENOTSUP, ELAUNCH = -22, -14, -95, -5
+
+c_i32, c_i64, c_f32, c_ptr = ctypes.c_int32, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
+
+
+class HycDesc(ctypes.Structure):
+    """struct hyc_desc"""
+    _fields_ = [
+        ("mode", c_i32), ("bits", c_i32), ("group", c_i32), ("k", c_i32),
+        ("chan_plan", c_ptr),
+        ("threshold", c_f32),
+        ("scale", c_ptr),
+        ("scale_stride_token", c_i64), ("scale_stride_channel", c_i64), ("S", c_i64),
+        ("L", c_ptr), ("R", c_ptr),
+        ("rank", c_i32), ("reserved", c_i32),
+        ("csr_row_ptr", c_ptr), ("csr_cols", c_ptr), ("csr_vals", c_ptr),
+    ]
+
+
+# name -> (restype, argtypes); one line per declaration in include/hyc_abi.h
+SIGNATURES = {
+    "hyc_abi_version": (c_i32, []),
+    "hyc_last_error": (ctypes.c_char_p, []),
+    "hyc_check_shape": (c_i32, [c_i64, c_i32, c_i32, c_i32]),
+    "hyc_stored_row_bytes": (c_i64, [c_i64, c_i32]),
+    "hyc_rmsnorm_bwd_partials": (c_i64, [c_i64, c_i64]),
+    "hyc_channel_absmax": (c_i32, [c_ptr, c_i64, c_i64, c_ptr, c_ptr]),
+    "hyc_select_channels": (c_i32, [c_ptr, c_i64, c_i32, c_ptr, c_ptr, c_ptr]),
+    "hyc_compress": (c_i32, [c_ptr, c_i64, c_i64, ctypes.POINTER(HycDesc), c_ptr, c_ptr, c_ptr, c_ptr, c_ptr]),
+    "hyc_decompress": (c_i32, [c_ptr, c_ptr, c_ptr, c_i64, c_i64, ctypes.POINTER(HycDesc), c_ptr, c_ptr]),
+    "hyc_ref_outlier_count": (c_i32, [c_ptr, c_i64, c_i64, ctypes.POINTER(HycDesc), c_ptr, c_ptr]),
+    "hyc_ref_outlier_fill": (c_i32, [c_ptr, c_i64, c_i64, ctypes.POINTER(HycDesc), c_ptr, c_ptr, c_ptr, c_ptr]),
+    "hyc_rmsnorm_fwd_compress": (c_i32, [c_ptr, c_ptr, c_i32, c_f32, c_i64, c_i64, ctypes.POINTER(HycDesc),
+                                         c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr]),
+    "hyc_rmsnorm_bwd": (c_i32, [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_i32, c_ptr, c_i64, c_i64,
+                                ctypes.POINTER(HycDesc), c_i32, c_ptr, c_ptr, c_ptr, c_ptr]),
+    "hyc_act_bwd": (c_i32, [c_i32, c_ptr, c_ptr, c_ptr, c_ptr, c_i64, c_i64, ctypes.POINTER(HycDesc), c_ptr, c_ptr]),
+    "hyc_hadamard_bwd": (c_i32, [c_ptr, c_ptr, c_ptr, c_ptr, ctypes.POINTER(HycDesc), c_ptr, c_ptr, c_ptr,
+                                 ctypes.POINTER(HycDesc), c_i64, c_i64, c_ptr, c_ptr, c_ptr]),
+}
+
+_lib = None
+
+
+def load():
+    """dlopen the library once and attach the prototypes.  Raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            "HIP library %s is missing: build it with `python hyc-lora_amd/build.py` "
+            "(there is no CPU fallback)" % LIB_PATH)
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)           # AttributeError if a declared symbol is not exported
+        fn.restype = res
+        fn.argtypes = args
+    if lib.hyc_abi_version() != 1:
+        raise RuntimeError("libhyc ABI version %d, expected 1" % lib.hyc_abi_version())
+    _lib = lib
+    return lib
+
+
+class HycError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__("hyc error %d: %s" % (code, msg))
+        self.code = code
+
+
+def check(rc):
+    """raise the Python exception that corresponds to a negative return code"""
+    if rc == 0:
+        return
+    msg = load().hyc_last_error().decode("utf-8", "replace")
+    if rc == ENOTSUP:
+        raise NotImplementedError("hyc: " + msg)
+    if rc in (EINVAL, EFAULT):
+        raise ValueError("hyc: " + msg)
+    raise HycError(rc, msg)

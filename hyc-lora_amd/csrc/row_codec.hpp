@@ -1,0 +1,199 @@
+// Device-side building blocks shared by every kernel of the library (gfx950, wave64).
+//
+// Thread <-> data mapping of one row of H channels at `BITS` bits per code:
+//   the row is cut into NSEG = 8/BITS segments of SEG = H/NSEG channels (the reference's packing,
+//   operators/compress_function.py:175-197).  A segment is CPS = SEG/8 chunks of 8 channels.  In
+//   iteration `it` thread t owns chunk c = it*blockDim.x + t of EVERY segment: NSEG 16-byte loads of
+//   bf16 activations give exactly the 8 packed bytes [8c, 8c+8) of the stored row - one 8-byte store.
+//   A scale group of G channels is G/8 consecutive chunks = G/8 consecutive lanes (LPG), so group
+//   min/max are DPP butterflies inside a 16-lane row and never touch LDS.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace hyc {
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float floatx2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ float bf_lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf_hi(uint32_t w) { return __uint_as_float(w & 0xFFFF0000u); }
+__device__ __forceinline__ float bf_to_f(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
+
+// two floats -> packed bf16 pair, round to nearest even (v_cvt_pk_bf16_f32)
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  floatx2_t v = {lo, hi};
+  bf16x2_t b = __builtin_convertvector(v, bf16x2_t);
+  return __builtin_bit_cast(uint32_t, b);
+}
+__device__ __forceinline__ uint16_t f_to_bf(float f) {
+  __bf16 b = (__bf16)f;
+  return __builtin_bit_cast(uint16_t, b);
+}
+// round an fp32 value to the nearest bf16 and return it as fp32
+__device__ __forceinline__ float bfr(float f) { return (float)((__bf16)f); }
+
+// 8 consecutive bf16 <-> 8 floats
+__device__ __forceinline__ void unpack8(const uint4& r, float (&v)[8]) {
+  v[0] = bf_lo(r.x); v[1] = bf_hi(r.x); v[2] = bf_lo(r.y); v[3] = bf_hi(r.y);
+  v[4] = bf_lo(r.z); v[5] = bf_hi(r.z); v[6] = bf_lo(r.w); v[7] = bf_hi(r.w);
+}
+__device__ __forceinline__ uint4 pack8(const float (&v)[8]) {
+  uint4 r;
+  r.x = pack_bf16(v[0], v[1]); r.y = pack_bf16(v[2], v[3]);
+  r.z = pack_bf16(v[4], v[5]); r.w = pack_bf16(v[6], v[7]);
+  return r;
+}
+
+// ---- cross-lane -------------------------------------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
+}
+__device__ __forceinline__ float xor_lane(float v, int m) { return __shfl_xor(v, m, 64); }
+
+// butterfly over LPG consecutive lanes (LPG a power of two <= 64); every lane of the group gets the result.
+// Must be executed by all lanes of the wave (callers feed neutral values from lanes without data).
+template <int LPG, typename Op>
+__device__ __forceinline__ float group_reduce(float v, Op op) {
+  if (LPG >= 2) v = op(v, dpp_f<0xB1>(v));   // quad_perm [1,0,3,2]
+  if (LPG >= 4) v = op(v, dpp_f<0x4E>(v));   // quad_perm [2,3,0,1]
+  if (LPG >= 8) v = op(v, dpp_f<0x141>(v));  // row_half_mirror
+  if (LPG >= 16) v = op(v, dpp_f<0x140>(v)); // row_mirror
+  if (LPG >= 32) v = op(v, xor_lane(v, 16));
+  if (LPG >= 64) v = op(v, xor_lane(v, 32));
+  return v;
+}
+// runtime-width variant (lpg in {4, 8, 16, 32, 64}; the branches are uniform)
+template <typename Op>
+__device__ __forceinline__ float group_reduce_rt(float v, int lpg, Op op) {
+  v = op(v, dpp_f<0xB1>(v));
+  v = op(v, dpp_f<0x4E>(v));
+  if (lpg >= 8) v = op(v, dpp_f<0x141>(v));
+  if (lpg >= 16) v = op(v, dpp_f<0x140>(v));
+  if (lpg >= 32) v = op(v, xor_lane(v, 16));
+  if (lpg >= 64) v = op(v, xor_lane(v, 32));
+  return v;
+}
+struct OpMax { __device__ __forceinline__ float operator()(float a, float b) const { return a > b ? a : b; } };
+struct OpMin { __device__ __forceinline__ float operator()(float a, float b) const { return a < b ? a : b; } };
+struct OpAdd { __device__ __forceinline__ float operator()(float a, float b) const { return a + b; } };
+
+__device__ __forceinline__ float wave_sum(float v) { return group_reduce<64>(v, OpAdd()); }
+
+// sum over the whole workgroup; `red` is LDS scratch of >= 16 floats per reduction slot.
+// All threads return the total.  Contains two barriers.
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+  if ((threadIdx.x & 63) == 0) red[wave] = v;
+  __syncthreads();
+  float t = 0.f;
+  for (int i = 0; i < nw; ++i) t += red[i];
+  __syncthreads();
+  return t;
+}
+
+// ---- quantise one chunk -------------------------------------------------------------------------
+template <int BITS>
+struct Q {
+  static constexpr int NSEG = 8 / BITS;
+  static constexpr int OFF = 1 << (BITS - 1);
+  static constexpr float LO = -(float)OFF;
+  static constexpr float HI = (float)(OFF - 1);
+  static constexpr float INV_LEVELS = 1.0f / (float)((1 << BITS) - 1);
+  static constexpr uint32_t CODE_MASK = (1u << BITS) - 1;
+};
+
+// reciprocal used for q = bf16(x / s).  For bf16 x and s in the normal range the exact quotient is a
+// ratio of two integers below 256, which can never sit closer than 2^-17 (relative) to a bf16
+// rounding boundary, so bf16(x * fl(1/s)) equals bf16(fl(x / s)); outside that range fall back to the
+// IEEE division (`exact` = true).
+struct Recip {
+  float r;
+  float s;
+  bool exact;
+};
+__device__ __forceinline__ Recip make_recip(float s) {
+  Recip k;
+  k.s = s;
+  k.exact = !(s > 1e-30f && s < 1e30f);   // also true for negative, zero, NaN scales
+  k.r = 1.0f / s;
+  return k;
+}
+// signed code q (as float, already clamped) of one element.  x / 0 = +-inf clamps like any large quotient;
+// 0 / 0 = NaN, whose integer cast the reference leaves undefined, is given q = 0 (code = offset).
+template <int BITS>
+__device__ __forceinline__ float quant1(float x, const Recip& k) {
+  float t = k.exact ? (x / k.s) : (x * k.r);
+  t = __builtin_rintf(bfr(t));
+  t = (t != t) ? 0.f : t;
+  return __builtin_fminf(__builtin_fmaxf(t, Q<BITS>::LO), Q<BITS>::HI);
+}
+
+// 8 signed codes -> OR into the packed 8-byte word at bit field `seg`
+template <int BITS>
+__device__ __forceinline__ void put_codes(const float (&q)[8], int seg, uint32_t& lo, uint32_t& hi) {
+  if (BITS == 8) {
+    lo = ((uint32_t)(int)q[0] & 0xFF) | (((uint32_t)(int)q[1] & 0xFF) << 8) | (((uint32_t)(int)q[2] & 0xFF) << 16) |
+         (((uint32_t)(int)q[3] & 0xFF) << 24);
+    hi = ((uint32_t)(int)q[4] & 0xFF) | (((uint32_t)(int)q[5] & 0xFF) << 8) | (((uint32_t)(int)q[6] & 0xFF) << 16) |
+         (((uint32_t)(int)q[7] & 0xFF) << 24);
+  } else {
+    const int sh = seg * BITS;
+    uint32_t a = (uint32_t)((int)q[0] + Q<BITS>::OFF) | ((uint32_t)((int)q[1] + Q<BITS>::OFF) << 8) |
+                 ((uint32_t)((int)q[2] + Q<BITS>::OFF) << 16) | ((uint32_t)((int)q[3] + Q<BITS>::OFF) << 24);
+    uint32_t b = (uint32_t)((int)q[4] + Q<BITS>::OFF) | ((uint32_t)((int)q[5] + Q<BITS>::OFF) << 8) |
+                 ((uint32_t)((int)q[6] + Q<BITS>::OFF) << 16) | ((uint32_t)((int)q[7] + Q<BITS>::OFF) << 24);
+    lo |= a << sh;
+    hi |= b << sh;
+  }
+}
+
+// signed value (code - offset, or the int8 itself) of element j of segment `seg` in a packed word
+template <int BITS>
+__device__ __forceinline__ float get_code(uint32_t lo, uint32_t hi, int seg, int j) {
+  const uint32_t w = (j < 4) ? lo : hi;
+  const int byte = (int)((w >> ((j & 3) * 8)) & 0xFF);
+  if (BITS == 8) return (float)(int)(int8_t)byte;
+  return (float)((int)((byte >> (seg * BITS)) & Q<BITS>::CODE_MASK) - Q<BITS>::OFF);
+}
+
+// ---- descriptors as the kernels see them -------------------------------------------------------
+struct ChanArgs {           // HYC_MODE_CHANNEL
+  const uint32_t* plan;     // [H/8]
+  int k;                    // outlier channels
+  int groups_per_row;       // H / G
+  int chunk_to_group_shift; // log2(G/8)
+};
+
+struct ThrArgs {            // HYC_MODE_THRESHOLD
+  float thr;                // already a bf16 value
+  const uint16_t* scale;
+  int64_t sst, ssc;         // scale strides (token, channel)
+  int64_t S;
+  const uint16_t* L;        // [S, rank]
+  const uint16_t* R;        // [rank, H]
+  int rank;
+  const int32_t* row_ptr;
+  const int32_t* cols;
+  const uint16_t* vals;
+};
+
+// base[c..c+8) = bf16(sum_r L[s,r] * R[r,c]) accumulated in fp32 in increasing r
+__device__ __forceinline__ void base8(const ThrArgs& a, int64_t s, int64_t col, int64_t H, float (&b)[8]) {
+#pragma unroll
+  for (int j = 0; j < 8; ++j) b[j] = 0.f;
+  for (int r = 0; r < a.rank; ++r) {
+    const float l = bf_to_f(a.L[s * a.rank + r]);
+    const uint4 rr = *reinterpret_cast<const uint4*>(a.R + (int64_t)r * H + col);
+    float rv[8];
+    unpack8(rr, rv);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) b[j] = __builtin_fmaf(l, rv[j], b[j]);
+  }
+#pragma unroll
+  for (int j = 0; j < 8; ++j) b[j] = bfr(b[j]);
+}
+
+}  // namespace hyc

@@ -1,0 +1,341 @@
+"""Host-side launchers: torch tensors in, torch tensors out, every computation done by the HIP library.
+
+torch is used for device memory and the current stream only.  Nothing here computes on the CPU and
+nothing falls back to torch ops for the hot path: inputs that are not CUDA tensors raise.
+"""
+import ctypes
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+
+from . import _abi
+from ._abi import HycDesc, check
+
+BF16 = torch.bfloat16
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _p(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _need(t, dtype, name):
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise ValueError("%s must be a CUDA (ROCm) tensor: the hot path runs on the GPU only" % name)
+    if t.dtype != dtype:
+        raise ValueError("%s must be %s, got %s" % (name, dtype, t.dtype))
+    if not t.is_contiguous():
+        raise ValueError("%s must be contiguous" % name)
+    return t
+
+
+def num_outlier_channels(H, ratio):
+    """k = floor(ratio*H + 1/2)"""
+    import math
+    return int(math.floor(ratio * H + 0.5))
+
+
+# ----------------------------------------------------------------------------------------------------
+# channel mode
+# ----------------------------------------------------------------------------------------------------
+@dataclass
+class ChannelPlan:
+    """the static outlier-channel set of one activation site"""
+    H: int
+    k: int
+    idx: torch.Tensor    # int32 [k], ascending
+    plan: torch.Tensor   # int32 [H/8] (bit pattern of the uint32 lookup words)
+
+
+def channel_absmax(x2d, amax=None):
+    """running per-channel max |x| (fp32 [H]); pass the previous result to accumulate"""
+    _need(x2d, BF16, "x")
+    M, H = x2d.shape
+    if amax is None:
+        amax = torch.zeros(H, dtype=torch.float32, device=x2d.device)
+    check(_abi.load().hyc_channel_absmax(_p(x2d), M, H, _p(amax), _stream()))
+    return amax
+
+
+def select_channels(amax, k):
+    _need(amax, torch.float32, "amax")
+    H = amax.numel()
+    idx = torch.empty(max(k, 1), dtype=torch.int32, device=amax.device)[:k]
+    plan = torch.empty(H // 8, dtype=torch.int32, device=amax.device)
+    check(_abi.load().hyc_select_channels(_p(amax), H, k, _p(idx), _p(plan), _stream()))
+    return ChannelPlan(H, k, idx, plan)
+
+
+def channel_desc(plan: ChannelPlan, bits, group):
+    d = HycDesc()
+    d.mode, d.bits, d.group, d.k = _abi.MODE_CHANNEL, bits, group, plan.k
+    d.chan_plan = plan.plan.data_ptr()
+    return d
+
+
+def dense_desc(bits=4):
+    d = HycDesc()
+    d.mode, d.bits = _abi.MODE_DENSE, bits
+    return d
+
+
+@dataclass
+class ChannelCompressed:
+    """a [M,H] bf16 activation held as codes + outlier channels + group scales"""
+    stored: torch.Tensor   # uint8 [M, H*bits/8] (int8 [M,H] for 8 bits)
+    vals: torch.Tensor     # bf16 [M, k]
+    scales: torch.Tensor   # bf16 [M, H/group]
+    plan: ChannelPlan
+    bits: int
+    group: int
+    M: int
+    H: int
+
+    def desc(self):
+        return channel_desc(self.plan, self.bits, self.group)
+
+    def nbytes(self):
+        return self.stored.numel() * self.stored.element_size() + 2 * self.vals.numel() + 2 * self.scales.numel()
+
+
+def alloc_channel(M, H, plan, bits, group, device):
+    stored = torch.empty((M, H * bits // 8), dtype=torch.int8 if bits == 8 else torch.uint8, device=device)
+    vals = torch.empty((M, plan.k), dtype=BF16, device=device)
+    scales = torch.empty((M, H // group), dtype=BF16, device=device)
+    return ChannelCompressed(stored, vals, scales, plan, bits, group, M, H)
+
+
+def compress_channel(x2d, plan, bits, group):
+    _need(x2d, BF16, "x")
+    M, H = x2d.shape
+    lib = _abi.load()
+    check(lib.hyc_check_shape(H, bits, group, _abi.MODE_CHANNEL))
+    out = alloc_channel(M, H, plan, bits, group, x2d.device)
+    d = out.desc()
+    check(lib.hyc_compress(_p(x2d), M, H, ctypes.byref(d), _p(out.stored), _p(out.vals), _p(out.scales), None, _stream()))
+    return out
+
+
+def decompress_channel(c: ChannelCompressed):
+    xhat = torch.empty((c.M, c.H), dtype=BF16, device=c.stored.device)
+    d = c.desc()
+    check(_abi.load().hyc_decompress(_p(c.stored), _p(c.vals), _p(c.scales), c.M, c.H, ctypes.byref(d), _p(xhat), _stream()))
+    return xhat
+
+
+# ----------------------------------------------------------------------------------------------------
+# threshold mode (the scheme of the reference snapshot)
+# ----------------------------------------------------------------------------------------------------
+def scale_strides(scale, S, H):
+    """(stride_token, stride_channel) of a per-tensor [] / per-channel [1,H] / per-token [S,1] scale"""
+    n = scale.numel()
+    if n == 1:
+        return 0, 0
+    if scale.dim() >= 2 and scale.shape[-1] == H and n == H:
+        return 0, 1
+    if scale.dim() >= 2 and scale.shape[-1] == 1 and n == S:
+        return 1, 0
+    raise ValueError("scale of shape %s is neither per-tensor, per-channel [1,%d] nor per-token [%d,1]"
+                     % (tuple(scale.shape), H, S))
+
+
+@dataclass
+class ThresholdCompressed:
+    stored: torch.Tensor               # uint8 [M, H*bits/8] / int8 [M,H]
+    row_ptr: torch.Tensor              # int32 [M+1]
+    cols: torch.Tensor                 # int32 [nnz]
+    vals: torch.Tensor                 # bf16 [nnz]
+    threshold: float
+    scale: torch.Tensor
+    L: Optional[torch.Tensor]
+    R: Optional[torch.Tensor]
+    bits: int
+    M: int
+    H: int
+    S: int
+
+    def desc(self):
+        return threshold_desc(self.threshold, self.scale, self.bits, self.S, self.H, self.L, self.R,
+                              self.row_ptr, self.cols, self.vals)
+
+
+def threshold_desc(threshold, scale, bits, S, H, L=None, R=None, row_ptr=None, cols=None, vals=None):
+    d = HycDesc()
+    d.mode, d.bits = _abi.MODE_THRESHOLD, bits
+    d.threshold = float(threshold)
+    d.scale = scale.data_ptr()
+    d.scale_stride_token, d.scale_stride_channel = scale_strides(scale, S, H)
+    d.S = S
+    rank = 0 if L is None else L.shape[-1]
+    d.rank = rank
+    if rank:
+        d.L, d.R = L.data_ptr(), R.data_ptr()
+    if row_ptr is not None:
+        d.csr_row_ptr = row_ptr.data_ptr()
+        d.csr_cols = cols.data_ptr() if cols.numel() else None
+        d.csr_vals = vals.data_ptr() if vals.numel() else None
+    return d
+
+
+def fit_rows(L, S):
+    """pad with zero rows / cut L [S', r] to S rows (the reference's pad_cut_L); L is tiny"""
+    have = L.shape[0]
+    if have == S:
+        return L.contiguous()
+    if have > S:
+        return L[:S].contiguous()
+    out = torch.zeros((S, L.shape[1]), dtype=L.dtype, device=L.device)
+    out[:have] = L
+    return out
+
+
+def compress_threshold(x2d, S, threshold, scale, bits, L=None, R=None):
+    """codes + CSR outliers of x [M,H] (row m is sequence position m mod S).  One host read-back
+    (the outlier total) sizes the CSR arrays, as `.to_sparse()` does in the reference."""
+    _need(x2d, BF16, "x")
+    _need(scale, BF16, "scale")
+    M, H = x2d.shape
+    lib = _abi.load()
+    check(lib.hyc_check_shape(H, bits, 0, _abi.MODE_THRESHOLD))
+    dev = x2d.device
+    if L is not None:
+        L = fit_rows(_need(L, BF16, "L"), S)
+        _need(R, BF16, "R")
+    stored = torch.empty((M, H * bits // 8), dtype=torch.int8 if bits == 8 else torch.uint8, device=dev)
+    counts = torch.empty(M, dtype=torch.int32, device=dev)
+    d = threshold_desc(threshold, scale, bits, S, H, L, R)
+    check(lib.hyc_compress(_p(x2d), M, H, ctypes.byref(d), _p(stored), None, None, _p(counts), _stream()))
+    row_ptr = torch.zeros(M + 1, dtype=torch.int32, device=dev)
+    torch.cumsum(counts, 0, out=row_ptr[1:])
+    nnz = int(row_ptr[-1].item())
+    cols = torch.empty(nnz, dtype=torch.int32, device=dev)
+    vals = torch.empty(nnz, dtype=BF16, device=dev)
+    check(lib.hyc_ref_outlier_fill(_p(x2d), M, H, ctypes.byref(d), _p(row_ptr), _p(cols) if nnz else None,
+                                   _p(vals) if nnz else None, _stream()))
+    return ThresholdCompressed(stored, row_ptr, cols, vals, float(threshold), scale, L, R, bits, M, H, S)
+
+
+def outlier_counts(x2d, S, threshold, bits=8, L=None, R=None):
+    _need(x2d, BF16, "x")
+    M, H = x2d.shape
+    counts = torch.empty(M, dtype=torch.int32, device=x2d.device)
+    one = torch.ones(1, dtype=BF16, device=x2d.device)
+    if L is not None:
+        L = fit_rows(L, S)
+    d = threshold_desc(threshold, one, bits, S, H, L, R)
+    check(_abi.load().hyc_ref_outlier_count(_p(x2d), M, H, ctypes.byref(d), _p(counts), _stream()))
+    return counts
+
+
+def decompress_threshold(c: ThresholdCompressed):
+    xhat = torch.empty((c.M, c.H), dtype=BF16, device=c.stored.device)
+    d = c.desc()
+    check(_abi.load().hyc_decompress(_p(c.stored), None, None, c.M, c.H, ctypes.byref(d), _p(xhat), _stream()))
+    return xhat
+
+
+# ----------------------------------------------------------------------------------------------------
+# fused operators
+# ----------------------------------------------------------------------------------------------------
+def _wdtype(w):
+    if w.dtype == torch.float32:
+        return _abi.DTYPE_F32
+    if w.dtype == BF16:
+        return _abi.DTYPE_BF16
+    raise ValueError("RMSNorm weight must be bf16 or fp32, got %s" % w.dtype)
+
+
+def rmsnorm_fwd_compress_channel(x2d, w, eps, plan, bits, group):
+    """-> (y bf16 [M,H], rstd fp32 [M], ChannelCompressed of x)"""
+    _need(x2d, BF16, "x")
+    if not (w.is_cuda and w.is_contiguous()):
+        raise ValueError("weight must be a contiguous CUDA tensor")
+    M, H = x2d.shape
+    lib = _abi.load()
+    check(lib.hyc_check_shape(H, bits, group, _abi.MODE_CHANNEL))
+    y = torch.empty_like(x2d)
+    rstd = torch.empty(M, dtype=torch.float32, device=x2d.device)
+    c = alloc_channel(M, H, plan, bits, group, x2d.device)
+    d = c.desc()
+    check(lib.hyc_rmsnorm_fwd_compress(_p(x2d), _p(w), _wdtype(w), float(eps), M, H, ctypes.byref(d), _p(y), _p(rstd),
+                                       _p(c.stored), _p(c.vals), _p(c.scales), None, _stream()))
+    return y, rstd, c
+
+
+def rmsnorm_fwd_compress_threshold(x2d, w, eps, S, threshold, scale, bits, L=None, R=None):
+    """-> (y, rstd, ThresholdCompressed of x)"""
+    _need(x2d, BF16, "x")
+    _need(scale, BF16, "scale")
+    M, H = x2d.shape
+    lib = _abi.load()
+    dev = x2d.device
+    if L is not None:
+        L = fit_rows(_need(L, BF16, "L"), S)
+        _need(R, BF16, "R")
+    y = torch.empty_like(x2d)
+    rstd = torch.empty(M, dtype=torch.float32, device=dev)
+    stored = torch.empty((M, H * bits // 8), dtype=torch.int8 if bits == 8 else torch.uint8, device=dev)
+    counts = torch.empty(M, dtype=torch.int32, device=dev)
+    d = threshold_desc(threshold, scale, bits, S, H, L, R)
+    check(lib.hyc_rmsnorm_fwd_compress(_p(x2d), _p(w), _wdtype(w), float(eps), M, H, ctypes.byref(d), _p(y), _p(rstd),
+                                       _p(stored), None, None, _p(counts), _stream()))
+    row_ptr = torch.zeros(M + 1, dtype=torch.int32, device=dev)
+    torch.cumsum(counts, 0, out=row_ptr[1:])
+    nnz = int(row_ptr[-1].item())
+    cols = torch.empty(nnz, dtype=torch.int32, device=dev)
+    vals = torch.empty(nnz, dtype=BF16, device=dev)
+    check(lib.hyc_ref_outlier_fill(_p(x2d), M, H, ctypes.byref(d), _p(row_ptr), _p(cols) if nnz else None,
+                                   _p(vals) if nnz else None, _stream()))
+    return y, rstd, ThresholdCompressed(stored, row_ptr, cols, vals, float(threshold), scale, L, R, bits, M, H, S)
+
+
+def _source(c):
+    """(stored, vals, scales, desc) of a ChannelCompressed, or of a dense bf16 x_hat"""
+    if isinstance(c, ChannelCompressed):
+        return c.stored, c.vals, c.scales, c.desc()
+    if isinstance(c, ThresholdCompressed):
+        c = decompress_threshold(c)
+    _need(c, BF16, "x_hat")
+    return c, None, None, dense_desc()
+
+
+def rmsnorm_bwd(dy2d, src, w, rstd, c2_quirk=True):
+    """-> (dx bf16 [M,H], dw in w's dtype [H]); src is a ChannelCompressed, ThresholdCompressed or dense x_hat"""
+    _need(dy2d, BF16, "dy")
+    M, H = dy2d.shape
+    lib = _abi.load()
+    stored, vals, scales, d = _source(src)
+    P = lib.hyc_rmsnorm_bwd_partials(M, H)
+    partials = torch.empty((max(P, 1), H), dtype=torch.float32, device=dy2d.device)
+    dx = torch.empty_like(dy2d)
+    dw = torch.empty(H, dtype=w.dtype, device=dy2d.device)
+    check(lib.hyc_rmsnorm_bwd(_p(dy2d), _p(stored), _p(vals), _p(scales), _p(w), _wdtype(w), _p(rstd), M, H,
+                              ctypes.byref(d), 1 if c2_quirk else 0, _p(dx), _p(partials), _p(dw), _stream()))
+    return dx, dw
+
+
+def act_bwd(act, g2d, src):
+    """act in {'silu', 'gelu'} -> dx bf16 [M,H]"""
+    _need(g2d, BF16, "grad_output")
+    M, H = g2d.shape
+    stored, vals, scales, d = _source(src)
+    dx = torch.empty_like(g2d)
+    code = {"silu": _abi.ACT_SILU, "gelu": _abi.ACT_GELU_TANH}[act]
+    check(_abi.load().hyc_act_bwd(code, _p(g2d), _p(stored), _p(vals), _p(scales), M, H, ctypes.byref(d), _p(dx), _stream()))
+    return dx
+
+
+def hadamard_bwd(g2d, src1, src2):
+    """-> (g * x2_hat, x1_hat * g)"""
+    _need(g2d, BF16, "grad_output")
+    M, H = g2d.shape
+    s1, v1, c1, d1 = _source(src1)
+    s2, v2, c2, d2 = _source(src2)
+    dx1, dx2 = torch.empty_like(g2d), torch.empty_like(g2d)
+    check(_abi.load().hyc_hadamard_bwd(_p(g2d), _p(s1), _p(v1), _p(c1), ctypes.byref(d1), _p(s2), _p(v2), _p(c2),
+                                       ctypes.byref(d2), M, H, _p(dx1), _p(dx2), _stream()))
+    return dx1, dx2

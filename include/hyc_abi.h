@@ -1,0 +1,155 @@
+/*
+ * hyc_abi.h - C ABI of the MI355X (gfx950) hybrid activation-compression library.
+ *
+ * Plain pointers and sizes only; every pointer named "device" is HBM memory of the current HIP
+ * device, every entry point is asynchronous on the given stream (a hipStream_t passed as void*,
+ * NULL = the default stream), returns 0 on success or a negative HYC_E* code, never throws,
+ * never synchronises, and never allocates device memory: outputs and workspaces belong to the
+ * caller.  hyc_last_error() returns a thread-local description of the last failure.
+ *
+ * What each entry point stands in for (paths relative to the HyC-LoRA reference checkout):
+ *   hyc_compress / hyc_decompress
+ *       true_divide_outlier_suboutlier_svd_compress / _decompress,
+ *       operators/compress_function.py:136-200 and :203-261
+ *   hyc_ref_outlier_count / hyc_ref_outlier_fill
+ *       the `.to_sparse()` of the element-threshold outliers, operators/compress_function.py:149-156
+ *   hyc_channel_absmax / hyc_select_channels
+ *       the calibration statistics, operators/compress_function.py:292-340 (get_statistics), for the
+ *       channel-structured outlier rule
+ *   hyc_rmsnorm_fwd_compress
+ *       EfficientMemoryRMSNormFunc.forward + _rms_norm_fwd_fused, operators/efficient_rmsnorm.py:147-212, :15-60
+ *   hyc_rmsnorm_bwd
+ *       EfficientMemoryRMSNormFunc.backward + _rms_norm_bwd_dx_fused + _rms_norm_bwd_dwdb,
+ *       operators/efficient_rmsnorm.py:215-269, :63-143
+ *   hyc_act_bwd
+ *       EfficientMemorySiLUFunc.backward operators/efficient_silu.py:44-53,
+ *       EfficientMemoryGELUFunc.backward operators/efficient_gelu.py:44-64,
+ *       EfficientMemoryHadamardFunc.backward operators/efficient_hadamard.py:55-83
+ *   hyc_softmax_fwd_compress / hyc_softmax_bwd
+ *       EfficientMemorySoftmaxFunc operators/efficient_softmax.py:10-45 with
+ *       true_compress_softmax / true_decompress_softmax operators/compress_function.py:264-275
+ *   hyc_gradw_gemm
+ *       grad_weight = grad_output^T @ decompress(x), operators/efficient_linear.py:56-67
+ *   hyc_low_rank_update
+ *       low_rank_extraction / low_rank_addition, operators/fused_compression.py:80-99, :184-210
+ *
+ * Compressed activation of a [M, H] bf16 matrix (M tokens, H channels), `bits` in {1,2,4,8}:
+ *   stored   uint8 [M, H*bits/8]   (bits == 8: int8 [M, H], the signed code itself)
+ *            byte j of a row = sum_i code[j + i*H/n] << (i*bits), n = 8/bits, code = q + 2^(bits-1),
+ *            q = clamp(rint(bf16(x / scale)), -2^(bits-1), 2^(bits-1)-1)   (compress_function.py:170-197)
+ *   HYC_MODE_CHANNEL   k outlier channels kept verbatim: vals bf16 [M, k] (column i = channel idx[i],
+ *            idx ascending); scales bf16 [M, H/group], scale = bf16(bf16(max-min) / (2^bits-1)) over
+ *            the group's channels after the outlier channels were zeroed.
+ *   HYC_MODE_THRESHOLD outliers are the elements with |x - base| > threshold (CSR: row_ptr int32 [M+1],
+ *            cols int32 [nnz] ascending within a row, vals bf16 [nnz]); static scale read through two
+ *            strides (per-tensor 0/0, per-channel 0/1, per-token 1/0) at row (m mod S);
+ *            base = bf16(L[m mod S, :] @ R) with L bf16 [S, rank], R bf16 [rank, H] (rank may be 0).
+ */
+#ifndef HYC_ABI_H
+#define HYC_ABI_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HYC_ABI_VERSION 1
+
+/* error codes (negative errno values) */
+#define HYC_OK 0
+#define HYC_EINVAL (-22)  /* bad shape, misaligned pointer, inconsistent descriptor */
+#define HYC_EFAULT (-14)  /* null pointer where data is required */
+#define HYC_ENOTSUP (-95) /* bits / group / H combination the kernels do not cover */
+#define HYC_ELAUNCH (-5)  /* the HIP runtime refused the launch */
+
+#define HYC_MODE_CHANNEL 0
+#define HYC_MODE_THRESHOLD 1
+#define HYC_MODE_DENSE 2 /* consumers only: `stored` is the already decompressed bf16 [M,H] */
+
+#define HYC_DTYPE_BF16 0
+#define HYC_DTYPE_F32 1
+
+#define HYC_ACT_SILU 0
+#define HYC_ACT_GELU_TANH 1
+
+typedef struct hyc_desc {
+  int32_t mode;  /* HYC_MODE_* */
+  int32_t bits;  /* 1, 2, 4, 8 */
+  /* ---- HYC_MODE_CHANNEL ---- */
+  int32_t group; /* channels per scale group */
+  int32_t k;     /* number of outlier channels (may be 0) */
+  const uint32_t* chan_plan; /* device [H/8]: bits 0-7 = outlier mask of channels 8c..8c+7,
+                                bits 16-31 = number of outlier channels below 8c; from hyc_select_channels */
+  /* ---- HYC_MODE_THRESHOLD ---- */
+  float threshold;            /* compared as bf16: the library rounds it to bf16 (nearest even) */
+  const void* scale;          /* device bf16 */
+  int64_t scale_stride_token; /* element (s, c) is scale[s*stride_token + c*stride_channel] */
+  int64_t scale_stride_channel;
+  int64_t S;                  /* rows per batch element: row m uses sequence position m mod S */
+  const void* L;              /* device bf16 [S, rank] or NULL when rank == 0 */
+  const void* R;              /* device bf16 [rank, H] */
+  int32_t rank;
+  int32_t reserved;
+  /* outliers as CSR; consumed by decompress / backward entry points, produced by hyc_ref_outlier_fill */
+  const int32_t* csr_row_ptr; /* device [M+1] */
+  const int32_t* csr_cols;    /* device [nnz] */
+  const void* csr_vals;       /* device bf16 [nnz] */
+} hyc_desc;
+
+int hyc_abi_version(void);
+const char* hyc_last_error(void);
+
+/* 0 when the kernels cover (H, bits, group) in the given mode, else HYC_ENOTSUP / HYC_EINVAL.  Pure host code. */
+int hyc_check_shape(int64_t H, int32_t bits, int32_t group, int32_t mode);
+/* bytes of one stored row: H*bits/8 */
+int64_t hyc_stored_row_bytes(int64_t H, int32_t bits);
+/* number of fp32 [H] partial rows hyc_rmsnorm_bwd needs in dw_partials for M tokens */
+int64_t hyc_rmsnorm_bwd_partials(int64_t M, int64_t H);
+
+/* ---- calibration, channel mode --------------------------------------------------------------- */
+/* amax[c] = max(amax[c], max_m |x[m, c]|); the caller zero-fills amax (fp32 [H]) before the first call. */
+int hyc_channel_absmax(const void* x, int64_t M, int64_t H, float* amax, void* stream);
+/* the k largest amax, ties to the lower channel, written ascending to idx [k]; plan [H/8] as described above. */
+int hyc_select_channels(const float* amax, int64_t H, int32_t k, int32_t* idx, uint32_t* plan, void* stream);
+
+/* ---- standalone compress / decompress -------------------------------------------------------- */
+/* x bf16 [M,H] -> stored; channel mode also writes vals [M,k] and scales [M,H/group];
+ * threshold mode writes per-row outlier counts to row_counts (int32 [M], may be NULL). */
+int hyc_compress(const void* x, int64_t M, int64_t H, const hyc_desc* d, void* stored, void* vals, void* scales,
+                 int32_t* row_counts, void* stream);
+/* -> xhat bf16 [M,H]; channel mode reads vals/scales, threshold mode reads the CSR in the descriptor. */
+int hyc_decompress(const void* stored, const void* vals, const void* scales, int64_t M, int64_t H, const hyc_desc* d,
+                   void* xhat, void* stream);
+
+/* ---- threshold-mode outliers as CSR ---------------------------------------------------------- */
+/* counts[m] = #{c : |x[m,c] - base[m,c]| > threshold} */
+int hyc_ref_outlier_count(const void* x, int64_t M, int64_t H, const hyc_desc* d, int32_t* counts, void* stream);
+/* row_ptr int32 [M+1] = exclusive prefix sums of the counts; fills cols / vals in ascending column order */
+int hyc_ref_outlier_fill(const void* x, int64_t M, int64_t H, const hyc_desc* d, const int32_t* row_ptr,
+                         int32_t* cols, void* vals, void* stream);
+
+/* ---- RMSNorm ----------------------------------------------------------------------------------- */
+/* y = bf16((x*rstd)*w), rstd = 1/sqrt(mean(x^2)+eps) [M] fp32, and x compressed as hyc_compress does. */
+int hyc_rmsnorm_fwd_compress(const void* x, const void* w, int32_t w_dtype, float eps, int64_t M, int64_t H,
+                             const hyc_desc* d, void* y, float* rstd, void* stored, void* vals, void* scales,
+                             int32_t* row_counts, void* stream);
+/* dx = (w*dy - (xn*c1 + c2))*rstd with xn = xhat*rstd, c1 = mean(xn*w*dy), c2 = c2_quirk ? mean(w*dy) : 0;
+ * dw = sum_m dy*xn (fp32 accumulation, fixed order) written in w's dtype. */
+int hyc_rmsnorm_bwd(const void* dy, const void* stored, const void* vals, const void* scales, const void* w,
+                    int32_t w_dtype, const float* rstd, int64_t M, int64_t H, const hyc_desc* d, int32_t c2_quirk,
+                    void* dx, float* dw_partials, void* dw, void* stream);
+
+/* ---- activation backward ------------------------------------------------------------------- */
+/* dx = act'(xhat) * g evaluated op by op in bf16 as the reference expressions are. */
+int hyc_act_bwd(int32_t act, const void* g, const void* stored, const void* vals, const void* scales, int64_t M,
+                int64_t H, const hyc_desc* d, void* dx, void* stream);
+/* dx1 = g * x2hat, dx2 = x1hat * g */
+int hyc_hadamard_bwd(const void* g, const void* stored1, const void* vals1, const void* scales1, const hyc_desc* d1,
+                     const void* stored2, const void* vals2, const void* scales2, const hyc_desc* d2, int64_t M,
+                     int64_t H, void* dx1, void* dx2, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HYC_ABI_H */

@@ -105,16 +105,16 @@ def unpack_codes(packed_u8, bits):
 # --------------------------------------------------------------------------------------
 # quantise / dequantise primitives              operators/compress_function.py:170, 221-255
 # --------------------------------------------------------------------------------------
-def quantize_q(x, scale, bits, guard_zero_scale=False):
+def quantize_q(x, scale, bits, define_nan=False):
     """q = clamp(round(x / scale), -2^(b-1), 2^(b-1)-1); x, scale bf16 (broadcastable).
 
     The division result is a bf16 tensor (fp32 divide rounded to nearest even), round is
-    half-to-even, then the clamp.  With guard_zero_scale, positions whose scale is 0
-    give q = 0 instead of the reference's undefined NaN -> integer cast."""
+    half-to-even, then the clamp.  0/0 gives NaN, whose cast to an integer type the reference
+    leaves to the platform; with define_nan those positions get q = 0 (what the HIP kernels do)."""
     off = 2 ** (bits - 1)
     q = torch.clamp(torch.round(x / scale), min=-off, max=off - 1)
-    if guard_zero_scale:
-        q = torch.where((scale == 0).expand_as(q), torch.zeros_like(q), q)
+    if define_nan:
+        q = torch.where(torch.isnan(q), torch.zeros_like(q), q)
     return q
 
 
@@ -204,8 +204,9 @@ def running_mean_update(static, fresh, iteration):
 # ref-mode compress / decompress                 operators/compress_function.py:136-261
 # --------------------------------------------------------------------------------------
 @torch.no_grad()
-def ref_compress(x, thr, scale, bits=8, sub_outlier_ratio=1., L=None, R=None):
-    """-> (coo sparse bf16 of the outliers, stored codes, scale).  x is [B,S,H] or [B,nh,S,hd]."""
+def ref_compress(x, thr, scale, bits=8, sub_outlier_ratio=1., L=None, R=None, define_nan=False):
+    """-> (coo sparse bf16 of the outliers, stored codes, scale).  x is [B,S,H] or [B,nh,S,hd].
+    define_nan=True replaces the platform-defined integer cast of 0/0 by q = 0 (see quantize_q)."""
     if x.dim() == 4:
         x = head_to_hidden_shape(x)
     S = x.shape[-2]
@@ -220,7 +221,7 @@ def ref_compress(x, thr, scale, bits=8, sub_outlier_ratio=1., L=None, R=None):
         big_c = big
     assert sub_outlier_ratio != 0., "the no-quantisation branch is not part of the path"
     assert bits in (1, 2, 4, 8), "bits must be 1, 2, 4 or 8 on this path"
-    q = quantize_q(x, scale, bits)
+    q = quantize_q(x, scale, bits, define_nan)
     return big_c, encode_q(q, bits), scale
 
 
@@ -291,7 +292,7 @@ def hyc_compress(x, idx, bits, group):
     Composition of the reference steps (:149-151 zero-out, :170 quantise, :175-197 pack) with
     the channel mask in place of the threshold mask, and the reference scale formula
     (max - min) / (2^b - 1) (:328-334) evaluated per token and group of G channels.
-    A group whose scale is 0 (constant group) is given code = offset (q = 0)."""
+    0/0 (an all-zero group) is given q = 0, i.e. code = offset."""
     M, H = x.shape
     idx = idx.long()
     hot = torch.zeros(H, dtype=torch.bool)
@@ -301,7 +302,7 @@ def hyc_compress(x, idx, bits, group):
     rest = x - big
     g = rest.reshape(M, H // group, group)
     scales = (g.amax(dim=-1) - g.amin(dim=-1)) / (2 ** bits - 1)
-    q = quantize_q(g, scales[..., None], bits, guard_zero_scale=True).reshape(M, H)
+    q = quantize_q(g, scales[..., None], bits, define_nan=True).reshape(M, H)
     return vals, encode_q(q, bits), scales
 
 

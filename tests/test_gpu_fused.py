@@ -1,0 +1,163 @@
+"""GPU parity of the fused operators (RMSNorm forward + compress, RMSNorm backward, activation backward)
+against the CPU oracle.  Tolerances: compressed outputs bit-exact; y and dx within 1 bf16 ulp of the oracle
+(fp32 reduction order differs), gradients within rtol 1e-2 / atol 1e-3."""
+import pytest
+import torch
+
+from conftest import bf16_ulp_diff, bits_equal
+from oracle import hyc_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def K(hyc):
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    return hyc.kernels
+
+
+def make_x(seed, M, H, n_hot, gain):
+    gen = torch.Generator().manual_seed(seed)
+    x = torch.randn(M, H, generator=gen)
+    hot = torch.randperm(H, generator=gen)[:n_hot]
+    x[:, hot] *= gain
+    return x.bfloat16(), gen
+
+
+def close_bf16(got, want, max_ulp=1, frac=1e-3):
+    """all elements within max_ulp bf16 ulps, or (for values rounding to different binades near zero) tiny abs error"""
+    d = bf16_ulp_diff(got, want)
+    bad = (d > max_ulp) & ((got.float() - want.float()).abs() > 1e-6)
+    return int(bad.sum()) <= frac * got.numel() and torch.allclose(got.float(), want.float(), rtol=1e-2, atol=1e-3)
+
+
+NORM_CASES = [(4, 128, 96, 4096, 41, torch.float32), (4, 128, 96, 4096, 41, torch.bfloat16),
+              (2, 64, 40, 4096, 41, torch.float32), (4, 128, 20, 11008, 110, torch.float32),
+              (8, 128, 33, 2048, 20, torch.bfloat16), (1, 64, 16, 1024, 10, torch.float32),
+              (4, 128, 5, 16384, 164, torch.float32), (8, 256, 3, 32768, 300, torch.float32)]
+
+
+@pytest.mark.parametrize("bits,group,M,H,k,wdt", NORM_CASES)
+def test_rmsnorm_channel(K, bits, group, M, H, k, wdt):
+    x, gen = make_x(H + bits, M, H, k // 2, 30.0)
+    w = (1 + 0.1 * torch.randn(H, generator=gen)).to(wdt)
+    dy = (0.02 * torch.randn(M, H, generator=gen)).bfloat16()
+    eps = 1e-6
+    xd = x.cuda()
+    plan = K.select_channels(K.channel_absmax(xd), k)
+    idx = plan.idx.cpu()
+    assert torch.equal(idx, O.hyc_select_channels(O.hyc_channel_scores(x), k))
+    y, rstd, c = K.rmsnorm_fwd_compress_channel(xd, w.cuda(), eps, plan, bits, group)
+    y_o, rstd_o = O.rmsnorm_fwd(x, w, eps)
+    assert torch.allclose(rstd.cpu(), rstd_o, rtol=2e-6, atol=0)
+    assert bf16_ulp_diff(y.cpu(), y_o).max() <= 1
+    vals, stored, scales = O.hyc_compress(x, idx, bits, group)
+    assert torch.equal(c.stored.cpu(), stored) and bits_equal(c.scales.cpu(), scales) and bits_equal(c.vals.cpu(), vals)
+    # backward
+    xh = O.hyc_decompress(vals, stored, idx, scales, bits, group)
+    for quirk in (True, False):
+        dx, dw = K.rmsnorm_bwd(dy.cuda(), c, w.cuda(), rstd, c2_quirk=quirk)
+        dx_o, dw_o = O.rmsnorm_bwd(dy, xh, w, rstd_o, c2_quirk=quirk)
+        assert close_bf16(dx.cpu(), dx_o)
+        assert dw.dtype == w.dtype
+        assert torch.allclose(dw.cpu().float(), dw_o.float(), rtol=1e-2, atol=1e-3)
+    # the dense-source variant gives the same result as the fused one
+    dx2, dw2 = K.rmsnorm_bwd(dy.cuda(), xh.cuda(), w.cuda(), rstd, c2_quirk=True)
+    dx1, dw1 = K.rmsnorm_bwd(dy.cuda(), c, w.cuda(), rstd, c2_quirk=True)
+    assert bits_equal(dx1, dx2) and torch.equal(dw1, dw2)
+
+
+def test_rmsnorm_bwd_is_deterministic(K):
+    x, gen = make_x(9, 512, 4096, 20, 30.0)
+    w = (1 + 0.1 * torch.randn(4096, generator=gen))
+    dy = (0.02 * torch.randn(512, 4096, generator=gen)).bfloat16().cuda()
+    xd = x.cuda()
+    plan = K.select_channels(K.channel_absmax(xd), 41)
+    y, rstd, c = K.rmsnorm_fwd_compress_channel(xd, w.cuda(), 1e-6, plan, 4, 128)
+    a = K.rmsnorm_bwd(dy, c, w.cuda(), rstd)
+    b = K.rmsnorm_bwd(dy, c, w.cuda(), rstd)
+    assert bits_equal(a[0], b[0]) and torch.equal(a[1], b[1])
+
+
+@pytest.mark.parametrize("bits,method,rank", [(8, "per-channel", 2), (4, "per-token", 0), (2, "per-tensor", 0), (1, "per-channel", 0)])
+def test_rmsnorm_threshold(K, bits, method, rank):
+    B, S, H = 2, 24, 1024
+    gen = torch.Generator().manual_seed(bits)
+    x = torch.randn(B, S, H, generator=gen)
+    x[..., :3] *= 15
+    x = x.bfloat16()
+    w = (1 + 0.1 * torch.randn(H, generator=gen))
+    dy = (0.02 * torch.randn(B * S, H, generator=gen)).bfloat16()
+    torch.manual_seed(1)
+    thr, L, R, scale = O.get_statistics(x, 0, 0.005, 1.0, bits, method, rank)
+    coo, stored, _ = O.ref_compress(x, thr, scale, bits, 1.0, L, R)
+    xh = O.ref_decompress(coo, stored, bits, scale, L=L, R=R).reshape(-1, H)
+    y, rstd, c = K.rmsnorm_fwd_compress_threshold(x.reshape(-1, H).cuda(), w.cuda(), 1e-6, S, float(thr), scale.cuda(), bits,
+                                                  L.cuda() if rank else None, R.cuda() if rank else None)
+    y_o, rstd_o = O.rmsnorm_fwd(x.reshape(-1, H), w, 1e-6)
+    assert bf16_ulp_diff(y.cpu(), y_o).max() <= 1
+    assert torch.equal(c.stored.cpu().reshape(stored.shape), stored)
+    assert c.cols.numel() == coo.coalesce().values().numel()
+    assert bits_equal(K.decompress_threshold(c).cpu(), xh)
+    dx, dw = K.rmsnorm_bwd(dy.cuda(), c, w.cuda(), rstd)
+    dx_o, dw_o = O.rmsnorm_bwd(dy, xh, w, rstd_o)
+    assert close_bf16(dx.cpu(), dx_o)
+    assert torch.allclose(dw.cpu(), dw_o, rtol=1e-2, atol=1e-3)
+
+
+ACT_CASES = [(4, 128, 40, 11008, 110), (4, 128, 64, 4096, 41), (2, 64, 16, 4096, 41), (8, 32, 9, 512, 5), (1, 64, 9, 512, 5)]
+
+
+@pytest.mark.parametrize("bits,group,M,H,k", ACT_CASES)
+def test_act_bwd_channel(K, bits, group, M, H, k):
+    x, gen = make_x(bits + H, M, H, k, 20.0)
+    g = (0.1 * torch.randn(M, H, generator=gen)).bfloat16()
+    xd = x.cuda()
+    plan = K.select_channels(K.channel_absmax(xd), k)
+    c = K.compress_channel(xd, plan, bits, group)
+    xh = K.decompress_channel(c).cpu()
+    for act, fn in (("silu", O.silu_bwd), ("gelu", O.gelu_bwd)):
+        got = K.act_bwd(act, g.cuda(), c).cpu()
+        want = fn(xh, g)
+        # exp / tanh differ in the last fp32 bit between the host and device math libraries: allow 1 bf16 ulp on a
+        # small fraction of elements through each rounding of the chain, never more than the stated tolerance
+        assert close_bf16(got, want, max_ulp=2, frac=2e-3), act
+        same = (bf16_ulp_diff(got, want) == 0).float().mean()
+        assert same > 0.99, (act, float(same))
+        assert bits_equal(K.act_bwd(act, g.cuda(), xh.cuda()), K.act_bwd(act, g.cuda(), c))
+
+
+def test_hadamard_bwd(K):
+    M, H = 48, 4096
+    x1, gen = make_x(1, M, H, 41, 20.0)
+    x2, _ = make_x(2, M, H, 41, 20.0)
+    g = (0.1 * torch.randn(M, H, generator=gen)).bfloat16()
+    p1 = K.select_channels(K.channel_absmax(x1.cuda()), 41)
+    p2 = K.select_channels(K.channel_absmax(x2.cuda()), 41)
+    c1 = K.compress_channel(x1.cuda(), p1, 4, 128)
+    c2 = K.compress_channel(x2.cuda(), p2, 2, 64)
+    d1, d2 = K.hadamard_bwd(g.cuda(), c1, c2)
+    w1, w2 = O.hadamard_bwd(K.decompress_channel(c1).cpu(), K.decompress_channel(c2).cpu(), g)
+    assert bits_equal(d1.cpu(), w1) and bits_equal(d2.cpu(), w2)
+
+
+def test_config2_shape(K):
+    """BASELINE config 2: x [4,1024,4096] with 20 channels x30, w ~ N(1, 0.1), eps 1e-6, dy ~ N(0, 0.02), 1 % / INT4 / 128."""
+    M, H = 4096, 4096
+    x, gen = make_x(0, M, H, 20, 30.0)
+    w = 1 + 0.1 * torch.randn(H, generator=gen)
+    dy = (0.02 * torch.randn(M, H, generator=gen)).bfloat16()
+    xd = x.cuda()
+    plan = K.select_channels(K.channel_absmax(xd), 41)
+    y, rstd, c = K.rmsnorm_fwd_compress_channel(xd, w.cuda(), 1e-6, plan, 4, 128)
+    idx = plan.idx.cpu()
+    vals, stored, scales = O.hyc_compress(x, idx, 4, 128)
+    assert torch.equal(c.stored.cpu(), stored) and bits_equal(c.scales.cpu(), scales) and bits_equal(c.vals.cpu(), vals)
+    y_o, rstd_o = O.rmsnorm_fwd(x, w, 1e-6)
+    assert bf16_ulp_diff(y.cpu(), y_o).max() <= 1
+    xh = O.hyc_decompress(vals, stored, idx, scales, 4, 128)
+    dx, dw = K.rmsnorm_bwd(dy.cuda(), c, w.cuda(), rstd)
+    dx_o, dw_o = O.rmsnorm_bwd(dy, xh, w, rstd_o)
+    assert torch.allclose(dx.cpu().float(), dx_o.float(), rtol=1e-2, atol=1e-3)
+    assert torch.allclose(dw.cpu(), dw_o, rtol=1e-2, atol=1e-3)

@@ -184,7 +184,9 @@ def test_hyc_constant_group_is_defined():
     idx = torch.tensor([], dtype=torch.int32)
     vals, stored, scales = O.hyc_compress(x, idx, 4, 128)
     assert torch.all(scales == 0)
-    assert torch.all(O.unpack_codes(stored, 4) == 8)
+    codes = O.unpack_codes(stored, 4)
+    assert torch.all(codes[0, :128] == 15)          # 3/0 = +inf clamps to the top code
+    assert torch.all(codes[0, 128:] == 8) and torch.all(codes[1] == 8)   # 0/0 is defined as q = 0
     assert torch.all(O.hyc_decompress(vals, stored, idx, scales, 4, 128) == 0)
 
 
