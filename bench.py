@@ -1,0 +1,232 @@
+"""Benchmark of the hybrid activation-compression hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step = one pass of the path over one batch of synthetic input, BASELINE config 2: fused RMSNorm forward +
+compress (1 % outlier channels, INT4, group 128) of x [4,1024,4096] bf16, then the RMSNorm backward that
+decompresses it.  Inputs are resident in HBM before the timed region.  Prints ONE JSON line.
+"""
+import argparse
+import ctypes
+import importlib
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def algorithmic_bytes(M, H, bits, group, k):
+    """per-launch bytes a perfect kernel must move (no re-reads): see DESIGN.md for the derivation"""
+    side = H * bits // 8 + 2 * k + 2 * (H // group)          # packed codes + outlier values + group scales
+    fwd = M * (2 * H + 2 * H + side + 4)                       # read x, write y, side data, rstd
+    bwd = M * (2 * H + side + 4 + 2 * H)                       # read dy, side data, rstd; write dx
+    return fwd, bwd, M * side
+
+
+class Workload:
+    """device buffers + prebuilt ctypes calls for fwd and bwd of the fused RMSNorm path"""
+
+    def __init__(self, pkg, torch, M, H, bits, group, n_hot, gain, seed=0):
+        K, abi = pkg.kernels, pkg._abi
+        self.torch, self.lib, self.M, self.H = torch, abi.load(), M, H
+        gen = torch.Generator().manual_seed(seed)
+        k = K.num_outlier_channels(H, 0.01)
+        self.k, self.bits, self.group = k, bits, group
+        # generate on the host in slabs (identical bits for the oracle), then move to the device
+        xs = []
+        hot = torch.randperm(H, generator=gen)[:n_hot]
+        for r in range(0, M, 4096):
+            m = min(4096, M - r)
+            xs_ = torch.randn(m, H, generator=gen)
+            xs_[:, hot] *= gain
+            xs.append(xs_.bfloat16())
+        self.x_host = xs[0] if len(xs) == 1 else None
+        self.x = torch.cat([t.cuda() for t in xs])
+        self.w_host = 1 + 0.1 * torch.randn(H, generator=gen)
+        self.w = self.w_host.cuda()
+        self.dy = torch.cat([(0.02 * torch.randn(min(4096, M - r), H, generator=gen)).bfloat16().cuda()
+                             for r in range(0, M, 4096)])
+        self.plan = K.select_channels(K.channel_absmax(self.x), k)
+        self.c = K.alloc_channel(M, H, self.plan, bits, group, self.x.device)
+        self.y = torch.empty_like(self.x)
+        self.rstd = torch.empty(M, dtype=torch.float32, device="cuda")
+        self.dx = torch.empty_like(self.x)
+        P = self.lib.hyc_rmsnorm_bwd_partials(M, H)
+        self.partials = torch.empty((P, H), dtype=torch.float32, device="cuda")
+        self.dw = torch.empty(H, dtype=torch.float32, device="cuda")
+        self.desc = self.c.desc()
+        p = lambda t: ctypes.c_void_p(t.data_ptr())
+        self._fwd_args = (p(self.x), p(self.w), abi.DTYPE_F32, ctypes.c_float(1e-6), M, H, ctypes.byref(self.desc),
+                          p(self.y), p(self.rstd), p(self.c.stored), p(self.c.vals), p(self.c.scales), None)
+        self._bwd_args = (p(self.dy), p(self.c.stored), p(self.c.vals), p(self.c.scales), p(self.w), abi.DTYPE_F32,
+                          p(self.rstd), M, H, ctypes.byref(self.desc), 1, p(self.dx), p(self.partials), p(self.dw))
+        self._check = abi.check
+
+    def _stream(self):
+        return ctypes.c_void_p(self.torch.cuda.current_stream().cuda_stream)
+
+    def fwd(self):
+        self._check(self.lib.hyc_rmsnorm_fwd_compress(*self._fwd_args, self._stream()))
+
+    def bwd(self):
+        self._check(self.lib.hyc_rmsnorm_bwd(*self._bwd_args, self._stream()))
+
+    def step(self):
+        self.fwd()
+        self.bwd()
+
+
+def time_events(torch, fn, iters, warmup):
+    """average milliseconds of fn() over `iters` back-to-back launches, HIP events on the launch stream"""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / iters
+
+
+def cpu_baseline(torch, wl, rows, seconds):
+    """the oracle (CPU PyTorch restatement of the path) on the host cores, bounded sample of the same workload"""
+    from oracle import hyc_oracle as O
+    threads = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(threads)
+    x = wl.x[:rows].cpu()
+    dy = wl.dy[:rows].cpu()
+    w = wl.w_host
+    idx = wl.plan.idx.cpu()
+    H, bits, group = wl.H, wl.bits, wl.group
+
+    def one():
+        y, rstd = O.rmsnorm_fwd(x, w, 1e-6)
+        vals, stored, scales = O.hyc_compress(x, idx, bits, group)
+        xh = O.hyc_decompress(vals, stored, idx, scales, bits, group)
+        return O.rmsnorm_bwd(dy, xh, w, rstd)
+
+    one()
+    t0 = time.perf_counter()
+    reps = 0
+    while time.perf_counter() - t0 < seconds:
+        one()
+        reps += 1
+    dt = (time.perf_counter() - t0) / reps
+    fwd_b, bwd_b, _ = algorithmic_bytes(rows, H, bits, group, wl.k)
+    return {"value": round((fwd_b + bwd_b) / dt / 1e9, 4), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": "oracle rmsnorm_fwd + hyc_compress + hyc_decompress + rmsnorm_bwd on the first %d of %d tokens "
+                      "(H=%d), mean of %d passes, %.3f s per pass" % (rows, wl.M, H, reps, dt)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-scaled", action="store_true", help="skip the 16x token-scaled run")
+    ap.add_argument("--pmc-probe", action="store_true",
+                    help="for rocprofv3 --pmc: 5x a plain 32 MiB device copy, 5x fwd, 5x bwd, then exit")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this path runs on ONE GPU (no sharding, no collectives); run with --gpus 1")
+
+    import torch
+    pkg = importlib.import_module("hyc-lora_amd")
+    if not os.path.exists(pkg._abi.LIB_PATH):
+        import __graft_entry__
+        __graft_entry__.build()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+
+    M, H, bits, group = 4 * 1024, 4096, 4, 128
+    wl = Workload(pkg, torch, M, H, bits, group, n_hot=20, gain=30.0)
+    fwd_b, bwd_b, saved_b = algorithmic_bytes(M, H, bits, group, wl.k)
+
+    if args.pmc_probe:
+        dst = torch.empty_like(wl.x)
+        for _ in range(5):
+            dst.copy_(wl.x)          # reads 2*M*H bytes, writes 2*M*H bytes: the counters' yardstick
+        for _ in range(5):
+            wl.fwd()
+        for _ in range(5):
+            wl.bwd()
+        torch.cuda.synchronize()
+        print(json.dumps({"pmc_probe": True, "copy_bytes_each_way": 2 * M * H, "fwd_bytes": fwd_b, "bwd_bytes": bwd_b}))
+        return
+
+    # the step as a HIP graph (three launches; removes the host launch cost from the timed loop)
+    wl.step()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        wl.step()
+    torch.cuda.current_stream().wait_stream(side)
+    with torch.cuda.graph(graph):
+        wl.step()
+    for _ in range(args.warmup):
+        graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        graph.replay()
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # eager launches for comparison, and per-kernel durations with events on the launch stream
+    eager_ms = time_events(torch, wl.step, args.steps, args.warmup)
+    fwd_ms = time_events(torch, wl.fwd, args.steps, args.warmup)
+    bwd_ms = time_events(torch, wl.bwd, args.steps, args.warmup)
+
+    value = (fwd_b + bwd_b) / (ms_step * 1e-3) / 1e9
+    dom_name, dom_ms, dom_b = ("hyc_rmsnorm_bwd", bwd_ms, bwd_b) if bwd_ms >= fwd_ms else ("hyc_rmsnorm_fwd_compress", fwd_ms, fwd_b)
+    achieved = dom_b / (dom_ms * 1e-3) / 1e9
+    extra = {
+        "eager_ms_per_step": round(eager_ms, 5),
+        "fwd_kernel_ms": round(fwd_ms, 5), "fwd_GBps": round(fwd_b / fwd_ms / 1e6, 1),
+        "bwd_kernels_ms": round(bwd_ms, 5), "bwd_GBps": round(bwd_b / bwd_ms / 1e6, 1),
+        "act_mem_bytes_saved_tensor": saved_b + 4 * M, "act_mem_bytes_bf16": 2 * M * H,
+        "act_mem_ratio": round(2 * M * H / (saved_b + 4 * M), 3),
+    }
+    if not args.no_scaled:
+        # the config-size working set (~150 MB) fits the 256 MB Infinity Cache; 16x the tokens does not
+        del graph
+        Ms = 16 * M
+        wls = Workload(pkg, torch, Ms, H, bits, group, n_hot=20, gain=30.0, seed=1)
+        fs, bs, _ = algorithmic_bytes(Ms, H, bits, group, wls.k)
+        f_ms = time_events(torch, wls.fwd, 30, 5)
+        b_ms = time_events(torch, wls.bwd, 30, 5)
+        extra["scaled16x"] = {"tokens": Ms, "fwd_ms": round(f_ms, 4), "fwd_GBps": round(fs / f_ms / 1e6, 1),
+                              "bwd_ms": round(b_ms, 4), "bwd_GBps": round(bs / b_ms / 1e6, 1),
+                              "fwd_frac_of_hbm_peak": round(fs / f_ms / 1e6 / HBM_PEAK_GBPS, 4),
+                              "bwd_frac_of_hbm_peak": round(bs / b_ms / 1e6 / HBM_PEAK_GBPS, 4)}
+        del wls
+    out = {
+        "metric": "compress+decompress GB/s", "value": round(value, 2), "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "BASELINE configs[1]: fused RMSNorm fwd+compress and bwd(decompress), x bf16 [4,1024,4096], "
+                               "20 hot channels x30, 1% outlier channels kept bf16, INT4 codes, group 128, w fp32, eps 1e-6",
+                   "tokens": M, "hidden": H, "bits": bits, "group": group, "outlier_channels": wl.k,
+                   "launch": "hip graph replay of fwd + bwd + dw-reduce"},
+        "roofline": {"bound": "hbm", "kernel": dom_name, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None},
+        "extra": extra,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(torch, wl, rows=M, seconds=12.0)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -61,6 +61,9 @@ def load():
     global _lib
     if _lib is not None:
         return _lib
+    # torch first: it ships its own HIP runtime (same soname as the system one); the library must bind to the
+    # runtime instance that owns the caller's streams and allocations, so torch's has to be resident already.
+    import torch  # noqa: F401
     if not os.path.exists(LIB_PATH):
         raise RuntimeError(
             "HIP library %s is missing: build it with `python hyc-lora_amd/build.py` "

@@ -66,6 +66,15 @@ inline int chan_geom(const RowGeom& g, int group, int* lpg) {
   return HYC_OK;
 }
 
+// The HIP runtime keeps the last error of the thread until it is read; other code in the process (the
+// framework that owns the streams) may have left one behind.  Entry points call this before they launch so
+// that check_launch() reports only their own failure.
+inline void drop_stale_error() { (void)hipGetLastError(); }
+inline hipStream_t begin_launch(void* stream) {
+  drop_stale_error();
+  return static_cast<hipStream_t>(stream);
+}
+
 inline int check_launch(const char* what) {
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(HYC_ELAUNCH, "%s: %s", what, hipGetErrorString(e));

@@ -97,7 +97,7 @@ static int launch_act(const void* g, const void* stored, const void* vals, const
     return fail(HYC_EINVAL, "%s: g, dx must be 16-byte aligned, stored 8-byte (16 when dense)", who);
   const int64_t cap = 256 * (geo.threads >= 512 ? 3 : 8);
   const int grid = (int)(M < cap ? M : cap);
-  hipStream_t st = static_cast<hipStream_t>(stream);
+  hipStream_t st = begin_launch(stream);
 #define HYC_ACT_LAUNCH(B_, S_)                                                                            \
   hipLaunchKernelGGL((k_act_bwd<B_, S_, ACT>), dim3(grid), dim3(geo.threads), 0, st,                      \
                      static_cast<const uint16_t*>(g), static_cast<const uint8_t*>(stored),                \

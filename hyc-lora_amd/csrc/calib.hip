@@ -101,7 +101,7 @@ int hyc_channel_absmax(const void* x, int64_t M, int64_t H, float* amax, void* s
     return HYC_OK;
   }
   dim3 grid((unsigned)((H / 8 + 255) / 256), (unsigned)tiles);
-  hipLaunchKernelGGL(k_channel_absmax, grid, dim3(256), 0, static_cast<hipStream_t>(stream),
+  hipLaunchKernelGGL(k_channel_absmax, grid, dim3(256), 0, begin_launch(stream),
                      static_cast<const uint16_t*>(x), M, H, reinterpret_cast<unsigned int*>(amax));
   return check_launch("hyc_channel_absmax");
 }
@@ -110,7 +110,7 @@ int hyc_select_channels(const float* amax, int64_t H, int32_t k, int32_t* idx, u
   if (H <= 0 || H % 8 != 0 || H > 65536) return fail(HYC_EINVAL, "hyc_select_channels: H=%lld", (long long)H);
   if (k < 0 || k > H || k > 65535) return fail(HYC_EINVAL, "hyc_select_channels: k=%d", k);
   if (!amax || !plan || (k > 0 && !idx)) return fail(HYC_EFAULT, "hyc_select_channels: null buffer");
-  hipStream_t st = static_cast<hipStream_t>(stream);
+  hipStream_t st = begin_launch(stream);
   hipLaunchKernelGGL(k_select_rank, dim3((unsigned)((H + 255) / 256)), dim3(256), 0, st, amax, (int)H, (int)k, plan);
   hipLaunchKernelGGL(k_select_finish, dim3(1), dim3(1024), 0, st, (int)H, plan, idx);
   return check_launch("hyc_select_channels");

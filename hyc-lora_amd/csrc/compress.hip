@@ -248,7 +248,7 @@ int hyc_compress(const void* x, int64_t M, int64_t H, const hyc_desc* d, void* s
   RowGeom g;
   int rc = row_geom(H, d->bits, &g);
   if (rc) return rc;
-  hipStream_t st = static_cast<hipStream_t>(stream);
+  hipStream_t st = begin_launch(stream);
   if (d->mode == HYC_MODE_CHANNEL) {
     ChanArgs a; int lpg;
     if ((rc = make_chan_args(d, g, &a, &lpg))) return rc;
@@ -288,7 +288,7 @@ int hyc_decompress(const void* stored, const void* vals, const void* scales, int
   RowGeom g;
   int rc = row_geom(H, d->bits, &g);
   if (rc) return rc;
-  hipStream_t st = static_cast<hipStream_t>(stream);
+  hipStream_t st = begin_launch(stream);
   if (d->mode == HYC_MODE_CHANNEL) {
     ChanArgs a; int lpg;
     if ((rc = make_chan_args(d, g, &a, &lpg))) return rc;
@@ -342,7 +342,7 @@ int hyc_ref_outlier_count(const void* x, int64_t M, int64_t H, const hyc_desc* d
   if (M == 0) return HYC_OK;
   if (!x || !counts) return fail(HYC_EFAULT, "hyc_ref_outlier_count: null buffer");
   if (!aligned16(x)) return fail(HYC_EINVAL, "hyc_ref_outlier_count: x must be 16-byte aligned");
-  hipLaunchKernelGGL(k_outlier_count, dim3((unsigned)((M + 3) / 4)), dim3(256), 0, static_cast<hipStream_t>(stream),
+  hipLaunchKernelGGL(k_outlier_count, dim3((unsigned)((M + 3) / 4)), dim3(256), 0, begin_launch(stream),
                      static_cast<const uint16_t*>(x), M, H, a, counts);
   return check_launch("hyc_ref_outlier_count");
 }
@@ -355,7 +355,7 @@ int hyc_ref_outlier_fill(const void* x, int64_t M, int64_t H, const hyc_desc* d,
   if (M == 0) return HYC_OK;
   if (!x || !row_ptr) return fail(HYC_EFAULT, "hyc_ref_outlier_fill: null buffer");
   if (!aligned16(x)) return fail(HYC_EINVAL, "hyc_ref_outlier_fill: x must be 16-byte aligned");
-  hipLaunchKernelGGL(k_outlier_fill, dim3((unsigned)((M + 3) / 4)), dim3(256), 0, static_cast<hipStream_t>(stream),
+  hipLaunchKernelGGL(k_outlier_fill, dim3((unsigned)((M + 3) / 4)), dim3(256), 0, begin_launch(stream),
                      static_cast<const uint16_t*>(x), M, H, a, row_ptr, cols, static_cast<uint16_t*>(vals));
   return check_launch("hyc_ref_outlier_fill");
 }

@@ -201,15 +201,33 @@ k_rmsnorm_bwd(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ store
   }
 }
 
-// dw[c] = sum_p partials[p, c], fixed order
+// dw[c] = sum_p partials[p, c] in a fixed order: 32 columns x 8 row lanes per workgroup, each lane sums rows
+// p = lane, lane+8, ... and the 8 lane sums are added in lane order.
 __global__ void __launch_bounds__(256)
 k_colsum(const float* __restrict__ partials, int64_t P, int64_t H, void* __restrict__ dw, bool wf32) {
-  const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (c >= H) return;
-  float s = 0.f;
-  for (int64_t p = 0; p < P; ++p) s += partials[p * H + c];
-  if (wf32) static_cast<float*>(dw)[c] = s;
-  else static_cast<uint16_t*>(dw)[c] = f_to_bf(s);
+  __shared__ float part[8][33];
+  const int cx = threadIdx.x & 31, lane = threadIdx.x >> 5;
+  const int64_t c = (int64_t)blockIdx.x * 32 + cx;
+  float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+  if (c < H) {
+    int64_t p = lane;
+    for (; p + 24 < P; p += 32) {
+      s0 += partials[p * H + c];
+      s1 += partials[(p + 8) * H + c];
+      s2 += partials[(p + 16) * H + c];
+      s3 += partials[(p + 24) * H + c];
+    }
+    for (; p < P; p += 8) s0 += partials[p * H + c];
+  }
+  part[lane][cx] = (s0 + s1) + (s2 + s3);
+  __syncthreads();
+  if (lane == 0 && c < H) {
+    float s = 0.f;
+#pragma unroll
+    for (int l = 0; l < 8; ++l) s += part[l][cx];
+    if (wf32) static_cast<float*>(dw)[c] = s;
+    else static_cast<uint16_t*>(dw)[c] = f_to_bf(s);
+  }
 }
 
 static inline int64_t bwd_rows_per_block(int64_t M) {
@@ -269,7 +287,7 @@ int hyc_rmsnorm_fwd_compress(const void* x, const void* w, int32_t w_dtype, floa
   const bool wf32 = w_dtype == HYC_DTYPE_F32;
   const int64_t cap = 256 * (g.threads >= 512 ? 3 : 8);
   const int grid = (int)(M < cap ? M : cap);
-  hipStream_t st = static_cast<hipStream_t>(stream);
+  hipStream_t st = begin_launch(stream);
   const uint16_t* xp = static_cast<const uint16_t*>(x);
   if (d->mode == HYC_MODE_CHANNEL) {
     HYC_BITS_ITERS_MAXT(d->bits, round_iters(g.iters), g.threads,
@@ -300,7 +318,7 @@ int hyc_rmsnorm_bwd(const void* dy, const void* stored, const void* vals, const 
   ChanArgs ca = {}; int lpg = 16;
   if (d->mode == HYC_MODE_CHANNEL && (rc = make_chan_args(d, g, &ca, &lpg))) return rc;
   if (!dw) return fail(HYC_EFAULT, "hyc_rmsnorm_bwd: null dw");
-  hipStream_t st = static_cast<hipStream_t>(stream);
+  hipStream_t st = begin_launch(stream);
   const bool wf32 = w_dtype == HYC_DTYPE_F32;
   const int64_t P = hyc_rmsnorm_bwd_partials(M, H);
   if (M > 0) {
@@ -326,7 +344,7 @@ int hyc_rmsnorm_bwd(const void* dy, const void* stored, const void* vals, const 
     }
     if ((rc = check_launch("hyc_rmsnorm_bwd"))) return rc;
   }
-  hipLaunchKernelGGL(k_colsum, dim3((unsigned)((H + 255) / 256)), dim3(256), 0, st, dw_partials, P, H, dw, wf32);
+  hipLaunchKernelGGL(k_colsum, dim3((unsigned)((H + 31) / 32)), dim3(256), 0, st, dw_partials, P, H, dw, wf32);
   return check_launch("hyc_rmsnorm_bwd (dw)");
 }
 
