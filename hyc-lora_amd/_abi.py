@@ -51,6 +51,14 @@ SIGNATURES = {
     "hyc_act_bwd": (c_i32, [c_i32, c_ptr, c_ptr, c_ptr, c_ptr, c_i64, c_i64, ctypes.POINTER(HycDesc), c_ptr, c_ptr]),
     "hyc_hadamard_bwd": (c_i32, [c_ptr, c_ptr, c_ptr, c_ptr, ctypes.POINTER(HycDesc), c_ptr, c_ptr, c_ptr,
                                  ctypes.POINTER(HycDesc), c_i64, c_i64, c_ptr, c_ptr, c_ptr]),
+    "hyc_softmax_fwd": (c_i32, [c_ptr, c_i64, c_i64, c_f32, c_ptr, c_ptr, c_ptr]),
+    "hyc_softmax_fill": (c_i32, [c_ptr, c_i64, c_i64, c_f32, c_ptr, c_ptr, c_ptr, c_ptr]),
+    "hyc_softmax_bwd": (c_i32, [c_ptr, c_i64, c_i64, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr]),
+    "hyc_softmax_dense": (c_i32, [c_i64, c_i64, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr]),
+    "hyc_gradw_workspace_bytes": (c_i64, [c_i64, c_i64, c_i64]),
+    "hyc_gradw_gemm": (c_i32, [c_ptr, c_i64, c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_i64, ctypes.POINTER(HycDesc),
+                               c_f32, c_f32, c_ptr, c_i32, c_ptr, c_ptr]),
+    "hyc_low_rank_update": (c_i32, [c_ptr, c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_i64, c_i32, c_i32, c_ptr]),
 }
 
 _lib = None

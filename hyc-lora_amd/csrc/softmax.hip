@@ -1,0 +1,226 @@
+// Softmax over the last dimension with the sparsified copy for backward.
+//   forward   y = softmax(x) (fp32 math, one rounding to bf16); per-row count of y > threshold
+//   fill      the kept probabilities as CSR (cols ascending within a row, values verbatim)
+//   backward  dx = (g - sum_j g_j*yh_j) * yh, yh = the kept probabilities, zero elsewhere
+//   dense     yh as a dense matrix (what true_decompress_softmax returns)
+// Reference: operators/efficient_softmax.py:10-45, operators/compress_function.py:264-275.
+#include "abi_util.hpp"
+
+namespace hyc {
+
+// one workgroup (256 threads) per row, grid-stride; N a multiple of 8
+__global__ void __launch_bounds__(256)
+k_softmax_fwd(const uint16_t* __restrict__ x, int64_t rows, int64_t N, float thr, uint16_t* __restrict__ y,
+              int32_t* __restrict__ counts) {
+  __shared__ float red[32];
+  const int64_t nch = N / 8;
+  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+    const uint16_t* xr = x + row * N;
+    // pass 1: row maximum
+    float m = -INFINITY;
+    for (int64_t c = threadIdx.x; c < nch; c += 256) {
+      float v[8];
+      unpack8(*reinterpret_cast<const uint4*>(xr + 8 * c), v);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) m = v[j] > m ? v[j] : m;
+    }
+    m = group_reduce<64>(m, OpMax());
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    __syncthreads();
+    // pass 2: sum of exp(x - m)   (the row is re-read from cache)
+    float l = 0.f;
+    for (int64_t c = threadIdx.x; c < nch; c += 256) {
+      float v[8];
+      unpack8(*reinterpret_cast<const uint4*>(xr + 8 * c), v);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) l += expf(v[j] - m);
+    }
+    l = block_sum(l, red);
+    // pass 3: y and the count of kept entries
+    int kept = 0;
+    uint16_t* yr = y + row * N;
+    for (int64_t c = threadIdx.x; c < nch; c += 256) {
+      float v[8];
+      unpack8(*reinterpret_cast<const uint4*>(xr + 8 * c), v);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        v[j] = bfr(expf(v[j] - m) / l);
+        kept += (v[j] > thr) ? 1 : 0;
+      }
+      *reinterpret_cast<uint4*>(yr + 8 * c) = pack8(v);
+    }
+    if (counts) {
+      const float total = block_sum((float)kept, red);
+      if (threadIdx.x == 0) counts[row] = (int32_t)total;
+    }
+  }
+}
+
+// counts only, for probabilities computed elsewhere; one wave per row
+__global__ void __launch_bounds__(256)
+k_softmax_count(const uint16_t* __restrict__ y, int64_t rows, int64_t N, float thr, int32_t* __restrict__ counts) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const uint16_t* yr = y + row * N;
+  int kept = 0;
+  for (int64_t c = lane; c < N / 8; c += 64) {
+    float v[8];
+    unpack8(*reinterpret_cast<const uint4*>(yr + 8 * c), v);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) kept += (v[j] > thr) ? 1 : 0;
+  }
+  const float total = wave_sum((float)kept);
+  if (lane == 0) counts[row] = (int32_t)total;
+}
+
+// one wave per row: ordered compaction of the kept entries
+__global__ void __launch_bounds__(256)
+k_softmax_fill(const uint16_t* __restrict__ y, int64_t rows, int64_t N, float thr, const int32_t* __restrict__ row_ptr,
+               int32_t* __restrict__ cols, uint16_t* __restrict__ vals) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const uint16_t* yr = y + row * N;
+  const int64_t nch = N / 8;
+  int running = row_ptr[row];
+  for (int64_t c0 = 0; c0 < nch; c0 += 64) {
+    const int64_t c = c0 + lane;
+    uint4 raw = make_uint4(0, 0, 0, 0);
+    float v[8];
+    uint32_t m = 0;
+    if (c < nch) {
+      raw = *reinterpret_cast<const uint4*>(yr + 8 * c);
+      unpack8(raw, v);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) m |= (v[j] > thr) ? (1u << j) : 0u;
+    }
+    const int cnt = __popc(m);
+    int incl = cnt;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int t = __shfl_up(incl, d, 64);
+      if (lane >= d) incl += t;
+    }
+    int pos = running + incl - cnt;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if ((m >> j) & 1u) {
+        cols[pos] = (int32_t)(8 * c + j);
+        vals[pos] = f_to_bf(v[j]);
+        ++pos;
+      }
+    }
+    running += __shfl(incl, 63, 64);
+  }
+}
+
+// one wave per row; the output row is assembled in LDS (zeros + kept entries) and written out coalesced.
+// BWD: dx = (g - s) * yh with s = bf16(sum_j bf16(g_j * yh_j)), every product rounded to bf16 as torch does.
+template <bool BWD>
+__global__ void __launch_bounds__(256)
+k_softmax_rows(const uint16_t* __restrict__ g, int64_t rows, int64_t N, const int32_t* __restrict__ row_ptr,
+               const int32_t* __restrict__ cols, const uint16_t* __restrict__ vals, uint16_t* __restrict__ out) {
+  extern __shared__ __align__(16) uint16_t lds[];          // [4][N]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t row = (int64_t)blockIdx.x * 4 + wave;
+  if (row >= rows) return;
+  uint16_t* buf = lds + (int64_t)wave * N;
+  const int e0 = row_ptr[row], e1 = row_ptr[row + 1];
+  float s = 0.f;
+  if (BWD) {
+    float part = 0.f;
+    for (int e = e0 + lane; e < e1; e += 64)
+      part += bfr(bf_to_f(g[row * N + cols[e]]) * bf_to_f(vals[e]));
+    s = bfr(wave_sum(part));
+  }
+  for (int64_t c = lane; c < N / 8; c += 64) *reinterpret_cast<uint4*>(buf + 8 * c) = make_uint4(0, 0, 0, 0);
+  __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");  // order this wave's LDS writes (other lanes) before the next ones
+  __builtin_amdgcn_wave_barrier();
+  for (int e = e0 + lane; e < e1; e += 64) {
+    const int col = cols[e];
+    const float yh = bf_to_f(vals[e]);
+    buf[col] = BWD ? f_to_bf(bfr(bf_to_f(g[row * N + col]) - s) * yh) : vals[e];
+  }
+  __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  uint16_t* orow = out + row * N;
+  for (int64_t c = lane; c < N / 8; c += 64)
+    *reinterpret_cast<uint4*>(orow + 8 * c) = *reinterpret_cast<const uint4*>(buf + 8 * c);
+}
+
+static int softmax_shape(const char* who, int64_t rows, int64_t N) {
+  if (rows < 0 || N <= 0 || N % 8 != 0 || N > 8192)
+    return fail(rows < 0 || N <= 0 ? HYC_EINVAL : HYC_ENOTSUP, "%s: rows=%lld N=%lld (N must be a multiple of 8, at most 8192)",
+                who, (long long)rows, (long long)N);
+  return HYC_OK;
+}
+
+}  // namespace hyc
+
+using namespace hyc;
+
+extern "C" {
+
+int hyc_softmax_fwd(const void* x, int64_t rows, int64_t N, float threshold, void* y, int32_t* counts, void* stream) {
+  int rc = softmax_shape("hyc_softmax_fwd", rows, N);
+  if (rc) return rc;
+  if (rows == 0) return HYC_OK;
+  if (!y) return fail(HYC_EFAULT, "hyc_softmax_fwd: null y");
+  if ((x && !aligned16(x)) || !aligned16(y)) return fail(HYC_EINVAL, "hyc_softmax_fwd: x and y must be 16-byte aligned");
+  hipStream_t st = begin_launch(stream);
+  const float thr = round_to_bf16(threshold);
+  if (x) {
+    const int64_t cap = 256 * 8;
+    hipLaunchKernelGGL(k_softmax_fwd, dim3((unsigned)(rows < cap ? rows : cap)), dim3(256), 0, st,
+                       static_cast<const uint16_t*>(x), rows, N, thr, static_cast<uint16_t*>(y), counts);
+  } else {
+    if (!counts) return fail(HYC_EFAULT, "hyc_softmax_fwd: nothing to do (x and counts both null)");
+    hipLaunchKernelGGL(k_softmax_count, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st,
+                       static_cast<const uint16_t*>(y), rows, N, thr, counts);
+  }
+  return check_launch("hyc_softmax_fwd");
+}
+
+int hyc_softmax_fill(const void* y, int64_t rows, int64_t N, float threshold, const int32_t* row_ptr, int32_t* cols,
+                     void* vals, void* stream) {
+  int rc = softmax_shape("hyc_softmax_fill", rows, N);
+  if (rc) return rc;
+  if (rows == 0) return HYC_OK;
+  if (!y || !row_ptr) return fail(HYC_EFAULT, "hyc_softmax_fill: null buffer");
+  if (!aligned16(y)) return fail(HYC_EINVAL, "hyc_softmax_fill: y must be 16-byte aligned");
+  hipLaunchKernelGGL(k_softmax_fill, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, begin_launch(stream),
+                     static_cast<const uint16_t*>(y), rows, N, round_to_bf16(threshold), row_ptr, cols,
+                     static_cast<uint16_t*>(vals));
+  return check_launch("hyc_softmax_fill");
+}
+
+int hyc_softmax_bwd(const void* g, int64_t rows, int64_t N, const int32_t* row_ptr, const int32_t* cols,
+                    const void* vals, void* dx, void* stream) {
+  int rc = softmax_shape("hyc_softmax_bwd", rows, N);
+  if (rc) return rc;
+  if (rows == 0) return HYC_OK;
+  if (!g || !row_ptr || !dx) return fail(HYC_EFAULT, "hyc_softmax_bwd: null buffer");
+  if (!aligned16(dx)) return fail(HYC_EINVAL, "hyc_softmax_bwd: dx must be 16-byte aligned");
+  hipLaunchKernelGGL((k_softmax_rows<true>), dim3((unsigned)((rows + 3) / 4)), dim3(256), (size_t)N * 8, begin_launch(stream),
+                     static_cast<const uint16_t*>(g), rows, N, row_ptr, cols, static_cast<const uint16_t*>(vals),
+                     static_cast<uint16_t*>(dx));
+  return check_launch("hyc_softmax_bwd");
+}
+
+int hyc_softmax_dense(int64_t rows, int64_t N, const int32_t* row_ptr, const int32_t* cols, const void* vals,
+                      void* y_hat, void* stream) {
+  int rc = softmax_shape("hyc_softmax_dense", rows, N);
+  if (rc) return rc;
+  if (rows == 0) return HYC_OK;
+  if (!row_ptr || !y_hat) return fail(HYC_EFAULT, "hyc_softmax_dense: null buffer");
+  if (!aligned16(y_hat)) return fail(HYC_EINVAL, "hyc_softmax_dense: y_hat must be 16-byte aligned");
+  hipLaunchKernelGGL((k_softmax_rows<false>), dim3((unsigned)((rows + 3) / 4)), dim3(256), (size_t)N * 8, begin_launch(stream),
+                     static_cast<const uint16_t*>(nullptr), rows, N, row_ptr, cols, static_cast<const uint16_t*>(vals),
+                     static_cast<uint16_t*>(y_hat));
+  return check_launch("hyc_softmax_dense");
+}
+
+}  // extern "C"

@@ -339,3 +339,158 @@ def hadamard_bwd(g2d, src1, src2):
     check(_abi.load().hyc_hadamard_bwd(_p(g2d), _p(s1), _p(v1), _p(c1), ctypes.byref(d1), _p(s2), _p(v2), _p(c2),
                                        ctypes.byref(d2), M, H, _p(dx1), _p(dx2), _stream()))
     return dx1, dx2
+
+
+# ----------------------------------------------------------------------------------------------------
+# weight gradient
+# ----------------------------------------------------------------------------------------------------
+def gradw_gemm(dy2d, src, out_dtype=BF16, alpha=1.0, out=None, beta=0.0):
+    """dW [N_out, H] = alpha * dy^T @ x_hat (+ beta * out); src as for rmsnorm_bwd"""
+    _need(dy2d, BF16, "grad_output")
+    M, N_out = dy2d.shape
+    stored, vals, scales, d = _source(src)
+    H = src.H if isinstance(src, (ChannelCompressed, ThresholdCompressed)) else stored.shape[-1]
+    lib = _abi.load()
+    if out is None:
+        out = torch.empty((N_out, H), dtype=out_dtype, device=dy2d.device)
+    ws_bytes = lib.hyc_gradw_workspace_bytes(M, N_out, H)
+    ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=dy2d.device) if ws_bytes else None
+    code = _abi.DTYPE_F32 if out.dtype == torch.float32 else _abi.DTYPE_BF16
+    check(lib.hyc_gradw_gemm(_p(dy2d), dy2d.stride(0), _p(stored), _p(vals), _p(scales), M, N_out, H, ctypes.byref(d),
+                             float(alpha), float(beta), _p(out), code, _p(ws), _stream()))
+    return out
+
+
+# ----------------------------------------------------------------------------------------------------
+# softmax
+# ----------------------------------------------------------------------------------------------------
+@dataclass
+class SparseRows:
+    """probabilities above the threshold, CSR over the flattened leading dims"""
+    row_ptr: torch.Tensor   # int32 [rows+1]
+    cols: torch.Tensor      # int32 [nnz]
+    vals: torch.Tensor      # bf16 [nnz]
+    shape: tuple
+
+    @property
+    def rows(self):
+        return self.row_ptr.numel() - 1
+
+
+def _csr_from_counts(lib, y2d, threshold, counts):
+    rows, N = y2d.shape
+    dev = y2d.device
+    row_ptr = torch.zeros(rows + 1, dtype=torch.int32, device=dev)
+    torch.cumsum(counts, 0, out=row_ptr[1:])
+    nnz = int(row_ptr[-1].item())
+    cols = torch.empty(nnz, dtype=torch.int32, device=dev)
+    vals = torch.empty(nnz, dtype=BF16, device=dev)
+    check(lib.hyc_softmax_fill(_p(y2d), rows, N, float(threshold), _p(row_ptr), _p(cols) if nnz else None,
+                               _p(vals) if nnz else None, _stream()))
+    return row_ptr, cols, vals
+
+
+def softmax_fwd(x, threshold=None):
+    """y = softmax(x, -1) bf16; with a threshold also the kept entries (y > bf16(threshold)) as SparseRows"""
+    _need(x, BF16, "x")
+    N = x.shape[-1]
+    x2 = x.reshape(-1, N)
+    rows = x2.shape[0]
+    lib = _abi.load()
+    y = torch.empty_like(x2)
+    if threshold is None:
+        check(lib.hyc_softmax_fwd(_p(x2), rows, N, 0.0, _p(y), None, _stream()))
+        return y.reshape(x.shape), None
+    counts = torch.empty(rows, dtype=torch.int32, device=x.device)
+    check(lib.hyc_softmax_fwd(_p(x2), rows, N, float(threshold), _p(y), _p(counts), _stream()))
+    row_ptr, cols, vals = _csr_from_counts(lib, y, threshold, counts)
+    return y.reshape(x.shape), SparseRows(row_ptr, cols, vals, tuple(x.shape))
+
+
+def softmax_sparsify(y, threshold):
+    """kept entries of already computed probabilities"""
+    _need(y, BF16, "y")
+    N = y.shape[-1]
+    y2 = y.reshape(-1, N)
+    lib = _abi.load()
+    counts = torch.empty(y2.shape[0], dtype=torch.int32, device=y.device)
+    check(lib.hyc_softmax_fwd(None, y2.shape[0], N, float(threshold), _p(y2), _p(counts), _stream()))
+    row_ptr, cols, vals = _csr_from_counts(lib, y2, threshold, counts)
+    return SparseRows(row_ptr, cols, vals, tuple(y.shape))
+
+
+def softmax_bwd(g, sp: SparseRows):
+    _need(g, BF16, "grad_output")
+    N = g.shape[-1]
+    g2 = g.reshape(-1, N)
+    dx = torch.empty_like(g2)
+    check(_abi.load().hyc_softmax_bwd(_p(g2), g2.shape[0], N, _p(sp.row_ptr), _p(sp.cols) if sp.cols.numel() else None,
+                                      _p(sp.vals) if sp.vals.numel() else None, _p(dx), _stream()))
+    return dx.reshape(g.shape)
+
+
+def softmax_dense(sp: SparseRows):
+    N = sp.shape[-1]
+    out = torch.empty((sp.rows, N), dtype=BF16, device=sp.row_ptr.device)
+    check(_abi.load().hyc_softmax_dense(sp.rows, N, _p(sp.row_ptr), _p(sp.cols) if sp.cols.numel() else None,
+                                        _p(sp.vals) if sp.vals.numel() else None, _p(out), _stream()))
+    return out.reshape(sp.shape)
+
+
+def sparse_rows_to_coo(sp: SparseRows):
+    """the sparse COO tensor `.to_sparse()` gives for the pruned probabilities (int64 indices, row-major)"""
+    counts = (sp.row_ptr[1:] - sp.row_ptr[:-1]).long()
+    rows = torch.repeat_interleave(torch.arange(sp.rows, device=counts.device), counts)
+    lead = []
+    for dim in reversed(sp.shape[:-1]):
+        lead.append(rows % dim)
+        rows = rows // dim
+    idx = torch.stack(list(reversed(lead)) + [sp.cols.long()])
+    return torch.sparse_coo_tensor(idx, sp.vals, sp.shape, is_coalesced=True)
+
+
+def coo_to_sparse_rows(coo):
+    coo = coo.coalesce()
+    shape = tuple(coo.shape)
+    idx = coo.indices()
+    rows = torch.zeros_like(idx[0])
+    for i, dim in enumerate(shape[:-1]):
+        rows = rows * dim + idx[i]
+    n_rows = 1
+    for dim in shape[:-1]:
+        n_rows *= dim
+    row_ptr = torch.zeros(n_rows + 1, dtype=torch.int32, device=idx.device)
+    if rows.numel():
+        torch.cumsum(torch.bincount(rows, minlength=n_rows), 0, out=row_ptr[1:])
+    return SparseRows(row_ptr, idx[-1].to(torch.int32).contiguous(), coo.values().to(BF16).contiguous(), shape)
+
+
+def softmax_sparse_coo(y, threshold):
+    return sparse_rows_to_coo(softmax_sparsify(y, threshold))
+
+
+def sparse_coo_to_dense(coo):
+    return softmax_dense(coo_to_sparse_rows(coo))
+
+
+def softmax_prune(y, threshold):
+    """y * (y > threshold) as a dense tensor (the reference's prune_softmax; not used by the softmax operator)"""
+    return softmax_dense(softmax_sparsify(y, threshold))
+
+
+# ----------------------------------------------------------------------------------------------------
+# low-rank base
+# ----------------------------------------------------------------------------------------------------
+def low_rank_update(l, r, x, subtract, out=None):
+    """out = bf16(x -/+ l @ r), x [B,S,H] (or [S,H]); in place when out is x"""
+    _need(x, BF16, "x")
+    _need(l, BF16, "l")
+    _need(r, BF16, "r")
+    S, H = x.shape[-2], x.shape[-1]
+    M = x.numel() // H
+    if l.shape[0] != S or r.shape[0] != l.shape[1] or r.shape[1] != H:
+        raise ValueError("Incompatible dimensions")
+    if out is None:
+        out = torch.empty_like(x)
+    check(_abi.load().hyc_low_rank_update(_p(l), _p(r), _p(x), _p(out), M, S, H, l.shape[1], 1 if subtract else 0, _stream()))
+    return out

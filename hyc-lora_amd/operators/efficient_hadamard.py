@@ -1,0 +1,93 @@
+"""Elementwise product with both operands saved compressed.  Reference: operators/efficient_hadamard.py:9-183."""
+import torch
+
+from .. import kernels as K
+from ._calibration import CompressionSite, as_rows, fold_statistics
+from .compress_function import compress_to_csr, get_statistics
+
+
+class EfficientMemoryHadamardFunc(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x1, x2, outlier_ratio_1, sub_outlier_ratio_1, sub_outlier_bit_1, sub_outlier_quantize_method_1,
+                outlier_ratio_2, sub_outlier_ratio_2, sub_outlier_bit_2, sub_outlier_quantize_method_2, rank, iteration,
+                static_value_1, static_value_2):
+        result = x1 * x2
+        stats = []
+        for x, ratio, sub, bit, method, static in (
+                (x1, outlier_ratio_1, sub_outlier_ratio_1, sub_outlier_bit_1, sub_outlier_quantize_method_1, static_value_1),
+                (x2, outlier_ratio_2, sub_outlier_ratio_2, sub_outlier_bit_2, sub_outlier_quantize_method_2, static_value_2)):
+            if iteration < 2:
+                outlier, L, R, scale = get_statistics(x, iteration, ratio, sub, bit, method, rank)
+            else:
+                outlier, L, scale, R = static[0], static[1], static[2], static[3]
+            c, shape = compress_to_csr(x, outlier, scale, bit, sub, L if rank > 0 else None, R if rank > 0 else None)
+            stats.append((outlier, L, R, scale, c, shape))
+        ctx.saved = (stats[0][4], stats[1][4])
+        ctx.shape = stats[0][5]
+        o1, L1, R1, s1 = stats[0][:4]
+        o2, L2, R2, s2 = stats[1][:4]
+        ctx.mark_non_differentiable(o1, o2, L1, R1, s1, L2, R2, s2)
+        return result, o1, L1, R1, s1, o2, L2, R2, s2
+
+    @staticmethod
+    def backward(ctx, grad_output, *unused):
+        g2, _ = as_rows(grad_output.to(torch.bfloat16))
+        d1, d2 = K.hadamard_bwd(g2, ctx.saved[0], ctx.saved[1])
+        return (d1.reshape(grad_output.shape), d2.reshape(grad_output.shape)) + (None,) * 12
+
+
+class _ChannelHadamardFunc(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x1, x2, plan1, plan2, bits1, bits2, group):
+        a, _ = as_rows(x1)
+        b, _ = as_rows(x2)
+        ctx.saved = (K.compress_channel(a, plan1, bits1, group), K.compress_channel(b, plan2, bits2, group))
+        return x1 * x2
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        g2, _ = as_rows(grad_output.to(torch.bfloat16))
+        d1, d2 = K.hadamard_bwd(g2, ctx.saved[0], ctx.saved[1])
+        return d1.reshape(grad_output.shape), d2.reshape(grad_output.shape), None, None, None, None, None
+
+
+class EfficientMemoryHadamard(torch.nn.Module):
+    def __init__(self, outlier_ratio_1: float = 0.01, sub_outlier_ratio_1: float = 0.2, sub_outlier_bit_1: int = 8,
+                 sub_outlier_quantize_method_1: str = 'per-tensor', outlier_ratio_2: float = 0.01,
+                 sub_outlier_ratio_2: float = 0.2, sub_outlier_bit_2: int = 8,
+                 sub_outlier_quantize_method_2: str = 'per-tensor', rank: int = 16, *, mode: str = "ref",
+                 group_size: int = 128):
+        super().__init__()
+        self.outlier_ratio_1, self.sub_outlier_ratio_1 = outlier_ratio_1, sub_outlier_ratio_1
+        self.sub_outlier_bit_1, self.sub_outlier_quantize_method_1 = sub_outlier_bit_1, sub_outlier_quantize_method_1
+        self.outlier_ratio_2, self.sub_outlier_ratio_2 = outlier_ratio_2, sub_outlier_ratio_2
+        self.sub_outlier_bit_2, self.sub_outlier_quantize_method_2 = sub_outlier_bit_2, sub_outlier_quantize_method_2
+        self.rank = rank
+        self.mode = mode
+        self.group_size = group_size
+        self.site_1 = CompressionSite(outlier_ratio_1, sub_outlier_ratio_1, sub_outlier_bit_1,
+                                      sub_outlier_quantize_method_1, rank, mode, group_size)
+        self.site_2 = CompressionSite(outlier_ratio_2, sub_outlier_ratio_2, sub_outlier_bit_2,
+                                      sub_outlier_quantize_method_2, rank, mode, group_size)
+        self.iteration = 0
+        self.static_value_1 = [None, None, None, None]
+        self.static_value_2 = [None, None, None, None]
+
+    def forward(self, x1, x2):
+        if self.mode == "hyc":
+            a, _ = as_rows(x1)
+            b, _ = as_rows(x2)
+            p1 = self.site_1.channel_plan(a, self.iteration)
+            p2 = self.site_2.channel_plan(b, self.iteration)
+            result = _ChannelHadamardFunc.apply(x1, x2, p1, p2, self.sub_outlier_bit_1, self.sub_outlier_bit_2, self.group_size)
+            self.iteration += 1
+            return result
+        result, o1, L1, R1, s1, o2, L2, R2, s2 = EfficientMemoryHadamardFunc.apply(
+            x1, x2, self.outlier_ratio_1, self.sub_outlier_ratio_1, self.sub_outlier_bit_1,
+            self.sub_outlier_quantize_method_1, self.outlier_ratio_2, self.sub_outlier_ratio_2, self.sub_outlier_bit_2,
+            self.sub_outlier_quantize_method_2, self.rank, self.iteration, self.static_value_1, self.static_value_2)
+        if self.iteration < 2:
+            self.static_value_1 = fold_statistics(self.static_value_1, self.iteration, o1, L1, s1, R1)
+            self.static_value_2 = fold_statistics(self.static_value_2, self.iteration, o2, L2, s2, R2)
+        self.iteration += 1
+        return result

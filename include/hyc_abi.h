@@ -149,6 +149,34 @@ int hyc_hadamard_bwd(const void* g, const void* stored1, const void* vals1, cons
                      const void* stored2, const void* vals2, const void* scales2, const hyc_desc* d2, int64_t M,
                      int64_t H, void* dx1, void* dx2, void* stream);
 
+/* ---- softmax -------------------------------------------------------------------------------- */
+/* x bf16 [rows, N] -> y = softmax(x, -1) bf16 and counts[r] = #{j : y[r,j] > bf16(threshold)} (counts may be
+ * NULL).  With x == NULL, y is taken as given and only the counts are produced. */
+int hyc_softmax_fwd(const void* x, int64_t rows, int64_t N, float threshold, void* y, int32_t* counts, void* stream);
+/* the kept probabilities as CSR: row_ptr int32 [rows+1] (exclusive prefix sums of counts), cols ascending per row */
+int hyc_softmax_fill(const void* y, int64_t rows, int64_t N, float threshold, const int32_t* row_ptr, int32_t* cols,
+                     void* vals, void* stream);
+/* dx = (g - sum_j g_j*yh_j) * yh, yh = the CSR probabilities (zero elsewhere) */
+int hyc_softmax_bwd(const void* g, int64_t rows, int64_t N, const int32_t* row_ptr, const int32_t* cols,
+                    const void* vals, void* dx, void* stream);
+/* yh as a dense bf16 [rows, N] matrix */
+int hyc_softmax_dense(int64_t rows, int64_t N, const int32_t* row_ptr, const int32_t* cols, const void* vals,
+                      void* y_hat, void* stream);
+
+/* ---- weight gradient ------------------------------------------------------------------------- */
+/* out[n, h] = alpha * sum_m dy[m, n] * x_hat[m, h] + beta * out[n, h]; dy bf16 [M, N_out] with row stride ldy,
+ * x_hat dequantised on the fly (channel mode) or read as bf16 (HYC_MODE_DENSE); out [N_out, H] bf16 or fp32.
+ * workspace: hyc_gradw_workspace_bytes() bytes of device memory (may be 0 -> NULL). */
+int64_t hyc_gradw_workspace_bytes(int64_t M, int64_t N_out, int64_t H);
+int hyc_gradw_gemm(const void* dy, int64_t ldy, const void* stored, const void* vals, const void* scales, int64_t M,
+                   int64_t N_out, int64_t H, const hyc_desc* d, float alpha, float beta, void* out, int32_t out_dtype,
+                   void* workspace, void* stream);
+
+/* ---- low-rank base ----------------------------------------------------------------------------- */
+/* out[m, :] = bf16(x[m, :] -/+ L[m mod S, :] @ R); L bf16 [S, rank], R bf16 [rank, H]; out may alias x */
+int hyc_low_rank_update(const void* L, const void* R, const void* x, void* out, int64_t M, int64_t S, int64_t H,
+                        int32_t rank, int32_t subtract, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
