@@ -1,0 +1,150 @@
+"""CPU-only checks of the boundary: the shared library loads, exports every symbol include/hyc_abi.h declares,
+rejects bad arguments with the documented codes without touching a GPU, and the host-side calibration logic
+follows the reference's running-mean protocol."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import ROOT, bits_equal, from_bits
+
+
+@pytest.fixture(scope="module")
+def abi(hyc):
+    if not os.path.exists(hyc._abi.LIB_PATH):
+        pytest.skip("library not built (python hyc-lora_amd/build.py)")
+    return hyc._abi
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "hyc_abi.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(hyc_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported_and_bound(abi):
+    lib = abi.load()
+    names = declared_symbols()
+    assert len(names) >= 20
+    for n in names:
+        assert hasattr(lib, n), n
+        assert n in abi.SIGNATURES, "no ctypes prototype for " + n
+    assert sorted(abi.SIGNATURES) == names
+    assert lib.hyc_abi_version() == 1
+
+
+def test_desc_layout_matches_header(abi):
+    d = abi.HycDesc
+    assert (d.mode.offset, d.bits.offset, d.group.offset, d.k.offset) == (0, 4, 8, 12)
+    assert d.chan_plan.offset == 16 and d.threshold.offset == 24 and d.scale.offset == 32
+    assert d.scale_stride_token.offset == 40 and d.S.offset == 56 and d.L.offset == 64 and d.rank.offset == 80
+    assert d.csr_row_ptr.offset == 88 and ctypes.sizeof(d) == 112
+
+
+def test_shape_queries(abi):
+    lib = abi.load()
+    assert lib.hyc_check_shape(4096, 4, 128, abi.MODE_CHANNEL) == 0
+    assert lib.hyc_check_shape(11008, 2, 64, abi.MODE_CHANNEL) == 0
+    assert lib.hyc_check_shape(4100, 4, 128, abi.MODE_CHANNEL) == abi.ENOTSUP
+    assert b"multiple of 16" in lib.hyc_last_error()
+    assert lib.hyc_check_shape(4096, 3, 128, abi.MODE_CHANNEL) == abi.ENOTSUP
+    assert lib.hyc_check_shape(4096, 4, 96, abi.MODE_CHANNEL) == abi.ENOTSUP
+    assert lib.hyc_check_shape(4096, 4, 0, abi.MODE_THRESHOLD) == 0
+    assert lib.hyc_check_shape(0, 4, 128, abi.MODE_CHANNEL) == abi.EINVAL
+    assert lib.hyc_check_shape(4096, 4, 128, 7) == abi.EINVAL
+    assert lib.hyc_stored_row_bytes(4096, 4) == 2048 and lib.hyc_stored_row_bytes(11008, 2) == 2752
+    assert lib.hyc_rmsnorm_bwd_partials(0, 4096) == 0 and lib.hyc_rmsnorm_bwd_partials(4096, 4096) >= 1
+    assert lib.hyc_gradw_workspace_bytes(4096, 4096, 4096) == 0
+    assert lib.hyc_gradw_workspace_bytes(4096, 16, 4096) % (16 * 4096 * 4) == 0
+
+
+def test_argument_errors_without_a_gpu(abi):
+    """every entry point validates before it launches: these calls return before any HIP call is made"""
+    lib = abi.load()
+    d = abi.HycDesc()
+    d.mode, d.bits, d.group, d.k = abi.MODE_CHANNEL, 4, 128, 0
+    null = None
+    assert lib.hyc_compress(null, 4, 4096, None, null, null, null, null, null) == abi.EFAULT
+    assert lib.hyc_compress(null, 4, 4096, ctypes.byref(d), null, null, null, null, null) == abi.EFAULT      # no plan
+    d.chan_plan = 0x1000
+    assert lib.hyc_compress(null, 4, 4096, ctypes.byref(d), null, null, null, null, null) == abi.EFAULT      # null x
+    assert lib.hyc_compress(null, -1, 4096, ctypes.byref(d), null, null, null, null, null) == abi.EINVAL
+    assert lib.hyc_compress(null, 0, 4096, ctypes.byref(d), null, null, null, null, null) == 0               # empty input
+    assert lib.hyc_compress(0x1001, 4, 4096, ctypes.byref(d), 0x2000, null, 0x3000, null, null) == abi.EINVAL  # misaligned
+    d.bits = 3
+    assert lib.hyc_decompress(null, null, null, 4, 4096, ctypes.byref(d), null, null) == abi.ENOTSUP
+    d.bits = 4
+    t = abi.HycDesc()
+    t.mode, t.bits = abi.MODE_THRESHOLD, 8
+    assert lib.hyc_rmsnorm_bwd(null, null, null, null, null, 0, null, 4, 4096, ctypes.byref(t), 1, null, null, 0x10, null) == abi.ENOTSUP
+    assert lib.hyc_act_bwd(9, null, null, null, null, 4, 4096, ctypes.byref(d), null, null) == abi.EINVAL
+    assert lib.hyc_gradw_gemm(null, 20, null, null, null, 4, 20, 4096, ctypes.byref(d), 1.0, 0.0, 0x10, 0, null, null) == abi.ENOTSUP
+    assert lib.hyc_softmax_fwd(null, 4, 12, 0.0, 0x10, null, null) == abi.ENOTSUP
+    assert lib.hyc_low_rank_update(null, null, null, null, 4, 0, 64, 2, 1, null) == abi.EINVAL
+    assert lib.hyc_select_channels(null, 4096, 5000, null, null, null) == abi.EINVAL
+    with pytest.raises(NotImplementedError):
+        abi.check(abi.ENOTSUP)
+    with pytest.raises(ValueError):
+        abi.check(abi.EINVAL)
+
+
+def test_launchers_refuse_cpu_tensors(hyc, abi):
+    K = hyc.kernels
+    with pytest.raises(ValueError, match="CUDA"):
+        K.channel_absmax(torch.zeros(4, 64, dtype=torch.bfloat16))
+    assert K.num_outlier_channels(4096, 0.01) == 41 and K.num_outlier_channels(11008, 0.01) == 110
+    assert K.num_outlier_channels(4096, 0.005) == 20
+    assert K.scale_strides(torch.zeros(()), 16, 64) == (0, 0)
+    assert K.scale_strides(torch.zeros(1, 64), 16, 64) == (0, 1)
+    assert K.scale_strides(torch.zeros(16, 1), 16, 64) == (1, 0)
+    with pytest.raises(ValueError):
+        K.scale_strides(torch.zeros(3, 5), 16, 64)
+
+
+def test_running_mean_protocol_against_reference(hyc, golden_modules):
+    """fold_statistics (host logic of every module) reproduces the reference modules' static values after calls 0
+    and 1 when fed the per-call statistics the reference computed"""
+    from oracle import hyc_oracle as O
+    fold = hyc.operators._calibration.fold_statistics
+    gm = golden_modules
+    tag = "silu_b8_pt_r2"
+    static = [None] * 4
+    for call in range(2):
+        p = f"{tag}_call{call}_"
+        x = from_bits(gm[p + "x0"])
+        torch.manual_seed(900 + call)
+        thr, L, R, scale = O.get_statistics(x, call, 0.05, 1.0, 8, 'per-token', 2)
+        static = fold(static, call, thr, L, scale, R)
+        assert torch.equal(static[0], from_bits(gm[p + "s0_thr"]))
+        assert bits_equal(static[1], from_bits(gm[p + "s0_L"])) and bits_equal(static[3], from_bits(gm[p + "s0_R"]))
+        assert bits_equal(static[2], from_bits(gm[p + "s0_scale"]))
+
+
+def test_module_constructors_mirror_the_reference(hyc):
+    ops = hyc.operators
+    m = ops.EfficientMemoryRMSNorm(64, eps=1e-6, elementwise_affine=True, bias=False, outlier_ratio=0.005,
+                                   sub_outlier_ratio=1.0, sub_outlier_bit=8, sub_outlier_quantize_method='per-channel', rank=2)
+    assert isinstance(m, torch.nn.LayerNorm) and m.iteration == 0 and m.static_value == [None] * 4 and m.bias is None
+    l = ops.EfficientMemoryLinear(128, 16, bias=False, outlier_ratio=0.01, sub_outlier_ratio=1.0, sub_outlier_bit=2,
+                                  sub_outlier_quantize_method='per-token', rank=0)
+    assert isinstance(l, torch.nn.Linear) and l.weight.shape == (16, 128)
+    for cls in (ops.EfficientMemorySiLU, ops.EfficientMemoryGELU):
+        a = cls(outlier_ratio=0.01, sub_outlier_ratio=0.2, sub_outlier_bit=8, sub_outlier_quantize_method='per-tensor', rank=16)
+        assert a.iteration == 0 and a.static_value == [None] * 4
+    s = ops.EfficientMemorySoftmax(outlier_ratio=0.05)
+    assert s.static_value is None and s.outlier_ratio == 0.05
+    h = ops.EfficientMemoryHadamard()
+    assert h.static_value_1 == [None] * 4 and h.sub_outlier_bit_2 == 8
+    with pytest.raises(ValueError):
+        ops.EfficientMemorySiLU(mode="bogus")
+    cf = ops.compress_function
+    for name in ("true_divide_outlier_suboutlier_svd_compress", "true_divide_outlier_suboutlier_svd_decompress",
+                 "true_compress_softmax", "true_decompress_softmax", "prune_softmax", "get_statistics",
+                 "get_statistics_softmax", "pad_cut_L", "hidden_to_head_shape", "head_to_hidden_shape"):
+        assert callable(getattr(cf, name))
+    assert callable(ops.fused_compression.low_rank_extraction) and callable(ops.fused_compression.low_rank_addition)
+    x = torch.arange(2 * 3 * 8, dtype=torch.float32).reshape(2, 3, 8)
+    assert torch.equal(cf.head_to_hidden_shape(cf.hidden_to_head_shape(x, 2)), x)
