@@ -28,6 +28,7 @@ class HycDesc(ctypes.Structure):
         ("L", c_ptr), ("R", c_ptr),
         ("rank", c_i32), ("reserved", c_i32),
         ("csr_row_ptr", c_ptr), ("csr_cols", c_ptr), ("csr_vals", c_ptr),
+        ("chan_idx", c_ptr),
     ]
 
 

@@ -15,7 +15,9 @@ int make_chan_args(const hyc_desc* d, const RowGeom& g, ChanArgs* a, int* lpg) {
   if (rc) return rc;
   if (d->k < 0 || d->k > g.H || d->k > 65535) return fail(HYC_EINVAL, "k=%d out of range for H=%lld", d->k, (long long)g.H);
   if (!d->chan_plan) return fail(HYC_EFAULT, "channel mode needs chan_plan (from hyc_select_channels)");
+  if (d->k > 0 && !d->chan_idx) return fail(HYC_EFAULT, "channel mode needs chan_idx (from hyc_select_channels) when k > 0");
   a->plan = d->chan_plan;
+  a->idx = d->chan_idx;
   a->k = d->k;
   a->groups_per_row = (int)(g.H / d->group);
   a->chunk_to_group_shift = ilog2(*lpg);

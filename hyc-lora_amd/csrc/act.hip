@@ -11,37 +11,167 @@ namespace hyc {
 
 constexpr int ACT_MUL = 100;   // dx = g * x_hat (one half of the Hadamard backward)
 
-__device__ __forceinline__ float silu_grad(float x, float g) {
-  const float s = bfr(1.0f / (1.0f + expf(-x)));
-  const float a = bfr(x + 1.0f);
-  const float b = bfr(x * s);
-  const float c = bfr(a - b);
-  const float d = bfr(s * c);
-  return bfr(d * g);
+// ---- math helpers ----------------------------------------------------------------------------------
+// round two fp32 values to bf16 with one v_cvt_pk_bf16_f32 and widen them again
+__device__ __forceinline__ void bfr2(float& a, float& b) {
+  const uint32_t pk = pack_bf16(a, b);
+  a = bf_lo(pk);
+  b = bf_hi(pk);
+}
+// e^x to about 2 ulp: v_exp_f32 on x*log2(e) with the rounding error of that product (and the low part of
+// log2(e)) applied as a first-order correction.  Arguments far below the fp32 range give 0, far above give inf.
+__device__ __forceinline__ float exp_fast(float x) {
+  const float L2E = 1.44269502162933349609375f, L2E_LO = 1.925963033500e-08f;
+  const float t = x * L2E;
+  float r = __builtin_fmaf(x, L2E, -t);
+  r = __builtin_fmaf(x, L2E_LO, r);
+  const float e = __builtin_amdgcn_exp2f(t);
+  return __builtin_fmaf(e, r * 0.693147182464599609375f, e);
+}
+// 1 / d for finite positive d to about 1 ulp; 0 for d = inf
+__device__ __forceinline__ float rcp_pos(float d) {
+  float r = __builtin_amdgcn_rcpf(d);
+  r = __builtin_fmaf(__builtin_fmaf(-d, r, 1.0f), r, r);
+  return d < 3.0e38f ? r : 0.f;
+}
+__device__ __forceinline__ float sigmoid_f(float x) { return rcp_pos(1.0f + exp_fast(-x)); }
+// tanh: odd polynomial below 0.05 (where 1 - e^{-2|y|} cancels), (1 - e)/(1 + e) above
+__device__ __forceinline__ float tanh_f(float y) {
+  const float a = __builtin_fabsf(y);
+  const float e = exp_fast(-2.0f * a);
+  const float big = (1.0f - e) * rcp_pos(1.0f + e);
+  const float y2 = a * a;
+  float p = __builtin_fmaf(y2, 0.13333333333f, -0.33333333333f);
+  p = __builtin_fmaf(y2 * p, a, a);
+  const float t = a < 0.05f ? p : big;
+  return __builtin_copysignf(t, y);
 }
 
-__device__ __forceinline__ float gelu_tanh_grad(float x, float g) {
+// two elements at a time: every intermediate is rounded to bf16 where torch rounds it, pairs share the conversion
+__device__ __forceinline__ void silu_grad2(float x0, float x1, float g0, float g1, float& o0, float& o1) {
+  float s0 = sigmoid_f(x0), s1 = sigmoid_f(x1);
+  bfr2(s0, s1);
+  float a0 = x0 + 1.0f, a1 = x1 + 1.0f;
+  bfr2(a0, a1);
+  float b0 = x0 * s0, b1 = x1 * s1;
+  bfr2(b0, b1);
+  float c0 = a0 - b0, c1 = a1 - b1;
+  bfr2(c0, c1);
+  float d0 = s0 * c0, d1 = s1 * c1;
+  bfr2(d0, d1);
+  o0 = d0 * g0;           // the caller's pack8 performs the last rounding
+  o1 = d1 * g1;
+}
+
+__device__ __forceinline__ void gelu_tanh_grad2(float x0, float x1, float g0, float g1, float& o0, float& o1) {
   const float gamma = 0.7978845608028654f;   // sqrt(2/pi)
   const float kappa = 0.044715f;
   const float kappa3 = (float)(3 * 0.044715);
-  const float x2 = bfr(x * x);
-  const float x3 = bfr(x2 * x);
-  const float inner = bfr(gamma * bfr(x + bfr(kappa * x3)));
-  const float t = bfr(tanhf(inner));
-  const float A = bfr(1.0f + t);
-  const float B = bfr(1.0f - bfr(t * t));
-  const float C = bfr(B * gamma);
-  const float E = bfr(1.0f + bfr(kappa3 * x2));
-  const float G = bfr(x * bfr(C * E));
-  const float I = bfr(0.5f * bfr(A + G));
-  return bfr(I * g);
+  float q0 = x0 * x0, q1 = x1 * x1;                      // x**2
+  bfr2(q0, q1);
+  float c0 = q0 * x0, c1 = q1 * x1;                      // x**3 = bf16(bf16(x*x)*x)
+  bfr2(c0, c1);
+  float k0 = kappa * c0, k1 = kappa * c1;
+  bfr2(k0, k1);
+  float s0 = x0 + k0, s1 = x1 + k1;
+  bfr2(s0, s1);
+  float i0 = gamma * s0, i1 = gamma * s1;
+  bfr2(i0, i1);
+  float t0 = tanh_f(i0), t1 = tanh_f(i1);
+  bfr2(t0, t1);
+  float A0 = 1.0f + t0, A1 = 1.0f + t1;
+  bfr2(A0, A1);
+  float u0 = t0 * t0, u1 = t1 * t1;
+  bfr2(u0, u1);
+  float B0 = 1.0f - u0, B1 = 1.0f - u1;
+  bfr2(B0, B1);
+  float C0 = B0 * gamma, C1 = B1 * gamma;
+  bfr2(C0, C1);
+  float D0 = kappa3 * q0, D1 = kappa3 * q1;
+  bfr2(D0, D1);
+  float E0 = 1.0f + D0, E1 = 1.0f + D1;
+  bfr2(E0, E1);
+  float F0 = C0 * E0, F1 = C1 * E1;
+  bfr2(F0, F1);
+  float G0 = x0 * F0, G1 = x1 * F1;
+  bfr2(G0, G1);
+  float H0 = A0 + G0, H1 = A1 + G1;
+  bfr2(H0, H1);
+  float I0 = 0.5f * H0, I1 = 0.5f * H1;                  // exact
+  o0 = I0 * g0;
+  o1 = I1 * g1;
 }
 
 template <int ACT>
-__device__ __forceinline__ float act_grad(float x, float g) {
-  if (ACT == HYC_ACT_SILU) return silu_grad(x, g);
-  if (ACT == HYC_ACT_GELU_TANH) return gelu_tanh_grad(x, g);
-  return bfr(g * x);
+__device__ __forceinline__ void act_grad8(const float (&x)[8], const float (&g)[8], float (&o)[8]) {
+#pragma unroll
+  for (int j = 0; j < 8; j += 2) {
+    if (ACT == HYC_ACT_SILU) silu_grad2(x[j], x[j + 1], g[j], g[j + 1], o[j], o[j + 1]);
+    else if (ACT == HYC_ACT_GELU_TANH) gelu_tanh_grad2(x[j], x[j + 1], g[j], g[j + 1], o[j], o[j + 1]);
+    else { o[j] = g[j] * x[j]; o[j + 1] = g[j + 1] * x[j + 1]; }
+  }
+}
+
+// fast path: channel source, every lane owns one chunk per segment, next row requested ahead
+template <int BITS, int ACT, int MAXT>
+__global__ void __launch_bounds__(MAXT)
+k_act_bwd_fast(const uint16_t* __restrict__ g, const uint8_t* __restrict__ stored, const uint16_t* __restrict__ vals,
+               const uint16_t* __restrict__ scales, int64_t M, int64_t H, ChanArgs ca, uint16_t* __restrict__ dx) {
+  constexpr int NSEG = Q<BITS>::NSEG;
+  const int c = threadIdx.x, CPS = blockDim.x;
+  const int64_t SEG = (int64_t)CPS * 8;
+  const int seg_groups = CPS >> ca.chunk_to_group_shift;
+  uint32_t plan[NSEG];
+#pragma unroll
+  for (int i = 0; i < NSEG; ++i) plan[i] = ca.plan[i * CPS + c];
+  ChunkOutliers<NSEG> co;
+  co.init(plan);
+  const int64_t stride = gridDim.x;
+  int64_t row = blockIdx.x;
+  const uint16_t* gp = g + row * H + 8 * c;
+  uint16_t* dxp = dx + row * H + 8 * c;
+  const uint8_t* sp = stored + row * SEG + 8 * c;
+  const uint16_t* vp = vals + row * ca.k;
+  const uint16_t* scp = scales + row * ca.groups_per_row + (c >> ca.chunk_to_group_shift);
+  const int64_t xstep = stride * H, sstep = stride * SEG, vstep = stride * ca.k, scstep = stride * ca.groups_per_row;
+  uint2 pk = make_uint2(0, 0);
+  uint4 graw[NSEG];
+  uint32_t sc[NSEG];   // one register each: a packed pair would be assembled right after the load and stall on it
+  uint32_t o0[NSEG], o1[NSEG];
+  if (row < M) {
+    pk = *reinterpret_cast<const uint2*>(sp);
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) { graw[i] = *reinterpret_cast<const uint4*>(gp + i * SEG); sc[i] = scp[i * seg_groups]; }
+    co.request(vp, o0, o1);
+  }
+  for (; row < M; row += stride) {
+    uint2 pk_n = make_uint2(0, 0);
+    uint4 g_n[NSEG];
+    uint32_t sc_n[NSEG], o0_n[NSEG], o1_n[NSEG];
+    if (row + stride < M) {
+      pk_n = *reinterpret_cast<const uint2*>(sp + sstep);
+#pragma unroll
+      for (int i = 0; i < NSEG; ++i) {
+        g_n[i] = *reinterpret_cast<const uint4*>(gp + xstep + i * SEG);
+        sc_n[i] = scp[scstep + i * seg_groups];
+      }
+      co.request(vp + vstep, o0_n, o1_n);
+    }
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) {
+      float xv[8], gv[8], o[8];
+      const float sf = bf_to_f((uint16_t)sc[i]);
+      if (!co.many) unpack8(co.splice(i, dequant8<BITS>(pk.x, pk.y, i, sf), o0[i], o1[i], sf), xv);
+      else unpack8(decode_seg<BITS>(pk.x, pk.y, i, sf, plan[i], vp), xv);
+      unpack8(graw[i], gv);
+      act_grad8<ACT>(xv, gv, o);
+      store_stream(dxp + i * SEG, pack8(o));
+    }
+    pk = pk_n;
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) { graw[i] = g_n[i]; sc[i] = sc_n[i]; o0[i] = o0_n[i]; o1[i] = o1_n[i]; }
+    gp += xstep; dxp += xstep; sp += sstep; vp += vstep; scp += scstep;
+  }
 }
 
 // SRC 0 = channel-compressed, 2 = dense bf16
@@ -68,8 +198,7 @@ k_act_bwd(const uint16_t* __restrict__ g, const uint8_t* __restrict__ stored, co
           if (SRC == 0) decode_chan<BITS>(pk.x, pk.y, i, c, CPS, ca, vals + row * ca.k, scales + row * ca.groups_per_row, xv);
           else unpack8(*reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(stored) + row * H + col), xv);
           unpack8(graw[i], gv);
-#pragma unroll
-          for (int j = 0; j < 8; ++j) o[j] = act_grad<ACT>(xv[j], gv[j]);
+          act_grad8<ACT>(xv, gv, o);
           *reinterpret_cast<uint4*>(dx + row * H + col) = pack8(o);
         }
       }
@@ -98,6 +227,26 @@ static int launch_act(const void* g, const void* stored, const void* vals, const
   const int64_t cap = 256 * (geo.threads >= 512 ? 3 : 8);
   const int grid = (int)(M < cap ? M : cap);
   hipStream_t st = begin_launch(stream);
+  if (d->mode == HYC_MODE_CHANNEL && geo.iters == 1 && geo.cps == geo.threads && d->bits != 1) {
+#define HYC_ACT_FAST(B_)                                                                                       \
+  do {                                                                                                         \
+    if (geo.threads <= 256)                                                                                    \
+      hipLaunchKernelGGL((k_act_bwd_fast<B_, ACT, 256>), dim3(grid), dim3(geo.threads), 0, st,                 \
+                         static_cast<const uint16_t*>(g), static_cast<const uint8_t*>(stored),                 \
+                         static_cast<const uint16_t*>(vals), static_cast<const uint16_t*>(scales), M, H, ca,   \
+                         static_cast<uint16_t*>(dx));                                                          \
+    else                                                                                                       \
+      hipLaunchKernelGGL((k_act_bwd_fast<B_, ACT, 1024>), dim3(grid), dim3(geo.threads), 0, st,                \
+                         static_cast<const uint16_t*>(g), static_cast<const uint8_t*>(stored),                 \
+                         static_cast<const uint16_t*>(vals), static_cast<const uint16_t*>(scales), M, H, ca,   \
+                         static_cast<uint16_t*>(dx));                                                          \
+  } while (0)
+    if (d->bits == 2) HYC_ACT_FAST(2);
+    else if (d->bits == 4) HYC_ACT_FAST(4);
+    else HYC_ACT_FAST(8);
+#undef HYC_ACT_FAST
+    return check_launch(who);
+  }
 #define HYC_ACT_LAUNCH(B_, S_)                                                                            \
   hipLaunchKernelGGL((k_act_bwd<B_, S_, ACT>), dim3(grid), dim3(geo.threads), 0, st,                      \
                      static_cast<const uint16_t*>(g), static_cast<const uint8_t*>(stored),                \

@@ -1,5 +1,7 @@
 // Standalone compress / decompress of a [M, H] bf16 activation, and the element-threshold outliers as CSR.
 // One workgroup walks rows (grid-stride); within a row the chunk mapping of row_codec.hpp applies.
+#include <stdlib.h>
+
 #include "abi_util.hpp"
 #include "row_kernels.hpp"
 
@@ -51,12 +53,136 @@ k_decompress_chan(const uint8_t* __restrict__ stored, const uint16_t* __restrict
         const uint2 w = *reinterpret_cast<const uint2*>(sr + 8 * c);
 #pragma unroll
         for (int i = 0; i < NSEG; ++i) {
-          float v[8];
-          decode_chan<BITS>(w.x, w.y, i, c, CPS, a, vr, scr, v);
-          *reinterpret_cast<uint4*>(xr + i * SEG + 8 * c) = pack8(v);
+          *reinterpret_cast<uint4*>(xr + i * SEG + 8 * c) = decode_chan_pk<BITS>(w.x, w.y, i, c, CPS, a, vr, scr);
         }
       }
     }
+  }
+}
+
+// Fast paths: every lane owns exactly one chunk per segment (CPS == blockDim.x), the group width is a template
+// parameter, plan words are loaded once, pointers advance by a constant and the next row is requested before the
+// current one is processed.
+template <int BITS, int LPGT, int MAXT>
+__global__ void __launch_bounds__(MAXT)
+k_compress_chan_fast(const uint16_t* __restrict__ x, int64_t M, int64_t H, ChanArgs a, uint8_t* __restrict__ stored,
+                     uint16_t* __restrict__ vals, uint16_t* __restrict__ scales) {
+  constexpr int NSEG = Q<BITS>::NSEG;
+  const int c = threadIdx.x, CPS = blockDim.x;
+  const int64_t SEG = (int64_t)CPS * 8;
+  const bool leader = (c & (LPGT - 1)) == 0;
+  const int seg_groups = CPS >> a.chunk_to_group_shift;
+  uint32_t km[NSEG][4];
+  {
+    uint32_t plan[NSEG];
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) plan[i] = a.plan[i * CPS + c];
+    ChunkOutliers<NSEG> co;
+    co.init(plan);
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) co.keep_masks(i, km[i]);
+  }
+  const bool gather = c < a.k;                          // thread c copies outlier channel idx[c] (+ CPS, ...) to vals
+  const int idx0 = gather ? a.idx[c] : 0;
+  const int64_t stride = gridDim.x;
+  int64_t row = blockIdx.x;
+  const uint16_t* xrow = x + row * H;
+  const uint16_t* xp = xrow + 8 * c;
+  uint8_t* sp = stored + row * SEG + 8 * c;
+  uint16_t* vp = vals + row * a.k;
+  uint16_t* scp = scales + row * a.groups_per_row + (c >> a.chunk_to_group_shift);
+  const int64_t xstep = stride * H, sstep = stride * SEG, vstep = stride * a.k, scstep = stride * a.groups_per_row;
+  uint4 raw[NSEG];
+  uint16_t o = 0;
+  if (row < M) {
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) raw[i] = *reinterpret_cast<const uint4*>(xp + i * SEG);
+    if (gather) o = xrow[idx0];
+  }
+  for (; row < M; row += stride) {
+    uint4 nxt[NSEG];
+    uint16_t o_n = 0;
+    if (row + stride < M) {
+#pragma unroll
+      for (int i = 0; i < NSEG; ++i) nxt[i] = *reinterpret_cast<const uint4*>(xp + xstep + i * SEG);
+      if (gather) o_n = xrow[xstep + idx0];
+    }
+    uint32_t lo = 0, hi = 0;
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) {
+      float v[8];
+      unpack8(make_uint4(raw[i].x & km[i][0], raw[i].y & km[i][1], raw[i].z & km[i][2], raw[i].w & km[i][3]), v);
+      uint32_t cl, ch;
+      const float s = quant_seg<BITS, LPGT>(v, LPGT, cl, ch);
+      if (leader) scp[i * seg_groups] = f_to_bf(s);
+      if (BITS == 8) { lo = cl; hi = ch; }
+      else { lo |= cl << (i * BITS); hi |= ch << (i * BITS); }
+    }
+    *reinterpret_cast<uint2*>(sp) = make_uint2(lo, hi);
+    if (gather) {
+      vp[c] = o;
+      for (int t = c + CPS; t < a.k; t += CPS) vp[t] = xrow[a.idx[t]];   // only when k exceeds the workgroup size
+    }
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) raw[i] = nxt[i];
+    o = o_n;
+    xrow += xstep; xp += xstep; sp += sstep; vp += vstep; scp += scstep;
+  }
+}
+
+template <int BITS, int MAXT>
+__global__ void __launch_bounds__(MAXT)
+k_decompress_chan_fast(const uint8_t* __restrict__ stored, const uint16_t* __restrict__ vals,
+                       const uint16_t* __restrict__ scales, int64_t M, int64_t H, ChanArgs a, uint16_t* __restrict__ xhat) {
+  constexpr int NSEG = Q<BITS>::NSEG;
+  const int c = threadIdx.x, CPS = blockDim.x;
+  const int64_t SEG = (int64_t)CPS * 8;
+  const int seg_groups = CPS >> a.chunk_to_group_shift;
+  uint32_t plan[NSEG];
+#pragma unroll
+  for (int i = 0; i < NSEG; ++i) plan[i] = a.plan[i * CPS + c];
+  ChunkOutliers<NSEG> co;
+  co.init(plan);
+  const int64_t stride = gridDim.x;
+  int64_t row = blockIdx.x;
+  const uint8_t* sp = stored + row * SEG + 8 * c;
+  const uint16_t* vp = vals + row * a.k;
+  const uint16_t* scp = scales + row * a.groups_per_row + (c >> a.chunk_to_group_shift);
+  uint16_t* xp = xhat + row * H + 8 * c;
+  const int64_t xstep = stride * H, sstep = stride * SEG, vstep = stride * a.k, scstep = stride * a.groups_per_row;
+  uint2 pk = make_uint2(0, 0);
+  uint32_t sc[NSEG];   // one register each: a packed pair would be assembled right after the load and stall on it
+  uint32_t o0[NSEG], o1[NSEG];
+  if (row < M) {
+    pk = *reinterpret_cast<const uint2*>(sp);
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) sc[i] = scp[i * seg_groups];
+    co.request(vp, o0, o1);
+  }
+  for (; row < M; row += stride) {
+    uint2 pk_n = make_uint2(0, 0);
+    uint32_t sc_n[NSEG], o0_n[NSEG], o1_n[NSEG];
+    if (row + stride < M) {
+      pk_n = *reinterpret_cast<const uint2*>(sp + sstep);
+#pragma unroll
+      for (int i = 0; i < NSEG; ++i) sc_n[i] = scp[scstep + i * seg_groups];
+      co.request(vp + vstep, o0_n, o1_n);
+    }
+    if (!co.many) {
+#pragma unroll
+      for (int i = 0; i < NSEG; ++i) {
+        const float sf = bf_to_f((uint16_t)sc[i]);
+        store_stream(xp + i * SEG, co.splice(i, dequant8<BITS>(pk.x, pk.y, i, sf), o0[i], o1[i], sf));
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NSEG; ++i)
+        store_stream(xp + i * SEG, decode_seg<BITS>(pk.x, pk.y, i, bf_to_f((uint16_t)sc[i]), plan[i], vp));
+    }
+    pk = pk_n;
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) { sc[i] = sc_n[i]; o0[i] = o0_n[i]; o1[i] = o1_n[i]; }
+    xp += xstep; sp += sstep; vp += vstep; scp += scstep;
   }
 }
 
@@ -223,7 +349,8 @@ k_outlier_fill(const uint16_t* __restrict__ x, int64_t M, int64_t H, ThrArgs a, 
 // ---- launch helpers -------------------------------------------------------------------------------
 static inline int row_grid(int64_t M, int threads) {
   // enough workgroups to keep 256 CUs busy with several rows in flight each
-  const int per_cu = threads >= 512 ? 3 : 8;
+  int per_cu = threads >= 512 ? 3 : 8;
+  if (const char* e = getenv("HYC_TUNE_ROW_GRID")) per_cu = atoi(e);   // tuning knob, not part of the interface
   const int64_t cap = (int64_t)256 * per_cu;
   return (int)(M < cap ? M : cap);
 }
@@ -256,6 +383,29 @@ int hyc_compress(const void* x, int64_t M, int64_t H, const hyc_desc* d, void* s
     if (!x || !stored || !scales || (d->k > 0 && !vals)) return fail(HYC_EFAULT, "hyc_compress: null buffer");
     if (!aligned16(x) || !aligned8(stored)) return fail(HYC_EINVAL, "hyc_compress: x must be 16-byte and stored 8-byte aligned");
     const int grid = row_grid(M, g.threads);
+    if (g.iters == 1 && g.cps == g.threads && (lpg == 8 || lpg == 16) && d->bits != 1) {
+#define HYC_CF(B_, L_)                                                                                             \
+  do {                                                                                                             \
+    if (g.threads <= 256)                                                                                          \
+      hipLaunchKernelGGL((k_compress_chan_fast<B_, L_, 256>), dim3(grid), dim3(g.threads), 0, st,                  \
+                         static_cast<const uint16_t*>(x), M, H, a, static_cast<uint8_t*>(stored),                  \
+                         static_cast<uint16_t*>(vals), static_cast<uint16_t*>(scales));                            \
+    else                                                                                                           \
+      hipLaunchKernelGGL((k_compress_chan_fast<B_, L_, 1024>), dim3(grid), dim3(g.threads), 0, st,                 \
+                         static_cast<const uint16_t*>(x), M, H, a, static_cast<uint8_t*>(stored),                  \
+                         static_cast<uint16_t*>(vals), static_cast<uint16_t*>(scales));                            \
+  } while (0)
+      switch (d->bits * 100 + lpg) {
+        case 208: HYC_CF(2, 8); break;
+        case 216: HYC_CF(2, 16); break;
+        case 408: HYC_CF(4, 8); break;
+        case 416: HYC_CF(4, 16); break;
+        case 808: HYC_CF(8, 8); break;
+        default: HYC_CF(8, 16); break;
+      }
+#undef HYC_CF
+      return check_launch("hyc_compress");
+    }
     HYC_DISPATCH_BITS(d->bits,
       hipLaunchKernelGGL((k_compress_chan<B>), dim3(grid), dim3(g.threads), 0, st,
                          static_cast<const uint16_t*>(x), M, H, g.cps, g.iters, lpg, a, static_cast<uint8_t*>(stored),
@@ -296,6 +446,24 @@ int hyc_decompress(const void* stored, const void* vals, const void* scales, int
     if (!stored || !xhat || !scales || (d->k > 0 && !vals)) return fail(HYC_EFAULT, "hyc_decompress: null buffer");
     if (!aligned16(xhat) || !aligned8(stored)) return fail(HYC_EINVAL, "hyc_decompress: xhat must be 16-byte and stored 8-byte aligned");
     const int grid = row_grid(M, g.threads);
+    if (g.iters == 1 && g.cps == g.threads && d->bits != 1) {
+#define HYC_DF(B_)                                                                                                 \
+  do {                                                                                                             \
+    if (g.threads <= 256)                                                                                          \
+      hipLaunchKernelGGL((k_decompress_chan_fast<B_, 256>), dim3(grid), dim3(g.threads), 0, st,                    \
+                         static_cast<const uint8_t*>(stored), static_cast<const uint16_t*>(vals),                  \
+                         static_cast<const uint16_t*>(scales), M, H, a, static_cast<uint16_t*>(xhat));             \
+    else                                                                                                           \
+      hipLaunchKernelGGL((k_decompress_chan_fast<B_, 1024>), dim3(grid), dim3(g.threads), 0, st,                   \
+                         static_cast<const uint8_t*>(stored), static_cast<const uint16_t*>(vals),                  \
+                         static_cast<const uint16_t*>(scales), M, H, a, static_cast<uint16_t*>(xhat));             \
+  } while (0)
+      if (d->bits == 2) HYC_DF(2);
+      else if (d->bits == 4) HYC_DF(4);
+      else HYC_DF(8);
+#undef HYC_DF
+      return check_launch("hyc_decompress");
+    }
     HYC_DISPATCH_BITS(d->bits,
       hipLaunchKernelGGL((k_decompress_chan<B>), dim3(grid), dim3(g.threads), 0, st,
                          static_cast<const uint8_t*>(stored), static_cast<const uint16_t*>(vals),

@@ -113,9 +113,8 @@ k_gradw(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_out, 
             const uint2 pk = *reinterpret_cast<const uint2*>(stored + m * SEG + 8 * c);
 #pragma unroll
             for (int i = 0; i < NSEG; ++i) {
-              float v[8];
-              decode_chan<BITS>(pk.x, pk.y, i, c, CPS, ca, vals + m * ca.k, scales + m * ca.groups_per_row, v);
-              *reinterpret_cast<uint4*>(Bs + row * BP + i * HS + 8 * cc) = pack8(v);
+              *reinterpret_cast<uint4*>(Bs + row * BP + i * HS + 8 * cc) =
+                  decode_chan_pk<BITS>(pk.x, pk.y, i, c, CPS, ca, vals + m * ca.k, scales + m * ca.groups_per_row);
             }
           } else {
 #pragma unroll

@@ -1,5 +1,6 @@
 // RMSNorm forward fused with the compression of its input, and RMSNorm backward fused with the
-// decompression.  One workgroup per row at a time; the row lives in registers (x is read from HBM once).
+// decompression.  A row lives in registers (x is read from HBM once); the next row's loads are issued before the
+// current row is processed so that memory requests stay in flight during the arithmetic.
 #include "abi_util.hpp"
 #include "row_kernels.hpp"
 
@@ -16,21 +17,287 @@ __device__ __forceinline__ void load_w8(const void* w, bool wf32, int64_t col, f
   }
 }
 
-// two block-wide sums at once; red holds >= 32 floats
-__device__ __forceinline__ void block_sum2(float& a, float& b, float* red) {
+// Sum of two values over the `nw` waves of one row slot with ONE barrier: partials go to a buffer that alternates
+// with `parity`, so the next reduction never overwrites values a slower wave is still reading.
+// red layout: [2 parities][slots][16 waves][2 values].
+__device__ __forceinline__ void slot_sum2(float& a, float& b, float* red, int parity, int slot, int nslots, int wave_in_slot,
+                                          int nw) {
   a = wave_sum(a);
   b = wave_sum(b);
-  const int wave = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
-  if ((threadIdx.x & 63) == 0) { red[wave] = a; red[16 + wave] = b; }
+  float* base = red + ((parity * nslots + slot) * 16) * 2;
+  if ((threadIdx.x & 63) == 0) { base[2 * wave_in_slot] = a; base[2 * wave_in_slot + 1] = b; }
   __syncthreads();
   float ta = 0.f, tb = 0.f;
-  for (int i = 0; i < nw; ++i) { ta += red[i]; tb += red[16 + i]; }
-  __syncthreads();
+  for (int i = 0; i < nw; ++i) { ta += base[2 * i]; tb += base[2 * i + 1]; }
   a = ta; b = tb;
 }
 
 // ------------------------------------------------------------------------------------------------
-// forward: y, rstd, and x compressed.  MODE 0 = channel, 1 = threshold.
+// Fast paths (channel mode, every lane owns exactly one chunk per segment: CPS == blockDim.x, LPG known at
+// compile time).  No per-lane predication, row-invariant data (weights, plan words) hoisted, pointers advanced
+// instead of recomputed, next row prefetched under a uniform branch.
+// ------------------------------------------------------------------------------------------------
+template <bool WF32>
+__device__ __forceinline__ void load_w8t(const void* w, int64_t col, float (&o)[8]) {
+  if (WF32) {
+    const float4 a = *reinterpret_cast<const float4*>(static_cast<const float*>(w) + col);
+    const float4 b = *reinterpret_cast<const float4*>(static_cast<const float*>(w) + col + 4);
+    o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w; o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+  } else {
+    unpack8(*reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(w) + col), o);
+  }
+}
+
+// sum over the waves of the workgroup, one barrier (alternating buffers, see slot_sum2)
+__device__ __forceinline__ float block_sum1(float a, float (*red)[16], int parity, int wave, int nw) {
+  a = wave_sum(a);
+  if ((threadIdx.x & 63) == 0) red[parity][wave] = a;
+  __syncthreads();
+  float t = red[parity][0];
+  for (int i = 1; i < nw; ++i) t += red[parity][i];
+  return t;
+}
+
+template <int BITS, int LPGT, bool WF32, int MAXT>
+__global__ void __launch_bounds__(MAXT)
+k_rmsnorm_fwd_fast(const uint16_t* __restrict__ x, const void* __restrict__ w, float eps, int64_t M, int64_t H,
+                   ChanArgs ca, uint16_t* __restrict__ y, float* __restrict__ rstd_out, uint8_t* __restrict__ stored,
+                   uint16_t* __restrict__ vals, uint16_t* __restrict__ scales) {
+  constexpr int NSEG = Q<BITS>::NSEG;
+  __shared__ float red[2][16];
+  const int c = threadIdx.x, CPS = blockDim.x;
+  const int64_t SEG = (int64_t)CPS * 8;
+  const float invH = 1.0f / (float)H;
+  const int wave = c >> 6, nw = CPS >> 6;
+  const bool leader = (c & (LPGT - 1)) == 0;
+
+  uint32_t km[NSEG][4];                                            // AND masks that zero the outlier channels
+  float wv[NSEG][8];
+  {
+    uint32_t plan[NSEG];
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) {
+      plan[i] = ca.plan[i * CPS + c];
+      load_w8t<WF32>(w, i * SEG + 8 * c, wv[i]);
+    }
+    ChunkOutliers<NSEG> co;
+    co.init(plan);
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) co.keep_masks(i, km[i]);
+  }
+  const bool gather = c < ca.k;                                   // thread c copies outlier channel idx[c] to vals
+  const int idx0 = gather ? ca.idx[c] : 0;
+  const int64_t stride = gridDim.x;
+  int64_t row = blockIdx.x;
+  const uint16_t* xrow = x + row * H;
+  const uint16_t* xp = xrow + 8 * c;
+  uint16_t* yp = y + row * H + 8 * c;
+  uint8_t* sp = stored + row * SEG + 8 * c;
+  uint16_t* vp = vals + row * ca.k;
+  uint16_t* scp = scales + row * ca.groups_per_row + (c >> ca.chunk_to_group_shift);
+  const int64_t xstep = stride * H, sstep = stride * SEG, vstep = stride * ca.k, scstep = stride * ca.groups_per_row;
+  const int seg_groups = CPS >> ca.chunk_to_group_shift;          // scale groups per segment
+
+  uint4 raw[NSEG];
+  uint16_t o = 0;
+  if (row < M) {
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) raw[i] = *reinterpret_cast<const uint4*>(xp + i * SEG);
+    if (gather) o = xrow[idx0];
+  }
+  int parity = 0;
+  for (; row < M; row += stride, parity ^= 1) {
+    uint4 nxt[NSEG];
+    uint16_t o_n = 0;
+    if (row + stride < M) {                                         // uniform
+#pragma unroll
+      for (int i = 0; i < NSEG; ++i) nxt[i] = *reinterpret_cast<const uint4*>(xp + xstep + i * SEG);
+      if (gather) o_n = xrow[xstep + idx0];
+    }
+    float ss = 0.f;
+    uint32_t lo = 0, hi = 0;
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) {
+      float v[8];
+      unpack8(raw[i], v);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ss = __builtin_fmaf(v[j], v[j], ss);
+      unpack8(make_uint4(raw[i].x & km[i][0], raw[i].y & km[i][1], raw[i].z & km[i][2], raw[i].w & km[i][3]), v);
+      uint32_t cl, ch;
+      const float s = quant_seg<BITS, LPGT>(v, LPGT, cl, ch);
+      if (leader) scp[i * seg_groups] = f_to_bf(s);
+      if (BITS == 8) { lo = cl; hi = ch; }
+      else { lo |= cl << (i * BITS); hi |= ch << (i * BITS); }
+    }
+    *reinterpret_cast<uint2*>(sp) = make_uint2(lo, hi);
+    if (gather) {
+      vp[c] = o;
+      for (int t = c + CPS; t < ca.k; t += CPS) vp[t] = xrow[ca.idx[t]];   // only when k exceeds the workgroup size
+    }
+    ss = block_sum1(ss, red, parity, wave, nw);
+    const float rstd = 1.0f / __builtin_sqrtf(ss * invH + eps);
+    if (c == 0) rstd_out[row] = rstd;
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) {
+      float v[8];
+      unpack8(raw[i], v);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = (v[j] * rstd) * wv[i][j];
+      store_stream(yp + i * SEG, pack8(v));
+    }
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) raw[i] = nxt[i];
+    o = o_n;
+    xrow += xstep; xp += xstep; yp += xstep; sp += sstep; vp += vstep; scp += scstep;
+  }
+}
+
+// Backward fast path.  A workgroup is `slots` row slots of CPS threads; slot s of workgroup b handles rows
+// b*slots + s, + gridDim.x*slots, ...: the rows in flight across the chip are adjacent in memory (rows that are far
+// apart would crowd onto a few memory channels).  Each slot keeps its own dw accumulators; they are added through
+// LDS at the end, in slot order, so a workgroup writes one fp32 partial row.
+template <int BITS, bool WF32, bool QUIRK, int MAXT>
+__global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(4, 8)))
+k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ stored, const uint16_t* __restrict__ vals,
+                   const uint16_t* __restrict__ scales, const void* __restrict__ w, const float* __restrict__ rstd,
+                   int64_t M, int64_t H, int CPS, int slots, ChanArgs ca, uint16_t* __restrict__ dx,
+                   float* __restrict__ dw_partials) {
+  constexpr int NSEG = Q<BITS>::NSEG;
+  __shared__ float red[2][16][2][16];                                 // [parity][slot][value][wave]
+  extern __shared__ __align__(16) float xslot[];                      // [slots-1][CPS][8]
+  const int slot = threadIdx.x / CPS, c = threadIdx.x - slot * CPS;
+  const int64_t SEG = (int64_t)CPS * 8;
+  const float invH = 1.0f / (float)H;
+  const int wave = c >> 6, nw = CPS >> 6;
+  const int seg_groups = CPS >> ca.chunk_to_group_shift;
+
+  uint32_t plan[NSEG];
+  float wv[NSEG][8], acc[NSEG][8];
+#pragma unroll
+  for (int i = 0; i < NSEG; ++i) {
+    plan[i] = ca.plan[i * CPS + c];
+    load_w8t<WF32>(w, i * SEG + 8 * c, wv[i]);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[i][j] = 0.f;
+  }
+  ChunkOutliers<NSEG> co;
+  co.init(plan);
+  const int64_t stride = (int64_t)gridDim.x * slots;
+  int64_t row = (int64_t)blockIdx.x * slots + slot;
+  const int64_t steps = (M + stride - 1) / stride;                    // the same for every slot: barriers stay matched
+  const uint16_t* gp = dy + row * H + 8 * c;
+  uint16_t* dxp = dx + row * H + 8 * c;
+  const uint8_t* sp = stored + row * SEG + 8 * c;
+  const uint16_t* vp = vals + row * ca.k;
+  const uint16_t* scp = scales + row * ca.groups_per_row + (c >> ca.chunk_to_group_shift);
+
+  uint2 pk = make_uint2(0, 0);
+  uint4 graw[NSEG];
+  uint32_t sc[NSEG];   // one register each: a packed pair would be assembled right after the load and stall on it
+  uint32_t o0[NSEG], o1[NSEG];
+  float rs = 0.f;
+#pragma unroll
+  for (int i = 0; i < NSEG; ++i) { graw[i] = make_uint4(0, 0, 0, 0); sc[i] = 0; o0[i] = 0; o1[i] = 0; }
+  if (row < M) {                                                      // uniform per wave
+    pk = *reinterpret_cast<const uint2*>(sp);
+    rs = rstd[row];
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) { graw[i] = *reinterpret_cast<const uint4*>(gp + i * SEG); sc[i] = scp[i * seg_groups]; }
+    co.request(vp, o0, o1);
+  }
+  int parity = 0;
+  for (int64_t step = 0; step < steps; ++step, row += stride, parity ^= 1) {
+    const bool valid = row < M;
+    uint2 pk_n = make_uint2(0, 0);
+    uint4 g_n[NSEG];
+    uint32_t sc_n[NSEG], o0_n[NSEG], o1_n[NSEG];
+    float rs_n = 0.f;
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) { g_n[i] = make_uint4(0, 0, 0, 0); sc_n[i] = 0; o0_n[i] = 0; o1_n[i] = 0; }
+    if (row + stride < M) {                                           // uniform per wave
+      pk_n = *reinterpret_cast<const uint2*>(sp + stride * SEG);
+      rs_n = rstd[row + stride];
+#pragma unroll
+      for (int i = 0; i < NSEG; ++i) {
+        g_n[i] = *reinterpret_cast<const uint4*>(gp + stride * H + i * SEG);
+        sc_n[i] = scp[stride * ca.groups_per_row + i * seg_groups];
+      }
+      co.request(vp + stride * ca.k, o0_n, o1_n);
+    }
+    float xn[NSEG][8], wdy[NSEG][8];
+    float p1 = 0.f, p2 = 0.f;
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) {
+      float g[8];
+      unpack8(graw[i], g);
+      const float sf = bf_to_f((uint16_t)sc[i]);
+      if (!co.many) unpack8(co.splice(i, dequant8<BITS>(pk.x, pk.y, i, sf), o0[i], o1[i], sf), xn[i]);
+      else unpack8(decode_seg<BITS>(pk.x, pk.y, i, sf, valid ? plan[i] : 0u, vp), xn[i]);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float n = xn[i][j] * rs;
+        const float t = wv[i][j] * g[j];
+        xn[i][j] = n;
+        wdy[i][j] = t;
+        p1 = __builtin_fmaf(n, t, p1);
+        if (QUIRK) p2 += t;
+        acc[i][j] = __builtin_fmaf(g[j], n, acc[i][j]);
+      }
+    }
+    // two sums per slot, one barrier
+    p1 = wave_sum(p1);
+    if (QUIRK) p2 = wave_sum(p2);
+    if ((c & 63) == 0) { red[parity][slot][0][wave] = p1; if (QUIRK) red[parity][slot][1][wave] = p2; }
+    __syncthreads();
+    float t1 = red[parity][slot][0][0], t2 = QUIRK ? red[parity][slot][1][0] : 0.f;
+    for (int i = 1; i < nw; ++i) { t1 += red[parity][slot][0][i]; if (QUIRK) t2 += red[parity][slot][1][i]; }
+    // dx = (wdy - (xn*c1 + c2)) * rstd, arranged as two fused multiply-adds
+    const float k1 = -(t1 * invH) * rs;
+    const float k2 = QUIRK ? -(t2 * invH) * rs : 0.f;
+    if (valid) {
+#pragma unroll
+      for (int i = 0; i < NSEG; ++i) {
+        float o[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) o[j] = __builtin_fmaf(xn[i][j], k1, __builtin_fmaf(wdy[i][j], rs, k2));
+        store_stream(dxp + i * SEG, pack8(o));
+      }
+    }
+    pk = pk_n; rs = rs_n;
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) { graw[i] = g_n[i]; sc[i] = sc_n[i]; o0[i] = o0_n[i]; o1[i] = o1_n[i]; }
+    gp += stride * H; dxp += stride * H; sp += stride * SEG; vp += stride * ca.k; scp += stride * ca.groups_per_row;
+  }
+  float* pr = dw_partials + (int64_t)blockIdx.x * H + 8 * c;
+#pragma unroll
+  for (int i = 0; i < NSEG; ++i) {
+    if (slots > 1) {
+      __syncthreads();
+      if (slot > 0) {
+        float4* o = reinterpret_cast<float4*>(xslot + ((int64_t)(slot - 1) * CPS + c) * 8);
+        o[0] = make_float4(acc[i][0], acc[i][1], acc[i][2], acc[i][3]);
+        o[1] = make_float4(acc[i][4], acc[i][5], acc[i][6], acc[i][7]);
+      }
+      __syncthreads();
+      if (slot == 0) {
+        for (int s2 = 1; s2 < slots; ++s2) {
+          const float4* o = reinterpret_cast<const float4*>(xslot + ((int64_t)(s2 - 1) * CPS + c) * 8);
+          const float4 a = o[0], b = o[1];
+          acc[i][0] += a.x; acc[i][1] += a.y; acc[i][2] += a.z; acc[i][3] += a.w;
+          acc[i][4] += b.x; acc[i][5] += b.y; acc[i][6] += b.z; acc[i][7] += b.w;
+        }
+      }
+    }
+    if (slot == 0) {
+      float4* o = reinterpret_cast<float4*>(pr + i * SEG);
+      o[0] = make_float4(acc[i][0], acc[i][1], acc[i][2], acc[i][3]);
+      o[1] = make_float4(acc[i][4], acc[i][5], acc[i][6], acc[i][7]);
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// forward: y, rstd, and x compressed.  MODE 0 = channel, 1 = threshold.  One workgroup = one row at a time.
 // ------------------------------------------------------------------------------------------------
 template <int BITS, int ITERS, int MAXT, int MODE>
 __global__ void __launch_bounds__(MAXT)
@@ -39,48 +306,79 @@ k_rmsnorm_fwd(const uint16_t* __restrict__ x, const void* __restrict__ w, bool w
               float* __restrict__ rstd_out, uint8_t* __restrict__ stored, uint16_t* __restrict__ vals,
               uint16_t* __restrict__ scales, int32_t* __restrict__ row_counts) {
   constexpr int NSEG = Q<BITS>::NSEG;
-  __shared__ float red[32];
+  __shared__ float red[2 * 16 * 2];
   const int64_t SEG = (int64_t)CPS * 8;
   const float invH = 1.0f / (float)H;
-  for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
-    const uint16_t* xr = x + row * H;
-    uint4 raw[ITERS][NSEG];
-    float ss = 0.f;
+  const int wave = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+
+  // what does not change from row to row: which chunks this thread owns and their outlier plan words
+  bool act[ITERS];
+  int cidx[ITERS];
+  uint32_t plan[ITERS][NSEG];
 #pragma unroll
-    for (int it = 0; it < ITERS; ++it) {
-      const int c = it * blockDim.x + threadIdx.x;
-      const bool active = c < CPS;
+  for (int it = 0; it < ITERS; ++it) {
+    cidx[it] = it * blockDim.x + threadIdx.x;
+    act[it] = cidx[it] < CPS;
 #pragma unroll
-      for (int i = 0; i < NSEG; ++i)
-        raw[it][i] = active ? *reinterpret_cast<const uint4*>(xr + i * SEG + 8 * c) : make_uint4(0, 0, 0, 0);
-    }
+    for (int i = 0; i < NSEG; ++i) plan[it][i] = (MODE == 0 && act[it]) ? ca.plan[i * CPS + cidx[it]] : 0u;
+  }
+
+  uint4 raw[ITERS][NSEG];
+  int64_t row = blockIdx.x;
+  if (row < M) {
 #pragma unroll
     for (int it = 0; it < ITERS; ++it)
 #pragma unroll
-      for (int i = 0; i < NSEG; ++i) {
-        float v[8];
-        unpack8(raw[it][i], v);
+      for (int i = 0; i < NSEG; ++i)
+        raw[it][i] = act[it] ? *reinterpret_cast<const uint4*>(x + row * H + i * SEG + 8 * cidx[it]) : make_uint4(0, 0, 0, 0);
+  }
+  int parity = 0;
+  for (; row < M; row += gridDim.x, parity ^= 1) {
+    // prefetch the next row
+    uint4 nxt[ITERS][NSEG];
+    const int64_t nrow = row + gridDim.x;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) ss = __builtin_fmaf(v[j], v[j], ss);
-      }
-    // compress x (independent of rstd)
-    float hot = 0.f;
+    for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+      for (int i = 0; i < NSEG; ++i)
+        nxt[it][i] = (nrow < M && act[it]) ? *reinterpret_cast<const uint4*>(x + nrow * H + i * SEG + 8 * cidx[it])
+                                           : make_uint4(0, 0, 0, 0);
+
+    float ss = 0.f, hot = 0.f;
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
-      const int c = it * blockDim.x + threadIdx.x;
-      const bool active = c < CPS;
-      uint32_t lo, hi;
+      const int c = cidx[it];
+      uint32_t lo = 0, hi = 0;
       if (MODE == 0) {
-        encode_chan<BITS>(raw[it], active, c, CPS, lpg, ca, vals + row * ca.k, scales + row * ca.groups_per_row, lo, hi);
+#pragma unroll
+        for (int i = 0; i < NSEG; ++i) {
+          float v[8];
+          unpack8(raw[it][i], v);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) ss = __builtin_fmaf(v[j], v[j], ss);
+          uint32_t cl, ch;
+          const float s = encode_seg<BITS>(raw[it][i], v, plan[it][i], lpg, vals + row * ca.k, cl, ch);
+          if (act[it] && (c & (lpg - 1)) == 0)
+            scales[row * ca.groups_per_row + ((i * CPS + c) >> ca.chunk_to_group_shift)] = f_to_bf(s);
+          if (BITS == 8) { lo = cl; hi = ch; }
+          else { lo |= cl << (i * BITS); hi |= ch << (i * BITS); }
+        }
       } else {
-        if (active) {
+#pragma unroll
+        for (int i = 0; i < NSEG; ++i) {
+          float v[8];
+          unpack8(raw[it][i], v);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) ss = __builtin_fmaf(v[j], v[j], ss);
+        }
+        if (act[it]) {
           hot += (float)(perchan ? encode_thr<BITS, true>(raw[it], c, CPS, H, row % ta.S, ta, lo, hi)
                                  : encode_thr<BITS, false>(raw[it], c, CPS, H, row % ta.S, ta, lo, hi));
         }
       }
-      if (active) *reinterpret_cast<uint2*>(stored + row * SEG + 8 * c) = make_uint2(lo, hi);
+      if (act[it]) *reinterpret_cast<uint2*>(stored + row * SEG + 8 * c) = make_uint2(lo, hi);
     }
-    block_sum2(ss, hot, red);
+    slot_sum2(ss, hot, red, parity, 0, 1, wave, nw);
     const float rstd = 1.0f / __builtin_sqrtf(ss * invH + eps);
     if (threadIdx.x == 0) {
       rstd_out[row] = rstd;
@@ -89,11 +387,10 @@ k_rmsnorm_fwd(const uint16_t* __restrict__ x, const void* __restrict__ w, bool w
     uint16_t* yr = y + row * H;
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
-      const int c = it * blockDim.x + threadIdx.x;
-      if (c < CPS) {
+      if (act[it]) {
 #pragma unroll
         for (int i = 0; i < NSEG; ++i) {
-          const int64_t col = i * SEG + 8 * c;
+          const int64_t col = i * SEG + 8 * cidx[it];
           float v[8], wv[8];
           unpack8(raw[it][i], v);
           load_w8(w, wf32, col, wv);
@@ -103,97 +400,170 @@ k_rmsnorm_fwd(const uint16_t* __restrict__ x, const void* __restrict__ w, bool w
         }
       }
     }
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+      for (int i = 0; i < NSEG; ++i) raw[it][i] = nxt[it][i];
   }
 }
 
 // ------------------------------------------------------------------------------------------------
-// backward.  SRC 0 = channel-compressed x, 2 = dense bf16 x_hat.  Rows [blockIdx.x*rpb, +rpb).
+// backward.  SRC 0 = channel-compressed x, 2 = dense bf16 x_hat.
+// A workgroup is `slots` row slots of T threads; slot s handles rows r0+s, r0+s+slots, ... of the workgroup's
+// range, keeps its own dw accumulators, and the slots are added up through LDS at the end (one fp32 partial row
+// per workgroup).  All slots walk the same number of iterations so that they meet at the same barriers.
 // ------------------------------------------------------------------------------------------------
 template <int BITS, int ITERS, int MAXT, int SRC>
 __global__ void __launch_bounds__(MAXT)
 k_rmsnorm_bwd(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ stored, const uint16_t* __restrict__ vals,
               const uint16_t* __restrict__ scales, const void* __restrict__ w, bool wf32,
-              const float* __restrict__ rstd, int64_t M, int64_t H, int CPS, int rows_per_block, ChanArgs ca,
-              bool quirk, uint16_t* __restrict__ dx, float* __restrict__ dw_partials) {
+              const float* __restrict__ rstd, int64_t M, int64_t H, int CPS, int T, int slots, int rows_per_block,
+              ChanArgs ca, bool quirk, uint16_t* __restrict__ dx, float* __restrict__ dw_partials) {
   constexpr int NSEG = Q<BITS>::NSEG;
-  __shared__ float red[32];
+  __shared__ float red[2 * 16 * 16 * 2];
+  extern __shared__ __align__(16) float xslot[];                        // [slots-1][T][8] for the final reduction
   const int64_t SEG = (int64_t)CPS * 8;
   const float invH = 1.0f / (float)H;
+  const int slot = threadIdx.x / T, tl = threadIdx.x - slot * T;
+  const int wave_in_slot = tl >> 6, nw = T >> 6;
+
+  bool act[ITERS];
+  int cidx[ITERS];
+  uint32_t plan[ITERS][NSEG];
   float wv[ITERS][NSEG][8], acc[ITERS][NSEG][8];
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
-    const int c = it * blockDim.x + threadIdx.x;
+    cidx[it] = it * T + tl;
+    act[it] = cidx[it] < CPS;
 #pragma unroll
     for (int i = 0; i < NSEG; ++i) {
-      if (c < CPS) load_w8(w, wf32, i * SEG + 8 * c, wv[it][i]);
+      plan[it][i] = (SRC == 0 && act[it]) ? ca.plan[i * CPS + cidx[it]] : 0u;
+      if (act[it]) load_w8(w, wf32, i * SEG + 8 * cidx[it], wv[it][i]);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) { acc[it][i][j] = 0.f; if (c >= CPS) wv[it][i][j] = 0.f; }
+      for (int j = 0; j < 8; ++j) { acc[it][i][j] = 0.f; if (!act[it]) wv[it][i][j] = 0.f; }
     }
   }
+
   const int64_t r0 = (int64_t)blockIdx.x * rows_per_block;
   const int64_t r1 = r0 + rows_per_block < M ? r0 + rows_per_block : M;
-  for (int64_t row = r0; row < r1; ++row) {
-    const float rs = rstd[row];
-    float xn[ITERS][NSEG][8], wdy[ITERS][NSEG][8];
+  const int steps = (rows_per_block + slots - 1) / slots;
+
+  // per-row inputs, loaded one step ahead
+  uint2 pk[ITERS];
+  uint4 graw[ITERS][NSEG];
+  uint4 xraw[ITERS][NSEG];        // SRC 2 only
+  uint16_t sc[ITERS][NSEG];       // SRC 0 only
+  float rs = 0.f;
+  auto load_row = [&](int64_t row, uint2 (&pk_)[ITERS], uint4 (&g_)[ITERS][NSEG], uint4 (&x_)[ITERS][NSEG],
+                      uint16_t (&sc_)[ITERS][NSEG], float& rs_) {
+    const bool valid = row < r1;
+    rs_ = valid ? rstd[row] : 0.f;
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const bool on = valid && act[it];
+      if (SRC == 0) pk_[it] = on ? *reinterpret_cast<const uint2*>(stored + row * SEG + 8 * cidx[it]) : make_uint2(0, 0);
+#pragma unroll
+      for (int i = 0; i < NSEG; ++i) {
+        const int64_t col = i * SEG + 8 * cidx[it];
+        g_[it][i] = on ? *reinterpret_cast<const uint4*>(dy + row * H + col) : make_uint4(0, 0, 0, 0);
+        if (SRC == 0) {
+          sc_[it][i] = on ? scales[row * ca.groups_per_row + ((i * CPS + cidx[it]) >> ca.chunk_to_group_shift)] : (uint16_t)0;
+        } else {
+          x_[it][i] = on ? *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(stored) + row * H + col)
+                         : make_uint4(0, 0, 0, 0);
+        }
+      }
+    }
+  };
+  load_row(r0 + slot, pk, graw, xraw, sc, rs);
+
+  int parity = 0;
+  for (int step = 0; step < steps; ++step, parity ^= 1) {
+    const int64_t row = r0 + (int64_t)step * slots + slot;
+    const bool valid = row < r1;
+    uint2 pk_n[ITERS];
+    uint4 g_n[ITERS][NSEG], x_n[ITERS][NSEG];
+    uint16_t sc_n[ITERS][NSEG];
+    float rs_n;
+    load_row(row + slots, pk_n, g_n, x_n, sc_n, rs_n);
+
+    float xn[ITERS][NSEG][8];
     float p1 = 0.f, p2 = 0.f;
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
-      const int c = it * blockDim.x + threadIdx.x;
-      const bool active = c < CPS;
-      uint2 pk = make_uint2(0, 0);
-      if (SRC == 0 && active) pk = *reinterpret_cast<const uint2*>(stored + row * SEG + 8 * c);
 #pragma unroll
       for (int i = 0; i < NSEG; ++i) {
-        const int64_t col = i * SEG + 8 * c;
         float g[8];
-        if (active) {
-          unpack8(*reinterpret_cast<const uint4*>(dy + row * H + col), g);
-          if (SRC == 0) {
-            decode_chan<BITS>(pk.x, pk.y, i, c, CPS, ca, vals + row * ca.k, scales + row * ca.groups_per_row, xn[it][i]);
-          } else {
-            unpack8(*reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(stored) + row * H + col), xn[it][i]);
-          }
+        unpack8(graw[it][i], g);
+        if (SRC == 0) {
+          unpack8(decode_seg<BITS>(pk[it].x, pk[it].y, i, bf_to_f(sc[it][i]), valid ? plan[it][i] : 0u, vals + row * ca.k),
+                  xn[it][i]);
         } else {
-#pragma unroll
-          for (int j = 0; j < 8; ++j) { g[j] = 0.f; xn[it][i][j] = 0.f; }
+          unpack8(xraw[it][i], xn[it][i]);
         }
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           const float n = xn[it][i][j] * rs;
           const float t = wv[it][i][j] * g[j];
           xn[it][i][j] = n;
-          wdy[it][i][j] = t;
           p1 = __builtin_fmaf(n, t, p1);
-          p2 += t;
+          if (quirk) p2 += t;
           acc[it][i][j] = __builtin_fmaf(g[j], n, acc[it][i][j]);
         }
       }
     }
-    block_sum2(p1, p2, red);
+    slot_sum2(p1, p2, red, parity, slot, slots, wave_in_slot, nw);
     const float c1 = p1 * invH;
     const float c2 = quirk ? p2 * invH : 0.f;
+    if (valid) {
 #pragma unroll
-    for (int it = 0; it < ITERS; ++it) {
-      const int c = it * blockDim.x + threadIdx.x;
-      if (c < CPS) {
+      for (int it = 0; it < ITERS; ++it) {
+        if (act[it]) {
 #pragma unroll
-        for (int i = 0; i < NSEG; ++i) {
-          float o[8];
+          for (int i = 0; i < NSEG; ++i) {
+            float o[8], g[8];
+            unpack8(graw[it][i], g);
 #pragma unroll
-          for (int j = 0; j < 8; ++j) o[j] = (wdy[it][i][j] - (xn[it][i][j] * c1 + c2)) * rs;
-          *reinterpret_cast<uint4*>(dx + row * H + i * SEG + 8 * c) = pack8(o);
+            for (int j = 0; j < 8; ++j) o[j] = (wv[it][i][j] * g[j] - __builtin_fmaf(xn[it][i][j], c1, c2)) * rs;
+            *reinterpret_cast<uint4*>(dx + row * H + i * SEG + 8 * cidx[it]) = pack8(o);
+          }
         }
       }
     }
+    rs = rs_n;
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      pk[it] = pk_n[it];
+#pragma unroll
+      for (int i = 0; i < NSEG; ++i) { graw[it][i] = g_n[it][i]; xraw[it][i] = x_n[it][i]; sc[it][i] = sc_n[it][i]; }
+    }
   }
+
+  // add the slots' accumulators (slot order) and write the workgroup's partial row
   float* pr = dw_partials + (int64_t)blockIdx.x * H;
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
-    const int c = it * blockDim.x + threadIdx.x;
-    if (c < CPS) {
 #pragma unroll
-      for (int i = 0; i < NSEG; ++i) {
-        float4* o = reinterpret_cast<float4*>(pr + i * SEG + 8 * c);
+    for (int i = 0; i < NSEG; ++i) {
+      if (slots > 1) {
+        __syncthreads();
+        if (slot > 0) {
+          float4* o = reinterpret_cast<float4*>(xslot + ((int64_t)(slot - 1) * T + tl) * 8);
+          o[0] = make_float4(acc[it][i][0], acc[it][i][1], acc[it][i][2], acc[it][i][3]);
+          o[1] = make_float4(acc[it][i][4], acc[it][i][5], acc[it][i][6], acc[it][i][7]);
+        }
+        __syncthreads();
+        if (slot == 0) {
+          for (int s = 1; s < slots; ++s) {
+            const float4* o = reinterpret_cast<const float4*>(xslot + ((int64_t)(s - 1) * T + tl) * 8);
+            const float4 a = o[0], b = o[1];
+            acc[it][i][0] += a.x; acc[it][i][1] += a.y; acc[it][i][2] += a.z; acc[it][i][3] += a.w;
+            acc[it][i][4] += b.x; acc[it][i][5] += b.y; acc[it][i][6] += b.z; acc[it][i][7] += b.w;
+          }
+        }
+      }
+      if (slot == 0 && act[it]) {
+        float4* o = reinterpret_cast<float4*>(pr + i * SEG + 8 * cidx[it]);
         o[0] = make_float4(acc[it][i][0], acc[it][i][1], acc[it][i][2], acc[it][i][3]);
         o[1] = make_float4(acc[it][i][4], acc[it][i][5], acc[it][i][6], acc[it][i][7]);
       }
@@ -230,40 +600,90 @@ k_colsum(const float* __restrict__ partials, int64_t P, int64_t H, void* __restr
   }
 }
 
-static inline int64_t bwd_rows_per_block(int64_t M) {
-  // about a thousand workgroups, at least four rows each
-  int64_t rpb = (M + 1023) / 1024;
-  return rpb < 4 ? 4 : rpb;
+// Row-slot geometry of the fused norm kernels: T threads per row, ITERS chunks per thread and segment.
+struct NormGeom {
+  int T, iters, iters_t;   // iters_t = the template value (1, 2 or 4) that covers `iters`
+};
+static inline int norm_geom(int cps, NormGeom* n) {
+  // one chunk per thread and segment whenever a workgroup can span the row: light threads, high occupancy
+  int T = cps <= 1024 ? ((cps + 63) / 64) * 64 : 1024;
+  int iters = (cps + T - 1) / T;
+  if (iters > 4) return fail(HYC_ENOTSUP, "row too long for the fused RMSNorm kernels (%d chunks per segment)", cps);
+  n->T = T;
+  n->iters = iters;
+  n->iters_t = iters <= 1 ? 1 : (iters <= 2 ? 2 : 4);
+  return HYC_OK;
+}
+
+#ifndef BWD_FAST_SLOTS_MAX
+#define BWD_FAST_SLOTS_MAX 4
+#endif
+#ifndef BWD_SLOTS_SMALL
+#define BWD_SLOTS_SMALL 1
+#endif
+// backward launch shape: slots per workgroup and rows per workgroup
+struct BwdShape {
+  int slots, threads, rpb;
+  int64_t P;
+  int fast_slots;      // fast path: row slots per workgroup and workgroups (= partial rows)
+  int64_t fast_P;
+};
+static inline BwdShape bwd_shape(int64_t M, int bits, const NormGeom& n) {
+  (void)bits;
+  BwdShape b;
+  b.slots = n.T <= 256 ? BWD_SLOTS_SMALL : 1;
+  b.threads = b.slots * n.T;
+  // about a thousand row slots in flight; each walks at least four rows so the partial rows stay few
+  int64_t rpb = (M * b.slots + 1023) / 1024;
+  if (rpb < 4 * b.slots) rpb = 4 * b.slots;
+  rpb = ((rpb + b.slots - 1) / b.slots) * b.slots;
+  b.rpb = (int)rpb;
+  b.P = M > 0 ? (M + rpb - 1) / rpb : 0;
+  // fast path: up to 1024 threads per workgroup, one workgroup per CU slot; every slot walks at least two rows
+  int fs = 1024 / n.T;
+  if (fs < 1) fs = 1;
+  if (fs > BWD_FAST_SLOTS_MAX) fs = BWD_FAST_SLOTS_MAX;
+  int64_t fp = 256 * (int64_t)(1024 / (fs * n.T) > 0 ? 1024 / (fs * n.T) : 1);
+  const int64_t need = (M + 2 * fs - 1) / (2 * fs);
+  if (fp > need) fp = need;
+  if (fp < 1) fp = 1;
+  b.fast_slots = fs;
+  b.fast_P = M > 0 ? fp : 0;
+  return b;
 }
 
 }  // namespace hyc
 
 using namespace hyc;
 
-#define HYC_BITS_ITERS_MAXT(BITS_, ITERS_, THREADS_, ...)                                   \
+#define HYC_BITS_ITERS(BITS_, ITERS_, ...)                                                  \
   do {                                                                                      \
-    const int key_ = (BITS_) * 100 + (ITERS_) * 10 + ((THREADS_) > 256 ? 1 : 0);            \
-    switch (key_) {                                                                         \
+    switch ((BITS_) * 10 + (ITERS_)) {                                                      \
       HYC_CASE_(1, 1, __VA_ARGS__) HYC_CASE_(1, 2, __VA_ARGS__) HYC_CASE_(1, 4, __VA_ARGS__)  \
       HYC_CASE_(2, 1, __VA_ARGS__) HYC_CASE_(2, 2, __VA_ARGS__) HYC_CASE_(2, 4, __VA_ARGS__)  \
       HYC_CASE_(4, 1, __VA_ARGS__) HYC_CASE_(4, 2, __VA_ARGS__) HYC_CASE_(4, 4, __VA_ARGS__)  \
       HYC_CASE_(8, 1, __VA_ARGS__) HYC_CASE_(8, 2, __VA_ARGS__) HYC_CASE_(8, 4, __VA_ARGS__)  \
-      default: return fail(HYC_ENOTSUP, "row too long for the fused kernels (bits=%d)", (BITS_)); \
+      default: return fail(HYC_ENOTSUP, "unsupported bits/iters combination (bits=%d)", (BITS_)); \
     }                                                                                       \
   } while (0)
-#define HYC_CASE_(B_, I_, ...)                                                              \
-  case (B_) * 100 + (I_) * 10 + 0: { constexpr int B = B_, IT = I_, MT = 256; __VA_ARGS__; } break;  \
-  case (B_) * 100 + (I_) * 10 + 1: { constexpr int B = B_, IT = I_, MT = 1024; __VA_ARGS__; } break;
-
-static inline int round_iters(int iters) { return iters <= 1 ? 1 : iters <= 2 ? 2 : iters <= 4 ? 4 : 99; }
+#define HYC_CASE_(B_, I_, ...) \
+  case (B_) * 10 + (I_): { constexpr int B = B_, IT = I_; __VA_ARGS__; } break;
 
 extern "C" {
 
 int64_t hyc_rmsnorm_bwd_partials(int64_t M, int64_t H) {
-  (void)H;
-  if (M <= 0) return 0;
-  const int64_t rpb = bwd_rows_per_block(M);
-  return (M + rpb - 1) / rpb;
+  // the partial count depends on the bit width only through the slot count; report the largest over all widths
+  if (M <= 0 || H <= 0) return 0;
+  int64_t best = 0;
+  for (int bits = 1; bits <= 8; bits *= 2) {
+    if (H % (64 / bits) != 0) continue;
+    NormGeom n;
+    if (norm_geom((int)(H * bits / 64), &n)) continue;
+    const BwdShape b = bwd_shape(M, bits, n);
+    if (b.P > best) best = b.P;
+    if (b.fast_P > best) best = b.fast_P;
+  }
+  return best;
 }
 
 int hyc_rmsnorm_fwd_compress(const void* x, const void* w, int32_t w_dtype, float eps, int64_t M, int64_t H,
@@ -279,27 +699,54 @@ int hyc_rmsnorm_fwd_compress(const void* x, const void* w, int32_t w_dtype, floa
   if (d->mode == HYC_MODE_CHANNEL) { if ((rc = make_chan_args(d, g, &ca, &lpg))) return rc; }
   else if (d->mode == HYC_MODE_THRESHOLD) { if ((rc = make_thr_args(d, g, &ta, &perchan))) return rc; }
   else return fail(HYC_EINVAL, "hyc_rmsnorm_fwd_compress: mode=%d", d->mode);
+  NormGeom n;
+  if ((rc = norm_geom(g.cps, &n))) return rc;
   if (M == 0) return HYC_OK;
   if (!x || !w || !y || !rstd || !stored) return fail(HYC_EFAULT, "hyc_rmsnorm_fwd_compress: null buffer");
   if (d->mode == HYC_MODE_CHANNEL && (!scales || (d->k > 0 && !vals))) return fail(HYC_EFAULT, "hyc_rmsnorm_fwd_compress: null vals/scales");
   if (!aligned16(x) || !aligned16(y) || !aligned16(w) || !aligned8(stored))
     return fail(HYC_EINVAL, "hyc_rmsnorm_fwd_compress: x, y, w must be 16-byte and stored 8-byte aligned");
   const bool wf32 = w_dtype == HYC_DTYPE_F32;
-  const int64_t cap = 256 * (g.threads >= 512 ? 3 : 8);
+  const int64_t cap = 256 * (n.T >= 512 ? 2 : 8);
   const int grid = (int)(M < cap ? M : cap);
   hipStream_t st = begin_launch(stream);
   const uint16_t* xp = static_cast<const uint16_t*>(x);
-  if (d->mode == HYC_MODE_CHANNEL) {
-    HYC_BITS_ITERS_MAXT(d->bits, round_iters(g.iters), g.threads,
-      hipLaunchKernelGGL((k_rmsnorm_fwd<B, IT, MT, 0>), dim3(grid), dim3(g.threads), 0, st, xp, w, wf32, eps, M, H, g.cps,
-                         ca, lpg, ta, perchan, static_cast<uint16_t*>(y), rstd, static_cast<uint8_t*>(stored),
-                         static_cast<uint16_t*>(vals), static_cast<uint16_t*>(scales), row_counts));
-  } else {
-    HYC_BITS_ITERS_MAXT(d->bits, round_iters(g.iters), g.threads,
-      hipLaunchKernelGGL((k_rmsnorm_fwd<B, IT, MT, 1>), dim3(grid), dim3(g.threads), 0, st, xp, w, wf32, eps, M, H, g.cps,
-                         ca, lpg, ta, perchan, static_cast<uint16_t*>(y), rstd, static_cast<uint8_t*>(stored),
-                         static_cast<uint16_t*>(vals), static_cast<uint16_t*>(scales), row_counts));
+  // fast path: every lane owns one chunk per segment, group width known at compile time
+  if (d->mode == HYC_MODE_CHANNEL && n.iters == 1 && g.cps == n.T && (lpg == 8 || lpg == 16) && d->bits != 1) {
+    uint16_t* yp = static_cast<uint16_t*>(y);
+    uint8_t* stp = static_cast<uint8_t*>(stored);
+    uint16_t* vp = static_cast<uint16_t*>(vals);
+    uint16_t* scp = static_cast<uint16_t*>(scales);
+#define HYC_FWD_FAST(B_, L_, W_, MT_)                                                                              \
+  hipLaunchKernelGGL((k_rmsnorm_fwd_fast<B_, L_, W_, MT_>), dim3(grid), dim3(n.T), 0, st, xp, w, eps, M, H, ca, yp, \
+                     rstd, stp, vp, scp)
+#define HYC_FWD_FAST_W(B_, L_)                                                        \
+  do {                                                                                \
+    if (n.T <= 256) { if (wf32) HYC_FWD_FAST(B_, L_, true, 256); else HYC_FWD_FAST(B_, L_, false, 256); }  \
+    else { if (wf32) HYC_FWD_FAST(B_, L_, true, 1024); else HYC_FWD_FAST(B_, L_, false, 1024); }           \
+  } while (0)
+    switch (d->bits * 100 + lpg) {
+      case 208: HYC_FWD_FAST_W(2, 8); break;
+      case 216: HYC_FWD_FAST_W(2, 16); break;
+      case 408: HYC_FWD_FAST_W(4, 8); break;
+      case 416: HYC_FWD_FAST_W(4, 16); break;
+      case 808: HYC_FWD_FAST_W(8, 8); break;
+      default: HYC_FWD_FAST_W(8, 16); break;
+    }
+#undef HYC_FWD_FAST_W
+#undef HYC_FWD_FAST
+    return check_launch("hyc_rmsnorm_fwd_compress");
   }
+#define HYC_FWD(MODE_, MT_)                                                                                        \
+  hipLaunchKernelGGL((k_rmsnorm_fwd<B, IT, MT_, MODE_>), dim3(grid), dim3(n.T), 0, st, xp, w, wf32, eps, M, H, g.cps, \
+                     ca, lpg, ta, perchan, static_cast<uint16_t*>(y), rstd, static_cast<uint8_t*>(stored),         \
+                     static_cast<uint16_t*>(vals), static_cast<uint16_t*>(scales), row_counts)
+  if (d->mode == HYC_MODE_CHANNEL) {
+    HYC_BITS_ITERS(d->bits, n.iters_t, if (n.T <= 256) HYC_FWD(0, 256); else HYC_FWD(0, 1024));
+  } else {
+    HYC_BITS_ITERS(d->bits, n.iters_t, if (n.T <= 256) HYC_FWD(1, 256); else HYC_FWD(1, 1024));
+  }
+#undef HYC_FWD
   return check_launch("hyc_rmsnorm_fwd_compress");
 }
 
@@ -317,34 +764,74 @@ int hyc_rmsnorm_bwd(const void* dy, const void* stored, const void* vals, const 
   if (rc) return rc;
   ChanArgs ca = {}; int lpg = 16;
   if (d->mode == HYC_MODE_CHANNEL && (rc = make_chan_args(d, g, &ca, &lpg))) return rc;
+  NormGeom n;
+  if ((rc = norm_geom(g.cps, &n))) return rc;
   if (!dw) return fail(HYC_EFAULT, "hyc_rmsnorm_bwd: null dw");
   hipStream_t st = begin_launch(stream);
   const bool wf32 = w_dtype == HYC_DTYPE_F32;
-  const int64_t P = hyc_rmsnorm_bwd_partials(M, H);
+  const BwdShape b = bwd_shape(M, d->bits, n);
+  const bool fast = d->mode == HYC_MODE_CHANNEL && n.iters == 1 && g.cps == n.T && d->bits != 1;
+  const int64_t used_P = fast ? b.fast_P : b.P;
   if (M > 0) {
     if (!dy || !stored || !w || !rstd || !dx || !dw_partials) return fail(HYC_EFAULT, "hyc_rmsnorm_bwd: null buffer");
     if (d->mode == HYC_MODE_CHANNEL && (!scales || (d->k > 0 && !vals))) return fail(HYC_EFAULT, "hyc_rmsnorm_bwd: null vals/scales");
     if (!aligned16(dy) || !aligned16(dx) || !aligned16(w) || !aligned16(dw_partials) || !aligned8(stored) ||
         (d->mode == HYC_MODE_DENSE && !aligned16(stored)))
       return fail(HYC_EINVAL, "hyc_rmsnorm_bwd: dy, dx, w, dw_partials must be 16-byte aligned, stored 8-byte (16 when dense)");
-    const int rpb = (int)bwd_rows_per_block(M);
     const uint16_t* gp = static_cast<const uint16_t*>(dy);
-    if (d->mode == HYC_MODE_CHANNEL) {
-      HYC_BITS_ITERS_MAXT(d->bits, round_iters(g.iters), g.threads,
-        hipLaunchKernelGGL((k_rmsnorm_bwd<B, IT, MT, 0>), dim3((unsigned)P), dim3(g.threads), 0, st, gp,
-                           static_cast<const uint8_t*>(stored), static_cast<const uint16_t*>(vals),
-                           static_cast<const uint16_t*>(scales), w, wf32, rstd, M, H, g.cps, rpb, ca, c2_quirk != 0,
-                           static_cast<uint16_t*>(dx), dw_partials));
+    const size_t lds = b.slots > 1 ? (size_t)(b.slots - 1) * n.T * 8 * sizeof(float) : 0;
+    if (fast) {
+      const int fthreads = b.fast_slots * n.T;
+      const size_t flds = b.fast_slots > 1 ? (size_t)(b.fast_slots - 1) * n.T * 8 * sizeof(float) : 0;
+#define HYC_BWD_FAST(B_, W_, Q_, MT_)                                                                              \
+  hipLaunchKernelGGL((k_rmsnorm_bwd_fast<B_, W_, Q_, MT_>), dim3((unsigned)b.fast_P), dim3(fthreads), flds, st, gp,  \
+                     static_cast<const uint8_t*>(stored), static_cast<const uint16_t*>(vals),                     \
+                     static_cast<const uint16_t*>(scales), w, rstd, M, H, n.T, b.fast_slots, ca,                   \
+                     static_cast<uint16_t*>(dx), dw_partials)
+#define HYC_BWD_FAST_WQ(B_)                                                                   \
+  do {                                                                                        \
+    const int key_ = (wf32 ? 4 : 0) + (c2_quirk ? 2 : 0) + (fthreads <= 256 ? 0 : 1);        \
+    switch (key_) {                                                                           \
+      case 0: HYC_BWD_FAST(B_, false, false, 256); break;                                     \
+      case 1: HYC_BWD_FAST(B_, false, false, 1024); break;                                    \
+      case 2: HYC_BWD_FAST(B_, false, true, 256); break;                                      \
+      case 3: HYC_BWD_FAST(B_, false, true, 1024); break;                                     \
+      case 4: HYC_BWD_FAST(B_, true, false, 256); break;                                      \
+      case 5: HYC_BWD_FAST(B_, true, false, 1024); break;                                     \
+      case 6: HYC_BWD_FAST(B_, true, true, 256); break;                                       \
+      default: HYC_BWD_FAST(B_, true, true, 1024); break;                                     \
+    }                                                                                         \
+  } while (0)
+      if (d->bits == 2) HYC_BWD_FAST_WQ(2);
+      else if (d->bits == 4) HYC_BWD_FAST_WQ(4);
+      else HYC_BWD_FAST_WQ(8);
+#undef HYC_BWD_FAST_WQ
+#undef HYC_BWD_FAST
+      if ((rc = check_launch("hyc_rmsnorm_bwd"))) return rc;
     } else {
-      HYC_BITS_ITERS_MAXT(d->bits, round_iters(g.iters), g.threads,
-        hipLaunchKernelGGL((k_rmsnorm_bwd<B, IT, MT, 2>), dim3((unsigned)P), dim3(g.threads), 0, st, gp,
-                           static_cast<const uint8_t*>(stored), static_cast<const uint16_t*>(vals),
-                           static_cast<const uint16_t*>(scales), w, wf32, rstd, M, H, g.cps, rpb, ca, c2_quirk != 0,
-                           static_cast<uint16_t*>(dx), dw_partials));
-    }
+#define HYC_BWD(SRC_)                                                                                             \
+  if (IT == 1 && b.threads <= 256)                                                                                \
+    hipLaunchKernelGGL((k_rmsnorm_bwd<B, IT, (IT == 1 ? 256 : 1024), SRC_>), dim3((unsigned)b.P), dim3(b.threads), lds, st, gp, \
+                       static_cast<const uint8_t*>(stored), static_cast<const uint16_t*>(vals),                   \
+                       static_cast<const uint16_t*>(scales), w, wf32, rstd, M, H, g.cps, n.T, b.slots, b.rpb, ca, \
+                       c2_quirk != 0, static_cast<uint16_t*>(dx), dw_partials);                                   \
+  else if (IT == 1 && b.threads <= 512)                                                                           \
+    hipLaunchKernelGGL((k_rmsnorm_bwd<B, IT, (IT == 1 ? 512 : 1024), SRC_>), dim3((unsigned)b.P), dim3(b.threads), lds, st, gp, \
+                       static_cast<const uint8_t*>(stored), static_cast<const uint16_t*>(vals),                   \
+                       static_cast<const uint16_t*>(scales), w, wf32, rstd, M, H, g.cps, n.T, b.slots, b.rpb, ca, \
+                       c2_quirk != 0, static_cast<uint16_t*>(dx), dw_partials);                                   \
+  else                                                                                                            \
+  hipLaunchKernelGGL((k_rmsnorm_bwd<B, IT, 1024, SRC_>), dim3((unsigned)b.P), dim3(b.threads), lds, st, gp,       \
+                     static_cast<const uint8_t*>(stored), static_cast<const uint16_t*>(vals),                     \
+                     static_cast<const uint16_t*>(scales), w, wf32, rstd, M, H, g.cps, n.T, b.slots, b.rpb, ca,   \
+                     c2_quirk != 0, static_cast<uint16_t*>(dx), dw_partials)
+    if (d->mode == HYC_MODE_CHANNEL) HYC_BITS_ITERS(d->bits, n.iters_t, HYC_BWD(0));
+    else HYC_BITS_ITERS(d->bits, n.iters_t, HYC_BWD(2));
+#undef HYC_BWD
     if ((rc = check_launch("hyc_rmsnorm_bwd"))) return rc;
+    }
   }
-  hipLaunchKernelGGL(k_colsum, dim3((unsigned)((H + 31) / 32)), dim3(256), 0, st, dw_partials, P, H, dw, wf32);
+  hipLaunchKernelGGL(k_colsum, dim3((unsigned)((H + 31) / 32)), dim3(256), 0, st, dw_partials, used_P, H, dw, wf32);
   return check_launch("hyc_rmsnorm_bwd (dw)");
 }
 

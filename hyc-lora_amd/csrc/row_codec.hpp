@@ -45,39 +45,81 @@ __device__ __forceinline__ uint4 pack8(const float (&v)[8]) {
   return r;
 }
 
+// 16-byte store of a streaming output (written once, not read again by this kernel): bypasses cache allocation.
+// Measured on MI355X: with loads in flight, plain 16-byte stores reach ~4.1 TB/s, these ~5.4 TB/s.
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void store_stream(uint16_t* p, const uint4& v) {
+  const u32x4_t t = {v.x, v.y, v.z, v.w};
+  __builtin_nontemporal_store(t, reinterpret_cast<u32x4_t*>(p));
+}
+
 // ---- cross-lane -------------------------------------------------------------------------------
-template <int CTRL>
+// value of another lane of the same 16-lane row.  OLD_ZERO: lanes without a source read 0 (lets the compiler fold
+// the move into v_add_f32_dpp).
+template <int CTRL, bool OLD_ZERO>
 __device__ __forceinline__ float dpp_f(float v) {
-  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
+  const int self = __builtin_bit_cast(int, v);
+  if (OLD_ZERO) return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, self, CTRL, 0xF, 0xF, false));
+  // every pattern used here (quad_perm, row_half_mirror, row_mirror) has a valid source lane for every lane, so the
+  // previous content of the destination is never read: leave it undefined (a single v_mov_b32_dpp)
+  return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(self, CTRL, 0xF, 0xF, false));
 }
 __device__ __forceinline__ float xor_lane(float v, int m) { return __shfl_xor(v, m, 64); }
+
+struct OpMax {
+  static constexpr bool ZERO = false;
+  __device__ __forceinline__ float operator()(float a, float b) const { return __builtin_elementwise_maximum(a, b); }
+};
+struct OpMin {
+  static constexpr bool ZERO = false;
+  __device__ __forceinline__ float operator()(float a, float b) const { return __builtin_elementwise_minimum(a, b); }
+};
+struct OpAdd {
+  static constexpr bool ZERO = true;
+  __device__ __forceinline__ float operator()(float a, float b) const { return a + b; }
+};
 
 // butterfly over LPG consecutive lanes (LPG a power of two <= 64); every lane of the group gets the result.
 // Must be executed by all lanes of the wave (callers feed neutral values from lanes without data).
 template <int LPG, typename Op>
 __device__ __forceinline__ float group_reduce(float v, Op op) {
-  if (LPG >= 2) v = op(v, dpp_f<0xB1>(v));   // quad_perm [1,0,3,2]
-  if (LPG >= 4) v = op(v, dpp_f<0x4E>(v));   // quad_perm [2,3,0,1]
-  if (LPG >= 8) v = op(v, dpp_f<0x141>(v));  // row_half_mirror
-  if (LPG >= 16) v = op(v, dpp_f<0x140>(v)); // row_mirror
+  if (LPG >= 2) v = op(v, dpp_f<0xB1, Op::ZERO>(v));   // quad_perm [1,0,3,2]
+  if (LPG >= 4) v = op(v, dpp_f<0x4E, Op::ZERO>(v));   // quad_perm [2,3,0,1]
+  if (LPG >= 8) v = op(v, dpp_f<0x141, Op::ZERO>(v));  // row_half_mirror
+  if (LPG >= 16) v = op(v, dpp_f<0x140, Op::ZERO>(v)); // row_mirror
   if (LPG >= 32) v = op(v, xor_lane(v, 16));
   if (LPG >= 64) v = op(v, xor_lane(v, 32));
   return v;
 }
+// max of `mx` and min of `mn` over LPG lanes, the two butterflies interleaved so that neither waits on the
+// read-after-write distance a DPP source needs
+template <int LPG>
+__device__ __forceinline__ void group_maxmin(float& mx, float& mn) {
+#define HYC_STEP(CTRL)                                                     \
+  {                                                                        \
+    const float a_ = dpp_f<CTRL, false>(mx), b_ = dpp_f<CTRL, false>(mn);  \
+    mx = __builtin_elementwise_maximum(mx, a_);                            \
+    mn = __builtin_elementwise_minimum(mn, b_);                            \
+  }
+  if (LPG >= 2) HYC_STEP(0xB1)
+  if (LPG >= 4) HYC_STEP(0x4E)
+  if (LPG >= 8) HYC_STEP(0x141)
+  if (LPG >= 16) HYC_STEP(0x140)
+#undef HYC_STEP
+  if (LPG >= 32) { mx = __builtin_elementwise_maximum(mx, xor_lane(mx, 16)); mn = __builtin_elementwise_minimum(mn, xor_lane(mn, 16)); }
+  if (LPG >= 64) { mx = __builtin_elementwise_maximum(mx, xor_lane(mx, 32)); mn = __builtin_elementwise_minimum(mn, xor_lane(mn, 32)); }
+}
 // runtime-width variant (lpg in {4, 8, 16, 32, 64}; the branches are uniform)
 template <typename Op>
 __device__ __forceinline__ float group_reduce_rt(float v, int lpg, Op op) {
-  v = op(v, dpp_f<0xB1>(v));
-  v = op(v, dpp_f<0x4E>(v));
-  if (lpg >= 8) v = op(v, dpp_f<0x141>(v));
-  if (lpg >= 16) v = op(v, dpp_f<0x140>(v));
+  v = op(v, dpp_f<0xB1, Op::ZERO>(v));
+  v = op(v, dpp_f<0x4E, Op::ZERO>(v));
+  if (lpg >= 8) v = op(v, dpp_f<0x141, Op::ZERO>(v));
+  if (lpg >= 16) v = op(v, dpp_f<0x140, Op::ZERO>(v));
   if (lpg >= 32) v = op(v, xor_lane(v, 16));
   if (lpg >= 64) v = op(v, xor_lane(v, 32));
   return v;
 }
-struct OpMax { __device__ __forceinline__ float operator()(float a, float b) const { return a > b ? a : b; } };
-struct OpMin { __device__ __forceinline__ float operator()(float a, float b) const { return a < b ? a : b; } };
-struct OpAdd { __device__ __forceinline__ float operator()(float a, float b) const { return a + b; } };
 
 __device__ __forceinline__ float wave_sum(float v) { return group_reduce<64>(v, OpAdd()); }
 
@@ -159,9 +201,82 @@ __device__ __forceinline__ float get_code(uint32_t lo, uint32_t hi, int seg, int
   return (float)((int)((byte >> (seg * BITS)) & Q<BITS>::CODE_MASK) - Q<BITS>::OFF);
 }
 
+// ---- lean forms used by the channel-mode kernels ------------------------------------------------
+// Same arithmetic as quant1 / put_codes / get_code above, arranged for few VALU operations per element.
+
+// Code bytes of 8 elements: byte j of {lo, hi} = q_j + OFF (BITS < 8) or the int8 q_j (BITS == 8).
+//   fast path  t = bf16(x * r), r = 1/s refined to full fp32 precision (see Recip); the clamp uses v_med3 and
+//              the round-half-even + offset + float->int conversion are one add of 1.5*2^23 + OFF, which leaves
+//              q + OFF in the low mantissa byte.  clamp(rint(t)) == rint(clamp(t)) because the bounds are integers.
+//   slow path  scales outside (1e-30, 1e30), zero included: IEEE division, NaN (0/0) -> q = 0.
+template <int BITS>
+__device__ __forceinline__ void codes8(const float (&v)[8], float s, uint32_t& lo, uint32_t& hi) {
+  // the added constant must stay even, or the tie-breaking of the half-even rounding flips: 1-bit codes
+  // (OFF = 1) are formed with an offset of 2 and corrected after the gather
+  constexpr int OFF_EVEN = (BITS == 8) ? 0 : ((Q<BITS>::OFF + 1) & ~1);
+  constexpr float MAGIC = 12582912.0f + (float)OFF_EVEN;
+  uint32_t u[8];
+  if (__builtin_expect(s > 1e-30f && s < 1e30f, 1)) {
+    float r = __builtin_amdgcn_rcpf(s);
+    r = __builtin_fmaf(__builtin_fmaf(-s, r, 1.0f), r, r);
+#pragma unroll
+    for (int j = 0; j < 8; j += 2) {
+      const uint32_t pk = pack_bf16(v[j] * r, v[j + 1] * r);
+      const float c0 = __builtin_amdgcn_fmed3f(bf_lo(pk), Q<BITS>::LO, Q<BITS>::HI);
+      const float c1 = __builtin_amdgcn_fmed3f(bf_hi(pk), Q<BITS>::LO, Q<BITS>::HI);
+      u[j] = __float_as_uint(c0 + MAGIC);
+      u[j + 1] = __float_as_uint(c1 + MAGIC);
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      float t = __builtin_rintf(bfr(v[j] / s));
+      t = (t != t) ? 0.f : t;
+      t = __builtin_fminf(__builtin_fmaxf(t, Q<BITS>::LO), Q<BITS>::HI);
+      u[j] = __float_as_uint(t + MAGIC);
+    }
+  }
+  // gather byte 0 of four words into one
+  const uint32_t p01 = __builtin_amdgcn_perm(u[1], u[0], 0x0c0c0400u);
+  const uint32_t p23 = __builtin_amdgcn_perm(u[3], u[2], 0x0c0c0400u);
+  const uint32_t p45 = __builtin_amdgcn_perm(u[5], u[4], 0x0c0c0400u);
+  const uint32_t p67 = __builtin_amdgcn_perm(u[7], u[6], 0x0c0c0400u);
+  lo = __builtin_amdgcn_perm(p23, p01, 0x05040100u);
+  hi = __builtin_amdgcn_perm(p67, p45, 0x05040100u);
+  if (BITS != 8 && OFF_EVEN != Q<BITS>::OFF) {
+    lo -= (uint32_t)(OFF_EVEN - Q<BITS>::OFF) * 0x01010101u;
+    hi -= (uint32_t)(OFF_EVEN - Q<BITS>::OFF) * 0x01010101u;
+  }
+}
+
+// Dequantised values of segment `seg` of a packed word, as four packed bf16 pairs:
+// x_hat = bf16((code - OFF) * s); (code - OFF) * s is exact in fp32, so one fma and one rounding.
+template <int BITS>
+__device__ __forceinline__ uint4 dequant8(uint32_t lo, uint32_t hi, int seg, float s) {
+  constexpr uint32_t REP = (BITS == 8) ? 0x80808080u : Q<BITS>::CODE_MASK * 0x01010101u;
+  uint32_t a, b;
+  if (BITS == 8) { a = lo ^ REP; b = hi ^ REP; }             // int8 -> biased unsigned (q + 128)
+  else { a = (lo >> (seg * BITS)) & REP; b = (hi >> (seg * BITS)) & REP; }
+  float c[8] = {(float)(a & 0xFFu), (float)((a >> 8) & 0xFFu), (float)((a >> 16) & 0xFFu), (float)(a >> 24),
+                (float)(b & 0xFFu), (float)((b >> 8) & 0xFFu), (float)((b >> 16) & 0xFFu), (float)(b >> 24)};
+  constexpr float OFFV = (BITS == 8) ? 128.f : (float)Q<BITS>::OFF;
+  if (__builtin_expect(s < 1e30f, 1)) {
+    const float ns = -OFFV * s;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) c[j] = __builtin_fmaf(c[j], s, ns);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) c[j] = (c[j] - OFFV) * s;
+  }
+  uint4 r;
+  r.x = pack_bf16(c[0], c[1]); r.y = pack_bf16(c[2], c[3]); r.z = pack_bf16(c[4], c[5]); r.w = pack_bf16(c[6], c[7]);
+  return r;
+}
+
 // ---- descriptors as the kernels see them -------------------------------------------------------
 struct ChanArgs {           // HYC_MODE_CHANNEL
   const uint32_t* plan;     // [H/8]
+  const int32_t* idx;       // [k] outlier channels, ascending
   int k;                    // outlier channels
   int groups_per_row;       // H / G
   int chunk_to_group_shift; // log2(G/8)

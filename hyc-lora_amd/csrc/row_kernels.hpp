@@ -14,6 +14,53 @@ __device__ __forceinline__ uint16_t raw16(const uint4& r, int j) {
 // ------------------------------------------------------------------------------------------------
 // channel mode
 // ------------------------------------------------------------------------------------------------
+// One segment-chunk of the encoder: 8 activations (already as floats, `rawseg` = their bf16 bits) -> 8 code bytes.
+// plan word `p` (see hyc_desc.chan_plan) marks the outlier channels of the chunk; their values go to vals_row and
+// they are quantised as exact zeros.  Cross-lane: every lane of the wave must take part.
+// Returns the group scale; the caller stores it from the first lane of each group.
+template <int BITS, int LPGT>
+__device__ __forceinline__ float quant_seg(float (&v)[8], int lpg, uint32_t& cl, uint32_t& ch);
+
+// LPGT: lanes per scale group when known at compile time, 0 = use the runtime value `lpg`.
+template <int BITS, int LPGT = 0>
+__device__ __forceinline__ float encode_seg(const uint4& rawseg, float (&v)[8], uint32_t p, int lpg, uint16_t* vals_row,
+                                            uint32_t& cl, uint32_t& ch) {
+  if (__builtin_expect((p & 0xFFu) != 0, 0)) {         // rare: ~k/(H/8) of the chunks
+    const uint32_t m8 = p & 0xFFu;
+    const int first = (int)(p >> 16);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if ((m8 >> j) & 1u) {
+        vals_row[first + __popc(m8 & ((1u << j) - 1u))] = raw16(rawseg, j);
+        v[j] = 0.f;                                    // x - x*mask is an exact zero
+      }
+    }
+  }
+  return quant_seg<BITS, LPGT>(v, lpg, cl, ch);
+}
+
+// group min/max -> scale -> 8 code bytes, no outlier handling (the caller has zeroed the outlier channels)
+template <int BITS, int LPGT>
+__device__ __forceinline__ float quant_seg(float (&v)[8], int lpg, uint32_t& cl, uint32_t& ch) {
+  float mx = __builtin_elementwise_maximum(__builtin_elementwise_maximum(v[0], v[1]), v[2]);
+  float mn = __builtin_elementwise_minimum(__builtin_elementwise_minimum(v[0], v[1]), v[2]);
+  mx = __builtin_elementwise_maximum(__builtin_elementwise_maximum(mx, v[3]), v[4]);
+  mn = __builtin_elementwise_minimum(__builtin_elementwise_minimum(mn, v[3]), v[4]);
+  mx = __builtin_elementwise_maximum(__builtin_elementwise_maximum(mx, v[5]), v[6]);
+  mn = __builtin_elementwise_minimum(__builtin_elementwise_minimum(mn, v[5]), v[6]);
+  mx = __builtin_elementwise_maximum(mx, v[7]);
+  mn = __builtin_elementwise_minimum(mn, v[7]);
+  if (LPGT > 0) {
+    group_maxmin<LPGT>(mx, mn);
+  } else {
+    mx = group_reduce_rt(mx, lpg, OpMax());
+    mn = group_reduce_rt(mn, lpg, OpMin());
+  }
+  const float s = bfr(bfr(mx - mn) * Q<BITS>::INV_LEVELS);   // == bf16(bf16(max-min)/levels): same integer-ratio argument
+  codes8<BITS>(v, s, cl, ch);
+  return s;
+}
+
 // Encode the NSEG chunks `raw` (chunk index c of each segment) of one row.  Every lane of the wave must
 // call this (inactive lanes pass active=false and zero data) because of the cross-lane reductions.
 // Writes the outlier values and the group scales; returns the packed word in lo/hi.
@@ -28,52 +75,116 @@ __device__ __forceinline__ void encode_chan(const uint4* raw, bool active, int c
     unpack8(raw[i], v);
     const int cg = i * CPS + c;                        // chunk index within the full row
     const uint32_t p = active ? a.plan[cg] : 0u;
-    const uint32_t m8 = p & 0xFFu;
-    if (m8) {                                          // rare: ~k/(H/8) of the chunks
-      const int first = (int)(p >> 16);
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        if ((m8 >> j) & 1u) {
-          vals_row[first + __popc(m8 & ((1u << j) - 1u))] = raw16(raw[i], j);
-          v[j] = 0.f;                                  // x - x*mask is an exact zero
-        }
-      }
-    }
-    float mx = v[0], mn = v[0];
-#pragma unroll
-    for (int j = 1; j < 8; ++j) { mx = v[j] > mx ? v[j] : mx; mn = v[j] < mn ? v[j] : mn; }
-    mx = group_reduce_rt(mx, lpg, OpMax());
-    mn = group_reduce_rt(mn, lpg, OpMin());
-    const float s = bfr(bfr(mx - mn) * Q<BITS>::INV_LEVELS);   // == bf16(bf16(max-min)/levels), see make_recip
+    uint32_t cl, ch;
+    const float s = encode_seg<BITS>(raw[i], v, p, lpg, vals_row, cl, ch);
     if (active && (c & (lpg - 1)) == 0) scales_row[cg >> a.chunk_to_group_shift] = f_to_bf(s);
-    const Recip k = make_recip(s);
-    float q[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) q[j] = quant1<BITS>(v[j], k);
-    put_codes<BITS>(q, i, lo, hi);
+    if (BITS == 8) { lo = cl; hi = ch; }
+    else { lo |= cl << (i * BITS); hi |= ch << (i * BITS); }
   }
 }
 
-// Decode chunk c of segment i of one row to 8 floats holding bf16 values.
+// Decode segment i of a packed word to 8 bf16 values (four packed pairs), given the group scale and the chunk's
+// plan word.
 template <int BITS>
-__device__ __forceinline__ void decode_chan(uint32_t lo, uint32_t hi, int i, int c, int CPS, const ChanArgs& a,
-                                            const uint16_t* vals_row, const uint16_t* scales_row, float (&v)[8]) {
-  const int cg = i * CPS + c;
-  const float s = bf_to_f(scales_row[cg >> a.chunk_to_group_shift]);
-#pragma unroll
-  for (int j = 0; j < 8; ++j) v[j] = bfr(get_code<BITS>(lo, hi, i, j) * s) + 0.f;   // 0 + d: a -0 becomes +0
-  const uint32_t p = a.plan[cg];
-  const uint32_t m8 = p & 0xFFu;
-  if (m8) {
+__device__ __forceinline__ uint4 decode_seg(uint32_t lo, uint32_t hi, int i, float s, uint32_t p, const uint16_t* vals_row) {
+  uint4 r = dequant8<BITS>(lo, hi, i, s);
+  if (__builtin_expect((p & 0xFFu) != 0, 0)) {
+    const uint32_t m8 = p & 0xFFu;
     const int first = (int)(p >> 16);
+    uint32_t w[4] = {r.x, r.y, r.z, r.w};
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       if ((m8 >> j) & 1u) {
+        // (0 + outlier) + dequant, where dequant is the zero the outlier position was quantised to
         const float o = bf_to_f(vals_row[first + __popc(m8 & ((1u << j) - 1u))]) + 0.f;
-        v[j] = bfr(o + v[j]);                          // (0 + outlier) + dequant; dequant is 0 here
+        const float d = (j & 1) ? bf_hi(w[j >> 1]) : bf_lo(w[j >> 1]);
+        const uint32_t nb = f_to_bf(o + d);
+        w[j >> 1] = (j & 1) ? ((w[j >> 1] & 0x0000FFFFu) | (nb << 16)) : ((w[j >> 1] & 0xFFFF0000u) | nb);
       }
     }
+    r = make_uint4(w[0], w[1], w[2], w[3]);
   }
+  return r;
+}
+
+// ---- outliers without per-element branches (fast kernels) -----------------------------------------------------
+// The outlier channel set is static, so what a thread has to do about outliers is the same for every row and is
+// worked out once from the plan words.
+//   decode side: the packed codes of outlier channels decode to 0 (they were quantised as zeros).  The thread
+//     requests the first two outlier values of each of its chunks together with the row's other loads and splices
+//     them into the decoded chunk with four byte-permutes whose selectors are per-lane constants.  A chunk with
+//     more than two outlier channels sends its whole wave (a static, wave-uniform choice) down decode_seg().
+//   encode side: the outlier channels are zeroed with precomputed AND masks, and the side tensor vals[m, :] is
+//     filled by the first k threads of the workgroup straight from x (gather through L1/L2, coalesced store).
+template <int NSEG>
+struct ChunkOutliers {
+  uint32_t sel[NSEG][4];   // v_perm selectors: bytes 0-3 = decoded word, 4-5 = first outlier, 6-7 = second
+  uint32_t m8[NSEG];       // outlier bit mask of the chunk
+  int vi[NSEG];            // index of the chunk's first outlier in vals[m, :]
+  bool has0[NSEG], has1[NSEG];
+  bool many;               // wave-uniform: some lane of the wave has a chunk with more than two
+
+  __device__ __forceinline__ void init(const uint32_t (&plan)[NSEG]) {
+    bool big = false;
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) {
+      m8[i] = plan[i] & 0xFFu;
+      vi[i] = (int)(plan[i] >> 16);
+      const int n = __popc(m8[i]);
+      has0[i] = n > 0; has1[i] = n > 1;
+      const int j0 = m8[i] ? __ffs(m8[i]) - 1 : 0;
+      const uint32_t rest = m8[i] & (m8[i] - 1);
+      const int j1 = rest ? __ffs(rest) - 1 : 0;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        uint32_t q = 0x03020100u;
+        if (has0[i] && (j0 >> 1) == w) q = (j0 & 1) ? ((q & 0x0000FFFFu) | 0x05040000u) : ((q & 0xFFFF0000u) | 0x00000504u);
+        if (has1[i] && (j1 >> 1) == w) q = (j1 & 1) ? ((q & 0x0000FFFFu) | 0x07060000u) : ((q & 0xFFFF0000u) | 0x00000706u);
+        sel[i][w] = q;
+      }
+      big = big || n > 2;
+    }
+    many = __ballot(big) != 0;
+  }
+  // AND masks that zero the outlier channels in the four bf16-pair words of chunk i
+  __device__ __forceinline__ void keep_masks(int i, uint32_t (&km)[4]) const {
+#pragma unroll
+    for (int w = 0; w < 4; ++w)
+      km[w] = (((m8[i] >> (2 * w)) & 1u) ? 0u : 0x0000FFFFu) | (((m8[i] >> (2 * w + 1)) & 1u) ? 0u : 0xFFFF0000u);
+  }
+  // request the first two outlier values of every chunk from vals[m, :] (no wait here)
+  __device__ __forceinline__ void request(const uint16_t* vals_row, uint32_t (&o0)[NSEG], uint32_t (&o1)[NSEG]) const {
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) {
+      o0[i] = 0; o1[i] = 0;
+      if (has0[i]) o0[i] = vals_row[vi[i]];
+      if (has1[i]) o1[i] = vals_row[vi[i] + 1];
+    }
+  }
+  // Splice the outliers into decoded chunk i.  The reconstruction is (0 + outlier) + dequant(zero code): a -0
+  // outlier comes out as +0, and a group whose scale is inf/NaN is NaN at the outlier channels too.
+  __device__ __forceinline__ uint4 splice(int i, const uint4& r, uint32_t o0, uint32_t o1, float s) const {
+    o0 = o0 == 0x8000u ? 0u : o0;
+    o1 = o1 == 0x8000u ? 0u : o1;
+    uint32_t oo = o0 | (o1 << 16);
+    oo = (0.f * s == 0.f) ? oo : 0x7FC07FC0u;
+    return make_uint4(__builtin_amdgcn_perm(oo, r.x, sel[i][0]), __builtin_amdgcn_perm(oo, r.y, sel[i][1]),
+                      __builtin_amdgcn_perm(oo, r.z, sel[i][2]), __builtin_amdgcn_perm(oo, r.w, sel[i][3]));
+  }
+};
+
+// Decode chunk c of segment i of one row (loads the scale and the plan word itself).
+template <int BITS>
+__device__ __forceinline__ uint4 decode_chan_pk(uint32_t lo, uint32_t hi, int i, int c, int CPS, const ChanArgs& a,
+                                                const uint16_t* vals_row, const uint16_t* scales_row) {
+  const int cg = i * CPS + c;
+  return decode_seg<BITS>(lo, hi, i, bf_to_f(scales_row[cg >> a.chunk_to_group_shift]), a.plan[cg], vals_row);
+}
+
+template <int BITS>
+__device__ __forceinline__ void decode_chan(uint32_t lo, uint32_t hi, int i, int c, int CPS, const ChanArgs& a,
+                                            const uint16_t* vals_row, const uint16_t* scales_row, float (&v)[8]) {
+  unpack8(decode_chan_pk<BITS>(lo, hi, i, c, CPS, a, vals_row, scales_row), v);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -103,8 +214,8 @@ __device__ __forceinline__ int encode_thr(const uint4* raw, int c, int CPS, int6
       hot += h ? 1 : 0;
       v[j] = h ? 0.f : v[j];
     }
-    float q[8];
     if (PERCHAN) {
+      float q[8];
       const uint4 sr = *reinterpret_cast<const uint4*>(a.scale + s_pos * a.sst + col);   // ssc == 1
       float sv[8];
       unpack8(sr, sv);
@@ -113,12 +224,13 @@ __device__ __forceinline__ int encode_thr(const uint4* raw, int c, int CPS, int6
         Recip k; k.s = sv[j]; k.r = 0.f; k.exact = true;
         q[j] = quant1<BITS>(v[j], k);
       }
+      put_codes<BITS>(q, i, lo, hi);
     } else {
-      const Recip k = make_recip(bf_to_f(a.scale[s_pos * a.sst]));
-#pragma unroll
-      for (int j = 0; j < 8; ++j) q[j] = quant1<BITS>(v[j], k);
+      uint32_t cl, ch;
+      codes8<BITS>(v, bf_to_f(a.scale[s_pos * a.sst]), cl, ch);
+      if (BITS == 8) { lo = cl; hi = ch; }
+      else { lo |= cl << (i * BITS); hi |= ch << (i * BITS); }
     }
-    put_codes<BITS>(q, i, lo, hi);
   }
   return hot;
 }

@@ -74,6 +74,7 @@ def channel_desc(plan: ChannelPlan, bits, group):
     d = HycDesc()
     d.mode, d.bits, d.group, d.k = _abi.MODE_CHANNEL, bits, group, plan.k
     d.chan_plan = plan.plan.data_ptr()
+    d.chan_idx = plan.idx.data_ptr() if plan.k else None
     return d
 
 

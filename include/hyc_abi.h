@@ -95,6 +95,8 @@ typedef struct hyc_desc {
   const int32_t* csr_row_ptr; /* device [M+1] */
   const int32_t* csr_cols;    /* device [nnz] */
   const void* csr_vals;       /* device bf16 [nnz] */
+  /* ---- HYC_MODE_CHANNEL (continued) ---- */
+  const int32_t* chan_idx;    /* device [k]: the outlier channels, ascending (from hyc_select_channels); needed when k > 0 */
 } hyc_desc;
 
 int hyc_abi_version(void);

@@ -41,7 +41,7 @@ def test_desc_layout_matches_header(abi):
     assert (d.mode.offset, d.bits.offset, d.group.offset, d.k.offset) == (0, 4, 8, 12)
     assert d.chan_plan.offset == 16 and d.threshold.offset == 24 and d.scale.offset == 32
     assert d.scale_stride_token.offset == 40 and d.S.offset == 56 and d.L.offset == 64 and d.rank.offset == 80
-    assert d.csr_row_ptr.offset == 88 and ctypes.sizeof(d) == 112
+    assert d.csr_row_ptr.offset == 88 and d.chan_idx.offset == 112 and ctypes.sizeof(d) == 120
 
 
 def test_shape_queries(abi):

@@ -65,7 +65,9 @@ def test_rmsnorm_channel(K, bits, group, M, H, k, wdt):
     # the dense-source variant gives the same result as the fused one
     dx2, dw2 = K.rmsnorm_bwd(dy.cuda(), xh.cuda(), w.cuda(), rstd, c2_quirk=True)
     dx1, dw1 = K.rmsnorm_bwd(dy.cuda(), c, w.cuda(), rstd, c2_quirk=True)
-    assert bits_equal(dx1, dx2) and torch.equal(dw1, dw2)
+    # the two variants may split the row over a different number of waves: sums agree to fp32 rounding
+    assert bf16_ulp_diff(dx1.cpu(), dx2.cpu()).max() <= 1
+    assert torch.allclose(dw1.float(), dw2.float(), rtol=1e-2 if wdt == torch.bfloat16 else 1e-4, atol=1e-5)
 
 
 def test_rmsnorm_bwd_is_deterministic(K):
