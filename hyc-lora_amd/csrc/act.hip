@@ -116,9 +116,11 @@ __device__ __forceinline__ void act_grad8(const float (&x)[8], const float (&g)[
 template <int BITS, int ACT, int MAXT>
 __global__ void __launch_bounds__(MAXT)
 k_act_bwd_fast(const uint16_t* __restrict__ g, const uint8_t* __restrict__ stored, const uint16_t* __restrict__ vals,
-               const uint16_t* __restrict__ scales, int64_t M, int64_t H, ChanArgs ca, uint16_t* __restrict__ dx) {
+               const uint16_t* __restrict__ scales, int64_t M, int64_t H, int CPS, ChanArgs ca,
+               uint16_t* __restrict__ dx) {
   constexpr int NSEG = Q<BITS>::NSEG;
-  const int c = threadIdx.x, CPS = blockDim.x;
+  const int c = threadIdx.x;
+  if (c >= CPS) return;                                 // tail of the last wave
   const int64_t SEG = (int64_t)CPS * 8;
   const int seg_groups = CPS >> ca.chunk_to_group_shift;
   uint32_t plan[NSEG];
@@ -227,18 +229,18 @@ static int launch_act(const void* g, const void* stored, const void* vals, const
   const int64_t cap = 256 * (geo.threads >= 512 ? 3 : 8);
   const int grid = (int)(M < cap ? M : cap);
   hipStream_t st = begin_launch(stream);
-  if (d->mode == HYC_MODE_CHANNEL && geo.iters == 1 && geo.cps == geo.threads && d->bits != 1) {
+  if (d->mode == HYC_MODE_CHANNEL && geo.iters == 1 && d->bits != 1) {
 #define HYC_ACT_FAST(B_)                                                                                       \
   do {                                                                                                         \
     if (geo.threads <= 256)                                                                                    \
       hipLaunchKernelGGL((k_act_bwd_fast<B_, ACT, 256>), dim3(grid), dim3(geo.threads), 0, st,                 \
                          static_cast<const uint16_t*>(g), static_cast<const uint8_t*>(stored),                 \
-                         static_cast<const uint16_t*>(vals), static_cast<const uint16_t*>(scales), M, H, ca,   \
+                         static_cast<const uint16_t*>(vals), static_cast<const uint16_t*>(scales), M, H, geo.cps, ca, \
                          static_cast<uint16_t*>(dx));                                                          \
     else                                                                                                       \
       hipLaunchKernelGGL((k_act_bwd_fast<B_, ACT, 1024>), dim3(grid), dim3(geo.threads), 0, st,                \
                          static_cast<const uint16_t*>(g), static_cast<const uint8_t*>(stored),                 \
-                         static_cast<const uint16_t*>(vals), static_cast<const uint16_t*>(scales), M, H, ca,   \
+                         static_cast<const uint16_t*>(vals), static_cast<const uint16_t*>(scales), M, H, geo.cps, ca, \
                          static_cast<uint16_t*>(dx));                                                          \
   } while (0)
     if (d->bits == 2) HYC_ACT_FAST(2);

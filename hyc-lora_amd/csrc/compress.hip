@@ -65,10 +65,11 @@ k_decompress_chan(const uint8_t* __restrict__ stored, const uint16_t* __restrict
 // current one is processed.
 template <int BITS, int LPGT, int MAXT>
 __global__ void __launch_bounds__(MAXT)
-k_compress_chan_fast(const uint16_t* __restrict__ x, int64_t M, int64_t H, ChanArgs a, uint8_t* __restrict__ stored,
-                     uint16_t* __restrict__ vals, uint16_t* __restrict__ scales) {
+k_compress_chan_fast(const uint16_t* __restrict__ x, int64_t M, int64_t H, int CPS, ChanArgs a,
+                     uint8_t* __restrict__ stored, uint16_t* __restrict__ vals, uint16_t* __restrict__ scales) {
   constexpr int NSEG = Q<BITS>::NSEG;
-  const int c = threadIdx.x, CPS = blockDim.x;
+  const int c = threadIdx.x;
+  if (c >= CPS) return;                                 // tail of the last wave; scale groups never straddle it
   const int64_t SEG = (int64_t)CPS * 8;
   const bool leader = (c & (LPGT - 1)) == 0;
   const int seg_groups = CPS >> a.chunk_to_group_shift;
@@ -133,9 +134,11 @@ k_compress_chan_fast(const uint16_t* __restrict__ x, int64_t M, int64_t H, ChanA
 template <int BITS, int MAXT>
 __global__ void __launch_bounds__(MAXT)
 k_decompress_chan_fast(const uint8_t* __restrict__ stored, const uint16_t* __restrict__ vals,
-                       const uint16_t* __restrict__ scales, int64_t M, int64_t H, ChanArgs a, uint16_t* __restrict__ xhat) {
+                       const uint16_t* __restrict__ scales, int64_t M, int64_t H, int CPS, ChanArgs a,
+                       uint16_t* __restrict__ xhat) {
   constexpr int NSEG = Q<BITS>::NSEG;
-  const int c = threadIdx.x, CPS = blockDim.x;
+  const int c = threadIdx.x;
+  if (c >= CPS) return;
   const int64_t SEG = (int64_t)CPS * 8;
   const int seg_groups = CPS >> a.chunk_to_group_shift;
   uint32_t plan[NSEG];
@@ -383,16 +386,16 @@ int hyc_compress(const void* x, int64_t M, int64_t H, const hyc_desc* d, void* s
     if (!x || !stored || !scales || (d->k > 0 && !vals)) return fail(HYC_EFAULT, "hyc_compress: null buffer");
     if (!aligned16(x) || !aligned8(stored)) return fail(HYC_EINVAL, "hyc_compress: x must be 16-byte and stored 8-byte aligned");
     const int grid = row_grid(M, g.threads);
-    if (g.iters == 1 && g.cps == g.threads && (lpg == 8 || lpg == 16) && d->bits != 1) {
+    if (g.iters == 1 && (lpg == 8 || lpg == 16) && d->bits != 1) {
 #define HYC_CF(B_, L_)                                                                                             \
   do {                                                                                                             \
     if (g.threads <= 256)                                                                                          \
       hipLaunchKernelGGL((k_compress_chan_fast<B_, L_, 256>), dim3(grid), dim3(g.threads), 0, st,                  \
-                         static_cast<const uint16_t*>(x), M, H, a, static_cast<uint8_t*>(stored),                  \
+                         static_cast<const uint16_t*>(x), M, H, g.cps, a, static_cast<uint8_t*>(stored),                 \
                          static_cast<uint16_t*>(vals), static_cast<uint16_t*>(scales));                            \
     else                                                                                                           \
       hipLaunchKernelGGL((k_compress_chan_fast<B_, L_, 1024>), dim3(grid), dim3(g.threads), 0, st,                 \
-                         static_cast<const uint16_t*>(x), M, H, a, static_cast<uint8_t*>(stored),                  \
+                         static_cast<const uint16_t*>(x), M, H, g.cps, a, static_cast<uint8_t*>(stored),                 \
                          static_cast<uint16_t*>(vals), static_cast<uint16_t*>(scales));                            \
   } while (0)
       switch (d->bits * 100 + lpg) {
@@ -446,17 +449,17 @@ int hyc_decompress(const void* stored, const void* vals, const void* scales, int
     if (!stored || !xhat || !scales || (d->k > 0 && !vals)) return fail(HYC_EFAULT, "hyc_decompress: null buffer");
     if (!aligned16(xhat) || !aligned8(stored)) return fail(HYC_EINVAL, "hyc_decompress: xhat must be 16-byte and stored 8-byte aligned");
     const int grid = row_grid(M, g.threads);
-    if (g.iters == 1 && g.cps == g.threads && d->bits != 1) {
+    if (g.iters == 1 && d->bits != 1) {
 #define HYC_DF(B_)                                                                                                 \
   do {                                                                                                             \
     if (g.threads <= 256)                                                                                          \
       hipLaunchKernelGGL((k_decompress_chan_fast<B_, 256>), dim3(grid), dim3(g.threads), 0, st,                    \
                          static_cast<const uint8_t*>(stored), static_cast<const uint16_t*>(vals),                  \
-                         static_cast<const uint16_t*>(scales), M, H, a, static_cast<uint16_t*>(xhat));             \
+                         static_cast<const uint16_t*>(scales), M, H, g.cps, a, static_cast<uint16_t*>(xhat));         \
     else                                                                                                           \
       hipLaunchKernelGGL((k_decompress_chan_fast<B_, 1024>), dim3(grid), dim3(g.threads), 0, st,                   \
                          static_cast<const uint8_t*>(stored), static_cast<const uint16_t*>(vals),                  \
-                         static_cast<const uint16_t*>(scales), M, H, a, static_cast<uint16_t*>(xhat));             \
+                         static_cast<const uint16_t*>(scales), M, H, g.cps, a, static_cast<uint16_t*>(xhat));         \
   } while (0)
       if (d->bits == 2) HYC_DF(2);
       else if (d->bits == 4) HYC_DF(4);

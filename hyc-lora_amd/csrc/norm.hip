@@ -61,15 +61,16 @@ __device__ __forceinline__ float block_sum1(float a, float (*red)[16], int parit
 template <int BITS, int LPGT, bool WF32, int MAXT>
 __global__ void __launch_bounds__(MAXT)
 k_rmsnorm_fwd_fast(const uint16_t* __restrict__ x, const void* __restrict__ w, float eps, int64_t M, int64_t H,
-                   ChanArgs ca, uint16_t* __restrict__ y, float* __restrict__ rstd_out, uint8_t* __restrict__ stored,
+                   int CPS, ChanArgs ca, uint16_t* __restrict__ y, float* __restrict__ rstd_out, uint8_t* __restrict__ stored,
                    uint16_t* __restrict__ vals, uint16_t* __restrict__ scales) {
   constexpr int NSEG = Q<BITS>::NSEG;
   __shared__ float red[2][16];
-  const int c = threadIdx.x, CPS = blockDim.x;
+  const int c = threadIdx.x;
+  const bool active = c < CPS;                                    // false only in the tail of the last wave
   const int64_t SEG = (int64_t)CPS * 8;
   const float invH = 1.0f / (float)H;
-  const int wave = c >> 6, nw = CPS >> 6;
-  const bool leader = (c & (LPGT - 1)) == 0;
+  const int wave = c >> 6, nw = blockDim.x >> 6;
+  const bool leader = active && (c & (LPGT - 1)) == 0;
 
   uint32_t km[NSEG][4];                                            // AND masks that zero the outlier channels
   float wv[NSEG][8];
@@ -77,15 +78,20 @@ k_rmsnorm_fwd_fast(const uint16_t* __restrict__ x, const void* __restrict__ w, f
     uint32_t plan[NSEG];
 #pragma unroll
     for (int i = 0; i < NSEG; ++i) {
-      plan[i] = ca.plan[i * CPS + c];
-      load_w8t<WF32>(w, i * SEG + 8 * c, wv[i]);
+      plan[i] = 0;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) wv[i][j] = 0.f;
+      if (active) {
+        plan[i] = ca.plan[i * CPS + c];
+        load_w8t<WF32>(w, i * SEG + 8 * c, wv[i]);
+      }
     }
     ChunkOutliers<NSEG> co;
     co.init(plan);
 #pragma unroll
     for (int i = 0; i < NSEG; ++i) co.keep_masks(i, km[i]);
   }
-  const bool gather = c < ca.k;                                   // thread c copies outlier channel idx[c] to vals
+  const bool gather = active && c < ca.k;                                  // thread c copies outlier channel idx[c] to vals
   const int idx0 = gather ? ca.idx[c] : 0;
   const int64_t stride = gridDim.x;
   int64_t row = blockIdx.x;
@@ -100,7 +106,9 @@ k_rmsnorm_fwd_fast(const uint16_t* __restrict__ x, const void* __restrict__ w, f
 
   uint4 raw[NSEG];
   uint16_t o = 0;
-  if (row < M) {
+#pragma unroll
+  for (int i = 0; i < NSEG; ++i) raw[i] = make_uint4(0, 0, 0, 0);
+  if (row < M && active) {
 #pragma unroll
     for (int i = 0; i < NSEG; ++i) raw[i] = *reinterpret_cast<const uint4*>(xp + i * SEG);
     if (gather) o = xrow[idx0];
@@ -109,7 +117,7 @@ k_rmsnorm_fwd_fast(const uint16_t* __restrict__ x, const void* __restrict__ w, f
   for (; row < M; row += stride, parity ^= 1) {
     uint4 nxt[NSEG];
     uint16_t o_n = 0;
-    if (row + stride < M) {                                         // uniform
+    if (row + stride < M && active) {
 #pragma unroll
       for (int i = 0; i < NSEG; ++i) nxt[i] = *reinterpret_cast<const uint4*>(xp + xstep + i * SEG);
       if (gather) o_n = xrow[xstep + idx0];
@@ -129,12 +137,12 @@ k_rmsnorm_fwd_fast(const uint16_t* __restrict__ x, const void* __restrict__ w, f
       if (BITS == 8) { lo = cl; hi = ch; }
       else { lo |= cl << (i * BITS); hi |= ch << (i * BITS); }
     }
-    *reinterpret_cast<uint2*>(sp) = make_uint2(lo, hi);
+    if (active) *reinterpret_cast<uint2*>(sp) = make_uint2(lo, hi);
     if (gather) {
       vp[c] = o;
       for (int t = c + CPS; t < ca.k; t += CPS) vp[t] = xrow[ca.idx[t]];   // only when k exceeds the workgroup size
     }
-    ss = block_sum1(ss, red, parity, wave, nw);
+    ss = block_sum1(active ? ss : 0.f, red, parity, wave, nw);      // inactive lanes hold no data
     const float rstd = 1.0f / __builtin_sqrtf(ss * invH + eps);
     if (c == 0) rstd_out[row] = rstd;
 #pragma unroll
@@ -143,7 +151,7 @@ k_rmsnorm_fwd_fast(const uint16_t* __restrict__ x, const void* __restrict__ w, f
       unpack8(raw[i], v);
 #pragma unroll
       for (int j = 0; j < 8; ++j) v[j] = (v[j] * rstd) * wv[i][j];
-      store_stream(yp + i * SEG, pack8(v));
+      if (active) store_stream(yp + i * SEG, pack8(v));
     }
 #pragma unroll
     for (int i = 0; i < NSEG; ++i) raw[i] = nxt[i];
@@ -160,36 +168,45 @@ template <int BITS, bool WF32, bool QUIRK, int MAXT>
 __global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(4, 8)))
 k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ stored, const uint16_t* __restrict__ vals,
                    const uint16_t* __restrict__ scales, const void* __restrict__ w, const float* __restrict__ rstd,
-                   int64_t M, int64_t H, int CPS, int slots, ChanArgs ca, uint16_t* __restrict__ dx,
+                   int64_t M, int64_t H, int T, int CPS, int slots, ChanArgs ca, uint16_t* __restrict__ dx,
                    float* __restrict__ dw_partials) {
-  constexpr int NSEG = Q<BITS>::NSEG;
+  // A thread decodes at most two segments of its packed word: with four segments (2-bit codes) two threads share
+  // a word, which keeps the per-thread state (and so the occupancy) the same for every bit width.
+  constexpr int NSEG = Q<BITS>::NSEG > 2 ? 2 : Q<BITS>::NSEG;         // segments per thread
+  constexpr int PARTS = Q<BITS>::NSEG / NSEG;                         // threads per packed word
   __shared__ float red[2][16][2][16];                                 // [parity][slot][value][wave]
-  extern __shared__ __align__(16) float xslot[];                      // [slots-1][CPS][8]
-  const int slot = threadIdx.x / CPS, c = threadIdx.x - slot * CPS;
+  extern __shared__ __align__(16) float xslot[];                      // [slots-1][T][8]
+  const int slot = threadIdx.x / T, u = threadIdx.x - slot * T;       // T = PARTS*CPS rounded up to whole waves
+  const bool active = u < PARTS * CPS;
+  const int part = PARTS > 1 ? u / CPS : 0, c = u - part * CPS;
+  const int seg0 = part * NSEG;                                       // first segment of this thread
   const int64_t SEG = (int64_t)CPS * 8;
   const float invH = 1.0f / (float)H;
-  const int wave = c >> 6, nw = CPS >> 6;
+  const int wave = u >> 6, nw = T >> 6;
   const int seg_groups = CPS >> ca.chunk_to_group_shift;
 
   uint32_t plan[NSEG];
   float wv[NSEG][8], acc[NSEG][8];
 #pragma unroll
   for (int i = 0; i < NSEG; ++i) {
-    plan[i] = ca.plan[i * CPS + c];
-    load_w8t<WF32>(w, i * SEG + 8 * c, wv[i]);
+    plan[i] = 0;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc[i][j] = 0.f;
+    for (int j = 0; j < 8; ++j) { acc[i][j] = 0.f; wv[i][j] = 0.f; }
+    if (active) {
+      plan[i] = ca.plan[(seg0 + i) * CPS + c];
+      load_w8t<WF32>(w, (seg0 + i) * SEG + 8 * c, wv[i]);
+    }
   }
   ChunkOutliers<NSEG> co;
   co.init(plan);
   const int64_t stride = (int64_t)gridDim.x * slots;
   int64_t row = (int64_t)blockIdx.x * slots + slot;
   const int64_t steps = (M + stride - 1) / stride;                    // the same for every slot: barriers stay matched
-  const uint16_t* gp = dy + row * H + 8 * c;
-  uint16_t* dxp = dx + row * H + 8 * c;
+  const uint16_t* gp = dy + row * H + seg0 * SEG + 8 * c;
+  uint16_t* dxp = dx + row * H + seg0 * SEG + 8 * c;
   const uint8_t* sp = stored + row * SEG + 8 * c;
   const uint16_t* vp = vals + row * ca.k;
-  const uint16_t* scp = scales + row * ca.groups_per_row + (c >> ca.chunk_to_group_shift);
+  const uint16_t* scp = scales + row * ca.groups_per_row + seg0 * seg_groups + (c >> ca.chunk_to_group_shift);
 
   uint2 pk = make_uint2(0, 0);
   uint4 graw[NSEG];
@@ -198,7 +215,7 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
   float rs = 0.f;
 #pragma unroll
   for (int i = 0; i < NSEG; ++i) { graw[i] = make_uint4(0, 0, 0, 0); sc[i] = 0; o0[i] = 0; o1[i] = 0; }
-  if (row < M) {                                                      // uniform per wave
+  if (row < M && active) {
     pk = *reinterpret_cast<const uint2*>(sp);
     rs = rstd[row];
 #pragma unroll
@@ -207,14 +224,14 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
   }
   int parity = 0;
   for (int64_t step = 0; step < steps; ++step, row += stride, parity ^= 1) {
-    const bool valid = row < M;
+    const bool valid = row < M && active;
     uint2 pk_n = make_uint2(0, 0);
     uint4 g_n[NSEG];
     uint32_t sc_n[NSEG], o0_n[NSEG], o1_n[NSEG];
     float rs_n = 0.f;
 #pragma unroll
     for (int i = 0; i < NSEG; ++i) { g_n[i] = make_uint4(0, 0, 0, 0); sc_n[i] = 0; o0_n[i] = 0; o1_n[i] = 0; }
-    if (row + stride < M) {                                           // uniform per wave
+    if (row + stride < M && active) {
       pk_n = *reinterpret_cast<const uint2*>(sp + stride * SEG);
       rs_n = rstd[row + stride];
 #pragma unroll
@@ -231,8 +248,8 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
       float g[8];
       unpack8(graw[i], g);
       const float sf = bf_to_f((uint16_t)sc[i]);
-      if (!co.many) unpack8(co.splice(i, dequant8<BITS>(pk.x, pk.y, i, sf), o0[i], o1[i], sf), xn[i]);
-      else unpack8(decode_seg<BITS>(pk.x, pk.y, i, sf, valid ? plan[i] : 0u, vp), xn[i]);
+      if (!co.many) unpack8(co.splice(i, dequant8<BITS>(pk.x, pk.y, seg0 + i, sf), o0[i], o1[i], sf), xn[i]);
+      else unpack8(decode_seg<BITS>(pk.x, pk.y, seg0 + i, sf, valid ? plan[i] : 0u, vp), xn[i]);
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const float n = xn[i][j] * rs;
@@ -247,7 +264,7 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
     // two sums per slot, one barrier
     p1 = wave_sum(p1);
     if (QUIRK) p2 = wave_sum(p2);
-    if ((c & 63) == 0) { red[parity][slot][0][wave] = p1; if (QUIRK) red[parity][slot][1][wave] = p2; }
+    if ((u & 63) == 0) { red[parity][slot][0][wave] = p1; if (QUIRK) red[parity][slot][1][wave] = p2; }
     __syncthreads();
     float t1 = red[parity][slot][0][0], t2 = QUIRK ? red[parity][slot][1][0] : 0.f;
     for (int i = 1; i < nw; ++i) { t1 += red[parity][slot][0][i]; if (QUIRK) t2 += red[parity][slot][1][i]; }
@@ -268,27 +285,27 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
     for (int i = 0; i < NSEG; ++i) { graw[i] = g_n[i]; sc[i] = sc_n[i]; o0[i] = o0_n[i]; o1[i] = o1_n[i]; }
     gp += stride * H; dxp += stride * H; sp += stride * SEG; vp += stride * ca.k; scp += stride * ca.groups_per_row;
   }
-  float* pr = dw_partials + (int64_t)blockIdx.x * H + 8 * c;
+  float* pr = dw_partials + (int64_t)blockIdx.x * H + seg0 * SEG + 8 * c;
 #pragma unroll
   for (int i = 0; i < NSEG; ++i) {
     if (slots > 1) {
       __syncthreads();
       if (slot > 0) {
-        float4* o = reinterpret_cast<float4*>(xslot + ((int64_t)(slot - 1) * CPS + c) * 8);
+        float4* o = reinterpret_cast<float4*>(xslot + ((int64_t)(slot - 1) * T + u) * 8);
         o[0] = make_float4(acc[i][0], acc[i][1], acc[i][2], acc[i][3]);
         o[1] = make_float4(acc[i][4], acc[i][5], acc[i][6], acc[i][7]);
       }
       __syncthreads();
       if (slot == 0) {
         for (int s2 = 1; s2 < slots; ++s2) {
-          const float4* o = reinterpret_cast<const float4*>(xslot + ((int64_t)(s2 - 1) * CPS + c) * 8);
+          const float4* o = reinterpret_cast<const float4*>(xslot + ((int64_t)(s2 - 1) * T + u) * 8);
           const float4 a = o[0], b = o[1];
           acc[i][0] += a.x; acc[i][1] += a.y; acc[i][2] += a.z; acc[i][3] += a.w;
           acc[i][4] += b.x; acc[i][5] += b.y; acc[i][6] += b.z; acc[i][7] += b.w;
         }
       }
     }
-    if (slot == 0) {
+    if (slot == 0 && active) {
       float4* o = reinterpret_cast<float4*>(pr + i * SEG);
       o[0] = make_float4(acc[i][0], acc[i][1], acc[i][2], acc[i][3]);
       o[1] = make_float4(acc[i][4], acc[i][5], acc[i][6], acc[i][7]);
@@ -626,11 +643,15 @@ struct BwdShape {
   int slots, threads, rpb;
   int64_t P;
   int fast_slots;      // fast path: row slots per workgroup and workgroups (= partial rows)
+  int fast_T;          //   threads per row slot (two threads share a packed word of 2-bit codes)
+  bool fast_ok;
   int64_t fast_P;
 };
-static inline BwdShape bwd_shape(int64_t M, int bits, const NormGeom& n) {
-  (void)bits;
+static inline BwdShape bwd_shape(int64_t M, int bits, int cps, const NormGeom& n) {
   BwdShape b;
+  const int parts = bits == 2 ? 2 : 1;
+  b.fast_T = ((parts * cps + 63) / 64) * 64;
+  b.fast_ok = n.iters == 1 && bits != 1 && b.fast_T <= 1024;
   b.slots = n.T <= 256 ? BWD_SLOTS_SMALL : 1;
   b.threads = b.slots * n.T;
   // about a thousand row slots in flight; each walks at least four rows so the partial rows stay few
@@ -640,10 +661,11 @@ static inline BwdShape bwd_shape(int64_t M, int bits, const NormGeom& n) {
   b.rpb = (int)rpb;
   b.P = M > 0 ? (M + rpb - 1) / rpb : 0;
   // fast path: up to 1024 threads per workgroup, one workgroup per CU slot; every slot walks at least two rows
-  int fs = 1024 / n.T;
+  const int ft = b.fast_ok ? b.fast_T : 1024;
+  int fs = 1024 / ft;
   if (fs < 1) fs = 1;
   if (fs > BWD_FAST_SLOTS_MAX) fs = BWD_FAST_SLOTS_MAX;
-  int64_t fp = 256 * (int64_t)(1024 / (fs * n.T) > 0 ? 1024 / (fs * n.T) : 1);
+  int64_t fp = 256 * (int64_t)(1024 / (fs * ft) > 0 ? 1024 / (fs * ft) : 1);
   const int64_t need = (M + 2 * fs - 1) / (2 * fs);
   if (fp > need) fp = need;
   if (fp < 1) fp = 1;
@@ -679,7 +701,7 @@ int64_t hyc_rmsnorm_bwd_partials(int64_t M, int64_t H) {
     if (H % (64 / bits) != 0) continue;
     NormGeom n;
     if (norm_geom((int)(H * bits / 64), &n)) continue;
-    const BwdShape b = bwd_shape(M, bits, n);
+    const BwdShape b = bwd_shape(M, bits, (int)(H * bits / 64), n);
     if (b.P > best) best = b.P;
     if (b.fast_P > best) best = b.fast_P;
   }
@@ -712,13 +734,13 @@ int hyc_rmsnorm_fwd_compress(const void* x, const void* w, int32_t w_dtype, floa
   hipStream_t st = begin_launch(stream);
   const uint16_t* xp = static_cast<const uint16_t*>(x);
   // fast path: every lane owns one chunk per segment, group width known at compile time
-  if (d->mode == HYC_MODE_CHANNEL && n.iters == 1 && g.cps == n.T && (lpg == 8 || lpg == 16) && d->bits != 1) {
+  if (d->mode == HYC_MODE_CHANNEL && n.iters == 1 && (lpg == 8 || lpg == 16) && d->bits != 1) {
     uint16_t* yp = static_cast<uint16_t*>(y);
     uint8_t* stp = static_cast<uint8_t*>(stored);
     uint16_t* vp = static_cast<uint16_t*>(vals);
     uint16_t* scp = static_cast<uint16_t*>(scales);
 #define HYC_FWD_FAST(B_, L_, W_, MT_)                                                                              \
-  hipLaunchKernelGGL((k_rmsnorm_fwd_fast<B_, L_, W_, MT_>), dim3(grid), dim3(n.T), 0, st, xp, w, eps, M, H, ca, yp, \
+  hipLaunchKernelGGL((k_rmsnorm_fwd_fast<B_, L_, W_, MT_>), dim3(grid), dim3(n.T), 0, st, xp, w, eps, M, H, g.cps, ca, yp, \
                      rstd, stp, vp, scp)
 #define HYC_FWD_FAST_W(B_, L_)                                                        \
   do {                                                                                \
@@ -769,8 +791,8 @@ int hyc_rmsnorm_bwd(const void* dy, const void* stored, const void* vals, const 
   if (!dw) return fail(HYC_EFAULT, "hyc_rmsnorm_bwd: null dw");
   hipStream_t st = begin_launch(stream);
   const bool wf32 = w_dtype == HYC_DTYPE_F32;
-  const BwdShape b = bwd_shape(M, d->bits, n);
-  const bool fast = d->mode == HYC_MODE_CHANNEL && n.iters == 1 && g.cps == n.T && d->bits != 1;
+  const BwdShape b = bwd_shape(M, d->bits, g.cps, n);
+  const bool fast = d->mode == HYC_MODE_CHANNEL && b.fast_ok;
   const int64_t used_P = fast ? b.fast_P : b.P;
   if (M > 0) {
     if (!dy || !stored || !w || !rstd || !dx || !dw_partials) return fail(HYC_EFAULT, "hyc_rmsnorm_bwd: null buffer");
@@ -781,12 +803,12 @@ int hyc_rmsnorm_bwd(const void* dy, const void* stored, const void* vals, const 
     const uint16_t* gp = static_cast<const uint16_t*>(dy);
     const size_t lds = b.slots > 1 ? (size_t)(b.slots - 1) * n.T * 8 * sizeof(float) : 0;
     if (fast) {
-      const int fthreads = b.fast_slots * n.T;
-      const size_t flds = b.fast_slots > 1 ? (size_t)(b.fast_slots - 1) * n.T * 8 * sizeof(float) : 0;
+      const int fthreads = b.fast_slots * b.fast_T;
+      const size_t flds = b.fast_slots > 1 ? (size_t)(b.fast_slots - 1) * b.fast_T * 8 * sizeof(float) : 0;
 #define HYC_BWD_FAST(B_, W_, Q_, MT_)                                                                              \
   hipLaunchKernelGGL((k_rmsnorm_bwd_fast<B_, W_, Q_, MT_>), dim3((unsigned)b.fast_P), dim3(fthreads), flds, st, gp,  \
                      static_cast<const uint8_t*>(stored), static_cast<const uint16_t*>(vals),                     \
-                     static_cast<const uint16_t*>(scales), w, rstd, M, H, n.T, b.fast_slots, ca,                   \
+                     static_cast<const uint16_t*>(scales), w, rstd, M, H, b.fast_T, g.cps, b.fast_slots, ca,       \
                      static_cast<uint16_t*>(dx), dw_partials)
 #define HYC_BWD_FAST_WQ(B_)                                                                   \
   do {                                                                                        \

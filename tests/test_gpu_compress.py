@@ -62,6 +62,11 @@ CH_CASES = [
     (8, 128, 32, 4096, 41), (1, 64, 32, 4096, 41), (4, 32, 17, 512, 5), (4, 256, 17, 2048, 20),
     (8, 512, 9, 4096, 0), (2, 32, 5, 256, 3), (1, 32, 3, 256, 2), (8, 32, 1, 64, 1), (4, 64, 130, 1024, 10),
     (8, 128, 20, 16384, 164), (4, 128, 6, 32768, 328),
+    # more rows than workgroups (rows are walked with the next one requested ahead), full and partial last wave
+    (4, 128, 4133, 4096, 41), (2, 64, 4133, 4096, 41), (4, 128, 800, 11008, 110), (2, 64, 2100, 11008, 110),
+    (8, 64, 900, 4096, 41),
+    # more outlier channels than threads in a workgroup; several outliers per chunk
+    (2, 32, 40, 1024, 200), (4, 32, 40, 512, 300), (4, 64, 40, 512, 300), (8, 128, 40, 1024, 700),
 ]
 
 
@@ -84,6 +89,38 @@ def test_channel_roundtrip(K, bits, group, M, H, k):
     want = O.hyc_decompress(vals, stored, idx, scales, bits, group)
     assert bits_equal(xh, want)
     assert bits_equal(xh[:, idx.long()], x[:, idx.long()])
+
+
+@pytest.mark.parametrize("bits,group", [(4, 64), (2, 64), (8, 128)])
+def test_channel_special_values(K, bits, group):
+    """A -0 in an outlier channel comes back as +0 (the reconstruction is a sum with a +0); a group that holds an
+    inf has a non-finite scale and reconstructs as NaN everywhere, its outlier channels included."""
+    M, H, k = 8, 1024, 10
+    x, _ = make_x(77, M, H, k, 30.0)
+    amax = O.hyc_channel_scores(x)
+    idx = O.hyc_select_channels(amax, k)
+    ch = int(idx[0])
+    other = next(c for c in range(ch - ch % group, ch - ch % group + group) if c not in set(idx.tolist()))
+    x[3, ch] = -0.0
+    x[4, other] = float("inf")
+    x[5, other] = float("-inf")
+    plan = K.select_channels(amax.cuda(), k)
+    assert torch.equal(plan.idx.cpu(), idx)
+    c = K.compress_channel(x.cuda(), plan, bits, group)
+    vals, stored, scales = O.hyc_compress(x, idx, bits, group)
+    assert bits_equal(c.vals.cpu(), vals)
+    # The reference zeroes outliers as x - x*mask, which turns a non-outlier inf into NaN before the scale is taken;
+    # the kernel masks bits and keeps the inf.  Either way the group's scale is non-finite and the group decodes to NaN.
+    rows = [r for r in range(M) if r not in (4, 5)]
+    assert bits_equal(c.scales.cpu()[rows], scales[rows]) and torch.equal(c.stored.cpu()[rows], stored[rows])
+    assert not bool(c.scales.cpu()[4, ch // group].float().isfinite())
+    got = K.decompress_channel(c).cpu()
+    want = O.hyc_decompress(vals, stored, idx, scales, bits, group)
+    assert torch.equal(got.isnan(), want.isnan())
+    assert bool(want[4, ch].isnan()) and bool(want[5, ch].isnan())
+    ok = ~want.isnan()
+    assert torch.equal(got.view(torch.int16)[ok], want.view(torch.int16)[ok])
+    assert got[3, ch].view(torch.int16).item() == 0          # +0, not the stored -0
 
 
 def test_channel_config1_shape(K):
