@@ -19,6 +19,11 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes per launch at the bench workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# `bench.py --pmc-probe`, scaled by what the same counters read for a plain copy of known size
+# (profiles/rmsnorm_fwd_bwd_config2.md).  None until measured for the current kernels.
+TRAFFIC_FWD = None
+TRAFFIC_BWD = None
 
 
 def algorithmic_bytes(M, H, bits, group, k):
@@ -66,6 +71,7 @@ class Workload:
                           p(self.y), p(self.rstd), p(self.c.stored), p(self.c.vals), p(self.c.scales), None)
         self._bwd_args = (p(self.dy), p(self.c.stored), p(self.c.vals), p(self.c.scales), p(self.w), abi.DTYPE_F32,
                           p(self.rstd), M, H, ctypes.byref(self.desc), 1, p(self.dx), p(self.partials), p(self.dw))
+        self._bwd_main_args = self._bwd_args[:-1] + (None,)     # dw = NULL: the row kernel alone, no column sum
         self._check = abi.check
 
     def _stream(self):
@@ -76,6 +82,9 @@ class Workload:
 
     def bwd(self):
         self._check(self.lib.hyc_rmsnorm_bwd(*self._bwd_args, self._stream()))
+
+    def bwd_main(self):
+        self._check(self.lib.hyc_rmsnorm_bwd(*self._bwd_main_args, self._stream()))
 
     def step(self):
         self.fwd()
@@ -159,6 +168,9 @@ def main():
             wl.fwd()
         for _ in range(5):
             wl.bwd()
+        for case in (("silu", 4), ("gelu", 4)):
+            for _ in range(5):
+                pkg.kernels.act_bwd(case[0], wl.dy, wl.c)
         torch.cuda.synchronize()
         print(json.dumps({"pmc_probe": True, "copy_bytes_each_way": 2 * M * H, "fwd_bytes": fwd_b, "bwd_bytes": bwd_b}))
         return
@@ -187,14 +199,19 @@ def main():
     eager_ms = time_events(torch, wl.step, args.steps, args.warmup)
     fwd_ms = time_events(torch, wl.fwd, args.steps, args.warmup)
     bwd_ms = time_events(torch, wl.bwd, args.steps, args.warmup)
+    bwd_main_ms = time_events(torch, wl.bwd_main, args.steps, args.warmup)   # k_rmsnorm_bwd_fast alone
 
     value = (fwd_b + bwd_b) / (ms_step * 1e-3) / 1e9
-    dom_name, dom_ms, dom_b = ("hyc_rmsnorm_bwd", bwd_ms, bwd_b) if bwd_ms >= fwd_ms else ("hyc_rmsnorm_fwd_compress", fwd_ms, fwd_b)
+    if bwd_main_ms >= fwd_ms:
+        dom_name, dom_ms, dom_b, dom_traffic = "hyc::k_rmsnorm_bwd_fast<4,true,true,1024>", bwd_main_ms, bwd_b, TRAFFIC_BWD
+    else:
+        dom_name, dom_ms, dom_b, dom_traffic = "hyc::k_rmsnorm_fwd_fast<4,16,true,256>", fwd_ms, fwd_b, TRAFFIC_FWD
     achieved = dom_b / (dom_ms * 1e-3) / 1e9
     extra = {
         "eager_ms_per_step": round(eager_ms, 5),
         "fwd_kernel_ms": round(fwd_ms, 5), "fwd_GBps": round(fwd_b / fwd_ms / 1e6, 1),
         "bwd_kernels_ms": round(bwd_ms, 5), "bwd_GBps": round(bwd_b / bwd_ms / 1e6, 1),
+        "bwd_row_kernel_ms": round(bwd_main_ms, 5), "bwd_row_kernel_GBps": round(bwd_b / bwd_main_ms / 1e6, 1),
         "act_mem_bytes_saved_tensor": saved_b + 4 * M, "act_mem_bytes_bf16": 2 * M * H,
         "act_mem_ratio": round(2 * M * H / (saved_b + 4 * M), 3),
     }
@@ -220,7 +237,8 @@ def main():
                    "tokens": M, "hidden": H, "bits": bits, "group": group, "outlier_channels": wl.k,
                    "launch": "hip graph replay of fwd + bwd + dw-reduce"},
         "roofline": {"bound": "hbm", "kernel": dom_name, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None},
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "algorithmic_bytes": dom_b,
+                     "traffic": dom_traffic},
         "extra": extra,
     }
     if not args.no_cpu_baseline:

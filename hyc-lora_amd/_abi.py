@@ -39,6 +39,7 @@ SIGNATURES = {
     "hyc_check_shape": (c_i32, [c_i64, c_i32, c_i32, c_i32]),
     "hyc_stored_row_bytes": (c_i64, [c_i64, c_i32]),
     "hyc_rmsnorm_bwd_partials": (c_i64, [c_i64, c_i64]),
+    "hyc_rmsnorm_bwd_partial_rows": (c_i64, [c_i64, c_i64, ctypes.POINTER(HycDesc)]),
     "hyc_channel_absmax": (c_i32, [c_ptr, c_i64, c_i64, c_ptr, c_ptr]),
     "hyc_select_channels": (c_i32, [c_ptr, c_i64, c_i32, c_ptr, c_ptr, c_ptr]),
     "hyc_compress": (c_i32, [c_ptr, c_i64, c_i64, ctypes.POINTER(HycDesc), c_ptr, c_ptr, c_ptr, c_ptr, c_ptr]),

@@ -163,8 +163,9 @@ k_act_bwd_fast(const uint16_t* __restrict__ g, const uint8_t* __restrict__ store
     for (int i = 0; i < NSEG; ++i) {
       float xv[8], gv[8], o[8];
       const float sf = bf_to_f((uint16_t)sc[i]);
-      if (!co.many) unpack8(co.splice(i, dequant8<BITS>(pk.x, pk.y, i, sf), o0[i], o1[i], sf), xv);
-      else unpack8(decode_seg<BITS>(pk.x, pk.y, i, sf, plan[i], vp), xv);
+      uint4 r = co.splice(i, dequant8<BITS>(pk.x, pk.y, i, sf), o0[i], o1[i], sf);
+      if (co.more_pairs) r = splice_more(r, co.more_pairs, ca.plan[i * CPS + c], vp, true, sf);
+      unpack8(r, xv);
       unpack8(graw[i], gv);
       act_grad8<ACT>(xv, gv, o);
       store_stream(dxp + i * SEG, pack8(o));

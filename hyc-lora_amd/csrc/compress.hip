@@ -171,16 +171,12 @@ k_decompress_chan_fast(const uint8_t* __restrict__ stored, const uint16_t* __res
       for (int i = 0; i < NSEG; ++i) sc_n[i] = scp[scstep + i * seg_groups];
       co.request(vp + vstep, o0_n, o1_n);
     }
-    if (!co.many) {
 #pragma unroll
-      for (int i = 0; i < NSEG; ++i) {
-        const float sf = bf_to_f((uint16_t)sc[i]);
-        store_stream(xp + i * SEG, co.splice(i, dequant8<BITS>(pk.x, pk.y, i, sf), o0[i], o1[i], sf));
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < NSEG; ++i)
-        store_stream(xp + i * SEG, decode_seg<BITS>(pk.x, pk.y, i, bf_to_f((uint16_t)sc[i]), plan[i], vp));
+    for (int i = 0; i < NSEG; ++i) {
+      const float sf = bf_to_f((uint16_t)sc[i]);
+      uint4 r = co.splice(i, dequant8<BITS>(pk.x, pk.y, i, sf), o0[i], o1[i], sf);
+      if (co.more_pairs) r = splice_more(r, co.more_pairs, a.plan[i * CPS + c], vp, true, sf);
+      store_stream(xp + i * SEG, r);
     }
     pk = pk_n;
 #pragma unroll

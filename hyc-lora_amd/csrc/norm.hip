@@ -175,38 +175,57 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
   constexpr int NSEG = Q<BITS>::NSEG > 2 ? 2 : Q<BITS>::NSEG;         // segments per thread
   constexpr int PARTS = Q<BITS>::NSEG / NSEG;                         // threads per packed word
   __shared__ float red[2][16][2][16];                                 // [parity][slot][value][wave]
-  extern __shared__ __align__(16) float xslot[];                      // [slots-1][T][8]
-  const int slot = threadIdx.x / T, u = threadIdx.x - slot * T;       // T = PARTS*CPS rounded up to whole waves
+  // dynamic LDS: the weight row as fp32 [segment][half chunk][CPS] float4 (read again for every row: sixteen
+  // registers fewer than keeping the thread's weights live), then [slots-1][T][8] floats for the final dw sum
+  extern __shared__ __align__(16) float lds_dyn[];
+  float4* wl4 = reinterpret_cast<float4*>(lds_dyn);
+  float* xslot = lds_dyn + H;
+  // T = PARTS*CPS rounded up to whole waves, so the slot is the same for a whole wave: row bases stay scalar
+  const int slot = __builtin_amdgcn_readfirstlane((int)threadIdx.x / T);
+  const int u = (int)threadIdx.x - slot * T;
   const bool active = u < PARTS * CPS;
   const int part = PARTS > 1 ? u / CPS : 0, c = u - part * CPS;
   const int seg0 = part * NSEG;                                       // first segment of this thread
-  const int64_t SEG = (int64_t)CPS * 8;
+  const int SEG = CPS * 8;                                            // channels per segment = bytes per stored row
   const float invH = 1.0f / (float)H;
   const int wave = u >> 6, nw = T >> 6;
   const int seg_groups = CPS >> ca.chunk_to_group_shift;
+  // byte offsets of the thread inside a row of each tensor; 32 bits, added to a scalar row base by the load itself
+  const uint32_t xo = (uint32_t)(seg0 * SEG + 8 * c) * 2u;
+  const uint32_t so = 8u * (uint32_t)c;
+  const uint32_t go = (uint32_t)(seg0 * seg_groups + (c >> ca.chunk_to_group_shift)) * 2u;
+  const int64_t seg_b = (int64_t)SEG * 2, grp_b = (int64_t)seg_groups * 2;
 
   uint32_t plan[NSEG];
-  float wv[NSEG][8], acc[NSEG][8];
+  float acc[NSEG][8];
 #pragma unroll
   for (int i = 0; i < NSEG; ++i) {
     plan[i] = 0;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) { acc[i][j] = 0.f; wv[i][j] = 0.f; }
+    for (int j = 0; j < 8; ++j) acc[i][j] = 0.f;
     if (active) {
       plan[i] = ca.plan[(seg0 + i) * CPS + c];
-      load_w8t<WF32>(w, (seg0 + i) * SEG + 8 * c, wv[i]);
+      if (slot == 0) {
+        float wv[8];
+        load_w8t<WF32>(w, (int64_t)(seg0 + i) * SEG + 8 * c, wv);
+        wl4[((seg0 + i) * 2 + 0) * CPS + c] = make_float4(wv[0], wv[1], wv[2], wv[3]);
+        wl4[((seg0 + i) * 2 + 1) * CPS + c] = make_float4(wv[4], wv[5], wv[6], wv[7]);
+      }
     }
   }
   ChunkOutliers<NSEG> co;
   co.init(plan);
+  __syncthreads();                                                    // the weight row is in LDS
+  const uint32_t wbase = active ? (uint32_t)(seg0 * 2 * CPS + c) : 0u;
   const int64_t stride = (int64_t)gridDim.x * slots;
   int64_t row = (int64_t)blockIdx.x * slots + slot;
   const int64_t steps = (M + stride - 1) / stride;                    // the same for every slot: barriers stay matched
-  const uint16_t* gp = dy + row * H + seg0 * SEG + 8 * c;
-  uint16_t* dxp = dx + row * H + seg0 * SEG + 8 * c;
-  const uint8_t* sp = stored + row * SEG + 8 * c;
-  const uint16_t* vp = vals + row * ca.k;
-  const uint16_t* scp = scales + row * ca.groups_per_row + seg0 * seg_groups + (c >> ca.chunk_to_group_shift);
+  const int64_t xstep = stride * H * 2, sstep = stride * SEG, vstep = stride * ca.k * 2, gstep = stride * ca.groups_per_row * 2;
+  const char* gq = reinterpret_cast<const char*>(dy) + row * H * 2;
+  char* dq = reinterpret_cast<char*>(dx) + row * H * 2;
+  const char* sq = reinterpret_cast<const char*>(stored) + row * SEG;
+  const char* vq = reinterpret_cast<const char*>(vals) + row * ca.k * 2;
+  const char* cq = reinterpret_cast<const char*>(scales) + row * ca.groups_per_row * 2;
 
   uint2 pk = make_uint2(0, 0);
   uint4 graw[NSEG];
@@ -216,30 +235,27 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
 #pragma unroll
   for (int i = 0; i < NSEG; ++i) { graw[i] = make_uint4(0, 0, 0, 0); sc[i] = 0; o0[i] = 0; o1[i] = 0; }
   if (row < M && active) {
-    pk = *reinterpret_cast<const uint2*>(sp);
+    pk = *reinterpret_cast<const uint2*>(sq + so);
     rs = rstd[row];
 #pragma unroll
-    for (int i = 0; i < NSEG; ++i) { graw[i] = *reinterpret_cast<const uint4*>(gp + i * SEG); sc[i] = scp[i * seg_groups]; }
-    co.request(vp, o0, o1);
+    for (int i = 0; i < NSEG; ++i) {
+      graw[i] = *reinterpret_cast<const uint4*>(gq + i * seg_b + xo);
+      sc[i] = *reinterpret_cast<const uint16_t*>(cq + i * grp_b + go);
+    }
+    co.request(reinterpret_cast<const uint16_t*>(vq), o0, o1);
   }
   int parity = 0;
   for (int64_t step = 0; step < steps; ++step, row += stride, parity ^= 1) {
     const bool valid = row < M && active;
-    uint2 pk_n = make_uint2(0, 0);
-    uint4 g_n[NSEG];
-    uint32_t sc_n[NSEG], o0_n[NSEG], o1_n[NSEG];
+    const bool more = row + stride < M && active;
+    uint4 g_n[NSEG];                                                  // the bulk of the next row: requested a row ahead
     float rs_n = 0.f;
 #pragma unroll
-    for (int i = 0; i < NSEG; ++i) { g_n[i] = make_uint4(0, 0, 0, 0); sc_n[i] = 0; o0_n[i] = 0; o1_n[i] = 0; }
-    if (row + stride < M && active) {
-      pk_n = *reinterpret_cast<const uint2*>(sp + stride * SEG);
+    for (int i = 0; i < NSEG; ++i) g_n[i] = make_uint4(0, 0, 0, 0);
+    if (more) {
       rs_n = rstd[row + stride];
 #pragma unroll
-      for (int i = 0; i < NSEG; ++i) {
-        g_n[i] = *reinterpret_cast<const uint4*>(gp + stride * H + i * SEG);
-        sc_n[i] = scp[stride * ca.groups_per_row + i * seg_groups];
-      }
-      co.request(vp + stride * ca.k, o0_n, o1_n);
+      for (int i = 0; i < NSEG; ++i) g_n[i] = *reinterpret_cast<const uint4*>(gq + xstep + i * seg_b + xo);
     }
     float xn[NSEG][8], wdy[NSEG][8];
     float p1 = 0.f, p2 = 0.f;
@@ -248,18 +264,32 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
       float g[8];
       unpack8(graw[i], g);
       const float sf = bf_to_f((uint16_t)sc[i]);
-      if (!co.many) unpack8(co.splice(i, dequant8<BITS>(pk.x, pk.y, seg0 + i, sf), o0[i], o1[i], sf), xn[i]);
-      else unpack8(decode_seg<BITS>(pk.x, pk.y, seg0 + i, sf, valid ? plan[i] : 0u, vp), xn[i]);
+      uint4 r = co.splice(i, dequant8<BITS>(pk.x, pk.y, seg0 + i, sf), o0[i], o1[i], sf);
+      if (co.more_pairs)
+        r = splice_more(r, co.more_pairs, ca.plan[(seg0 + i) * CPS + c], reinterpret_cast<const uint16_t*>(vq), valid, sf);
+      unpack8(r, xn[i]);
+      uint32_t wo = wbase + (uint32_t)(i * 2 * CPS);
+      asm volatile("" : "+v"(wo));                                    // re-read per row: do not keep the weights live
+      const float4 wa = wl4[wo], wb = wl4[wo + CPS];
+      const float wv[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const float n = xn[i][j] * rs;
-        const float t = wv[i][j] * g[j];
+        const float t = wv[j] * g[j];
         xn[i][j] = n;
         wdy[i][j] = t;
         p1 = __builtin_fmaf(n, t, p1);
         if (QUIRK) p2 += t;
         acc[i][j] = __builtin_fmaf(g[j], n, acc[i][j]);
       }
+    }
+    // The compressed row is decoded: its registers take the next row's codes, scales and outliers now (a row's
+    // worth of registers less than requesting them at the top; the barrier and the second pass cover the latency).
+    if (more) {
+      pk = *reinterpret_cast<const uint2*>(sq + sstep + so);
+#pragma unroll
+      for (int i = 0; i < NSEG; ++i) sc[i] = *reinterpret_cast<const uint16_t*>(cq + gstep + i * grp_b + go);
+      co.request(reinterpret_cast<const uint16_t*>(vq + vstep), o0, o1);
     }
     // two sums per slot, one barrier
     p1 = wave_sum(p1);
@@ -277,15 +307,15 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
         float o[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) o[j] = __builtin_fmaf(xn[i][j], k1, __builtin_fmaf(wdy[i][j], rs, k2));
-        store_stream(dxp + i * SEG, pack8(o));
+        store_stream(reinterpret_cast<uint16_t*>(dq + i * seg_b + xo), pack8(o));
       }
     }
-    pk = pk_n; rs = rs_n;
+    rs = rs_n;
 #pragma unroll
-    for (int i = 0; i < NSEG; ++i) { graw[i] = g_n[i]; sc[i] = sc_n[i]; o0[i] = o0_n[i]; o1[i] = o1_n[i]; }
-    gp += stride * H; dxp += stride * H; sp += stride * SEG; vp += stride * ca.k; scp += stride * ca.groups_per_row;
+    for (int i = 0; i < NSEG; ++i) graw[i] = g_n[i];
+    gq += xstep; dq += xstep; sq += sstep; vq += vstep; cq += gstep;
   }
-  float* pr = dw_partials + (int64_t)blockIdx.x * H + seg0 * SEG + 8 * c;
+  float* pr = dw_partials + (int64_t)blockIdx.x * H + (int64_t)seg0 * SEG + 8 * c;
 #pragma unroll
   for (int i = 0; i < NSEG; ++i) {
     if (slots > 1) {
@@ -306,7 +336,7 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
       }
     }
     if (slot == 0 && active) {
-      float4* o = reinterpret_cast<float4*>(pr + i * SEG);
+      float4* o = reinterpret_cast<float4*>(pr + (int64_t)i * SEG);
       o[0] = make_float4(acc[i][0], acc[i][1], acc[i][2], acc[i][3]);
       o[1] = make_float4(acc[i][4], acc[i][5], acc[i][6], acc[i][7]);
     }
@@ -708,6 +738,15 @@ int64_t hyc_rmsnorm_bwd_partials(int64_t M, int64_t H) {
   return best;
 }
 
+int64_t hyc_rmsnorm_bwd_partial_rows(int64_t M, int64_t H, const hyc_desc* d) {
+  if (!d || M <= 0 || H <= 0) return 0;
+  RowGeom g;
+  NormGeom n;
+  if (row_geom(H, d->bits, &g) || norm_geom(g.cps, &n)) return 0;
+  const BwdShape b = bwd_shape(M, d->bits, g.cps, n);
+  return (d->mode == HYC_MODE_CHANNEL && b.fast_ok) ? b.fast_P : b.P;
+}
+
 int hyc_rmsnorm_fwd_compress(const void* x, const void* w, int32_t w_dtype, float eps, int64_t M, int64_t H,
                              const hyc_desc* d, void* y, float* rstd, void* stored, void* vals, void* scales,
                              int32_t* row_counts, void* stream) {
@@ -788,7 +827,6 @@ int hyc_rmsnorm_bwd(const void* dy, const void* stored, const void* vals, const 
   if (d->mode == HYC_MODE_CHANNEL && (rc = make_chan_args(d, g, &ca, &lpg))) return rc;
   NormGeom n;
   if ((rc = norm_geom(g.cps, &n))) return rc;
-  if (!dw) return fail(HYC_EFAULT, "hyc_rmsnorm_bwd: null dw");
   hipStream_t st = begin_launch(stream);
   const bool wf32 = w_dtype == HYC_DTYPE_F32;
   const BwdShape b = bwd_shape(M, d->bits, g.cps, n);
@@ -804,7 +842,8 @@ int hyc_rmsnorm_bwd(const void* dy, const void* stored, const void* vals, const 
     const size_t lds = b.slots > 1 ? (size_t)(b.slots - 1) * n.T * 8 * sizeof(float) : 0;
     if (fast) {
       const int fthreads = b.fast_slots * b.fast_T;
-      const size_t flds = b.fast_slots > 1 ? (size_t)(b.fast_slots - 1) * b.fast_T * 8 * sizeof(float) : 0;
+      const size_t flds = (size_t)H * sizeof(float) +
+                          (b.fast_slots > 1 ? (size_t)(b.fast_slots - 1) * b.fast_T * 8 * sizeof(float) : 0);
 #define HYC_BWD_FAST(B_, W_, Q_, MT_)                                                                              \
   hipLaunchKernelGGL((k_rmsnorm_bwd_fast<B_, W_, Q_, MT_>), dim3((unsigned)b.fast_P), dim3(fthreads), flds, st, gp,  \
                      static_cast<const uint8_t*>(stored), static_cast<const uint16_t*>(vals),                     \
@@ -853,6 +892,7 @@ int hyc_rmsnorm_bwd(const void* dy, const void* stored, const void* vals, const 
     if ((rc = check_launch("hyc_rmsnorm_bwd"))) return rc;
     }
   }
+  if (!dw) return HYC_OK;                        // the caller adds up the partial rows itself
   hipLaunchKernelGGL(k_colsum, dim3((unsigned)((H + 31) / 32)), dim3(256), 0, st, dw_partials, used_P, H, dw, wf32);
   return check_launch("hyc_rmsnorm_bwd (dw)");
 }

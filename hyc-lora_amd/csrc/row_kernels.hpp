@@ -112,39 +112,57 @@ __device__ __forceinline__ uint4 decode_seg(uint32_t lo, uint32_t hi, int i, flo
 // worked out once from the plan words.
 //   decode side: the packed codes of outlier channels decode to 0 (they were quantised as zeros).  The thread
 //     requests the first two outlier values of each of its chunks together with the row's other loads and splices
-//     them into the decoded chunk with four byte-permutes whose selectors are per-lane constants.  A chunk with
-//     more than two outlier channels sends its whole wave (a static, wave-uniform choice) down decode_seg().
+//     them into the decoded chunk with four byte-permutes whose selectors are per-lane constants.  Chunks with
+//     more than two outlier channels are finished by splice_more(): a loop whose trip count is the same for the
+//     whole wave and zero unless one of its lanes owns such a chunk.
 //   encode side: the outlier channels are zeroed with precomputed AND masks, and the side tensor vals[m, :] is
 //     filled by the first k threads of the workgroup straight from x (gather through L1/L2, coalesced store).
+
+// v_perm selectors that put outlier j0 (bytes 4-5 of the outlier pair word) and, if has1, j1 (bytes 6-7) into the
+// four bf16-pair words of a decoded chunk; bytes 0-3 keep the decoded word
+__device__ __forceinline__ void splice_selectors(bool has0, int j0, bool has1, int j1, uint32_t (&sel)[4]) {
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    uint32_t q = 0x03020100u;
+    if (has0 && (j0 >> 1) == w) q = (j0 & 1) ? ((q & 0x0000FFFFu) | 0x05040000u) : ((q & 0xFFFF0000u) | 0x00000504u);
+    if (has1 && (j1 >> 1) == w) q = (j1 & 1) ? ((q & 0x0000FFFFu) | 0x07060000u) : ((q & 0xFFFF0000u) | 0x00000706u);
+    sel[w] = q;
+  }
+}
+// The reconstruction is (0 + outlier) + dequant(zero code): a -0 outlier comes out as +0, and a group whose scale
+// is inf/NaN is NaN at the outlier channels too.
+__device__ __forceinline__ uint4 splice_pair(const uint4& r, const uint32_t (&sel)[4], uint32_t o0, uint32_t o1, float s) {
+  o0 = o0 == 0x8000u ? 0u : o0;
+  o1 = o1 == 0x8000u ? 0u : o1;
+  uint32_t oo = o0 | (o1 << 16);
+  oo = (0.f * s == 0.f) ? oo : 0x7FC07FC0u;
+  return make_uint4(__builtin_amdgcn_perm(oo, r.x, sel[0]), __builtin_amdgcn_perm(oo, r.y, sel[1]),
+                    __builtin_amdgcn_perm(oo, r.z, sel[2]), __builtin_amdgcn_perm(oo, r.w, sel[3]));
+}
+
 template <int NSEG>
 struct ChunkOutliers {
-  uint32_t sel[NSEG][4];   // v_perm selectors: bytes 0-3 = decoded word, 4-5 = first outlier, 6-7 = second
+  uint32_t sel[NSEG][4];   // selectors of the first outlier pair
   uint32_t m8[NSEG];       // outlier bit mask of the chunk
-  int vi[NSEG];            // index of the chunk's first outlier in vals[m, :]
+  uint32_t vb[NSEG];       // byte offset of the chunk's first outlier in vals[m, :]
   bool has0[NSEG], has1[NSEG];
-  bool many;               // wave-uniform: some lane of the wave has a chunk with more than two
+  int more_pairs;          // wave-uniform: outlier pairs beyond the first in the fullest chunk of the wave (0..3)
 
   __device__ __forceinline__ void init(const uint32_t (&plan)[NSEG]) {
-    bool big = false;
+    int most = 0;
 #pragma unroll
     for (int i = 0; i < NSEG; ++i) {
       m8[i] = plan[i] & 0xFFu;
-      vi[i] = (int)(plan[i] >> 16);
+      vb[i] = (plan[i] >> 16) * 2u;
       const int n = __popc(m8[i]);
       has0[i] = n > 0; has1[i] = n > 1;
       const int j0 = m8[i] ? __ffs(m8[i]) - 1 : 0;
       const uint32_t rest = m8[i] & (m8[i] - 1);
       const int j1 = rest ? __ffs(rest) - 1 : 0;
-#pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        uint32_t q = 0x03020100u;
-        if (has0[i] && (j0 >> 1) == w) q = (j0 & 1) ? ((q & 0x0000FFFFu) | 0x05040000u) : ((q & 0xFFFF0000u) | 0x00000504u);
-        if (has1[i] && (j1 >> 1) == w) q = (j1 & 1) ? ((q & 0x0000FFFFu) | 0x07060000u) : ((q & 0xFFFF0000u) | 0x00000706u);
-        sel[i][w] = q;
-      }
-      big = big || n > 2;
+      splice_selectors(has0[i], j0, has1[i], j1, sel[i]);
+      most = n > most ? n : most;
     }
-    many = __ballot(big) != 0;
+    more_pairs = (__ballot(most > 2) != 0) + (__ballot(most > 4) != 0) + (__ballot(most > 6) != 0);
   }
   // AND masks that zero the outlier channels in the four bf16-pair words of chunk i
   __device__ __forceinline__ void keep_masks(int i, uint32_t (&km)[4]) const {
@@ -157,21 +175,34 @@ struct ChunkOutliers {
 #pragma unroll
     for (int i = 0; i < NSEG; ++i) {
       o0[i] = 0; o1[i] = 0;
-      if (has0[i]) o0[i] = vals_row[vi[i]];
-      if (has1[i]) o1[i] = vals_row[vi[i] + 1];
+      const char* b = reinterpret_cast<const char*>(vals_row);        // uniform base + 32-bit lane offset
+      if (has0[i]) o0[i] = *reinterpret_cast<const uint16_t*>(b + vb[i]);
+      if (has1[i]) o1[i] = *reinterpret_cast<const uint16_t*>((b + 2) + vb[i]);
     }
   }
-  // Splice the outliers into decoded chunk i.  The reconstruction is (0 + outlier) + dequant(zero code): a -0
-  // outlier comes out as +0, and a group whose scale is inf/NaN is NaN at the outlier channels too.
   __device__ __forceinline__ uint4 splice(int i, const uint4& r, uint32_t o0, uint32_t o1, float s) const {
-    o0 = o0 == 0x8000u ? 0u : o0;
-    o1 = o1 == 0x8000u ? 0u : o1;
-    uint32_t oo = o0 | (o1 << 16);
-    oo = (0.f * s == 0.f) ? oo : 0x7FC07FC0u;
-    return make_uint4(__builtin_amdgcn_perm(oo, r.x, sel[i][0]), __builtin_amdgcn_perm(oo, r.y, sel[i][1]),
-                      __builtin_amdgcn_perm(oo, r.z, sel[i][2]), __builtin_amdgcn_perm(oo, r.w, sel[i][3]));
+    return splice_pair(r, sel[i], o0, o1, s);
   }
 };
+
+// Outlier pairs 1..more_pairs of a chunk (plan word p); `ok` = the row exists.  Loads and waits in place: only
+// waves that own a chunk with more than two outlier channels come here.
+__device__ __forceinline__ uint4 splice_more(uint4 r, int more_pairs, uint32_t p, const uint16_t* vals_row, bool ok, float s) {
+  uint32_t m = p & 0xFFu;
+  int at = (int)(p >> 16);
+  for (int q = 1; q <= more_pairs; ++q) {
+    m &= m - 1; m &= m - 1;                              // drop the pair already spliced
+    at += 2;
+    if (m != 0 && ok) {
+      const uint32_t rest = m & (m - 1);
+      uint32_t sel[4];
+      splice_selectors(true, __ffs(m) - 1, rest != 0, rest ? __ffs(rest) - 1 : 0, sel);
+      const uint32_t o0 = vals_row[at], o1 = rest ? vals_row[at + 1] : 0u;
+      r = splice_pair(r, sel, o0, o1, s);
+    }
+  }
+  return r;
+}
 
 // Decode chunk c of segment i of one row (loads the scale and the plan word itself).
 template <int BITS>

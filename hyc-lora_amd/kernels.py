@@ -319,6 +319,20 @@ def rmsnorm_bwd(dy2d, src, w, rstd, c2_quirk=True):
     return dx, dw
 
 
+def rmsnorm_bwd_partial(dy2d, src, w, rstd, c2_quirk=True):
+    """-> (dx bf16 [M,H], fp32 partial rows [P,H] whose column sum is dw); the caller does the last reduction"""
+    _need(dy2d, BF16, "dy")
+    M, H = dy2d.shape
+    lib = _abi.load()
+    stored, vals, scales, d = _source(src)
+    P = lib.hyc_rmsnorm_bwd_partials(M, H)
+    partials = torch.empty((max(P, 1), H), dtype=torch.float32, device=dy2d.device)
+    dx = torch.empty_like(dy2d)
+    check(lib.hyc_rmsnorm_bwd(_p(dy2d), _p(stored), _p(vals), _p(scales), _p(w), _wdtype(w), _p(rstd), M, H,
+                              ctypes.byref(d), 1 if c2_quirk else 0, _p(dx), _p(partials), None, _stream()))
+    return dx, partials[:lib.hyc_rmsnorm_bwd_partial_rows(M, H, ctypes.byref(d))]
+
+
 def act_bwd(act, g2d, src):
     """act in {'silu', 'gelu'} -> dx bf16 [M,H]"""
     _need(g2d, BF16, "grad_output")

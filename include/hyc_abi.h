@@ -106,8 +106,10 @@ const char* hyc_last_error(void);
 int hyc_check_shape(int64_t H, int32_t bits, int32_t group, int32_t mode);
 /* bytes of one stored row: H*bits/8 */
 int64_t hyc_stored_row_bytes(int64_t H, int32_t bits);
-/* number of fp32 [H] partial rows hyc_rmsnorm_bwd needs in dw_partials for M tokens */
+/* number of fp32 [H] partial rows hyc_rmsnorm_bwd needs in dw_partials for M tokens (an upper bound over all
+ * descriptors), and the number it actually writes, rows [0, n), for one descriptor */
 int64_t hyc_rmsnorm_bwd_partials(int64_t M, int64_t H);
+int64_t hyc_rmsnorm_bwd_partial_rows(int64_t M, int64_t H, const hyc_desc* d);
 
 /* ---- calibration, channel mode --------------------------------------------------------------- */
 /* amax[c] = max(amax[c], max_m |x[m, c]|); the caller zero-fills amax (fp32 [H]) before the first call. */
@@ -137,7 +139,9 @@ int hyc_rmsnorm_fwd_compress(const void* x, const void* w, int32_t w_dtype, floa
                              const hyc_desc* d, void* y, float* rstd, void* stored, void* vals, void* scales,
                              int32_t* row_counts, void* stream);
 /* dx = (w*dy - (xn*c1 + c2))*rstd with xn = xhat*rstd, c1 = mean(xn*w*dy), c2 = c2_quirk ? mean(w*dy) : 0;
- * dw = sum_m dy*xn (fp32 accumulation, fixed order) written in w's dtype. */
+ * dw = sum_m dy*xn (fp32 accumulation, fixed order) written in w's dtype.  With dw == NULL the last step, the
+ * column sum of the partial rows, is left to the caller (e.g. to accumulate over micro-batches first):
+ * dw = sum of rows [0, hyc_rmsnorm_bwd_partial_rows(M, H, d)) of dw_partials. */
 int hyc_rmsnorm_bwd(const void* dy, const void* stored, const void* vals, const void* scales, const void* w,
                     int32_t w_dtype, const float* rstd, int64_t M, int64_t H, const hyc_desc* d, int32_t c2_quirk,
                     void* dx, float* dw_partials, void* dw, void* stream);

@@ -76,6 +76,20 @@ def test_rmsnorm_channel(K, bits, group, M, H, k, wdt):
     assert torch.allclose(dw1.float(), dw2.float(), rtol=1e-2 if wdt == torch.bfloat16 else 1e-4, atol=1e-5)
 
 
+@pytest.mark.parametrize("bits,M,H", [(4, 300, 4096), (2, 50, 11008), (1, 40, 1024)])
+def test_rmsnorm_bwd_partial_rows(K, bits, M, H):
+    """dw == NULL leaves the column sum to the caller: the partial rows add up to the dw of the full call"""
+    x, gen = make_x(3, M, H, 10, 30.0)
+    w = 1 + 0.1 * torch.randn(H, generator=gen)
+    dy = (0.02 * torch.randn(M, H, generator=gen)).bfloat16()
+    plan = K.select_channels(K.channel_absmax(x.cuda()), 10)
+    y, rstd, c = K.rmsnorm_fwd_compress_channel(x.cuda(), w.cuda(), 1e-6, plan, bits, 64)
+    dx, dw = K.rmsnorm_bwd(dy.cuda(), c, w.cuda(), rstd)
+    dx2, part = K.rmsnorm_bwd_partial(dy.cuda(), c, w.cuda(), rstd)
+    assert bits_equal(dx, dx2) and part.shape[0] >= 1
+    assert torch.allclose(part.sum(0), dw, rtol=1e-5, atol=1e-6)
+
+
 def test_rmsnorm_bwd_is_deterministic(K):
     x, gen = make_x(9, 512, 4096, 20, 30.0)
     w = (1 + 0.1 * torch.randn(4096, generator=gen))
