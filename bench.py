@@ -21,9 +21,9 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch at the bench workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
 # `bench.py --pmc-probe`, scaled by what the same counters read for a plain copy of known size
-# (profiles/rmsnorm_fwd_bwd_config2.md).  None until measured for the current kernels.
-TRAFFIC_FWD = None
-TRAFFIC_BWD = None
+# (profiles/rmsnorm_fwd_bwd_config2.md): FETCH_SIZE 16516.5 / 21039.0 KiB x 1.9986, WRITE_SIZE 41792.2 / 36888.7 KiB.
+TRAFFIC_FWD = int((16516.5 * 1.9986 + 41792.2) * 1024)
+TRAFFIC_BWD = int((21039.0 * 1.9986 + 36888.7) * 1024)
 
 
 def algorithmic_bytes(M, H, bits, group, k):
@@ -186,14 +186,20 @@ def main():
     torch.cuda.current_stream().wait_stream(side)
     with torch.cuda.graph(graph):
         wl.step()
-    for _ in range(args.warmup):
-        graph.replay()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        graph.replay()
-    torch.cuda.synchronize()
-    ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    def wall(fn):
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # the timed region: K steps between two synchronisations, launched back to back on one stream (the three
+    # kernels of a step are short enough that a graph replay per step costs more than it saves)
+    ms_step = wall(wl.step)
+    ms_graph = wall(graph.replay)
 
     # eager launches for comparison, and per-kernel durations with events on the launch stream
     eager_ms = time_events(torch, wl.step, args.steps, args.warmup)
@@ -208,7 +214,7 @@ def main():
         dom_name, dom_ms, dom_b, dom_traffic = "hyc::k_rmsnorm_fwd_fast<4,16,true,256>", fwd_ms, fwd_b, TRAFFIC_FWD
     achieved = dom_b / (dom_ms * 1e-3) / 1e9
     extra = {
-        "eager_ms_per_step": round(eager_ms, 5),
+        "graph_replay_ms_per_step": round(ms_graph, 5), "event_ms_per_step": round(eager_ms, 5),
         "fwd_kernel_ms": round(fwd_ms, 5), "fwd_GBps": round(fwd_b / fwd_ms / 1e6, 1),
         "bwd_kernels_ms": round(bwd_ms, 5), "bwd_GBps": round(bwd_b / bwd_ms / 1e6, 1),
         "bwd_row_kernel_ms": round(bwd_main_ms, 5), "bwd_row_kernel_GBps": round(bwd_b / bwd_main_ms / 1e6, 1),
@@ -235,7 +241,7 @@ def main():
         "config": {"workload": "BASELINE configs[1]: fused RMSNorm fwd+compress and bwd(decompress), x bf16 [4,1024,4096], "
                                "20 hot channels x30, 1% outlier channels kept bf16, INT4 codes, group 128, w fp32, eps 1e-6",
                    "tokens": M, "hidden": H, "bits": bits, "group": group, "outlier_channels": wl.k,
-                   "launch": "hip graph replay of fwd + bwd + dw-reduce"},
+                   "launch": "fwd + bwd (+ dw column sum) entry points back to back on one stream"},
         "roofline": {"bound": "hbm", "kernel": dom_name, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "algorithmic_bytes": dom_b,
                      "traffic": dom_traffic},
