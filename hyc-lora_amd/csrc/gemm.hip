@@ -172,6 +172,265 @@ k_gradw(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_out, 
     }
 }
 
+
+// ------------------------------------------------------------------------------------------------
+// Few output rows (N_out <= 32: the LoRA-A shape, dW [r, H]): a streaming kernel without LDS tiles.
+//
+// v_mfma_f32_16x16x32_bf16: per lane 8 consecutive tokens of ONE row (A, a feature of dY) or ONE column (B, a
+// channel of x_hat); lane L holds row/column L mod 16 and tokens 8*(L/16) .. +7 of the 32-token step.  A lane
+// therefore owns one chunk (8 channels = the 8 code bytes of a packed word) and loads that chunk's word for its 8
+// tokens; byte j of the 8 words is the operand fragment for channel 8c + j.  The 16 lanes of a quarter-wave own 16
+// neighbouring chunks, so MFMA number j covers the 16 channels {8c + j}: a strided column set, which only permutes
+// where results are stored.  The A operand is loaded the same way, one feature per lane.  A wave is self-contained
+// (no barriers in the token loop, two steps of loads in flight); the four waves of a workgroup take every fourth
+// step of the workgroup's token range and add their accumulators through LDS at the end.
+//
+// Outlier channels were quantised as zeros, so the main tiles contribute nothing there and do not store them;
+// their columns dW[:, idx[q]] = dY^T vals[:, q] come from a second launch that feeds vals [M, k] to the same loop,
+// 16 outlier channels per tile.
+// ------------------------------------------------------------------------------------------------
+constexpr int DK = 32;     // tokens per step = one MFMA k-step
+
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef float floatx4_t __attribute__((ext_vector_type(4)));
+
+struct DirectArgs {
+  const uint16_t* dy; int64_t ldy, M, N_out, H;
+  const uint8_t* stored; const uint16_t* vals; const uint16_t* scales;
+  ChanArgs ca; int CPS, c_tiles; int64_t tokens_per_split;
+  float alpha, beta; void* out; int out_f32; float* partial;
+};
+
+struct DirectRegs {          // what one lane loads for one step
+  uint32_t blo[8], bhi[8], sc[8];
+};
+
+// MAINT: true = a tile of 16 chunks of one segment (128 quantised channels), false = a tile of 16 outlier channels
+// NT = 16-row tiles of dY features (N_out <= 16*NT)
+template <int BITS, int NT, bool MAINT>
+__device__ __forceinline__ void gradw_direct_tile(const DirectArgs& A, float* red, int hy) {
+  constexpr uint32_t MASK = (BITS == 8) ? 0xFFu : Q<BITS>::CODE_MASK;
+  constexpr uint32_t REP = MASK * 0x01010101u;
+  constexpr float OFFV = (BITS == 8) ? 128.f : (float)Q<BITS>::OFF;
+  constexpr int NB = MAINT ? 8 : 1;                                              // 16-column MFMA tiles per wave
+  constexpr int RP = 17;                                                         // padded pitch of the reduction buffer
+  const ChanArgs& ca = A.ca;
+  const int CPS = A.CPS, c_tiles = A.c_tiles;
+  const int64_t ldy = A.ldy, N_out = A.N_out, H = A.H;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);                     // uniform: token bases stay scalar
+  const int l16 = lane & 15, kq = lane >> 4;                                     // column / token quarter
+  const int seg = MAINT ? hy / c_tiles : 0;
+  const int c = MAINT ? (hy - seg * c_tiles) * 16 + l16 : 0;                     // chunk inside the segment
+  const int q = MAINT ? 0 : hy * 16 + l16;                                       // outlier number
+  const bool lane_ok = MAINT ? c < CPS : q < ca.k;
+  const int shs = (BITS == 8) ? 0 : seg * BITS;
+  const int64_t m_begin = (int64_t)blockIdx.z * A.tokens_per_split;
+  const int64_t m_end = m_begin + A.tokens_per_split < A.M ? m_begin + A.tokens_per_split : A.M;
+
+  // Addresses = scalar base of (step, token e) + a 32-bit per-lane byte offset that never changes.
+  const int64_t tok_b = MAINT ? (int64_t)CPS * 8 : (int64_t)ca.k * 2;            // bytes per token of the B source
+  const int64_t sc_b = (int64_t)ca.groups_per_row * 2;
+  const int64_t dy_b = ldy * 2;
+  const char* bsrc = MAINT ? reinterpret_cast<const char*>(A.stored) : reinterpret_cast<const char*>(A.vals);
+  const char* ssrc = reinterpret_cast<const char*>(A.scales);
+  const char* asrc = reinterpret_cast<const char*>(A.dy);
+  const int cc = c < CPS ? c : CPS - 1, qc = q < ca.k ? q : ca.k - 1;           // clamped: see fetch()
+  const uint32_t lane_b = MAINT ? 8u * (uint32_t)cc : 2u * (uint32_t)qc;
+  const uint32_t lane_s = 2u * (uint32_t)((seg * CPS + cc) >> ca.chunk_to_group_shift);
+  uint32_t lane_a[NT], aoff[NT];                                                 // feature 16a + l16, clamped
+#pragma unroll
+  for (int a = 0; a < NT; ++a) {
+    lane_a[a] = 2u * (uint32_t)(16 * a + l16 < N_out ? 16 * a + l16 : N_out - 1);
+    aoff[a] = (uint32_t)(8 * kq * dy_b) + lane_a[a];
+  }
+  const uint32_t boff = (uint32_t)(8 * kq * tok_b) + lane_b;
+  const uint32_t soff = (uint32_t)(8 * kq * sc_b) + lane_s;
+
+  floatx4_t acc[NT][NB];
+#pragma unroll
+  for (int a = 0; a < NT; ++a)
+#pragma unroll
+    for (int b = 0; b < NB; ++b) acc[a][b] = (floatx4_t){0.f, 0.f, 0.f, 0.f};
+
+  // Every load is unconditional: lanes past the last chunk / outlier / feature read their neighbour's data (the
+  // results are dropped at the write-out), tokens past the end read the last token with a zeroed dY operand.
+  auto fetch = [&](int64_t m0, DirectRegs& R, uint32_t (&ar)[NT][8]) __attribute__((always_inline)) {
+    const int left = (int)(m_end - m0 < DK ? m_end - m0 : DK);                  // valid tokens of the step
+    const char* ab = asrc + m0 * dy_b;
+    const char* bb = bsrc + m0 * tok_b;
+    const char* sb = ssrc + m0 * sc_b;
+    if (left == DK) {                                                            // all steps but the last: scalar base + lane offset
+      uint32_t bo = boff, so = soff, ao[NT];
+      asm volatile("" : "+v"(bo), "+v"(so));                                     // keep them 32-bit values of this block
+#pragma unroll
+      for (int a = 0; a < NT; ++a) { ao[a] = aoff[a]; asm volatile("" : "+v"(ao[a])); }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        if (MAINT) {
+          const uint2 w = *reinterpret_cast<const uint2*>(bb + bo);
+          R.blo[e] = w.x; R.bhi[e] = w.y;
+          R.sc[e] = *reinterpret_cast<const uint16_t*>(sb + so);
+        } else {
+          R.blo[e] = *reinterpret_cast<const uint16_t*>(bb + bo);
+        }
+#pragma unroll
+        for (int a = 0; a < NT; ++a) ar[a][e] = *reinterpret_cast<const uint16_t*>(ab + ao[a]);
+        bb += tok_b; sb += sc_b; ab += dy_b;
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int t = 8 * kq + e;
+        const int tc = t < left ? t : left - 1;
+        if (MAINT) {
+          const uint2 w = *reinterpret_cast<const uint2*>(bb + tc * tok_b + lane_b);
+          R.blo[e] = w.x; R.bhi[e] = w.y;
+          R.sc[e] = *reinterpret_cast<const uint16_t*>(sb + tc * sc_b + lane_s);
+        } else {
+          R.blo[e] = *reinterpret_cast<const uint16_t*>(bb + tc * tok_b + lane_b);
+        }
+#pragma unroll
+        for (int a = 0; a < NT; ++a) {
+          const uint32_t v = *reinterpret_cast<const uint16_t*>(ab + tc * dy_b + lane_a[a]);
+          ar[a][e] = t < left ? v : 0u;
+        }
+      }
+    }
+  };
+  auto step = [&](DirectRegs& R, uint32_t (&ar)[NT][8]) __attribute__((always_inline)) {
+    bf16x8_t bfrag[NB];
+    if (MAINT) {
+      float s[8], ns[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        s[e] = bf_to_f((uint16_t)R.sc[e]); ns[e] = -OFFV * s[e];
+        // this segment's code of every byte, as a byte
+        R.blo[e] = (BITS == 8) ? R.blo[e] ^ 0x80808080u : (R.blo[e] >> shs) & REP;
+        R.bhi[e] = (BITS == 8) ? R.bhi[e] ^ 0x80808080u : (R.bhi[e] >> shs) & REP;
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        uint32_t wj[4];
+#pragma unroll
+        for (int e = 0; e < 8; e += 2) {
+          float f[2];
+#pragma unroll
+          for (int d = 0; d < 2; ++d) {
+            const uint32_t w = (j < 4) ? R.blo[e + d] : R.bhi[e + d];
+            f[d] = __builtin_fmaf((float)((w >> (8 * (j & 3))) & 0xFFu), s[e + d], ns[e + d]);
+          }
+          wj[e >> 1] = pack_bf16(f[0], f[1]);
+        }
+        bfrag[j] = __builtin_bit_cast(bf16x8_t, (u32x4_t){wj[0], wj[1], wj[2], wj[3]});
+      }
+    } else {
+      bfrag[0] = __builtin_bit_cast(bf16x8_t, (u32x4_t){R.blo[0] | (R.blo[1] << 16), R.blo[2] | (R.blo[3] << 16),
+                                                       R.blo[4] | (R.blo[5] << 16), R.blo[6] | (R.blo[7] << 16)});
+    }
+#pragma unroll
+    for (int a = 0; a < NT; ++a) {
+      const bf16x8_t af = __builtin_bit_cast(bf16x8_t, (u32x4_t){ar[a][0] | (ar[a][1] << 16), ar[a][2] | (ar[a][3] << 16),
+                                                                ar[a][4] | (ar[a][5] << 16), ar[a][6] | (ar[a][7] << 16)});
+#pragma unroll
+      for (int b = 0; b < NB; ++b) acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, bfrag[b], acc[a][b], 0, 0, 0);
+    }
+  };
+
+  // wave w takes steps w, w+4, ... of the workgroup's token range; two steps of loads are in flight
+  constexpr int64_t WS = 4 * DK;
+  DirectRegs R0, R1;
+  uint32_t a0[NT][8], a1[NT][8];
+  int64_t m0 = m_begin + (int64_t)wave * DK;
+  if (m0 < m_end) fetch(m0, R0, a0);
+  if (m0 + WS < m_end) fetch(m0 + WS, R1, a1);
+  for (; m0 < m_end; m0 += 2 * WS) {
+    step(R0, a0);
+    if (m0 + 2 * WS < m_end) fetch(m0 + 2 * WS, R0, a0);
+    if (m0 + WS < m_end) {
+      step(R1, a1);
+      if (m0 + 3 * WS < m_end) fetch(m0 + 3 * WS, R1, a1);
+    }
+  }
+
+  // ---- the four waves add up in LDS, in wave order; layout [row n][tile b][lane] with a padded pitch ----
+  // lane holds column (lane mod 16) and rows 4*(lane/16) + v of each 16x16 tile
+  for (int w = 0; w < 4; ++w) {
+    if (wave == w) {
+#pragma unroll
+      for (int a = 0; a < NT; ++a)
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) {
+            const int n = 16 * a + 4 * kq + v;
+            float* r = &red[(n * NB + b) * RP + l16];
+            *r = (w == 0) ? acc[a][b][v] : *r + acc[a][b][v];
+          }
+    }
+    __syncthreads();
+  }
+  // ---- write-out by all threads, neighbouring threads = neighbouring channels ----
+  constexpr int COLS = 16 * NB;                                                  // channels of the tile
+  const int mode = A.partial != nullptr ? 0 : (A.out_f32 ? 1 : 2);
+  const float alpha = A.alpha, beta = A.beta;
+  const int col = tid % COLS, nfirst = tid / COLS;                               // thread's channel, first row
+  constexpr int NSTEP = 256 / COLS;
+  const int tb = MAINT ? (col & 7) : 0, tl = MAINT ? (col >> 3) : col;           // tile (= byte of the word), lane
+  bool keep;
+  int64_t h;
+  if (MAINT) {
+    const int tc = (hy - seg * c_tiles) * 16 + tl;                               // chunk of this thread's channel
+    keep = tc < CPS;
+    const uint32_t pword = keep ? ca.plan[seg * CPS + tc] : 0u;
+    keep = keep && ((pword >> tb) & 1u) == 0;                                    // outlier channels belong to the outlier launch
+    h = (int64_t)seg * CPS * 8 + 8 * tc + tb;                                    // a segment spans CPS*8 channels
+  } else {
+    keep = hy * 16 + col < ca.k;
+    h = keep ? ca.idx[hy * 16 + col] : 0;
+  }
+  if (!keep) return;
+  for (int n = nfirst; n < (int)N_out; n += NSTEP) {
+    const float val = red[(n * NB + tb) * RP + tl];
+    if (mode == 0) {
+      A.partial[((int64_t)blockIdx.z * N_out + n) * H + h] = val;
+    } else if (mode == 1) {
+      float* o = static_cast<float*>(A.out) + n * H + h;
+      *o = (beta != 0.f) ? alpha * val + beta * *o : alpha * val;
+    } else {
+      uint16_t* o = static_cast<uint16_t*>(A.out) + n * H + h;
+      *o = f_to_bf((beta != 0.f) ? alpha * val + beta * bf_to_f(*o) : alpha * val);
+    }
+  }
+}
+
+// one launch: blockIdx.y < NSEG * c_tiles are the tiles of quantised channels, the rest the outlier tiles
+// (two waves per SIMD at least: with 256 registers or fewer the accumulators stay in ordinary vector registers)
+template <int BITS, int NT>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) k_gradw_direct(DirectArgs A) {
+  __shared__ float red[16 * NT * 8 * 17];
+  const int main_tiles = Q<BITS>::NSEG * A.c_tiles;
+  if ((int)blockIdx.y < main_tiles) gradw_direct_tile<BITS, NT, true>(A, red, (int)blockIdx.y);
+  else gradw_direct_tile<BITS, NT, false>(A, red, (int)blockIdx.y - main_tiles);
+}
+
+// the streaming kernel serves N_out <= DIRECT_MAX_N; its token splits are a function of the shape only
+constexpr int64_t DIRECT_MAX_N = 32;
+#ifndef DIRECT_BLOCKS
+#define DIRECT_BLOCKS 512                                 // workgroups to aim for (tiles x token splits)
+#endif
+static int direct_splits(int64_t M, int64_t N_out, int64_t H) {
+  (void)N_out;
+  const int64_t tiles = (H + 127) / 128;
+  int64_t s = (DIRECT_BLOCKS + tiles - 1) / tiles;
+  const int64_t max_by_tokens = (M + 8 * DK - 1) / (8 * DK);      // at least two steps per wave
+  if (s > max_by_tokens) s = max_by_tokens;
+  if (s < 1) s = 1;
+  if (s > 64) s = 64;
+  return (int)s;
+}
+
 // out = alpha * sum_z partial[z] + beta * out, splits added in increasing z
 __global__ void __launch_bounds__(256)
 k_gradw_finish(const float* __restrict__ partial, int splits, int64_t total, float alpha, float beta,
@@ -179,7 +438,15 @@ k_gradw_finish(const float* __restrict__ partial, int splits, int64_t total, flo
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= total) return;
   float s = 0.f;
-  for (int z = 0; z < splits; ++z) s += partial[(int64_t)z * total + i];
+  int z = 0;
+  for (; z + 8 <= splits; z += 8) {                       // eight loads in flight, added in increasing z
+    float t[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) t[u] = partial[(int64_t)(z + u) * total + i];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) s += t[u];
+  }
+  for (; z < splits; ++z) s += partial[(int64_t)z * total + i];
   if (out_f32) {
     float* o = static_cast<float*>(out) + i;
     *o = (beta != 0.f) ? alpha * s + beta * *o : alpha * s;
@@ -210,7 +477,11 @@ int64_t hyc_gradw_workspace_bytes(int64_t M, int64_t N_out, int64_t H) {
   if (M <= 0 || N_out <= 0 || H <= 0) return 0;
   const int BN = N_out <= 32 ? 32 : 128;
   const int64_t tiles = ((N_out + BN - 1) / BN) * (H / GH);
-  const int splits = choose_splits(M, tiles);
+  int splits = choose_splits(M, tiles);                   // dense source
+  if (N_out <= DIRECT_MAX_N) {                            // channel-compressed source, few output rows
+    const int ds = direct_splits(M, N_out, H);
+    if (ds > splits) splits = ds;
+  }
   return splits > 1 ? (int64_t)splits * N_out * H * 4 : 0;
 }
 
@@ -233,13 +504,50 @@ int hyc_gradw_gemm(const void* dy, int64_t ldy, const void* stored, const void* 
     if ((rc = row_geom(H, d->bits, &g))) return rc;
     if ((rc = make_chan_args(d, g, &ca, &lpg))) return rc;
     const int hs = GH / g.nseg;
-    if (g.seg % hs != 0) return fail(HYC_ENOTSUP, "hyc_gradw_gemm: H*bits/8=%lld must be a multiple of %d", (long long)g.seg, hs);
+    if (N_out > DIRECT_MAX_N && g.seg % hs != 0)
+      return fail(HYC_ENOTSUP, "hyc_gradw_gemm: H*bits/8=%lld must be a multiple of %d when N_out > %d", (long long)g.seg, hs, (int)DIRECT_MAX_N);
   } else {
     if (H <= 0 || H % GH != 0) return fail(HYC_ENOTSUP, "hyc_gradw_gemm: dense H=%lld must be a multiple of %d", (long long)H, GH);
     g.cps = (int)(H / 8);
   }
   if (!out) return fail(HYC_EFAULT, "hyc_gradw_gemm: null out");
   hipStream_t st = begin_launch(stream);
+  if (chan && N_out <= DIRECT_MAX_N) {
+    if (M > 0 && (!dy || !stored || !scales || (d->k > 0 && !vals))) return fail(HYC_EFAULT, "hyc_gradw_gemm: null buffer");
+    if (M > 0 && !aligned8(stored)) return fail(HYC_EINVAL, "hyc_gradw_gemm: stored must be 8-byte aligned");
+    const int splits = M > 0 ? direct_splits(M, N_out, H) : 1;
+    if (splits > 1 && !workspace) return fail(HYC_EFAULT, "hyc_gradw_gemm: workspace of hyc_gradw_workspace_bytes() bytes required");
+    int64_t tps = (M + splits - 1) / splits;
+    tps = ((tps + DK - 1) / DK) * DK;
+    if (tps < DK) tps = DK;
+    float* partial = splits > 1 ? static_cast<float*>(workspace) : nullptr;
+    const int c_tiles = (g.cps + 15) / 16, o_tiles = (d->k + 15) / 16;
+    const int nt = N_out <= 16 ? 1 : 2;
+    const dim3 grid(1, (unsigned)(g.nseg * c_tiles + o_tiles), (unsigned)splits);
+    const int of32 = out_dtype == HYC_DTYPE_F32;
+    DirectArgs da = {static_cast<const uint16_t*>(dy), ldy, M, N_out, H, static_cast<const uint8_t*>(stored),
+                     static_cast<const uint16_t*>(vals), static_cast<const uint16_t*>(scales), ca, g.cps, c_tiles, tps,
+                     alpha, beta, out, of32, partial};
+#define HYC_DIRECT_N(B_, N_) hipLaunchKernelGGL((k_gradw_direct<B_, N_>), grid, dim3(256), 0, st, da)
+#define HYC_DIRECT(B_)                                                                                 \
+  do { if (nt == 1) HYC_DIRECT_N(B_, 1); else HYC_DIRECT_N(B_, 2); } while (0)
+    switch (d->bits) {
+      case 1: HYC_DIRECT(1); break;
+      case 2: HYC_DIRECT(2); break;
+      case 4: HYC_DIRECT(4); break;
+      default: HYC_DIRECT(8); break;
+    }
+#undef HYC_DIRECT_N
+#undef HYC_DIRECT
+    if ((rc = check_launch("hyc_gradw_gemm"))) return rc;
+    if (splits > 1) {
+      const int64_t total = N_out * H;
+      hipLaunchKernelGGL(k_gradw_finish, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, partial, splits, total,
+                         alpha, beta, out, of32);
+      return check_launch("hyc_gradw_gemm (finish)");
+    }
+    return HYC_OK;
+  }
   const int BN = N_out <= 32 ? 32 : 128;
   const int64_t n_tiles = (N_out + BN - 1) / BN, h_tiles = H / GH;
   const int splits = M > 0 ? choose_splits(M, n_tiles * h_tiles) : 1;
