@@ -208,7 +208,7 @@ struct DirectRegs {          // what one lane loads for one step
 // MAINT: true = a tile of 16 chunks of one segment (128 quantised channels), false = a tile of 16 outlier channels
 // NT = 16-row tiles of dY features (N_out <= 16*NT)
 template <int BITS, int NT, bool MAINT>
-__device__ __forceinline__ void gradw_direct_tile(const DirectArgs& A, float* red, int hy) {
+__device__ __forceinline__ void gradw_direct_tile(const DirectArgs& A, float* red, int hy, int64_t n0) {
   constexpr uint32_t MASK = (BITS == 8) ? 0xFFu : Q<BITS>::CODE_MASK;
   constexpr uint32_t REP = MASK * 0x01010101u;
   constexpr float OFFV = (BITS == 8) ? 128.f : (float)Q<BITS>::OFF;
@@ -242,7 +242,7 @@ __device__ __forceinline__ void gradw_direct_tile(const DirectArgs& A, float* re
   uint32_t lane_a[NT], aoff[NT];                                                 // feature 16a + l16, clamped
 #pragma unroll
   for (int a = 0; a < NT; ++a) {
-    lane_a[a] = 2u * (uint32_t)(16 * a + l16 < N_out ? 16 * a + l16 : N_out - 1);
+    lane_a[a] = 2u * (uint32_t)(n0 + 16 * a + l16 < N_out ? n0 + 16 * a + l16 : N_out - 1);
     aoff[a] = (uint32_t)(8 * kq * dy_b) + lane_a[a];
   }
   const uint32_t boff = (uint32_t)(8 * kq * tok_b) + lane_b;
@@ -391,8 +391,9 @@ __device__ __forceinline__ void gradw_direct_tile(const DirectArgs& A, float* re
     h = keep ? ca.idx[hy * 16 + col] : 0;
   }
   if (!keep) return;
-  for (int n = nfirst; n < (int)N_out; n += NSTEP) {
-    const float val = red[(n * NB + tb) * RP + tl];
+  for (int nl = nfirst; nl < 16 * NT && n0 + nl < N_out; nl += NSTEP) {
+    const float val = red[(nl * NB + tb) * RP + tl];
+    const int64_t n = n0 + nl;
     if (mode == 0) {
       A.partial[((int64_t)blockIdx.z * N_out + n) * H + h] = val;
     } else if (mode == 1) {
@@ -411,8 +412,9 @@ template <int BITS, int NT>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) k_gradw_direct(DirectArgs A) {
   __shared__ float red[16 * NT * 8 * 17];
   const int main_tiles = Q<BITS>::NSEG * A.c_tiles;
-  if ((int)blockIdx.y < main_tiles) gradw_direct_tile<BITS, NT, true>(A, red, (int)blockIdx.y);
-  else gradw_direct_tile<BITS, NT, false>(A, red, (int)blockIdx.y - main_tiles);
+  const int64_t n0 = (int64_t)blockIdx.x * (16 * NT);                            // first feature of the workgroup
+  if ((int)blockIdx.y < main_tiles) gradw_direct_tile<BITS, NT, true>(A, red, (int)blockIdx.y, n0);
+  else gradw_direct_tile<BITS, NT, false>(A, red, (int)blockIdx.y - main_tiles, n0);
 }
 
 // the streaming kernel serves N_out <= DIRECT_MAX_N; its token splits are a function of the shape only
@@ -429,6 +431,265 @@ static int direct_splits(int64_t M, int64_t N_out, int64_t H) {
   if (s < 1) s = 1;
   if (s > 64) s = 64;
   return (int)s;
+}
+
+// ------------------------------------------------------------------------------------------------
+// Large output (N_out > 32): workgroup tile 128 (n) x 256 (h), four waves of 64 x 128, two LDS stages.
+// While the MFMAs of stage s run, the global loads of stage s+1 are in flight; they are decoded into the other LDS
+// buffer after the MFMAs have been issued, and one barrier per stage separates the two.  128 accumulator registers
+// per lane; at least two waves per SIMD so that they stay in ordinary vector registers and a second workgroup's
+// decode overlaps this one's MFMAs.
+// ------------------------------------------------------------------------------------------------
+constexpr int WK = 32;      // tokens per stage
+constexpr int WN = 128;     // dY features per workgroup
+constexpr int WH = 256;     // channels per workgroup
+
+template <int NSEG, int A_PER, int B_PER>
+struct WideRegs {            // one stage of global data per thread
+  uint4 a[A_PER];            // dY chunks
+  uint4 b[B_PER];            // channel scheme: .x/.y = packed word; dense: 8 bf16
+  uint32_t s[B_PER][NSEG];   // channel scheme: the group scale of each segment's chunk
+};
+
+template <int BITS, int SRC>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
+k_gradw_wide(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_out, int64_t H,
+             const uint8_t* __restrict__ stored, const uint16_t* __restrict__ vals, const uint16_t* __restrict__ scales,
+             ChanArgs ca, int CPS, int extra_tiles, int64_t tokens_per_split, float alpha, float beta,
+             void* __restrict__ out, int out_f32, float* __restrict__ partial) {
+  constexpr int NSEG = (SRC == 0) ? Q<BITS>::NSEG : 1;
+  constexpr int HS = WH / NSEG;               // columns of the tile that come from one segment
+  constexpr int CPR = HS / 8;                 // packed 8-byte chunks (channel scheme) / 16-byte chunks (dense) per token row and segment
+  constexpr int AP = WN + GPAD, BP = WH + GPAD;
+  __shared__ __align__(16) uint16_t As[2][WK * AP];
+  __shared__ __align__(16) uint16_t Bs[2][WK * BP];
+
+  // Workgroups past the main tiles compute the outlier columns dW[:, idx[q]] = dY^T vals[:, q] with the streaming
+  // tile: 16 outlier channels x 32 features each, four feature blocks per 128-feature tile of this grid.
+  // They come first in the grid: each walks the whole token range with little work per step, so they start early
+  // and run beside the main tiles instead of forming a tail.
+  if (SRC == 0 && (int)blockIdx.y < extra_tiles) {
+    const int e = (int)blockIdx.y;
+    DirectArgs A = {dy, ldy, M, N_out, H, stored, vals, scales, ca, CPS, 0, tokens_per_split, alpha, beta, out, out_f32, partial};
+    const int64_t nf = (int64_t)blockIdx.x * WN + 32 * (e & 3);
+    if (nf < N_out) gradw_direct_tile<BITS, 2, false>(A, reinterpret_cast<float*>(&Bs[0][0]), e >> 2, nf);
+    return;
+  }
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int64_t n0 = (int64_t)blockIdx.x * WN;
+  const int64_t SEG = (SRC == 0) ? (int64_t)CPS * 8 : H;
+  const int64_t j0 = (int64_t)((int)blockIdx.y - extra_tiles) * HS;   // first column of the tile inside each segment
+  const int64_t m_begin = (int64_t)blockIdx.z * tokens_per_split;
+  const int64_t m_end = m_begin + tokens_per_split < M ? m_begin + tokens_per_split : M;
+  const int wn = (wave >> 1) * 64, wh = (wave & 1) * 128;
+
+  floatx16_t acc[2][4];
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
+
+  constexpr int A_PER = WK * WN / 8 / 256;                // 16-byte chunks of the dY stage per thread (2)
+  constexpr int B_ITEMS = WK * CPR;
+  constexpr int B_PER = (B_ITEMS + 255) / 256;
+  static_assert(B_ITEMS % 256 == 0 || B_ITEMS < 256, "items per stage");
+  const bool b_thread = B_ITEMS >= 256 || tid < B_ITEMS;  // 1-bit codes: 128 items per stage
+  typedef WideRegs<NSEG, A_PER, B_PER> Regs;
+
+  // Loads past the token range re-read the last token with the dY operand zeroed; nothing is conditional.
+  auto fetch = [&](Regs& R, int64_t m0) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < A_PER; ++u) {
+      const int idx = tid + u * 256;
+      const int row = idx / (WN / 8), cc = idx % (WN / 8);
+      const int64_t m = m0 + row, n = n0 + 8 * cc;
+      const bool ok = m < m_end && n < N_out;
+      const uint4 v = *reinterpret_cast<const uint4*>(dy + (m < m_end ? m : m_end - 1) * ldy + (n < N_out ? n : 0));
+      R.a[u] = ok ? v : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int u = 0; u < B_PER; ++u) {
+      const int idx = b_thread ? tid + u * 256 : 0;
+      const int row = idx / CPR, cc = idx % CPR;
+      const int64_t m = m0 + row < m_end ? m0 + row : m_end - 1;
+      if (SRC == 0) {
+        const int c = (int)(j0 / 8) + cc;
+        const uint2 pk = *reinterpret_cast<const uint2*>(stored + m * SEG + 8 * c);
+        R.b[u] = make_uint4(pk.x, pk.y, 0, 0);
+#pragma unroll
+        for (int i = 0; i < NSEG; ++i)
+          R.s[u][i] = scales[m * ca.groups_per_row + ((i * CPS + c) >> ca.chunk_to_group_shift)];
+      } else {
+        R.b[u] = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(stored) + m * H + j0 + 8 * cc);
+      }
+    }
+  };
+  // decode one stage of registers into LDS buffer `buf`
+  auto stash = [&](int buf, const Regs& R) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < A_PER; ++u) {
+      const int idx = tid + u * 256;
+      const int row = idx / (WN / 8), cc = idx % (WN / 8);
+      *reinterpret_cast<uint4*>(&As[buf][row * AP + 8 * cc]) = R.a[u];
+    }
+    if (b_thread) {
+#pragma unroll
+      for (int u = 0; u < B_PER; ++u) {
+        const int idx = tid + u * 256;
+        const int row = idx / CPR, cc = idx % CPR;
+        if (SRC == 0) {
+          // outlier channels decode to 0 here; their columns of dW come from the outlier tiles (see the epilogue)
+#pragma unroll
+          for (int i = 0; i < NSEG; ++i)
+            *reinterpret_cast<uint4*>(&Bs[buf][row * BP + i * HS + 8 * cc]) =
+                dequant8_fast<BITS>(R.b[u].x, R.b[u].y, i, bf_to_f((uint16_t)R.s[u][i]));
+        } else {
+          *reinterpret_cast<uint4*>(&Bs[buf][row * BP + 8 * cc]) = R.b[u];
+        }
+      }
+    }
+  };
+  auto mfma_stage = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+    for (int kk = 0; kk < WK; kk += 16) {
+      bf16x8_t af[2], bfv[4];
+#pragma unroll
+      for (int a = 0; a < 2; ++a) af[a] = frag32(As[buf], AP, wn + 32 * a, kk);
+#pragma unroll
+      for (int b = 0; b < 4; ++b) bfv[b] = frag32(Bs[buf], BP, wh + 32 * b, kk);
+#pragma unroll
+      for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[a], bfv[b], acc[a][b], 0, 0, 0);
+    }
+  };
+
+  // Three stages in flight: stage s in LDS under the MFMAs, stage s+1 in registers being decoded into the other
+  // LDS buffer in the shadow of those MFMAs, stage s+2 on its way from memory.  One barrier per stage.
+  if (m_begin < m_end) {
+    Regs R0, R1;
+    int64_t m0 = m_begin;
+    fetch(R0, m0);
+    stash(0, R0);
+    if (m0 + WK < m_end) fetch(R0, m0 + WK);
+    // steady state: the next three stages exist, so nothing is conditional and the decode of stage s+1 shares a
+    // basic block with the MFMAs of stage s (the scheduling groups below interleave them)
+    // One MFMA takes 8 passes; the wave issues in order, so the decode is cut into 16 pieces (two elements each:
+    // convert, scale, round, pack) and one piece follows each of the stage's 16 MFMAs.
+    auto overlap = [&](int buf, const Regs& R) __attribute__((always_inline)) {
+      constexpr bool PIECES = SRC == 0 && B_PER * NSEG * 4 == 16;       // 2-, 4- and 8-bit codes
+      if (!PIECES) {
+        stash(buf ^ 1, R);
+        mfma_stage(buf);
+      } else {
+        constexpr uint32_t REP = (BITS == 8) ? 0x80808080u : Q<BITS>::CODE_MASK * 0x01010101u;
+        constexpr float OFFV = (BITS == 8) ? 128.f : (float)Q<BITS>::OFF;
+        uint32_t cw[B_PER][NSEG][2], res[B_PER][NSEG][4];
+        float sc[B_PER][NSEG], ns[B_PER][NSEG];
+#pragma unroll
+        for (int u = 0; u < B_PER; ++u)
+#pragma unroll
+          for (int i = 0; i < NSEG; ++i) {
+            cw[u][i][0] = (BITS == 8) ? R.b[u].x ^ REP : (R.b[u].x >> (i * BITS)) & REP;
+            cw[u][i][1] = (BITS == 8) ? R.b[u].y ^ REP : (R.b[u].y >> (i * BITS)) & REP;
+            sc[u][i] = bf_to_f((uint16_t)R.s[u][i]);
+            ns[u][i] = -OFFV * sc[u][i];
+          }
+        int piece = 0;
+#pragma unroll
+        for (int kk = 0; kk < WK; kk += 16) {
+          bf16x8_t af[2], bfv[4];
+#pragma unroll
+          for (int a = 0; a < 2; ++a) af[a] = frag32(As[buf], AP, wn + 32 * a, kk);
+#pragma unroll
+          for (int b = 0; b < 4; ++b) bfv[b] = frag32(Bs[buf], BP, wh + 32 * b, kk);
+#pragma unroll
+          for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+              __builtin_amdgcn_sched_barrier(0);
+              acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[a], bfv[b], acc[a][b], 0, 0, 0);
+              __builtin_amdgcn_sched_barrier(0);
+              const int u = piece / (4 * NSEG), i = (piece / 4) % NSEG, w = piece % 4;
+              const uint32_t src = cw[u][i][w >> 1] >> (16 * (w & 1));
+              const float f0 = __builtin_fmaf((float)(src & 0xFFu), sc[u][i], ns[u][i]);
+              const float f1 = __builtin_fmaf((float)((src >> 8) & 0xFFu), sc[u][i], ns[u][i]);
+              res[u][i][w] = pack_bf16(f0, f1);
+              ++piece;
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < A_PER; ++u) {
+          const int idx = tid + u * 256;
+          const int row = idx / (WN / 8), cc = idx % (WN / 8);
+          *reinterpret_cast<uint4*>(&As[buf ^ 1][row * AP + 8 * cc]) = R.a[u];
+        }
+#pragma unroll
+        for (int u = 0; u < B_PER; ++u) {
+          const int idx = tid + u * 256;
+          const int row = idx / CPR, cc = idx % CPR;
+#pragma unroll
+          for (int i = 0; i < NSEG; ++i)
+            *reinterpret_cast<uint4*>(&Bs[buf ^ 1][row * BP + i * HS + 8 * cc]) =
+                make_uint4(res[u][i][0], res[u][i][1], res[u][i][2], res[u][i][3]);
+        }
+      }
+    };
+    for (; m0 + 3 * WK < m_end; m0 += 2 * WK) {
+      fetch(R1, m0 + 2 * WK);
+      __syncthreads();                                    // buffer 0 is complete; buffer 1 is no longer read
+      overlap(0, R0);
+      fetch(R0, m0 + 3 * WK);
+      __syncthreads();
+      overlap(1, R1);
+    }
+    for (; m0 < m_end; m0 += 2 * WK) {
+      if (m0 + 2 * WK < m_end) fetch(R1, m0 + 2 * WK);
+      __syncthreads();                                    // buffer 0 is complete; buffer 1 is no longer read
+      if (m0 + WK < m_end) stash(1, R0);
+      mfma_stage(0);
+      if (m0 + WK < m_end) {
+        if (m0 + 3 * WK < m_end) fetch(R0, m0 + 3 * WK);
+        __syncthreads();
+        if (m0 + 2 * WK < m_end) stash(0, R1);
+        mfma_stage(1);
+      }
+    }
+  }
+
+  // ---- epilogue: lane holds column (lane mod 32), rows 8*(v/4) + 4*(lane/32) + (v mod 4) of each 32x32 tile ----
+  const bool direct = partial == nullptr;
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const int hl = wh + 32 * b + (lane & 31);              // column inside the tile
+      const int64_t hs = j0 + (hl % HS);                     // column inside its segment
+      const int64_t h = (int64_t)(hl / HS) * SEG + hs;
+      if (SRC == 0 && ((ca.plan[(hl / HS) * CPS + (int)(hs >> 3)] >> (hs & 7)) & 1u)) continue;   // an outlier channel
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int64_t n = n0 + wn + 32 * a + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+        if (n < N_out) {
+          const float val = acc[a][b][v];
+          if (!direct) {
+            partial[((int64_t)blockIdx.z * N_out + n) * H + h] = val;
+          } else if (out_f32) {
+            float* o = static_cast<float*>(out) + n * H + h;
+            *o = (beta != 0.f) ? alpha * val + beta * *o : alpha * val;
+          } else {
+            uint16_t* o = static_cast<uint16_t*>(out) + n * H + h;
+            *o = f_to_bf((beta != 0.f) ? alpha * val + beta * bf_to_f(*o) : alpha * val);
+          }
+        }
+      }
+    }
 }
 
 // out = alpha * sum_z partial[z] + beta * out, splits added in increasing z
@@ -550,8 +811,10 @@ int hyc_gradw_gemm(const void* dy, int64_t ldy, const void* stored, const void* 
   }
   const int BN = N_out <= 32 ? 32 : 128;
   const int64_t n_tiles = (N_out + BN - 1) / BN, h_tiles = H / GH;
-  const int splits = M > 0 ? choose_splits(M, n_tiles * h_tiles) : 1;
+  const int splits = M > 0 ? choose_splits(M, n_tiles * h_tiles) : 1;     // (the wide kernel has half the tiles: same value)
   if (M > 0 && (!dy || !stored)) return fail(HYC_EFAULT, "hyc_gradw_gemm: null buffer");
+  // wide tiles (128 x 256) when the output is large and the tile grid fits the packing
+  const bool wide = N_out >= WN && (chan ? g.seg % (WH / g.nseg) == 0 : H % WH == 0);
   if (chan && M > 0 && (!scales || (d->k > 0 && !vals))) return fail(HYC_EFAULT, "hyc_gradw_gemm: null vals/scales");
   if (M > 0 && (!aligned16(dy) || !aligned8(stored) || (!chan && !aligned16(stored))))
     return fail(HYC_EINVAL, "hyc_gradw_gemm: dy must be 16-byte aligned, stored 8-byte (16 when dense)");
@@ -561,6 +824,26 @@ int hyc_gradw_gemm(const void* dy, int64_t ldy, const void* stored, const void* 
   float* partial = splits > 1 ? static_cast<float*>(workspace) : nullptr;
   const dim3 grid((unsigned)n_tiles, (unsigned)h_tiles, (unsigned)splits);
   const int of32 = out_dtype == HYC_DTYPE_F32;
+  if (wide) {
+    const int main_h = (int)(H / WH);
+    const int extra = chan ? 4 * ((d->k + 15) / 16) : 0;   // outlier tiles: 16 channels x 32 features each
+    const dim3 wgrid((unsigned)n_tiles, (unsigned)(main_h + extra), (unsigned)splits);
+#define HYC_WIDE(B_, S_)                                                                                          \
+  hipLaunchKernelGGL((k_gradw_wide<B_, S_>), wgrid, dim3(256), 0, st, static_cast<const uint16_t*>(dy), ldy, M, N_out, H, \
+                     static_cast<const uint8_t*>(stored), static_cast<const uint16_t*>(vals),                    \
+                     static_cast<const uint16_t*>(scales), ca, g.cps, extra, tps, alpha, beta, out, of32, partial)
+    if (chan) {
+      switch (d->bits) {
+        case 1: HYC_WIDE(1, 0); break;
+        case 2: HYC_WIDE(2, 0); break;
+        case 4: HYC_WIDE(4, 0); break;
+        default: HYC_WIDE(8, 0); break;
+      }
+    } else {
+      HYC_WIDE(4, 2);
+    }
+#undef HYC_WIDE
+  } else {
 #define HYC_GEMM(B_, S_, N_)                                                                                     \
   hipLaunchKernelGGL((k_gradw<B_, S_, N_>), grid, dim3(256), 0, st, static_cast<const uint16_t*>(dy), ldy, M, N_out, H, \
                      static_cast<const uint8_t*>(stored), static_cast<const uint16_t*>(vals),                    \
@@ -578,6 +861,7 @@ int hyc_gradw_gemm(const void* dy, int64_t ldy, const void* stored, const void* 
   }
 #undef HYC_GEMM_BN
 #undef HYC_GEMM
+  }
   if ((rc = check_launch("hyc_gradw_gemm"))) return rc;
   if (splits > 1) {
     const int64_t total = N_out * H;

@@ -273,6 +273,25 @@ __device__ __forceinline__ uint4 dequant8(uint32_t lo, uint32_t hi, int seg, flo
   return r;
 }
 
+// The same without the branch for huge scales (s >= 1e30 overflows -OFF*s): for consumers that accumulate in fp32
+// and are compared to a tolerance, not bit for bit (the weight-gradient GEMM).
+template <int BITS>
+__device__ __forceinline__ uint4 dequant8_fast(uint32_t lo, uint32_t hi, int seg, float s) {
+  constexpr uint32_t REP = (BITS == 8) ? 0x80808080u : Q<BITS>::CODE_MASK * 0x01010101u;
+  uint32_t a, b;
+  if (BITS == 8) { a = lo ^ REP; b = hi ^ REP; }
+  else { a = (lo >> (seg * BITS)) & REP; b = (hi >> (seg * BITS)) & REP; }
+  float c[8] = {(float)(a & 0xFFu), (float)((a >> 8) & 0xFFu), (float)((a >> 16) & 0xFFu), (float)(a >> 24),
+                (float)(b & 0xFFu), (float)((b >> 8) & 0xFFu), (float)((b >> 16) & 0xFFu), (float)(b >> 24)};
+  constexpr float OFFV = (BITS == 8) ? 128.f : (float)Q<BITS>::OFF;
+  const float ns = -OFFV * s;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) c[j] = __builtin_fmaf(c[j], s, ns);
+  uint4 r;
+  r.x = pack_bf16(c[0], c[1]); r.y = pack_bf16(c[2], c[3]); r.z = pack_bf16(c[4], c[5]); r.w = pack_bf16(c[6], c[7]);
+  return r;
+}
+
 // ---- descriptors as the kernels see them -------------------------------------------------------
 struct ChanArgs {           // HYC_MODE_CHANNEL
   const uint32_t* plan;     // [H/8]
