@@ -105,6 +105,31 @@ def time_events(torch, fn, iters, warmup):
     return e0.elapsed_time(e1) / iters
 
 
+def gradw_extra(pkg, torch, wl):
+    """weight-gradient GEMM on the workload's compressed x (configs[2]/[3] shapes): full W and LoRA-A (r = 16)"""
+    K, abi = pkg.kernels, pkg._abi
+    lib = wl.lib
+    M, H = wl.M, wl.H
+    out = {}
+    p = lambda t: ctypes.c_void_p(t.data_ptr()) if t is not None else None
+    for name, N, iters in (("full_w", 4096, 20), ("lora_a_r16", 16, 100)):
+        dy = (0.01 * torch.randn(M, N, device="cuda")).bfloat16()
+        dw = torch.empty(N, H, dtype=torch.bfloat16, device="cuda")
+        ws_bytes = lib.hyc_gradw_workspace_bytes(M, N, H)
+        ws = torch.empty(max(ws_bytes // 4, 1), dtype=torch.float32, device="cuda")
+        args = (p(dy), N, p(wl.c.stored), p(wl.c.vals), p(wl.c.scales), M, N, H, ctypes.byref(wl.desc),
+                ctypes.c_float(1.0), ctypes.c_float(0.0), p(dw), abi.DTYPE_BF16, p(ws))
+        fn = lambda: abi.check(lib.hyc_gradw_gemm(*args, wl._stream()))
+        ms = time_events(torch, fn, iters, 3)
+        xh = K.decompress_channel(wl.c)
+        ms_lib = time_events(torch, lambda: torch.matmul(dy.t(), xh), iters, 3)
+        out[name] = {"M": M, "N_out": N, "H": H, "ms": round(ms, 5), "TFLOPs": round(2 * M * N * H / ms / 1e9, 1),
+                     "frac_of_bf16_mfma_peak": round(2 * M * N * H / ms / 1e9 / 2500.0, 4),
+                     "library_gemm_on_decompressed_ms": round(ms_lib, 5)}
+        del dy, dw, ws, xh
+    return out
+
+
 def cpu_baseline(torch, wl, rows, seconds):
     """the oracle (CPU PyTorch restatement of the path) on the host cores, bounded sample of the same workload"""
     from oracle import hyc_oracle as O
@@ -221,6 +246,7 @@ def main():
         "act_mem_bytes_saved_tensor": saved_b + 4 * M, "act_mem_bytes_bf16": 2 * M * H,
         "act_mem_ratio": round(2 * M * H / (saved_b + 4 * M), 3),
     }
+    extra["gradw_gemm_int4"] = gradw_extra(pkg, torch, wl)
     if not args.no_scaled:
         # the config-size working set (~150 MB) fits the 256 MB Infinity Cache; 16x the tokens does not
         del graph
