@@ -177,6 +177,97 @@ k_act_bwd_fast(const uint16_t* __restrict__ g, const uint8_t* __restrict__ store
   }
 }
 
+// Hadamard backward in one pass when both operands are channel-compressed with the same code width (the thread to
+// chunk mapping then agrees): g is read once, dx1 = g * x2_hat, dx2 = x1_hat * g.
+template <int BITS, int MAXT>
+__global__ void __launch_bounds__(MAXT)
+k_hadamard_bwd_fast(const uint16_t* __restrict__ g, const uint8_t* __restrict__ st1, const uint16_t* __restrict__ v1,
+                    const uint16_t* __restrict__ s1, ChanArgs c1, const uint8_t* __restrict__ st2,
+                    const uint16_t* __restrict__ v2, const uint16_t* __restrict__ s2, ChanArgs c2, int64_t M, int64_t H,
+                    int CPS, uint16_t* __restrict__ dx1, uint16_t* __restrict__ dx2) {
+  constexpr int NSEG = Q<BITS>::NSEG;
+  const int c = threadIdx.x;
+  if (c >= CPS) return;                                 // tail of the last wave
+  const int64_t SEG = (int64_t)CPS * 8;
+  const int sg1 = CPS >> c1.chunk_to_group_shift, sg2 = CPS >> c2.chunk_to_group_shift;
+  ChunkOutliers<NSEG> o1, o2;
+  {
+    uint32_t p1[NSEG], p2[NSEG];
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) { p1[i] = c1.plan[i * CPS + c]; p2[i] = c2.plan[i * CPS + c]; }
+    o1.init(p1);
+    o2.init(p2);
+  }
+  const int64_t stride = gridDim.x;
+  int64_t row = blockIdx.x;
+  const uint16_t* gp = g + row * H + 8 * c;
+  uint16_t* d1p = dx1 + row * H + 8 * c;
+  uint16_t* d2p = dx2 + row * H + 8 * c;
+  const uint8_t* sp1 = st1 + row * SEG + 8 * c;
+  const uint8_t* sp2 = st2 + row * SEG + 8 * c;
+  const uint16_t* vp1 = v1 + row * c1.k;
+  const uint16_t* vp2 = v2 + row * c2.k;
+  const uint16_t* scp1 = s1 + row * c1.groups_per_row + (c >> c1.chunk_to_group_shift);
+  const uint16_t* scp2 = s2 + row * c2.groups_per_row + (c >> c2.chunk_to_group_shift);
+  const int64_t xstep = stride * H, sstep = stride * SEG;
+  uint2 pk1 = make_uint2(0, 0), pk2 = make_uint2(0, 0);
+  uint4 graw[NSEG];
+  uint32_t sc1[NSEG], sc2[NSEG], a0[NSEG], a1[NSEG], b0[NSEG], b1[NSEG];
+  if (row < M) {
+    pk1 = *reinterpret_cast<const uint2*>(sp1);
+    pk2 = *reinterpret_cast<const uint2*>(sp2);
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) {
+      graw[i] = *reinterpret_cast<const uint4*>(gp + i * SEG);
+      sc1[i] = scp1[i * sg1]; sc2[i] = scp2[i * sg2];
+    }
+    o1.request(vp1, a0, a1);
+    o2.request(vp2, b0, b1);
+  }
+  for (; row < M; row += stride) {
+    uint2 pk1_n = make_uint2(0, 0), pk2_n = make_uint2(0, 0);
+    uint4 g_n[NSEG];
+    uint32_t sc1_n[NSEG], sc2_n[NSEG], a0_n[NSEG], a1_n[NSEG], b0_n[NSEG], b1_n[NSEG];
+    if (row + stride < M) {
+      pk1_n = *reinterpret_cast<const uint2*>(sp1 + sstep);
+      pk2_n = *reinterpret_cast<const uint2*>(sp2 + sstep);
+#pragma unroll
+      for (int i = 0; i < NSEG; ++i) {
+        g_n[i] = *reinterpret_cast<const uint4*>(gp + xstep + i * SEG);
+        sc1_n[i] = scp1[stride * c1.groups_per_row + i * sg1];
+        sc2_n[i] = scp2[stride * c2.groups_per_row + i * sg2];
+      }
+      o1.request(vp1 + stride * c1.k, a0_n, a1_n);
+      o2.request(vp2 + stride * c2.k, b0_n, b1_n);
+    }
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) {
+      float x1[8], x2[8], gv[8], r1[8], r2[8];
+      const float f1 = bf_to_f((uint16_t)sc1[i]), f2 = bf_to_f((uint16_t)sc2[i]);
+      uint4 q1 = o1.splice(i, dequant8<BITS>(pk1.x, pk1.y, i, f1), a0[i], a1[i], f1);
+      uint4 q2 = o2.splice(i, dequant8<BITS>(pk2.x, pk2.y, i, f2), b0[i], b1[i], f2);
+      if (o1.more_pairs) q1 = splice_more(q1, o1.more_pairs, c1.plan[i * CPS + c], vp1, true, f1);
+      if (o2.more_pairs) q2 = splice_more(q2, o2.more_pairs, c2.plan[i * CPS + c], vp2, true, f2);
+      unpack8(q1, x1);
+      unpack8(q2, x2);
+      unpack8(graw[i], gv);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) { r1[j] = gv[j] * x2[j]; r2[j] = x1[j] * gv[j]; }
+      store_stream(d1p + i * SEG, pack8(r1));
+      store_stream(d2p + i * SEG, pack8(r2));
+    }
+    pk1 = pk1_n; pk2 = pk2_n;
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) {
+      graw[i] = g_n[i]; sc1[i] = sc1_n[i]; sc2[i] = sc2_n[i];
+      a0[i] = a0_n[i]; a1[i] = a1_n[i]; b0[i] = b0_n[i]; b1[i] = b1_n[i];
+    }
+    gp += xstep; d1p += xstep; d2p += xstep; sp1 += sstep; sp2 += sstep;
+    vp1 += stride * c1.k; vp2 += stride * c2.k;
+    scp1 += stride * c1.groups_per_row; scp2 += stride * c2.groups_per_row;
+  }
+}
+
 // SRC 0 = channel-compressed, 2 = dense bf16
 template <int BITS, int SRC, int ACT>
 __global__ void __launch_bounds__(1024)
@@ -290,6 +381,39 @@ int hyc_act_bwd(int32_t act, const void* g, const void* stored, const void* vals
 int hyc_hadamard_bwd(const void* g, const void* stored1, const void* vals1, const void* scales1, const hyc_desc* d1,
                      const void* stored2, const void* vals2, const void* scales2, const hyc_desc* d2, int64_t M,
                      int64_t H, void* dx1, void* dx2, void* stream) {
+  // one pass when both operands use the channel scheme with the same code width and the row fits a workgroup
+  if (d1 && d2 && d1->mode == HYC_MODE_CHANNEL && d2->mode == HYC_MODE_CHANNEL && d1->bits == d2->bits && d1->bits != 1 &&
+      M > 0) {
+    RowGeom geo;
+    int rc = row_geom(H, d1->bits, &geo);
+    if (rc) return rc;
+    if (geo.iters == 1) {
+      ChanArgs c1 = {}, c2 = {};
+      int lpg = 16;
+      if ((rc = make_chan_args(d1, geo, &c1, &lpg)) || (rc = make_chan_args(d2, geo, &c2, &lpg))) return rc;
+      if (!g || !stored1 || !stored2 || !scales1 || !scales2 || !dx1 || !dx2 || (d1->k > 0 && !vals1) || (d2->k > 0 && !vals2))
+        return fail(HYC_EFAULT, "hyc_hadamard_bwd: null buffer");
+      if (!aligned16(g) || !aligned16(dx1) || !aligned16(dx2) || !aligned8(stored1) || !aligned8(stored2))
+        return fail(HYC_EINVAL, "hyc_hadamard_bwd: g, dx must be 16-byte aligned, stored 8-byte");
+      const int64_t cap = 256 * (geo.threads >= 512 ? 3 : 8);
+      const int grid = (int)(M < cap ? M : cap);
+      hipStream_t st = begin_launch(stream);
+#define HYC_HAD(B_, MT_)                                                                                           \
+  hipLaunchKernelGGL((k_hadamard_bwd_fast<B_, MT_>), dim3(grid), dim3(geo.threads), 0, st,                         \
+                     static_cast<const uint16_t*>(g), static_cast<const uint8_t*>(stored1),                        \
+                     static_cast<const uint16_t*>(vals1), static_cast<const uint16_t*>(scales1), c1,               \
+                     static_cast<const uint8_t*>(stored2), static_cast<const uint16_t*>(vals2),                    \
+                     static_cast<const uint16_t*>(scales2), c2, M, H, geo.cps, static_cast<uint16_t*>(dx1),        \
+                     static_cast<uint16_t*>(dx2))
+#define HYC_HAD_T(B_) do { if (geo.threads <= 256) HYC_HAD(B_, 256); else HYC_HAD(B_, 1024); } while (0)
+      if (d1->bits == 2) HYC_HAD_T(2);
+      else if (d1->bits == 4) HYC_HAD_T(4);
+      else HYC_HAD_T(8);
+#undef HYC_HAD_T
+#undef HYC_HAD
+      return check_launch("hyc_hadamard_bwd");
+    }
+  }
   int rc = launch_act<ACT_MUL>(g, stored2, vals2, scales2, M, H, d2, dx1, stream, "hyc_hadamard_bwd(dx1)");
   if (rc) return rc;
   return launch_act<ACT_MUL>(g, stored1, vals1, scales1, M, H, d1, dx2, stream, "hyc_hadamard_bwd(dx2)");

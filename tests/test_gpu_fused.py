@@ -153,15 +153,19 @@ def test_act_bwd_channel(K, bits, group, M, H, k):
         assert bits_equal(K.act_bwd(act, g.cuda(), xh.cuda()), K.act_bwd(act, g.cuda(), c))
 
 
-def test_hadamard_bwd(K):
-    M, H = 48, 4096
-    x1, gen = make_x(1, M, H, 41, 20.0)
-    x2, _ = make_x(2, M, H, 41, 20.0)
+@pytest.mark.parametrize("M,H,b1,g1,b2,g2", [(48, 4096, 4, 128, 2, 64),      # different code widths: two passes
+                                              (48, 4096, 4, 128, 4, 64),      # same width: one fused pass
+                                              (2100, 11008, 2, 64, 2, 32),    # partial last wave, several rows per workgroup
+                                              (33, 2048, 8, 128, 8, 128)])
+def test_hadamard_bwd(K, M, H, b1, g1, b2, g2):
+    k = K.num_outlier_channels(H, 0.01)
+    x1, gen = make_x(1, M, H, k, 20.0)
+    x2, _ = make_x(2, M, H, k, 20.0)
     g = (0.1 * torch.randn(M, H, generator=gen)).bfloat16()
-    p1 = K.select_channels(K.channel_absmax(x1.cuda()), 41)
-    p2 = K.select_channels(K.channel_absmax(x2.cuda()), 41)
-    c1 = K.compress_channel(x1.cuda(), p1, 4, 128)
-    c2 = K.compress_channel(x2.cuda(), p2, 2, 64)
+    p1 = K.select_channels(K.channel_absmax(x1.cuda()), k)
+    p2 = K.select_channels(K.channel_absmax(x2.cuda()), k)
+    c1 = K.compress_channel(x1.cuda(), p1, b1, g1)
+    c2 = K.compress_channel(x2.cuda(), p2, b2, g2)
     d1, d2 = K.hadamard_bwd(g.cuda(), c1, c2)
     w1, w2 = O.hadamard_bwd(K.decompress_channel(c1).cpu(), K.decompress_channel(c2).cpu(), g)
     assert bits_equal(d1.cpu(), w1) and bits_equal(d2.cpu(), w2)
