@@ -268,6 +268,109 @@ k_hadamard_bwd_fast(const uint16_t* __restrict__ g, const uint8_t* __restrict__ 
   }
 }
 
+// One channel-compressed operand of a fast row kernel: the thread's view of it (chunk c of every segment), with the
+// current row's codes / scales / outliers in registers; next() reloads them for the following row as soon as the
+// current one has been decoded (no second register set).
+template <int BITS>
+struct ChanSource {
+  static constexpr int NSEG = Q<BITS>::NSEG;
+  ChunkOutliers<NSEG> co;
+  const uint8_t* sp; const uint16_t* vp; const uint16_t* scp; const uint32_t* plan;
+  int64_t sstep, vstep, scstep;
+  int seg_groups;
+  uint2 pk;
+  uint32_t sc[NSEG], o0[NSEG], o1[NSEG];
+
+  __device__ __forceinline__ void init(const uint8_t* stored, const uint16_t* vals, const uint16_t* scales, const ChanArgs& a,
+                                       int c, int CPS, int64_t row, int64_t stride) {
+    uint32_t p[NSEG];
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) p[i] = a.plan[i * CPS + c];
+    co.init(p);
+    plan = a.plan + c;
+    seg_groups = CPS >> a.chunk_to_group_shift;
+    sp = stored + row * ((int64_t)CPS * 8) + 8 * c;
+    vp = vals + row * a.k;
+    scp = scales + row * a.groups_per_row + (c >> a.chunk_to_group_shift);
+    sstep = stride * (int64_t)CPS * 8; vstep = stride * a.k; scstep = stride * a.groups_per_row;
+    pk = make_uint2(0, 0);
+  }
+  __device__ __forceinline__ void request_first() {
+    pk = *reinterpret_cast<const uint2*>(sp);
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) sc[i] = scp[i * seg_groups];
+    co.request(vp, o0, o1);
+  }
+  __device__ __forceinline__ void next() {
+    sp += sstep; vp += vstep; scp += scstep;
+    request_first();
+  }
+  __device__ __forceinline__ void decode(int i, int CPS, float (&x)[8]) const {
+    const float f = bf_to_f((uint16_t)sc[i]);
+    uint4 q = co.splice(i, dequant8<BITS>(pk.x, pk.y, i, f), o0[i], o1[i], f);
+    if (co.more_pairs) q = splice_more(q, co.more_pairs, plan[i * CPS], vp, true, f);
+    unpack8(q, x);
+  }
+};
+
+// Backward of h = act(gate) * up in one pass, with the three saved activations the separate operators keep:
+// a_hat = decompress(act(gate)), up_hat, gate_hat.  d_up = a_hat * g;  d_gate = act'(gate_hat) * bf16(g * up_hat) -
+// the same roundings as hyc_hadamard_bwd followed by hyc_act_bwd, without the round trip of g * up_hat through memory.
+template <int BITS, int ACT, int MAXT>
+__global__ void __launch_bounds__(MAXT)
+k_gated_act_bwd_fast(const uint16_t* __restrict__ g, const uint8_t* __restrict__ st_a, const uint16_t* __restrict__ v_a,
+                     const uint16_t* __restrict__ s_a, ChanArgs c_a, const uint8_t* __restrict__ st_u,
+                     const uint16_t* __restrict__ v_u, const uint16_t* __restrict__ s_u, ChanArgs c_u,
+                     const uint8_t* __restrict__ st_g, const uint16_t* __restrict__ v_g, const uint16_t* __restrict__ s_g,
+                     ChanArgs c_g, int64_t M, int64_t H, int CPS, uint16_t* __restrict__ d_gate, uint16_t* __restrict__ d_up) {
+  constexpr int NSEG = Q<BITS>::NSEG;
+  const int c = threadIdx.x;
+  if (c >= CPS) return;                                 // tail of the last wave
+  const int64_t SEG = (int64_t)CPS * 8;
+  const int64_t stride = gridDim.x;
+  int64_t row = blockIdx.x;
+  ChanSource<BITS> A, U, G;
+  A.init(st_a, v_a, s_a, c_a, c, CPS, row, stride);
+  U.init(st_u, v_u, s_u, c_u, c, CPS, row, stride);
+  G.init(st_g, v_g, s_g, c_g, c, CPS, row, stride);
+  const uint16_t* gp = g + row * H + 8 * c;
+  uint16_t* dgp = d_gate + row * H + 8 * c;
+  uint16_t* dup = d_up + row * H + 8 * c;
+  const int64_t xstep = stride * H;
+  uint4 graw[NSEG];
+  if (row < M) {
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) graw[i] = *reinterpret_cast<const uint4*>(gp + i * SEG);
+    A.request_first(); U.request_first(); G.request_first();
+  }
+  for (; row < M; row += stride) {
+    uint4 g_n[NSEG];
+    const bool more = row + stride < M;
+    if (more) {
+#pragma unroll
+      for (int i = 0; i < NSEG; ++i) g_n[i] = *reinterpret_cast<const uint4*>(gp + xstep + i * SEG);
+    }
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) {
+      float xa[8], xu[8], xg[8], gv[8], t[8], r[8];
+      A.decode(i, CPS, xa);
+      U.decode(i, CPS, xu);
+      G.decode(i, CPS, xg);
+      if (i == NSEG - 1 && more) { A.next(); U.next(); G.next(); }   // the compressed rows are decoded: reload
+      unpack8(graw[i], gv);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) { r[j] = xa[j] * gv[j]; t[j] = gv[j] * xu[j]; }
+      store_stream(dup + i * SEG, pack8(r));
+      unpack8(pack8(t), t);                             // the gradient of act(gate), rounded to bf16 as a tensor would be
+      act_grad8<ACT>(xg, t, r);
+      store_stream(dgp + i * SEG, pack8(r));
+    }
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) graw[i] = g_n[i];
+    gp += xstep; dgp += xstep; dup += xstep;
+  }
+}
+
 // SRC 0 = channel-compressed, 2 = dense bf16
 template <int BITS, int SRC, int ACT>
 __global__ void __launch_bounds__(1024)
@@ -417,6 +520,60 @@ int hyc_hadamard_bwd(const void* g, const void* stored1, const void* vals1, cons
   int rc = launch_act<ACT_MUL>(g, stored2, vals2, scales2, M, H, d2, dx1, stream, "hyc_hadamard_bwd(dx1)");
   if (rc) return rc;
   return launch_act<ACT_MUL>(g, stored1, vals1, scales1, M, H, d1, dx2, stream, "hyc_hadamard_bwd(dx2)");
+}
+
+int hyc_gated_act_bwd(int32_t act, const void* g, const void* stored_a, const void* vals_a, const void* scales_a,
+                      const hyc_desc* d_a, const void* stored_u, const void* vals_u, const void* scales_u,
+                      const hyc_desc* d_u, const void* stored_g, const void* vals_g, const void* scales_g,
+                      const hyc_desc* d_g, int64_t M, int64_t H, void* d_gate, void* d_up, void* stream) {
+  if (act != HYC_ACT_SILU && act != HYC_ACT_GELU_TANH) return fail(HYC_EINVAL, "hyc_gated_act_bwd: act=%d", act);
+  if (!d_a || !d_u || !d_g) return fail(HYC_EFAULT, "hyc_gated_act_bwd: null descriptor");
+  if (M < 0) return fail(HYC_EINVAL, "hyc_gated_act_bwd: M=%lld", (long long)M);
+  if (d_a->mode != HYC_MODE_CHANNEL || d_u->mode != HYC_MODE_CHANNEL || d_g->mode != HYC_MODE_CHANNEL)
+    return fail(HYC_ENOTSUP, "hyc_gated_act_bwd: the three activations must be channel-compressed (use hyc_hadamard_bwd + hyc_act_bwd otherwise)");
+  if (d_a->bits != d_u->bits || d_a->bits != d_g->bits || d_a->bits == 1)
+    return fail(HYC_ENOTSUP, "hyc_gated_act_bwd: one code width (2, 4 or 8 bits) for the three activations");
+  RowGeom geo;
+  int rc = row_geom(H, d_a->bits, &geo);
+  if (rc) return rc;
+  if (geo.iters != 1) return fail(HYC_ENOTSUP, "hyc_gated_act_bwd: row too long (%d chunks per segment)", geo.cps);
+  ChanArgs c_a = {}, c_u = {}, c_g = {};
+  int lpg = 16;
+  if ((rc = make_chan_args(d_a, geo, &c_a, &lpg)) || (rc = make_chan_args(d_u, geo, &c_u, &lpg)) ||
+      (rc = make_chan_args(d_g, geo, &c_g, &lpg)))
+    return rc;
+  if (M == 0) return HYC_OK;
+  if (!g || !stored_a || !stored_u || !stored_g || !scales_a || !scales_u || !scales_g || !d_gate || !d_up ||
+      (d_a->k > 0 && !vals_a) || (d_u->k > 0 && !vals_u) || (d_g->k > 0 && !vals_g))
+    return fail(HYC_EFAULT, "hyc_gated_act_bwd: null buffer");
+  if (!aligned16(g) || !aligned16(d_gate) || !aligned16(d_up) || !aligned8(stored_a) || !aligned8(stored_u) || !aligned8(stored_g))
+    return fail(HYC_EINVAL, "hyc_gated_act_bwd: g, d_gate, d_up must be 16-byte aligned, stored 8-byte");
+  const int64_t cap = 256 * (geo.threads >= 512 ? 3 : 8);
+  const int grid = (int)(M < cap ? M : cap);
+  hipStream_t st = begin_launch(stream);
+#define HYC_GATED(B_, A_, MT_)                                                                                     \
+  hipLaunchKernelGGL((k_gated_act_bwd_fast<B_, A_, MT_>), dim3(grid), dim3(geo.threads), 0, st,                    \
+                     static_cast<const uint16_t*>(g), static_cast<const uint8_t*>(stored_a),                       \
+                     static_cast<const uint16_t*>(vals_a), static_cast<const uint16_t*>(scales_a), c_a,            \
+                     static_cast<const uint8_t*>(stored_u), static_cast<const uint16_t*>(vals_u),                  \
+                     static_cast<const uint16_t*>(scales_u), c_u, static_cast<const uint8_t*>(stored_g),           \
+                     static_cast<const uint16_t*>(vals_g), static_cast<const uint16_t*>(scales_g), c_g, M, H,      \
+                     geo.cps, static_cast<uint16_t*>(d_gate), static_cast<uint16_t*>(d_up))
+#define HYC_GATED_T(B_, A_)                                                       \
+  do {                                                                            \
+    if (geo.threads <= 256) HYC_GATED(B_, A_, 256);                               \
+    else if (geo.threads <= 768) HYC_GATED(B_, A_, 768); /* H = 11008: 704 threads, 168 registers each */ \
+    else HYC_GATED(B_, A_, 1024);                                                 \
+  } while (0)
+#define HYC_GATED_B(A_)                                                           \
+  do {                                                                            \
+    if (d_a->bits == 2) HYC_GATED_T(2, A_); else if (d_a->bits == 4) HYC_GATED_T(4, A_); else HYC_GATED_T(8, A_); \
+  } while (0)
+  if (act == HYC_ACT_SILU) HYC_GATED_B(HYC_ACT_SILU); else HYC_GATED_B(HYC_ACT_GELU_TANH);
+#undef HYC_GATED_B
+#undef HYC_GATED_T
+#undef HYC_GATED
+  return check_launch("hyc_gated_act_bwd");
 }
 
 }  // extern "C"

@@ -356,6 +356,21 @@ def hadamard_bwd(g2d, src1, src2):
     return dx1, dx2
 
 
+def gated_act_bwd(act, g2d, src_act, src_up, src_gate):
+    """backward of act(gate) * up in one pass -> (d_gate, d_up); the three sources are ChannelCompressed"""
+    _need(g2d, BF16, "grad_output")
+    M, H = g2d.shape
+    sa, va, ca, da = _source(src_act)
+    su, vu, cu, du = _source(src_up)
+    sg, vg, cg, dg = _source(src_gate)
+    d_gate, d_up = torch.empty_like(g2d), torch.empty_like(g2d)
+    code = {"silu": _abi.ACT_SILU, "gelu": _abi.ACT_GELU_TANH}[act]
+    check(_abi.load().hyc_gated_act_bwd(code, _p(g2d), _p(sa), _p(va), _p(ca), ctypes.byref(da), _p(su), _p(vu), _p(cu),
+                                        ctypes.byref(du), _p(sg), _p(vg), _p(cg), ctypes.byref(dg), M, H, _p(d_gate),
+                                        _p(d_up), _stream()))
+    return d_gate, d_up
+
+
 # ----------------------------------------------------------------------------------------------------
 # weight gradient
 # ----------------------------------------------------------------------------------------------------

@@ -1,7 +1,7 @@
 """Host-side mirror of the reference's operators/ package: same module, class and function names."""
 from . import compress_function, fused_compression  # noqa: F401
 from .efficient_gelu import EfficientMemoryGELU, EfficientMemoryGELUFunc  # noqa: F401
-from .efficient_hadamard import EfficientMemoryHadamard, EfficientMemoryHadamardFunc  # noqa: F401
+from .efficient_hadamard import EfficientMemoryGatedAct, EfficientMemoryHadamard, EfficientMemoryHadamardFunc  # noqa: F401
 from .efficient_linear import EfficientMemoryLinear, EfficientMemoryLinearFunc  # noqa: F401
 from .efficient_rmsnorm import EfficientMemoryRMSNorm, EfficientMemoryRMSNormFunc  # noqa: F401
 from .efficient_silu import EfficientMemorySiLU, EfficientMemorySiLUFunc  # noqa: F401

@@ -91,3 +91,52 @@ class EfficientMemoryHadamard(torch.nn.Module):
             self.static_value_2 = fold_statistics(self.static_value_2, self.iteration, o2, L2, s2, R2)
         self.iteration += 1
         return result
+
+
+class _ChannelGatedActFunc(torch.autograd.Function):
+    """h = act(gate) * up with the three activations EfficientMemorySiLU/GELU and EfficientMemoryHadamard would save
+    (gate; act(gate) and up), and one backward pass over them."""
+
+    @staticmethod
+    def forward(ctx, gate, up, act, plan_a, plan_u, plan_g, bits, group):
+        a = torch.nn.functional.silu(gate) if act == "silu" else torch.nn.functional.gelu(gate)
+        a2, _ = as_rows(a)
+        u2, _ = as_rows(up)
+        g2, _ = as_rows(gate)
+        ctx.saved = (K.compress_channel(a2, plan_a, bits, group), K.compress_channel(u2, plan_u, bits, group),
+                     K.compress_channel(g2, plan_g, bits, group))
+        ctx.act = act
+        return a * up
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        g2, _ = as_rows(grad_output.to(torch.bfloat16))
+        d_gate, d_up = K.gated_act_bwd(ctx.act, g2, *ctx.saved)
+        return d_gate.reshape(grad_output.shape), d_up.reshape(grad_output.shape), None, None, None, None, None, None
+
+
+class EfficientMemoryGatedAct(torch.nn.Module):
+    """SwiGLU / GeGLU product `act(gate) * up` as one module (channel scheme only).  The reference composes
+    EfficientMemorySiLU (efficient_silu.py:56-113) and EfficientMemoryHadamard (efficient_hadamard.py:86-183); this
+    module saves the same three compressed activations and gives bit-identical gradients, but its backward reads the
+    incoming gradient once and never writes the gradient of act(gate) to memory."""
+
+    def __init__(self, act: str = "silu", outlier_ratio: float = 0.01, sub_outlier_ratio: float = 1.0,
+                 sub_outlier_bit: int = 4, sub_outlier_quantize_method: str = 'per-token', rank: int = 0, *,
+                 group_size: int = 128):
+        super().__init__()
+        if act not in ("silu", "gelu"):
+            raise ValueError("act must be 'silu' or 'gelu'")
+        self.act, self.sub_outlier_bit, self.group_size = act, sub_outlier_bit, group_size
+        mk = lambda: CompressionSite(outlier_ratio, sub_outlier_ratio, sub_outlier_bit, sub_outlier_quantize_method,
+                                     rank, "hyc", group_size)
+        self.site_act, self.site_up, self.site_gate = mk(), mk(), mk()
+        self.iteration = 0
+
+    def forward(self, gate, up):
+        a = torch.nn.functional.silu(gate) if self.act == "silu" else torch.nn.functional.gelu(gate)
+        pa = self.site_act.channel_plan(as_rows(a)[0], self.iteration)
+        pu = self.site_up.channel_plan(as_rows(up)[0], self.iteration)
+        pg = self.site_gate.channel_plan(as_rows(gate)[0], self.iteration)
+        self.iteration += 1
+        return _ChannelGatedActFunc.apply(gate, up, self.act, pa, pu, pg, self.sub_outlier_bit, self.group_size)

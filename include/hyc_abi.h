@@ -155,6 +155,15 @@ int hyc_hadamard_bwd(const void* g, const void* stored1, const void* vals1, cons
                      const void* stored2, const void* vals2, const void* scales2, const hyc_desc* d2, int64_t M,
                      int64_t H, void* dx1, void* dx2, void* stream);
 
+/* Backward of h = act(gate) * up (SwiGLU / GeGLU) in one pass over the three activations that
+ * EfficientMemorySiLU/GELU (efficient_silu.py:11-53, efficient_gelu.py:11-64: saves gate) and EfficientMemoryHadamard
+ * (efficient_hadamard.py:9-83: saves act(gate) and up) keep: d_up = a_hat * g, d_gate = act'(gate_hat) * bf16(g * up_hat).
+ * Same results as hyc_hadamard_bwd followed by hyc_act_bwd; channel scheme, one code width for the three. */
+int hyc_gated_act_bwd(int32_t act, const void* g, const void* stored_a, const void* vals_a, const void* scales_a,
+                      const hyc_desc* d_a, const void* stored_u, const void* vals_u, const void* scales_u,
+                      const hyc_desc* d_u, const void* stored_g, const void* vals_g, const void* scales_g,
+                      const hyc_desc* d_g, int64_t M, int64_t H, void* d_gate, void* d_up, void* stream);
+
 /* ---- softmax -------------------------------------------------------------------------------- */
 /* x bf16 [rows, N] -> y = softmax(x, -1) bf16 and counts[r] = #{j : y[r,j] > bf16(threshold)} (counts may be
  * NULL).  With x == NULL, y is taken as given and only the counts are produced. */

@@ -171,6 +171,25 @@ def test_hadamard_bwd(K, M, H, b1, g1, b2, g2):
     assert bits_equal(d1.cpu(), w1) and bits_equal(d2.cpu(), w2)
 
 
+@pytest.mark.parametrize("act", ["silu", "gelu"])
+@pytest.mark.parametrize("M,H,bits,group", [(40, 4096, 4, 128), (2100, 11008, 2, 64), (33, 2048, 8, 64)])
+def test_gated_act_bwd_equals_the_two_steps(K, act, M, H, bits, group):
+    """one pass over (act(gate), up, gate) = hadamard backward followed by the activation backward, bit for bit"""
+    k = K.num_outlier_channels(H, 0.01)
+    gate, gen = make_x(5, M, H, k, 10.0)
+    up, _ = make_x(6, M, H, k, 10.0)
+    a = torch.nn.functional.silu(gate.float()).bfloat16() if act == "silu" else torch.nn.functional.gelu(gate.float()).bfloat16()
+    g = (0.1 * torch.randn(M, H, generator=gen)).bfloat16().cuda()
+    cs = []
+    for t in (a, up, gate):
+        td = t.cuda()
+        cs.append(K.compress_channel(td, K.select_channels(K.channel_absmax(td), k), bits, group))
+    d_h, d_up = K.hadamard_bwd(g, cs[0], cs[1])
+    d_gate = K.act_bwd(act, d_h, cs[2])
+    f_gate, f_up = K.gated_act_bwd(act, g, cs[0], cs[1], cs[2])
+    assert bits_equal(f_up, d_up) and bits_equal(f_gate, d_gate)
+
+
 def test_config2_shape(K):
     """BASELINE config 2: x [4,1024,4096] with 20 channels x30, w ~ N(1, 0.1), eps 1e-6, dy ~ N(0, 0.02), 1 % / INT4 / 128."""
     M, H = 4096, 4096

@@ -297,3 +297,25 @@ def test_linear_module(ops, K, mode, bits, group):
         dX, dW_lit, dW_f32, _ = O.linear_bwd(dy, xh, w)
         assert torch.allclose(xd.grad.cpu().float(), dX.float(), rtol=2e-2, atol=2e-3)
         assert torch.allclose(lin.weight.grad.cpu().float(), dW_f32, rtol=1e-2, atol=1e-3 + 4e-3 * float(dW_f32.abs().max()))
+
+
+@pytest.mark.gpu
+def test_gated_act_module_equals_silu_then_hadamard(ops):
+    """EfficientMemoryGatedAct = EfficientMemorySiLU followed by EfficientMemoryHadamard (channel scheme), bit for bit"""
+    gen = torch.Generator().manual_seed(11)
+    gate = torch.randn(2, 24, 4096, generator=gen).bfloat16().cuda()
+    up = torch.randn(2, 24, 4096, generator=gen).bfloat16().cuda()
+    gout = (0.1 * torch.randn(2, 24, 4096, generator=gen)).bfloat16().cuda()
+    kw = dict(outlier_ratio=0.01, sub_outlier_ratio=1.0, sub_outlier_bit=4, sub_outlier_quantize_method="per-token", rank=0)
+    fused = ops.EfficientMemoryGatedAct("silu", **kw)
+    silu = ops.EfficientMemorySiLU(mode="hyc", **kw)
+    had = ops.EfficientMemoryHadamard(0.01, 1.0, 4, "per-token", 0.01, 1.0, 4, "per-token", 0, mode="hyc")
+    for _ in range(3):                                    # two calibration calls, one steady-state call
+        g1, u1 = gate.clone().requires_grad_(), up.clone().requires_grad_()
+        g2, u2 = gate.clone().requires_grad_(), up.clone().requires_grad_()
+        y1 = fused(g1, u1)
+        y2 = had(silu(g2), u2)
+        assert torch.equal(y1, y2)
+        y1.backward(gout)
+        y2.backward(gout)
+        assert torch.equal(g1.grad, g2.grad) and torch.equal(u1.grad, u2.grad)
