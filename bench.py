@@ -130,6 +130,40 @@ def gradw_extra(pkg, torch, wl):
     return out
 
 
+def kernel_tour(pkg, torch, reps=5):
+    """every kernel of the path at the BASELINE config shapes (INT4 / group 128 and INT2 / group 64, 1 % outlier
+    channels): compress, decompress, activation / Hadamard / gated backward at H = 11008, weight gradient"""
+    K = pkg.kernels
+    gen = torch.Generator(device="cuda").manual_seed(0)
+
+    def mk(M, H, hot):
+        x = torch.randn(M, H, generator=gen, device="cuda")
+        x[:, torch.randperm(H, generator=gen, device="cuda")[:hot]] *= 30
+        return x.bfloat16()
+
+    for (M, H, bits, G) in ((4096, 4096, 4, 128), (4096, 4096, 2, 64), (4096, 11008, 4, 128)):
+        k = K.num_outlier_channels(H, 0.01)
+        x, up = mk(M, H, k // 2), mk(M, H, k // 2)
+        a = torch.nn.functional.silu(x)
+        g = (0.02 * torch.randn(M, H, generator=gen, device="cuda")).bfloat16()
+        cs = [K.compress_channel(t, K.select_channels(K.channel_absmax(t), k), bits, G) for t in (x, up, a)]
+        plan = K.select_channels(K.channel_absmax(x), k)
+        dy16 = (0.01 * torch.randn(M, 16, generator=gen, device="cuda")).bfloat16()
+        dyN = (0.01 * torch.randn(M, 4096, generator=gen, device="cuda")).bfloat16()
+        for _ in range(reps):
+            K.compress_channel(x, plan, bits, G)
+            K.decompress_channel(cs[0])
+            K.act_bwd("silu", g, cs[0])
+            K.act_bwd("gelu", g, cs[0])
+            K.hadamard_bwd(g, cs[2], cs[1])
+            K.gated_act_bwd("silu", g, cs[2], cs[1], cs[0])
+            K.gradw_gemm(dy16, cs[0])
+            K.gradw_gemm(dyN, cs[0])
+        torch.cuda.synchronize()
+        del x, up, a, g, cs
+    print(json.dumps({"kernel_tour": True}))
+
+
 def cpu_baseline(torch, wl, rows, seconds):
     """the oracle (CPU PyTorch restatement of the path) on the host cores, bounded sample of the same workload"""
     from oracle import hyc_oracle as O
@@ -167,6 +201,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-scaled", action="store_true", help="skip the 16x token-scaled run")
+    ap.add_argument("--kernel-tour", action="store_true",
+                    help="for rocprofv3 --kernel-trace: run every kernel of the path a few times at the config shapes, then exit")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="for rocprofv3 --pmc: 5x a plain 32 MiB device copy, 5x fwd, 5x bwd, then exit")
     args = ap.parse_args()
@@ -185,6 +221,9 @@ def main():
     wl = Workload(pkg, torch, M, H, bits, group, n_hot=20, gain=30.0)
     fwd_b, bwd_b, saved_b = algorithmic_bytes(M, H, bits, group, wl.k)
 
+    if args.kernel_tour:
+        kernel_tour(pkg, torch)
+        return
     if args.pmc_probe:
         dst = torch.empty_like(wl.x)
         for _ in range(5):
