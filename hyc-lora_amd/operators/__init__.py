@@ -6,3 +6,4 @@ from .efficient_linear import EfficientMemoryLinear, EfficientMemoryLinearFunc  
 from .efficient_rmsnorm import EfficientMemoryRMSNorm, EfficientMemoryRMSNormFunc  # noqa: F401
 from .efficient_silu import EfficientMemorySiLU, EfficientMemorySiLUFunc  # noqa: F401
 from .efficient_softmax import EfficientMemorySoftmax, EfficientMemorySoftmaxFunc  # noqa: F401
+from .swap import replace_module_for_quantization  # noqa: F401

@@ -1,0 +1,77 @@
+"""Swap a model's modules for their memory-efficient counterparts.
+
+Mirrors `replace_module_for_quantization` of the reference's training scripts (train_gsm8k.py:426-592,
+train_glue.py:391-493): same selection rules, same constructor keywords taken from the same `compress_config`
+sections ("linear", "silu", "layernorm", "softmax", "hadamard"), weights re-pointed, recursion into everything else.
+Module kinds this package does not provide (LayerNorm, Gemma RMSNorm, Dropout, the attention GEMM wrappers) are
+left as they are and reported, or raise with `strict=True`.
+"""
+import torch
+
+from .efficient_gelu import EfficientMemoryGELU
+from .efficient_hadamard import EfficientMemoryHadamard
+from .efficient_linear import EfficientMemoryLinear
+from .efficient_rmsnorm import EfficientMemoryRMSNorm
+from .efficient_silu import EfficientMemorySiLU
+from .efficient_softmax import EfficientMemorySoftmax
+
+
+def _knobs(section):
+    return dict(outlier_ratio=section["outlier_ratio"], sub_outlier_ratio=section["sub_outlier_ratio"],
+                rank=section["rank"], sub_outlier_bit=section["sub_outlier_bit"],
+                sub_outlier_quantize_method=section["sub_outlier_quant_method"])
+
+
+def replace_module_for_quantization(module, compress_config, model_args=None, *, mode="ref", group_size=128,
+                                    strict=False, _skipped=None):
+    """In place.  Returns the list of (qualified name, class name) of modules the reference would have swapped but this
+    package has no counterpart for.  `model_args` is accepted for signature compatibility (the reference reads
+    `model_name_or_path` from it to pick the Gemma RMSNorm)."""
+    skipped = [] if _skipped is None else _skipped
+    extra = dict(mode=mode, group_size=group_size)
+    gemma = model_args is not None and "gemma" in str(getattr(model_args, "model_name_or_path", ""))
+
+    def unsupported(name, child):
+        if strict:
+            raise NotImplementedError("no memory-efficient counterpart for %s (%s)" % (name, child.__class__.__name__))
+        skipped.append((name, child.__class__.__name__))
+
+    for name, child in module.named_children():
+        cls = child.__class__.__name__
+        if (isinstance(child, torch.nn.Linear) and child.weight.requires_grad and child.in_features > 100
+                and "lm_head" not in name):
+            new = EfficientMemoryLinear(in_features=child.in_features, out_features=child.out_features,
+                                        bias=child.bias is not None, **_knobs(compress_config["linear"]), **extra)
+            new.weight.data = child.weight.data
+            if child.bias is not None:
+                new.bias.data = child.bias.data
+            setattr(module, name, new)
+        elif "SiLU" in cls:
+            setattr(module, name, EfficientMemorySiLU(**_knobs(compress_config["silu"]), **extra))
+        elif "GELU" in cls:
+            setattr(module, name, EfficientMemoryGELU(**_knobs(compress_config["silu"]), **extra))   # sic: the "silu" section
+        elif "RMSNorm" in cls:
+            if gemma:
+                unsupported(name, child)
+                continue
+            eps = getattr(child, "variance_epsilon", getattr(child, "eps", 1e-5))
+            new = EfficientMemoryRMSNorm(normalized_shape=child.weight.data.shape, eps=eps, elementwise_affine=True,
+                                         bias=False, **_knobs(compress_config["layernorm"]), **extra)
+            new.weight.data = child.weight.data
+            setattr(module, name, new)
+        elif "LayerNorm" in cls or isinstance(child, torch.nn.Dropout) or "GEMM" in cls:
+            unsupported(name, child)
+        elif isinstance(child, torch.nn.Softmax):
+            setattr(module, name, EfficientMemorySoftmax(outlier_ratio=compress_config["softmax"]["outlier_ratio"]))
+        elif "Hadamard" in cls:
+            h = compress_config["hadamard"]
+            setattr(module, name, EfficientMemoryHadamard(
+                outlier_ratio_1=h["outlier_ratio"], sub_outlier_ratio_1=h["sub_outlier_ratio"],
+                sub_outlier_bit_1=h["sub_outlier_bit"], sub_outlier_quantize_method_1=h["sub_outlier_quant_method"],
+                outlier_ratio_2=h["outlier_ratio"], sub_outlier_ratio_2=h["sub_outlier_ratio"],
+                sub_outlier_bit_2=h["sub_outlier_bit"], sub_outlier_quantize_method_2=h["sub_outlier_quant_method"],
+                rank=h["rank"], **extra))
+        else:
+            replace_module_for_quantization(child, compress_config, model_args, mode=mode, group_size=group_size,
+                                            strict=strict, _skipped=skipped)
+    return skipped

@@ -148,3 +148,48 @@ def test_module_constructors_mirror_the_reference(hyc):
     assert callable(ops.fused_compression.low_rank_extraction) and callable(ops.fused_compression.low_rank_addition)
     x = torch.arange(2 * 3 * 8, dtype=torch.float32).reshape(2, 3, 8)
     assert torch.equal(cf.head_to_hidden_shape(cf.hidden_to_head_shape(x, 2)), x)
+
+
+def test_module_swap_follows_the_reference_rules(hyc):
+    """replace_module_for_quantization (train_gsm8k.py:426-592): trainable wide Linear, SiLU, RMSNorm, Softmax are
+    swapped with their weights shared; frozen / narrow Linear, lm_head, unsupported kinds are not"""
+    import torch
+    ops = hyc.operators
+
+    class TinyRMSNorm(torch.nn.Module):
+        def __init__(self, h):
+            super().__init__()
+            self.weight = torch.nn.Parameter(torch.ones(h))
+            self.variance_epsilon = 1e-6
+
+    class Block(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.norm = TinyRMSNorm(128)
+            self.lora_A = torch.nn.Linear(128, 16, bias=False)
+            self.lora_B = torch.nn.Linear(16, 128, bias=False)          # in_features <= 100: untouched
+            self.base = torch.nn.Linear(128, 128)
+            self.base.weight.requires_grad_(False)                      # frozen: untouched
+            self.act_fn = torch.nn.SiLU()
+            self.softmax = torch.nn.Softmax(dim=-1)
+            self.drop = torch.nn.Dropout(0.1)
+            self.lm_head = torch.nn.Linear(128, 128)
+
+    model = torch.nn.Sequential(Block(), Block())
+    cfg = {k: dict(outlier_ratio=0.01, sub_outlier_ratio=1.0, rank=0, sub_outlier_bit=4, sub_outlier_quant_method="per-token")
+           for k in ("linear", "silu", "layernorm", "hadamard")}
+    cfg["softmax"] = dict(outlier_ratio=0.05)
+    w_before = model[0].lora_A.weight.data_ptr()
+    skipped = ops.replace_module_for_quantization(model, cfg, mode="hyc", group_size=64)
+    b = model[1]
+    assert isinstance(b.lora_A, ops.EfficientMemoryLinear) and b.lora_A.mode == "hyc" and b.lora_A.group_size == 64
+    assert b.lora_A.sub_outlier_bit == 4 and b.lora_A.rank == 0
+    assert model[0].lora_A.weight.data_ptr() == w_before
+    assert type(b.lora_B) is torch.nn.Linear and type(b.base) is torch.nn.Linear and type(b.lm_head) is torch.nn.Linear
+    assert isinstance(b.norm, ops.EfficientMemoryRMSNorm) and b.norm.eps == 1e-6 and b.norm.bias is None
+    assert isinstance(b.act_fn, ops.EfficientMemorySiLU) and isinstance(b.softmax, ops.EfficientMemorySoftmax)
+    assert b.softmax.outlier_ratio == 0.05
+    assert sorted(skipped) == [("drop", "Dropout"), ("drop", "Dropout")]
+    import pytest
+    with pytest.raises(NotImplementedError):
+        ops.replace_module_for_quantization(torch.nn.Sequential(torch.nn.LayerNorm(8)), cfg, strict=True)
