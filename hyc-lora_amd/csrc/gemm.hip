@@ -441,7 +441,7 @@ static int direct_splits(int64_t M, int64_t N_out, int64_t H) {
 // decode overlaps this one's MFMAs.
 // ------------------------------------------------------------------------------------------------
 constexpr int WK = 32;      // tokens per stage
-constexpr int WN = 128;     // dY features per workgroup
+constexpr int WN = 128;     // dY features per workgroup: WN (four waves) or 2*WN (eight waves)
 constexpr int WH = 256;     // channels per workgroup
 
 template <int NSEG, int A_PER, int B_PER>
@@ -449,38 +449,28 @@ struct WideRegs {            // one stage of global data per thread
   uint4 a[A_PER];            // dY chunks
   uint4 b[B_PER];            // channel scheme: .x/.y = packed word; dense: 8 bf16
   uint32_t s[B_PER][NSEG];   // channel scheme: the group scale of each segment's chunk
+  uint32_t o0[B_PER][NSEG], o1[B_PER][NSEG];   // ... and the first two outlier values of the chunk
 };
 
-template <int BITS, int SRC>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
+template <int BITS, int SRC, int WNT>
+__global__ void __launch_bounds__(2 * WNT) __attribute__((amdgpu_waves_per_eu(2)))
 k_gradw_wide(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_out, int64_t H,
              const uint8_t* __restrict__ stored, const uint16_t* __restrict__ vals, const uint16_t* __restrict__ scales,
-             ChanArgs ca, int CPS, int extra_tiles, int64_t tokens_per_split, float alpha, float beta,
+             ChanArgs ca, int CPS, int64_t tokens_per_split, float alpha, float beta,
              void* __restrict__ out, int out_f32, float* __restrict__ partial) {
   constexpr int NSEG = (SRC == 0) ? Q<BITS>::NSEG : 1;
   constexpr int HS = WH / NSEG;               // columns of the tile that come from one segment
   constexpr int CPR = HS / 8;                 // packed 8-byte chunks (channel scheme) / 16-byte chunks (dense) per token row and segment
-  constexpr int AP = WN + GPAD, BP = WH + GPAD;
+  constexpr int THREADS = 2 * WNT;            // waves: WNT/64 along n x 2 along h, 64 x 128 each
+  constexpr int AP = WNT + GPAD, BP = WH + GPAD;
   __shared__ __align__(16) uint16_t As[2][WK * AP];
   __shared__ __align__(16) uint16_t Bs[2][WK * BP];
 
-  // Workgroups past the main tiles compute the outlier columns dW[:, idx[q]] = dY^T vals[:, q] with the streaming
-  // tile: 16 outlier channels x 32 features each, four feature blocks per 128-feature tile of this grid.
-  // They come first in the grid: each walks the whole token range with little work per step, so they start early
-  // and run beside the main tiles instead of forming a tail.
-  if (SRC == 0 && (int)blockIdx.y < extra_tiles) {
-    const int e = (int)blockIdx.y;
-    DirectArgs A = {dy, ldy, M, N_out, H, stored, vals, scales, ca, CPS, 0, tokens_per_split, alpha, beta, out, out_f32, partial};
-    const int64_t nf = (int64_t)blockIdx.x * WN + 32 * (e & 3);
-    if (nf < N_out) gradw_direct_tile<BITS, 2, false>(A, reinterpret_cast<float*>(&Bs[0][0]), e >> 2, nf);
-    return;
-  }
-
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int64_t n0 = (int64_t)blockIdx.x * WN;
+  const int64_t n0 = (int64_t)blockIdx.x * WNT;
   const int64_t SEG = (SRC == 0) ? (int64_t)CPS * 8 : H;
-  const int64_t j0 = (int64_t)((int)blockIdx.y - extra_tiles) * HS;   // first column of the tile inside each segment
+  const int64_t j0 = (int64_t)blockIdx.y * HS;          // first column of the tile inside each segment
   const int64_t m_begin = (int64_t)blockIdx.z * tokens_per_split;
   const int64_t m_end = m_begin + tokens_per_split < M ? m_begin + tokens_per_split : M;
   const int wn = (wave >> 1) * 64, wh = (wave & 1) * 128;
@@ -493,19 +483,35 @@ k_gradw_wide(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
 
-  constexpr int A_PER = WK * WN / 8 / 256;                // 16-byte chunks of the dY stage per thread (2)
+  constexpr int A_PER = WK * WNT / 8 / THREADS;           // 16-byte chunks of the dY stage per thread (2)
   constexpr int B_ITEMS = WK * CPR;
-  constexpr int B_PER = (B_ITEMS + 255) / 256;
-  static_assert(B_ITEMS % 256 == 0 || B_ITEMS < 256, "items per stage");
-  const bool b_thread = B_ITEMS >= 256 || tid < B_ITEMS;  // 1-bit codes: 128 items per stage
-  typedef WideRegs<NSEG, A_PER, B_PER> Regs;
+  constexpr int B_PER = (B_ITEMS + THREADS - 1) / THREADS;
+  static_assert(B_ITEMS % THREADS == 0 || B_ITEMS < THREADS, "items per stage");
+  // Narrow codes give fewer packed words per stage than threads: PARTS threads then share a word, NST segments each.
+  constexpr int PARTS = (SRC == 0 && B_ITEMS < THREADS) ? THREADS / B_ITEMS : 1;
+  constexpr int NST = NSEG / PARTS;                       // segments a thread decodes
+  static_assert(NSEG % PARTS == 0 && (PARTS == 1 || PARTS * B_ITEMS == THREADS), "threads per packed word");
+  const int seg0 = (PARTS > 1 ? tid / B_ITEMS : 0) * NST; // first of them
+  const int item0 = PARTS > 1 ? tid % B_ITEMS : tid;      // the thread's first item
+  constexpr bool b_thread = true;
+  typedef WideRegs<NST, A_PER, B_PER> Regs;
+  // A thread decodes the same chunk column of every row it touches (THREADS is a multiple of CPR), so its outlier
+  // work is static: selectors that splice up to two outlier values into a decoded chunk, as in the row kernels.
+  ChunkOutliers<NST> co;
+  {
+    uint32_t pw[NST];
+#pragma unroll
+    for (int i = 0; i < NST; ++i)
+      pw[i] = (SRC == 0) ? ca.plan[(seg0 + i) * CPS + (int)(j0 / 8) + item0 % CPR] : 0u;
+    co.init(pw);
+  }
 
   // Loads past the token range re-read the last token with the dY operand zeroed; nothing is conditional.
   auto fetch = [&](Regs& R, int64_t m0) __attribute__((always_inline)) {
 #pragma unroll
     for (int u = 0; u < A_PER; ++u) {
-      const int idx = tid + u * 256;
-      const int row = idx / (WN / 8), cc = idx % (WN / 8);
+      const int idx = tid + u * THREADS;
+      const int row = idx / (WNT / 8), cc = idx % (WNT / 8);
       const int64_t m = m0 + row, n = n0 + 8 * cc;
       const bool ok = m < m_end && n < N_out;
       const uint4 v = *reinterpret_cast<const uint4*>(dy + (m < m_end ? m : m_end - 1) * ldy + (n < N_out ? n : 0));
@@ -513,7 +519,7 @@ k_gradw_wide(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_
     }
 #pragma unroll
     for (int u = 0; u < B_PER; ++u) {
-      const int idx = b_thread ? tid + u * 256 : 0;
+      const int idx = item0 + u * THREADS;
       const int row = idx / CPR, cc = idx % CPR;
       const int64_t m = m0 + row < m_end ? m0 + row : m_end - 1;
       if (SRC == 0) {
@@ -521,32 +527,39 @@ k_gradw_wide(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_
         const uint2 pk = *reinterpret_cast<const uint2*>(stored + m * SEG + 8 * c);
         R.b[u] = make_uint4(pk.x, pk.y, 0, 0);
 #pragma unroll
-        for (int i = 0; i < NSEG; ++i)
-          R.s[u][i] = scales[m * ca.groups_per_row + ((i * CPS + c) >> ca.chunk_to_group_shift)];
+        for (int i = 0; i < NST; ++i)
+          R.s[u][i] = scales[m * ca.groups_per_row + (((seg0 + i) * CPS + c) >> ca.chunk_to_group_shift)];
+        co.request(vals + m * ca.k, R.o0[u], R.o1[u]);
       } else {
         R.b[u] = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(stored) + m * H + j0 + 8 * cc);
       }
     }
   };
-  // decode one stage of registers into LDS buffer `buf`
-  auto stash = [&](int buf, const Regs& R) __attribute__((always_inline)) {
+  // (chunks with more than two outlier channels: the remaining pairs, rare, loaded in place)
+  auto finish_chunk = [&](uint4 r, int i, int cc, int64_t m) __attribute__((always_inline)) {
+    if (co.more_pairs)
+      r = splice_more(r, co.more_pairs, ca.plan[(seg0 + i) * CPS + (int)(j0 / 8) + cc], vals + (m < m_end ? m : m_end - 1) * ca.k, true, 1.f);
+    return r;
+  };
+  // decode one stage of registers (tokens mb ..) into LDS buffer `buf`
+  auto stash = [&](int buf, const Regs& R, int64_t mb) __attribute__((always_inline)) {
 #pragma unroll
     for (int u = 0; u < A_PER; ++u) {
-      const int idx = tid + u * 256;
-      const int row = idx / (WN / 8), cc = idx % (WN / 8);
+      const int idx = tid + u * THREADS;
+      const int row = idx / (WNT / 8), cc = idx % (WNT / 8);
       *reinterpret_cast<uint4*>(&As[buf][row * AP + 8 * cc]) = R.a[u];
     }
     if (b_thread) {
 #pragma unroll
       for (int u = 0; u < B_PER; ++u) {
-        const int idx = tid + u * 256;
+        const int idx = item0 + u * THREADS;
         const int row = idx / CPR, cc = idx % CPR;
         if (SRC == 0) {
-          // outlier channels decode to 0 here; their columns of dW come from the outlier tiles (see the epilogue)
 #pragma unroll
-          for (int i = 0; i < NSEG; ++i)
-            *reinterpret_cast<uint4*>(&Bs[buf][row * BP + i * HS + 8 * cc]) =
-                dequant8_fast<BITS>(R.b[u].x, R.b[u].y, i, bf_to_f((uint16_t)R.s[u][i]));
+          for (int i = 0; i < NST; ++i)
+            *reinterpret_cast<uint4*>(&Bs[buf][row * BP + (seg0 + i) * HS + 8 * cc]) = finish_chunk(
+                co.splice(i, dequant8_fast<BITS>(R.b[u].x, R.b[u].y, seg0 + i, bf_to_f((uint16_t)R.s[u][i])), R.o0[u][i],
+                          R.o1[u][i], 1.f), i, cc, mb + row);
         } else {
           *reinterpret_cast<uint4*>(&Bs[buf][row * BP + 8 * cc]) = R.b[u];
         }
@@ -575,28 +588,30 @@ k_gradw_wide(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_
     Regs R0, R1;
     int64_t m0 = m_begin;
     fetch(R0, m0);
-    stash(0, R0);
+    stash(0, R0, m0);
     if (m0 + WK < m_end) fetch(R0, m0 + WK);
     // steady state: the next three stages exist, so nothing is conditional and the decode of stage s+1 shares a
     // basic block with the MFMAs of stage s (the scheduling groups below interleave them)
     // One MFMA takes 8 passes; the wave issues in order, so the decode is cut into 16 pieces (two elements each:
     // convert, scale, round, pack) and one piece follows each of the stage's 16 MFMAs.
-    auto overlap = [&](int buf, const Regs& R) __attribute__((always_inline)) {
-      constexpr bool PIECES = SRC == 0 && B_PER * NSEG * 4 == 16;       // 2-, 4- and 8-bit codes
+    auto overlap = [&](int buf, const Regs& R, int64_t mb) __attribute__((always_inline)) {
+      constexpr int NP = B_PER * NST * 4;                               // two-element pieces of a thread's decode
+      constexpr bool PIECES = SRC == 0 && (NP == 16 || NP == 8);        // 2-, 4- and 8-bit codes
+      constexpr int EVERY = PIECES ? 16 / NP : 1;                       // MFMAs per piece
       if (!PIECES) {
-        stash(buf ^ 1, R);
+        stash(buf ^ 1, R, mb);
         mfma_stage(buf);
       } else {
         constexpr uint32_t REP = (BITS == 8) ? 0x80808080u : Q<BITS>::CODE_MASK * 0x01010101u;
         constexpr float OFFV = (BITS == 8) ? 128.f : (float)Q<BITS>::OFF;
-        uint32_t cw[B_PER][NSEG][2], res[B_PER][NSEG][4];
-        float sc[B_PER][NSEG], ns[B_PER][NSEG];
+        uint32_t cw[B_PER][NST][2], res[B_PER][NST][4];
+        float sc[B_PER][NST], ns[B_PER][NST];
 #pragma unroll
         for (int u = 0; u < B_PER; ++u)
 #pragma unroll
-          for (int i = 0; i < NSEG; ++i) {
-            cw[u][i][0] = (BITS == 8) ? R.b[u].x ^ REP : (R.b[u].x >> (i * BITS)) & REP;
-            cw[u][i][1] = (BITS == 8) ? R.b[u].y ^ REP : (R.b[u].y >> (i * BITS)) & REP;
+          for (int i = 0; i < NST; ++i) {
+            cw[u][i][0] = (BITS == 8) ? R.b[u].x ^ REP : (R.b[u].x >> ((seg0 + i) * BITS)) & REP;
+            cw[u][i][1] = (BITS == 8) ? R.b[u].y ^ REP : (R.b[u].y >> ((seg0 + i) * BITS)) & REP;
             sc[u][i] = bf_to_f((uint16_t)R.s[u][i]);
             ns[u][i] = -OFFV * sc[u][i];
           }
@@ -615,49 +630,52 @@ k_gradw_wide(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_
               __builtin_amdgcn_sched_barrier(0);
               acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[a], bfv[b], acc[a][b], 0, 0, 0);
               __builtin_amdgcn_sched_barrier(0);
-              const int u = piece / (4 * NSEG), i = (piece / 4) % NSEG, w = piece % 4;
-              const uint32_t src = cw[u][i][w >> 1] >> (16 * (w & 1));
-              const float f0 = __builtin_fmaf((float)(src & 0xFFu), sc[u][i], ns[u][i]);
-              const float f1 = __builtin_fmaf((float)((src >> 8) & 0xFFu), sc[u][i], ns[u][i]);
-              res[u][i][w] = pack_bf16(f0, f1);
-              ++piece;
+              if ((a * 4 + b) % EVERY == 0) {
+                const int u = piece / (4 * NST), i = (piece / 4) % NST, w = piece % 4;
+                const uint32_t src = cw[u][i][w >> 1] >> (16 * (w & 1));
+                const float f0 = __builtin_fmaf((float)(src & 0xFFu), sc[u][i], ns[u][i]);
+                const float f1 = __builtin_fmaf((float)((src >> 8) & 0xFFu), sc[u][i], ns[u][i]);
+                res[u][i][w] = pack_bf16(f0, f1);
+                ++piece;
+              }
             }
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int u = 0; u < A_PER; ++u) {
-          const int idx = tid + u * 256;
-          const int row = idx / (WN / 8), cc = idx % (WN / 8);
+          const int idx = tid + u * THREADS;
+          const int row = idx / (WNT / 8), cc = idx % (WNT / 8);
           *reinterpret_cast<uint4*>(&As[buf ^ 1][row * AP + 8 * cc]) = R.a[u];
         }
 #pragma unroll
         for (int u = 0; u < B_PER; ++u) {
-          const int idx = tid + u * 256;
+          const int idx = item0 + u * THREADS;
           const int row = idx / CPR, cc = idx % CPR;
 #pragma unroll
-          for (int i = 0; i < NSEG; ++i)
-            *reinterpret_cast<uint4*>(&Bs[buf ^ 1][row * BP + i * HS + 8 * cc]) =
-                make_uint4(res[u][i][0], res[u][i][1], res[u][i][2], res[u][i][3]);
+          for (int i = 0; i < NST; ++i)
+            *reinterpret_cast<uint4*>(&Bs[buf ^ 1][row * BP + (seg0 + i) * HS + 8 * cc]) = finish_chunk(
+                co.splice(i, make_uint4(res[u][i][0], res[u][i][1], res[u][i][2], res[u][i][3]), R.o0[u][i], R.o1[u][i], 1.f),
+                i, cc, mb + row);
         }
       }
     };
     for (; m0 + 3 * WK < m_end; m0 += 2 * WK) {
       fetch(R1, m0 + 2 * WK);
       __syncthreads();                                    // buffer 0 is complete; buffer 1 is no longer read
-      overlap(0, R0);
+      overlap(0, R0, m0 + WK);
       fetch(R0, m0 + 3 * WK);
       __syncthreads();
-      overlap(1, R1);
+      overlap(1, R1, m0 + 2 * WK);
     }
     for (; m0 < m_end; m0 += 2 * WK) {
       if (m0 + 2 * WK < m_end) fetch(R1, m0 + 2 * WK);
       __syncthreads();                                    // buffer 0 is complete; buffer 1 is no longer read
-      if (m0 + WK < m_end) stash(1, R0);
+      if (m0 + WK < m_end) stash(1, R0, m0 + WK);
       mfma_stage(0);
       if (m0 + WK < m_end) {
         if (m0 + 3 * WK < m_end) fetch(R0, m0 + 3 * WK);
         __syncthreads();
-        if (m0 + 2 * WK < m_end) stash(0, R1);
+        if (m0 + 2 * WK < m_end) stash(0, R1, m0 + 2 * WK);
         mfma_stage(1);
       }
     }
@@ -672,7 +690,6 @@ k_gradw_wide(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_
       const int hl = wh + 32 * b + (lane & 31);              // column inside the tile
       const int64_t hs = j0 + (hl % HS);                     // column inside its segment
       const int64_t h = (int64_t)(hl / HS) * SEG + hs;
-      if (SRC == 0 && ((ca.plan[(hl / HS) * CPS + (int)(hs >> 3)] >> (hs & 7)) & 1u)) continue;   // an outlier channel
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int64_t n = n0 + wn + 32 * a + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
@@ -814,7 +831,8 @@ int hyc_gradw_gemm(const void* dy, int64_t ldy, const void* stored, const void* 
   const int splits = M > 0 ? choose_splits(M, n_tiles * h_tiles) : 1;     // (the wide kernel has half the tiles: same value)
   if (M > 0 && (!dy || !stored)) return fail(HYC_EFAULT, "hyc_gradw_gemm: null buffer");
   // wide tiles (128 x 256) when the output is large and the tile grid fits the packing
-  const bool wide = N_out >= WN && (chan ? g.seg % (WH / g.nseg) == 0 : H % WH == 0);
+  // (the channel scheme uses the eight-wave form only: its four-wave form runs out of registers)
+  const bool wide = chan ? (N_out >= 2 * WN && g.seg % (WH / g.nseg) == 0) : (N_out >= WN && H % WH == 0);
   if (chan && M > 0 && (!scales || (d->k > 0 && !vals))) return fail(HYC_EFAULT, "hyc_gradw_gemm: null vals/scales");
   if (M > 0 && (!aligned16(dy) || !aligned8(stored) || (!chan && !aligned16(stored))))
     return fail(HYC_EINVAL, "hyc_gradw_gemm: dy must be 16-byte aligned, stored 8-byte (16 when dense)");
@@ -825,24 +843,27 @@ int hyc_gradw_gemm(const void* dy, int64_t ldy, const void* stored, const void* 
   const dim3 grid((unsigned)n_tiles, (unsigned)h_tiles, (unsigned)splits);
   const int of32 = out_dtype == HYC_DTYPE_F32;
   if (wide) {
-    const int main_h = (int)(H / WH);
-    const int extra = chan ? 4 * ((d->k + 15) / 16) : 0;   // outlier tiles: 16 channels x 32 features each
-    const dim3 wgrid((unsigned)n_tiles, (unsigned)(main_h + extra), (unsigned)splits);
-#define HYC_WIDE(B_, S_)                                                                                          \
-  hipLaunchKernelGGL((k_gradw_wide<B_, S_>), wgrid, dim3(256), 0, st, static_cast<const uint16_t*>(dy), ldy, M, N_out, H, \
-                     static_cast<const uint8_t*>(stored), static_cast<const uint16_t*>(vals),                    \
-                     static_cast<const uint16_t*>(scales), ca, g.cps, extra, tps, alpha, beta, out, of32, partial)
+    // eight waves (256 features per workgroup) halve the decode work per MFMA; four waves fill the chip better
+    // when the output is small
+    const int wnt = chan || (N_out >= 2 * WN && ((N_out + 2 * WN - 1) / (2 * WN)) * (H / WH) >= 128) ? 2 * WN : WN;
+    const dim3 wgrid((unsigned)((N_out + wnt - 1) / wnt), (unsigned)(H / WH), (unsigned)splits);
+#define HYC_WIDE_W(B_, S_, W_)                                                                                    \
+  hipLaunchKernelGGL((k_gradw_wide<B_, S_, W_>), wgrid, dim3(2 * W_), 0, st, static_cast<const uint16_t*>(dy), ldy, M, \
+                     N_out, H, static_cast<const uint8_t*>(stored), static_cast<const uint16_t*>(vals),          \
+                     static_cast<const uint16_t*>(scales), ca, g.cps, tps, alpha, beta, out, of32, partial)
     if (chan) {
       switch (d->bits) {
-        case 1: HYC_WIDE(1, 0); break;
-        case 2: HYC_WIDE(2, 0); break;
-        case 4: HYC_WIDE(4, 0); break;
-        default: HYC_WIDE(8, 0); break;
+        case 1: HYC_WIDE_W(1, 0, 2 * WN); break;
+        case 2: HYC_WIDE_W(2, 0, 2 * WN); break;
+        case 4: HYC_WIDE_W(4, 0, 2 * WN); break;
+        default: HYC_WIDE_W(8, 0, 2 * WN); break;
       }
+    } else if (wnt == WN) {
+      HYC_WIDE_W(4, 2, WN);
     } else {
-      HYC_WIDE(4, 2);
+      HYC_WIDE_W(4, 2, 2 * WN);
     }
-#undef HYC_WIDE
+#undef HYC_WIDE_W
   } else {
 #define HYC_GEMM(B_, S_, N_)                                                                                     \
   hipLaunchKernelGGL((k_gradw<B_, S_, N_>), grid, dim3(256), 0, st, static_cast<const uint16_t*>(dy), ldy, M, N_out, H, \

@@ -31,7 +31,7 @@ def make_x(seed, M, H, n_hot, gain):
 
 
 # ------------------------------------------------------------------ weight gradient
-GEMM_CASES = [(4, 128, 200, 512, 16, 5), (4, 128, 4096, 4096, 16, 41), (2, 64, 1000, 4096, 16, 41),
+GEMM_CASES = [(4, 128, 200, 512, 16, 5), (2, 64, 300, 2048, 512, 20), (1, 64, 200, 2048, 256, 20), (8, 128, 150, 1024, 264, 30), (4, 32, 100, 512, 256, 300), (4, 128, 4096, 4096, 16, 41), (2, 64, 1000, 4096, 16, 41),
               (4, 128, 333, 1024, 256, 10), (8, 128, 130, 512, 136, 5), (1, 64, 96, 1024, 40, 10),
               (2, 64, 257, 2048, 128, 20), (4, 128, 64, 11008, 32, 110), (4, 128, 520, 1024, 4096, 10)]
 
