@@ -7,3 +7,4 @@ from .efficient_rmsnorm import EfficientMemoryRMSNorm, EfficientMemoryRMSNormFun
 from .efficient_silu import EfficientMemorySiLU, EfficientMemorySiLUFunc  # noqa: F401
 from .efficient_softmax import EfficientMemorySoftmax, EfficientMemorySoftmaxFunc  # noqa: F401
 from .swap import replace_module_for_quantization  # noqa: F401
+from .efficient_rmsnorm_gemma import EfficientMemoryRMSNormGemma, EfficientMemoryRMSNormGemmaFunc  # noqa: F401

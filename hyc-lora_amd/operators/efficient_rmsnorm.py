@@ -7,14 +7,21 @@ from ._calibration import CompressionSite, as_rows, fold_statistics
 from .compress_function import get_statistics
 
 
+def _effective_weight(weight, offset):
+    """the weight the kernels multiply by: w, or fp32(w) + 1 for the Gemma form (efficient_rmsnorm_gemma.py:59,100)"""
+    w = weight.detach()
+    return (w.float() + offset).contiguous() if offset else w.contiguous()
+
+
 class EfficientMemoryRMSNormFunc(torch.autograd.Function):
     """apply(x, normalized_shape, outlier_ratio, sub_outlier_ratio, sub_outlier_bit, sub_outlier_quantize_method, rank,
     weight, bias, eps, iteration, static_value) -> (y, outlier, L, R, scale); backward returns dx at slot 0 and dw at
     slot 7 (reference :147-269).  c2_quirk: the reference backward keeps LayerNorm's mean(w*dy) term (:102-104)."""
     c2_quirk = True
+    weight_offset = 0.0
 
-    @staticmethod
-    def forward(ctx, x, normalized_shape, outlier_ratio, sub_outlier_ratio, sub_outlier_bit, sub_outlier_quantize_method,
+    @classmethod
+    def forward(cls, ctx, x, normalized_shape, outlier_ratio, sub_outlier_ratio, sub_outlier_bit, sub_outlier_quantize_method,
                 rank, weight, bias, eps, iteration, static_value):
         x = x.contiguous()
         x2, S = as_rows(x)
@@ -27,7 +34,7 @@ class EfficientMemoryRMSNormFunc(torch.autograd.Function):
             outlier, L, scale, R = static_value[0], static_value[1], static_value[2], static_value[3]
         if sub_outlier_ratio == 0. or sub_outlier_bit == 16:
             raise NotImplementedError("the branches without a quantised part are outside the accelerated path")
-        y, rstd, c = K.rmsnorm_fwd_compress_threshold(x2, weight.detach().contiguous(), eps, S, float(outlier),
+        y, rstd, c = K.rmsnorm_fwd_compress_threshold(x2, _effective_weight(weight, cls.weight_offset), eps, S, float(outlier),
                                                       scale.contiguous(), sub_outlier_bit,
                                                       L.contiguous() if rank > 0 else None,
                                                       R.contiguous() if rank > 0 else None)
@@ -37,30 +44,33 @@ class EfficientMemoryRMSNormFunc(torch.autograd.Function):
         ctx.mark_non_differentiable(outlier, L, R, scale)
         return y.reshape(x.shape), outlier, L, R, scale
 
-    @staticmethod
-    def backward(ctx, dy, grad_outlier, grad_L, grad_R, grad_scale):
+    @classmethod
+    def backward(cls, ctx, dy, grad_outlier, grad_L, grad_R, grad_scale):
         dy2, _ = as_rows(dy.to(torch.bfloat16))
-        dx, dw = K.rmsnorm_bwd(dy2, ctx.saved, ctx.weight.detach().contiguous(), ctx.rstd,
-                               c2_quirk=EfficientMemoryRMSNormFunc.c2_quirk)
-        return dx.reshape(dy.shape), None, None, None, None, None, None, dw, None, None, None, None
+        dx, dw = K.rmsnorm_bwd(dy2, ctx.saved, _effective_weight(ctx.weight, cls.weight_offset), ctx.rstd,
+                               c2_quirk=cls.c2_quirk)
+        return dx.reshape(dy.shape), None, None, None, None, None, None, dw.to(ctx.weight.dtype), None, None, None, None
 
 
 class _ChannelRMSNormFunc(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, weight, eps, plan, bits, group, c2_quirk):
+    def forward(ctx, x, weight, eps, plan, bits, group, c2_quirk, weight_offset=0.0):
         x2, _ = as_rows(x)
-        y, rstd, c = K.rmsnorm_fwd_compress_channel(x2, weight.detach().contiguous(), eps, plan, bits, group)
-        ctx.saved, ctx.rstd, ctx.weight, ctx.c2_quirk = c, rstd, weight, c2_quirk
+        y, rstd, c = K.rmsnorm_fwd_compress_channel(x2, _effective_weight(weight, weight_offset), eps, plan, bits, group)
+        ctx.saved, ctx.rstd, ctx.weight, ctx.c2_quirk, ctx.weight_offset = c, rstd, weight, c2_quirk, weight_offset
         return y.reshape(x.shape)
 
     @staticmethod
     def backward(ctx, dy):
         dy2, _ = as_rows(dy.to(torch.bfloat16))
-        dx, dw = K.rmsnorm_bwd(dy2, ctx.saved, ctx.weight.detach().contiguous(), ctx.rstd, c2_quirk=ctx.c2_quirk)
-        return dx.reshape(dy.shape), dw, None, None, None, None, None
+        dx, dw = K.rmsnorm_bwd(dy2, ctx.saved, _effective_weight(ctx.weight, ctx.weight_offset), ctx.rstd,
+                               c2_quirk=ctx.c2_quirk)
+        return dx.reshape(dy.shape), dw.to(ctx.weight.dtype), None, None, None, None, None, None
 
 
 class EfficientMemoryRMSNorm(torch.nn.LayerNorm):
+    _func = EfficientMemoryRMSNormFunc
+
     def __init__(self, normalized_shape, eps=1e-05, elementwise_affine=True, bias=True, outlier_ratio: float = 0.01,
                  sub_outlier_ratio: float = 0.2, sub_outlier_bit: int = 8, sub_outlier_quantize_method: str = 'per-tensor',
                  rank: int = 16, *, mode: str = "ref", group_size: int = 128, ref_c2_quirk: bool = True):
@@ -83,11 +93,11 @@ class EfficientMemoryRMSNorm(torch.nn.LayerNorm):
             x2, _ = as_rows(x)
             plan = self.site.channel_plan(x2, self.iteration)
             y = _ChannelRMSNormFunc.apply(x, self.weight, self.eps, plan, self.sub_outlier_bit, self.group_size,
-                                          self.ref_c2_quirk)
+                                          self.ref_c2_quirk, self._func.weight_offset)
             self.iteration += 1
             return y
-        EfficientMemoryRMSNormFunc.c2_quirk = self.ref_c2_quirk
-        result, outlier, L, R, scale = EfficientMemoryRMSNormFunc.apply(
+        self._func.c2_quirk = self.ref_c2_quirk
+        result, outlier, L, R, scale = self._func.apply(
             x, self.normalized_shape, self.outlier_ratio, self.sub_outlier_ratio, self.sub_outlier_bit,
             self.sub_outlier_quantize_method, self.rank, self.weight, self.bias, self.eps, self.iteration,
             self.static_value)

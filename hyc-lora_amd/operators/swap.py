@@ -3,7 +3,7 @@
 Mirrors `replace_module_for_quantization` of the reference's training scripts (train_gsm8k.py:426-592,
 train_glue.py:391-493): same selection rules, same constructor keywords taken from the same `compress_config`
 sections ("linear", "silu", "layernorm", "softmax", "hadamard"), weights re-pointed, recursion into everything else.
-Module kinds this package does not provide (LayerNorm, Gemma RMSNorm, Dropout, the attention GEMM wrappers) are
+Module kinds this package does not provide (LayerNorm, Dropout, the attention GEMM wrappers) are
 left as they are and reported, or raise with `strict=True`.
 """
 import torch
@@ -12,6 +12,7 @@ from .efficient_gelu import EfficientMemoryGELU
 from .efficient_hadamard import EfficientMemoryHadamard
 from .efficient_linear import EfficientMemoryLinear
 from .efficient_rmsnorm import EfficientMemoryRMSNorm
+from .efficient_rmsnorm_gemma import EfficientMemoryRMSNormGemma
 from .efficient_silu import EfficientMemorySiLU
 from .efficient_softmax import EfficientMemorySoftmax
 
@@ -51,11 +52,8 @@ def replace_module_for_quantization(module, compress_config, model_args=None, *,
         elif "GELU" in cls:
             setattr(module, name, EfficientMemoryGELU(**_knobs(compress_config["silu"]), **extra))   # sic: the "silu" section
         elif "RMSNorm" in cls:
-            if gemma:
-                unsupported(name, child)
-                continue
             eps = getattr(child, "variance_epsilon", getattr(child, "eps", 1e-5))
-            new = EfficientMemoryRMSNorm(normalized_shape=child.weight.data.shape, eps=eps, elementwise_affine=True,
+            new = (EfficientMemoryRMSNormGemma if gemma else EfficientMemoryRMSNorm)(normalized_shape=child.weight.data.shape, eps=eps, elementwise_affine=True,
                                          bias=False, **_knobs(compress_config["layernorm"]), **extra)
             new.weight.data = child.weight.data
             setattr(module, name, new)

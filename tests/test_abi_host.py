@@ -190,6 +190,12 @@ def test_module_swap_follows_the_reference_rules(hyc):
     assert isinstance(b.act_fn, ops.EfficientMemorySiLU) and isinstance(b.softmax, ops.EfficientMemorySoftmax)
     assert b.softmax.outlier_ratio == 0.05
     assert sorted(skipped) == [("drop", "Dropout"), ("drop", "Dropout")]
+
+    class Args:
+        model_name_or_path = "google/gemma-7b"
+    gm = torch.nn.Sequential(Block())
+    ops.replace_module_for_quantization(gm, cfg, Args())
+    assert isinstance(gm[0].norm, ops.EfficientMemoryRMSNormGemma)
     import pytest
     with pytest.raises(NotImplementedError):
         ops.replace_module_for_quantization(torch.nn.Sequential(torch.nn.LayerNorm(8)), cfg, strict=True)

@@ -274,6 +274,34 @@ def test_rmsnorm_module(ops, K, mode):
     assert mod.iteration == 3
 
 
+@pytest.mark.parametrize("mode", ["ref", "hyc"])
+def test_rmsnorm_gemma_module(ops, K, mode):
+    """y = x * rstd * (1 + w) (efficient_rmsnorm_gemma.py:59,100): the RMSNorm path with fp32(w) + 1, bf16 weight"""
+    B, S, H = 2, 48, 1024
+    gen = torch.Generator().manual_seed(9)
+    mod = ops.EfficientMemoryRMSNormGemma(H, eps=1e-6, bias=False, outlier_ratio=0.01, sub_outlier_ratio=1.0,
+                                          sub_outlier_bit=4, sub_outlier_quantize_method='per-token', rank=0, mode=mode,
+                                          group_size=128).cuda().to(torch.bfloat16)
+    with torch.no_grad():
+        mod.weight.copy_(0.1 * torch.randn(H, generator=gen))
+    for call in range(3):
+        x = torch.randn(B, S, H, generator=gen).bfloat16()
+        dy = (0.02 * torch.randn(B, S, H, generator=gen)).bfloat16()
+        xd = x.cuda().requires_grad_(True)
+        mod.weight.grad = None
+        y = mod(xd)
+        saved = y.grad_fn.saved
+        y.backward(dy.cuda())
+        w1 = mod.weight.detach().cpu().float() + 1.0
+        y_o, rstd_o = O.rmsnorm_fwd(x, w1, 1e-6)
+        assert bf16_ulp_diff(y.detach().cpu(), y_o).max() <= 1
+        xh = (K.decompress_threshold(saved) if mode == "ref" else K.decompress_channel(saved)).cpu().reshape(B, S, H)
+        dx_o, dw_o = O.rmsnorm_bwd(dy, xh, w1, rstd_o)
+        assert torch.allclose(xd.grad.cpu().float(), dx_o.float(), rtol=1e-2, atol=1e-3)
+        assert mod.weight.grad.dtype == torch.bfloat16
+        assert torch.allclose(mod.weight.grad.cpu().float(), dw_o.float(), rtol=1e-2, atol=2e-3)
+
+
 @pytest.mark.parametrize("mode,bits,group", [("ref", 8, 128), ("hyc", 2, 64), ("hyc", 4, 128)])
 def test_linear_module(ops, K, mode, bits, group):
     B, S, H, N = 2, 96, 512, 16
