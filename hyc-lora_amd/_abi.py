@@ -50,6 +50,8 @@ SIGNATURES = {
                                          c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr]),
     "hyc_rmsnorm_bwd": (c_i32, [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_i32, c_ptr, c_i64, c_i64,
                                 ctypes.POINTER(HycDesc), c_i32, c_ptr, c_ptr, c_ptr, c_ptr]),
+    "hyc_layernorm_bwd": (c_i32, [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_i32, c_ptr, c_ptr, c_i64, c_i64,
+                                  ctypes.POINTER(HycDesc), c_ptr, c_ptr, c_ptr, c_ptr]),
     "hyc_act_bwd": (c_i32, [c_i32, c_ptr, c_ptr, c_ptr, c_ptr, c_i64, c_i64, ctypes.POINTER(HycDesc), c_ptr, c_ptr]),
     "hyc_hadamard_bwd": (c_i32, [c_ptr, c_ptr, c_ptr, c_ptr, ctypes.POINTER(HycDesc), c_ptr, c_ptr, c_ptr,
                                  ctypes.POINTER(HycDesc), c_i64, c_i64, c_ptr, c_ptr, c_ptr]),

@@ -168,8 +168,8 @@ template <int BITS, bool WF32, bool QUIRK, int MAXT>
 __global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(4, 8)))
 k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ stored, const uint16_t* __restrict__ vals,
                    const uint16_t* __restrict__ scales, const void* __restrict__ w, const float* __restrict__ rstd,
-                   int64_t M, int64_t H, int T, int CPS, int slots, ChanArgs ca, uint16_t* __restrict__ dx,
-                   float* __restrict__ dw_partials) {
+                   const float* __restrict__ mean, int64_t M, int64_t H, int T, int CPS, int slots, ChanArgs ca,
+                   uint16_t* __restrict__ dx, float* __restrict__ dw_partials) {
   // A thread decodes at most two segments of its packed word: with four segments (2-bit codes) two threads share
   // a word, which keeps the per-thread state (and so the occupancy) the same for every bit width.
   constexpr int NSEG = Q<BITS>::NSEG > 2 ? 2 : Q<BITS>::NSEG;         // segments per thread
@@ -231,12 +231,13 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
   uint4 graw[NSEG];
   uint32_t sc[NSEG];   // one register each: a packed pair would be assembled right after the load and stall on it
   uint32_t o0[NSEG], o1[NSEG];
-  float rs = 0.f;
+  float rs = 0.f, mu = 0.f;                                           // mu: LayerNorm's row mean (0 for RMSNorm)
 #pragma unroll
   for (int i = 0; i < NSEG; ++i) { graw[i] = make_uint4(0, 0, 0, 0); sc[i] = 0; o0[i] = 0; o1[i] = 0; }
   if (row < M && active) {
     pk = *reinterpret_cast<const uint2*>(sq + so);
     rs = rstd[row];
+    if (mean) mu = mean[row];
 #pragma unroll
     for (int i = 0; i < NSEG; ++i) {
       graw[i] = *reinterpret_cast<const uint4*>(gq + i * seg_b + xo);
@@ -249,16 +250,18 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
     const bool valid = row < M && active;
     const bool more = row + stride < M && active;
     uint4 g_n[NSEG];                                                  // the bulk of the next row: requested a row ahead
-    float rs_n = 0.f;
+    float rs_n = 0.f, mu_n = 0.f;
 #pragma unroll
     for (int i = 0; i < NSEG; ++i) g_n[i] = make_uint4(0, 0, 0, 0);
     if (more) {
       rs_n = rstd[row + stride];
+      if (mean) mu_n = mean[row + stride];
 #pragma unroll
       for (int i = 0; i < NSEG; ++i) g_n[i] = *reinterpret_cast<const uint4*>(gq + xstep + i * seg_b + xo);
     }
     float xn[NSEG][8], wdy[NSEG][8];
     float p1 = 0.f, p2 = 0.f;
+    const float nm = -mu * rs;                                        // xn = (x_hat - mean) * rstd as one fma
 #pragma unroll
     for (int i = 0; i < NSEG; ++i) {
       float g[8];
@@ -274,7 +277,7 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
       const float wv[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        const float n = xn[i][j] * rs;
+        const float n = __builtin_fmaf(xn[i][j], rs, nm);
         const float t = wv[j] * g[j];
         xn[i][j] = n;
         wdy[i][j] = t;
@@ -310,7 +313,7 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
         store_stream(reinterpret_cast<uint16_t*>(dq + i * seg_b + xo), pack8(o));
       }
     }
-    rs = rs_n;
+    rs = rs_n; mu = mu_n;
 #pragma unroll
     for (int i = 0; i < NSEG; ++i) graw[i] = g_n[i];
     gq += xstep; dq += xstep; sq += sstep; vq += vstep; cq += gstep;
@@ -464,8 +467,9 @@ template <int BITS, int ITERS, int MAXT, int SRC>
 __global__ void __launch_bounds__(MAXT)
 k_rmsnorm_bwd(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ stored, const uint16_t* __restrict__ vals,
               const uint16_t* __restrict__ scales, const void* __restrict__ w, bool wf32,
-              const float* __restrict__ rstd, int64_t M, int64_t H, int CPS, int T, int slots, int rows_per_block,
-              ChanArgs ca, bool quirk, uint16_t* __restrict__ dx, float* __restrict__ dw_partials) {
+              const float* __restrict__ rstd, const float* __restrict__ mean, int64_t M, int64_t H, int CPS, int T,
+              int slots, int rows_per_block, ChanArgs ca, bool quirk, uint16_t* __restrict__ dx,
+              float* __restrict__ dw_partials) {
   constexpr int NSEG = Q<BITS>::NSEG;
   __shared__ float red[2 * 16 * 16 * 2];
   extern __shared__ __align__(16) float xslot[];                        // [slots-1][T][8] for the final reduction
@@ -536,6 +540,7 @@ k_rmsnorm_bwd(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ store
 
     float xn[ITERS][NSEG][8];
     float p1 = 0.f, p2 = 0.f;
+    const float nm = (mean && valid) ? -mean[row] * rs : 0.f;        // LayerNorm: xn = (x_hat - mean) * rstd as one fma
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
 #pragma unroll
@@ -550,7 +555,7 @@ k_rmsnorm_bwd(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ store
         }
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          const float n = xn[it][i][j] * rs;
+          const float n = __builtin_fmaf(xn[it][i][j], rs, nm);
           const float t = wv[it][i][j] * g[j];
           xn[it][i][j] = n;
           p1 = __builtin_fmaf(n, t, p1);
@@ -811,9 +816,9 @@ int hyc_rmsnorm_fwd_compress(const void* x, const void* w, int32_t w_dtype, floa
   return check_launch("hyc_rmsnorm_fwd_compress");
 }
 
-int hyc_rmsnorm_bwd(const void* dy, const void* stored, const void* vals, const void* scales, const void* w,
-                    int32_t w_dtype, const float* rstd, int64_t M, int64_t H, const hyc_desc* d, int32_t c2_quirk,
-                    void* dx, float* dw_partials, void* dw, void* stream) {
+static int norm_bwd_impl(const void* dy, const void* stored, const void* vals, const void* scales, const void* w,
+                         int32_t w_dtype, const float* rstd, const float* mean, int64_t M, int64_t H, const hyc_desc* d,
+                         int32_t c2_quirk, void* dx, float* dw_partials, void* dw, void* stream) {
   if (!d) return fail(HYC_EFAULT, "hyc_rmsnorm_bwd: null descriptor");
   if (M < 0) return fail(HYC_EINVAL, "hyc_rmsnorm_bwd: M=%lld", (long long)M);
   if (w_dtype != HYC_DTYPE_BF16 && w_dtype != HYC_DTYPE_F32) return fail(HYC_EINVAL, "hyc_rmsnorm_bwd: w_dtype=%d", w_dtype);
@@ -847,7 +852,7 @@ int hyc_rmsnorm_bwd(const void* dy, const void* stored, const void* vals, const 
 #define HYC_BWD_FAST(B_, W_, Q_, MT_)                                                                              \
   hipLaunchKernelGGL((k_rmsnorm_bwd_fast<B_, W_, Q_, MT_>), dim3((unsigned)b.fast_P), dim3(fthreads), flds, st, gp,  \
                      static_cast<const uint8_t*>(stored), static_cast<const uint16_t*>(vals),                     \
-                     static_cast<const uint16_t*>(scales), w, rstd, M, H, b.fast_T, g.cps, b.fast_slots, ca,       \
+                     static_cast<const uint16_t*>(scales), w, rstd, mean, M, H, b.fast_T, g.cps, b.fast_slots, ca, \
                      static_cast<uint16_t*>(dx), dw_partials)
 #define HYC_BWD_FAST_WQ(B_)                                                                   \
   do {                                                                                        \
@@ -874,17 +879,17 @@ int hyc_rmsnorm_bwd(const void* dy, const void* stored, const void* vals, const 
   if (IT == 1 && b.threads <= 256)                                                                                \
     hipLaunchKernelGGL((k_rmsnorm_bwd<B, IT, (IT == 1 ? 256 : 1024), SRC_>), dim3((unsigned)b.P), dim3(b.threads), lds, st, gp, \
                        static_cast<const uint8_t*>(stored), static_cast<const uint16_t*>(vals),                   \
-                       static_cast<const uint16_t*>(scales), w, wf32, rstd, M, H, g.cps, n.T, b.slots, b.rpb, ca, \
+                       static_cast<const uint16_t*>(scales), w, wf32, rstd, mean, M, H, g.cps, n.T, b.slots, b.rpb, ca, \
                        c2_quirk != 0, static_cast<uint16_t*>(dx), dw_partials);                                   \
   else if (IT == 1 && b.threads <= 512)                                                                           \
     hipLaunchKernelGGL((k_rmsnorm_bwd<B, IT, (IT == 1 ? 512 : 1024), SRC_>), dim3((unsigned)b.P), dim3(b.threads), lds, st, gp, \
                        static_cast<const uint8_t*>(stored), static_cast<const uint16_t*>(vals),                   \
-                       static_cast<const uint16_t*>(scales), w, wf32, rstd, M, H, g.cps, n.T, b.slots, b.rpb, ca, \
+                       static_cast<const uint16_t*>(scales), w, wf32, rstd, mean, M, H, g.cps, n.T, b.slots, b.rpb, ca, \
                        c2_quirk != 0, static_cast<uint16_t*>(dx), dw_partials);                                   \
   else                                                                                                            \
   hipLaunchKernelGGL((k_rmsnorm_bwd<B, IT, 1024, SRC_>), dim3((unsigned)b.P), dim3(b.threads), lds, st, gp,       \
                      static_cast<const uint8_t*>(stored), static_cast<const uint16_t*>(vals),                     \
-                     static_cast<const uint16_t*>(scales), w, wf32, rstd, M, H, g.cps, n.T, b.slots, b.rpb, ca,   \
+                     static_cast<const uint16_t*>(scales), w, wf32, rstd, mean, M, H, g.cps, n.T, b.slots, b.rpb, ca, \
                      c2_quirk != 0, static_cast<uint16_t*>(dx), dw_partials)
     if (d->mode == HYC_MODE_CHANNEL) HYC_BITS_ITERS(d->bits, n.iters_t, HYC_BWD(0));
     else HYC_BITS_ITERS(d->bits, n.iters_t, HYC_BWD(2));
@@ -895,6 +900,19 @@ int hyc_rmsnorm_bwd(const void* dy, const void* stored, const void* vals, const 
   if (!dw) return HYC_OK;                        // the caller adds up the partial rows itself
   hipLaunchKernelGGL(k_colsum, dim3((unsigned)((H + 31) / 32)), dim3(256), 0, st, dw_partials, used_P, H, dw, wf32);
   return check_launch("hyc_rmsnorm_bwd (dw)");
+}
+
+int hyc_rmsnorm_bwd(const void* dy, const void* stored, const void* vals, const void* scales, const void* w,
+                    int32_t w_dtype, const float* rstd, int64_t M, int64_t H, const hyc_desc* d, int32_t c2_quirk,
+                    void* dx, float* dw_partials, void* dw, void* stream) {
+  return norm_bwd_impl(dy, stored, vals, scales, w, w_dtype, rstd, nullptr, M, H, d, c2_quirk, dx, dw_partials, dw, stream);
+}
+
+int hyc_layernorm_bwd(const void* dy, const void* stored, const void* vals, const void* scales, const void* w,
+                      int32_t w_dtype, const float* mean, const float* rstd, int64_t M, int64_t H, const hyc_desc* d,
+                      void* dx, float* dw_partials, void* dw, void* stream) {
+  if (M > 0 && !mean) return fail(HYC_EFAULT, "hyc_layernorm_bwd: null mean");
+  return norm_bwd_impl(dy, stored, vals, scales, w, w_dtype, rstd, mean, M, H, d, 1, dx, dw_partials, dw, stream);
 }
 
 }  // extern "C"

@@ -319,6 +319,21 @@ def rmsnorm_bwd(dy2d, src, w, rstd, c2_quirk=True):
     return dx, dw
 
 
+def layernorm_bwd(dy2d, src, w, mean, rstd):
+    """-> (dx bf16 [M,H], dw in w's dtype [H]) with xn = (x_hat - mean) * rstd; db = dy.sum(0) is the caller's"""
+    _need(dy2d, BF16, "dy")
+    M, H = dy2d.shape
+    lib = _abi.load()
+    stored, vals, scales, d = _source(src)
+    P = lib.hyc_rmsnorm_bwd_partials(M, H)
+    partials = torch.empty((max(P, 1), H), dtype=torch.float32, device=dy2d.device)
+    dx = torch.empty_like(dy2d)
+    dw = torch.empty(H, dtype=w.dtype, device=dy2d.device)
+    check(lib.hyc_layernorm_bwd(_p(dy2d), _p(stored), _p(vals), _p(scales), _p(w), _wdtype(w), _p(mean), _p(rstd), M, H,
+                                ctypes.byref(d), _p(dx), _p(partials), _p(dw), _stream()))
+    return dx, dw
+
+
 def rmsnorm_bwd_partial(dy2d, src, w, rstd, c2_quirk=True):
     """-> (dx bf16 [M,H], fp32 partial rows [P,H] whose column sum is dw); the caller does the last reduction"""
     _need(dy2d, BF16, "dy")

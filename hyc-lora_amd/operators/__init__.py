@@ -8,3 +8,4 @@ from .efficient_silu import EfficientMemorySiLU, EfficientMemorySiLUFunc  # noqa
 from .efficient_softmax import EfficientMemorySoftmax, EfficientMemorySoftmaxFunc  # noqa: F401
 from .swap import replace_module_for_quantization  # noqa: F401
 from .efficient_rmsnorm_gemma import EfficientMemoryRMSNormGemma, EfficientMemoryRMSNormGemmaFunc  # noqa: F401
+from .efficient_layernorm import EfficientMemoryLayerNorm, EfficientMemoryLayerNormFunc  # noqa: F401

@@ -3,13 +3,14 @@
 Mirrors `replace_module_for_quantization` of the reference's training scripts (train_gsm8k.py:426-592,
 train_glue.py:391-493): same selection rules, same constructor keywords taken from the same `compress_config`
 sections ("linear", "silu", "layernorm", "softmax", "hadamard"), weights re-pointed, recursion into everything else.
-Module kinds this package does not provide (LayerNorm, Dropout, the attention GEMM wrappers) are
+Module kinds this package does not provide (Dropout, the attention GEMM wrappers) are
 left as they are and reported, or raise with `strict=True`.
 """
 import torch
 
 from .efficient_gelu import EfficientMemoryGELU
 from .efficient_hadamard import EfficientMemoryHadamard
+from .efficient_layernorm import EfficientMemoryLayerNorm
 from .efficient_linear import EfficientMemoryLinear
 from .efficient_rmsnorm import EfficientMemoryRMSNorm
 from .efficient_rmsnorm_gemma import EfficientMemoryRMSNormGemma
@@ -57,7 +58,15 @@ def replace_module_for_quantization(module, compress_config, model_args=None, *,
                                          bias=False, **_knobs(compress_config["layernorm"]), **extra)
             new.weight.data = child.weight.data
             setattr(module, name, new)
-        elif "LayerNorm" in cls or isinstance(child, torch.nn.Dropout) or "GEMM" in cls:
+        elif "LayerNorm" in cls:
+            new = EfficientMemoryLayerNorm(normalized_shape=child.weight.data.shape, elementwise_affine=True,
+                                           bias=child.bias is not None, **_knobs(compress_config["layernorm"]), **extra)
+            new.eps = child.eps                           # (the reference leaves its own default, 1e-5)
+            new.weight.data = child.weight.data
+            if child.bias is not None:
+                new.bias.data = child.bias.data
+            setattr(module, name, new)
+        elif isinstance(child, torch.nn.Dropout) or "GEMM" in cls:
             unsupported(name, child)
         elif isinstance(child, torch.nn.Softmax):
             setattr(module, name, EfficientMemorySoftmax(outlier_ratio=compress_config["softmax"]["outlier_ratio"]))

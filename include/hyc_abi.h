@@ -146,6 +146,13 @@ int hyc_rmsnorm_bwd(const void* dy, const void* stored, const void* vals, const 
                     int32_t w_dtype, const float* rstd, int64_t M, int64_t H, const hyc_desc* d, int32_t c2_quirk,
                     void* dx, float* dw_partials, void* dw, void* stream);
 
+/* LayerNorm backward (efficient_layernorm.py:66-148, 262-330): xn = (xhat - mean)*rstd, dx as above with both
+ * means (c1, c2), dw = sum_m dy*xn.  db = sum_m dy and the forward (mean, rstd, y) are plain reductions / one
+ * library call and are left to the caller; x is compressed with hyc_compress.  Buffers as for hyc_rmsnorm_bwd. */
+int hyc_layernorm_bwd(const void* dy, const void* stored, const void* vals, const void* scales, const void* w,
+                      int32_t w_dtype, const float* mean, const float* rstd, int64_t M, int64_t H, const hyc_desc* d,
+                      void* dx, float* dw_partials, void* dw, void* stream);
+
 /* ---- activation backward ------------------------------------------------------------------- */
 /* dx = act'(xhat) * g evaluated op by op in bf16 as the reference expressions are. */
 int hyc_act_bwd(int32_t act, const void* g, const void* stored, const void* vals, const void* scales, int64_t M,

@@ -351,6 +351,39 @@ def rmsnorm_bwd(dy, x_hat, w, rstd, c2_quirk=True):
 
 
 # --------------------------------------------------------------------------------------
+# LayerNorm                                      operators/efficient_layernorm.py:15-148
+# --------------------------------------------------------------------------------------
+def layernorm_fwd(x, w, b, eps):
+    """two-pass statistics in fp32 (:27-41): mean, var = mean((x-mean)^2), rstd = 1/sqrt(var+eps);
+    y = bf16(((x-mean)*rstd)*w + b) (:55-56).  Returns (y, mean fp32 [M], rstd fp32 [M])."""
+    H = x.shape[-1]
+    xf = x.reshape(-1, H).float()
+    mean = xf.sum(dim=-1) / H
+    xc = xf - mean[:, None]
+    var = (xc * xc).sum(dim=-1) / H
+    rstd = 1.0 / torch.sqrt(var + eps)
+    y = (xc * rstd[:, None]) * w.float()[None, :]
+    if b is not None:
+        y = y + b.float()[None, :]
+    return y.to(x.dtype).reshape(x.shape), mean, rstd
+
+
+def layernorm_bwd(dy, x_hat, w, mean, rstd):
+    """xhat = (x_hat-mean)*rstd; dx = (w*dy - (xhat*c1 + c2))*rstd, c1 = mean(xhat*w*dy), c2 = mean(w*dy) (:113-121);
+    dw = sum_rows dy*xhat, db = sum_rows dy, accumulated in fp32 (the reference sums bf16 partials in lock order,
+    :123-137).  Returns (dx bf16, dw, db in w's dtype)."""
+    H = x_hat.shape[-1]
+    xf = x_hat.reshape(-1, H).float()
+    g = dy.reshape(-1, H).to(BF16).float()
+    xn = (xf - mean[:, None]) * rstd[:, None]
+    wdy = w.float()[None, :] * g
+    c1 = (xn * wdy).sum(dim=-1, keepdim=True) / H
+    c2 = wdy.sum(dim=-1, keepdim=True) / H
+    dx = ((wdy - (xn * c1 + c2)) * rstd[:, None]).to(BF16).reshape(dy.shape)
+    return dx, (g * xn).sum(dim=0).to(w.dtype), g.sum(dim=0).to(w.dtype)
+
+
+# --------------------------------------------------------------------------------------
 # activation / elementwise backward (bf16 op-by-op, as torch evaluates the expressions)
 # --------------------------------------------------------------------------------------
 def silu_bwd(x_hat, g):

@@ -197,5 +197,8 @@ def test_module_swap_follows_the_reference_rules(hyc):
     ops.replace_module_for_quantization(gm, cfg, Args())
     assert isinstance(gm[0].norm, ops.EfficientMemoryRMSNormGemma)
     import pytest
+    ln = torch.nn.Sequential(torch.nn.LayerNorm(128, eps=1e-12))
+    ops.replace_module_for_quantization(ln, cfg)
+    assert isinstance(ln[0], ops.EfficientMemoryLayerNorm) and ln[0].eps == 1e-12
     with pytest.raises(NotImplementedError):
-        ops.replace_module_for_quantization(torch.nn.Sequential(torch.nn.LayerNorm(8)), cfg, strict=True)
+        ops.replace_module_for_quantization(torch.nn.Sequential(torch.nn.Dropout(0.1)), cfg, strict=True)

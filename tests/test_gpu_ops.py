@@ -274,6 +274,37 @@ def test_rmsnorm_module(ops, K, mode):
     assert mod.iteration == 3
 
 
+@pytest.mark.parametrize("mode,H", [("ref", 768), ("hyc", 768), ("hyc", 4096)])
+def test_layernorm_module(ops, K, mode, H):
+    """EfficientMemoryLayerNorm (efficient_layernorm.py:333-405): y, dx, dw, db against the oracle on the activation the
+    backward actually sees"""
+    B, S = 2, 40
+    gen = torch.Generator().manual_seed(13)
+    mod = ops.EfficientMemoryLayerNorm(H, eps=1e-5, outlier_ratio=0.01, sub_outlier_ratio=1.0, sub_outlier_bit=4,
+                                       sub_outlier_quantize_method='per-token', rank=0, mode=mode, group_size=64).cuda()
+    with torch.no_grad():
+        mod.weight.copy_(1 + 0.1 * torch.randn(H, generator=gen))
+        mod.bias.copy_(0.1 * torch.randn(H, generator=gen))
+    for call in range(3):
+        x = (0.5 + torch.randn(B, S, H, generator=gen)).bfloat16()
+        dy = (0.02 * torch.randn(B, S, H, generator=gen)).bfloat16()
+        xd = x.cuda().requires_grad_(True)
+        mod.weight.grad = mod.bias.grad = None
+        y = mod(xd)
+        saved = y.grad_fn.saved
+        y.backward(dy.cuda())
+        w, b = mod.weight.detach().cpu(), mod.bias.detach().cpu()
+        y_o, mean_o, rstd_o = O.layernorm_fwd(x, w, b, 1e-5)
+        # y is the framework's own fused layer norm (it folds mean and rstd into per-row coefficients): a rounding
+        # or two away from the reference's expression order where the terms cancel
+        assert torch.allclose(y.detach().cpu().float(), y_o.float(), rtol=2 ** -6, atol=4e-3)
+        xh = (K.decompress_threshold(saved) if mode == "ref" else K.decompress_channel(saved)).cpu().reshape(B, S, H)
+        dx_o, dw_o, db_o = O.layernorm_bwd(dy, xh, w, mean_o, rstd_o)
+        assert torch.allclose(xd.grad.cpu().float(), dx_o.float(), rtol=1e-2, atol=1e-3)
+        assert torch.allclose(mod.weight.grad.cpu(), dw_o, rtol=1e-2, atol=1e-3)
+        assert torch.allclose(mod.bias.grad.cpu(), db_o, rtol=1e-2, atol=1e-3)
+
+
 @pytest.mark.parametrize("mode", ["ref", "hyc"])
 def test_rmsnorm_gemma_module(ops, K, mode):
     """y = x * rstd * (1 + w) (efficient_rmsnorm_gemma.py:59,100): the RMSNorm path with fp32(w) + 1, bf16 weight"""

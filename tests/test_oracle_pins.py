@@ -274,3 +274,30 @@ def test_low_rank_helpers():
     assert bf16_ulp_diff(O.low_rank_extraction(l, r, x), want.bfloat16()).max() <= 1
     want = (x.double() + (l.double() @ r.double())[None])
     assert bf16_ulp_diff(O.low_rank_addition(l, r, x), want.bfloat16()).max() <= 1
+
+
+def test_layernorm_against_torch_and_autograd():
+    """layernorm_fwd against torch's own layer norm; layernorm_bwd against float64 autograd of the same function
+    evaluated at the (rounded) activation the backward sees"""
+    gen = torch.Generator().manual_seed(21)
+    M, H = 24, 96
+    x = (3 + 2 * torch.randn(M, H, generator=gen)).bfloat16()
+    w = 1 + 0.1 * torch.randn(H, generator=gen)
+    b = 0.1 * torch.randn(H, generator=gen)
+    dy = (0.1 * torch.randn(M, H, generator=gen)).bfloat16()
+    y, mean, rstd = O.layernorm_fwd(x, w, b, 1e-5)
+    ref = torch.nn.functional.layer_norm(x.double(), (H,), w.double(), b.double(), 1e-5)
+    assert torch.allclose(y.double(), ref, rtol=2 ** -7, atol=1e-6)
+    assert torch.allclose(mean.double(), x.double().mean(-1), rtol=1e-6, atol=1e-6)
+    assert torch.allclose(rstd.double(), 1 / torch.sqrt(x.double().var(-1, unbiased=False) + 1e-5), rtol=1e-5)
+    xd = x.double().requires_grad_(True)
+    wd, bd = w.double().requires_grad_(True), b.double().requires_grad_(True)
+    torch.nn.functional.layer_norm(xd, (H,), wd, bd, 1e-5).backward(dy.double())
+    dx, dw, db = O.layernorm_bwd(dy, x, w, mean, rstd)
+    assert torch.allclose(dx.double(), xd.grad, rtol=2 ** -6, atol=1e-4)
+    assert torch.allclose(dw.double(), wd.grad, rtol=1e-4, atol=1e-4)
+    assert torch.allclose(db.double(), bd.grad, rtol=1e-5, atol=1e-5)
+    # a dropped mean term or a swapped c1/c2 must fail: shift invariance of the input
+    y1, _, _ = O.layernorm_fwd(x.float(), w, b, 1e-5)
+    y2, _, _ = O.layernorm_fwd(x.float() + 64, w, b, 1e-5)
+    assert torch.allclose(y2, y1, rtol=1e-3, atol=1e-3)
