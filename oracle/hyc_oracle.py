@@ -27,6 +27,8 @@ Pinning status (see tests/test_oracle_*.py):
                                - golden vectors written by importing the reference
 * rmsnorm_fwd / rmsnorm_bwd    - closed form + torch.autograd (reference kernels are
                                  Triton and cannot run without a GPU)
+* layernorm_fwd / layernorm_bwd - torch's own layer norm + float64 torch.autograd (reference
+                                 kernels are Triton): parity unpinned by reference outputs
 * linear_bwd                   - torch.matmul in fp32
 * hyc_select_channels / hyc group scales - parity unpinned (no reference code)
 """
