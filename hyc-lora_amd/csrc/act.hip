@@ -18,16 +18,6 @@ __device__ __forceinline__ void bfr2(float& a, float& b) {
   a = bf_lo(pk);
   b = bf_hi(pk);
 }
-// e^x to about 2 ulp: v_exp_f32 on x*log2(e) with the rounding error of that product (and the low part of
-// log2(e)) applied as a first-order correction.  Arguments far below the fp32 range give 0, far above give inf.
-__device__ __forceinline__ float exp_fast(float x) {
-  const float L2E = 1.44269502162933349609375f, L2E_LO = 1.925963033500e-08f;
-  const float t = x * L2E;
-  float r = __builtin_fmaf(x, L2E, -t);
-  r = __builtin_fmaf(x, L2E_LO, r);
-  const float e = __builtin_amdgcn_exp2f(t);
-  return __builtin_fmaf(e, r * 0.693147182464599609375f, e);
-}
 // 1 / d for finite positive d to about 1 ulp; 0 for d = inf
 __device__ __forceinline__ float rcp_pos(float d) {
   float r = __builtin_amdgcn_rcpf(d);

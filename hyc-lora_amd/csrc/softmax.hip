@@ -58,6 +58,73 @@ k_softmax_fwd(const uint16_t* __restrict__ x, int64_t rows, int64_t N, float thr
   }
 }
 
+// Rows of up to 4096 entries: one wave per row, the row stays in registers (CPL chunks of 8 per lane), wave-level
+// reductions only (no barrier), exp evaluated once per element, the next row requested before this one is processed.
+template <int CPL>
+__global__ void __launch_bounds__(256)
+k_softmax_fwd_wave(const uint16_t* __restrict__ x, int64_t rows, int64_t N, float thr, uint16_t* __restrict__ y,
+                   int32_t* __restrict__ counts) {
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+  const int nch = (int)(N / 8);
+  const int64_t stride = (int64_t)gridDim.x * 4;
+  int64_t row = (int64_t)blockIdx.x * 4 + wave;
+  bool on[CPL];
+#pragma unroll
+  for (int u = 0; u < CPL; ++u) on[u] = lane + 64 * u < nch;
+  uint4 raw[CPL];
+  if (row < rows) {
+#pragma unroll
+    for (int u = 0; u < CPL; ++u)
+      raw[u] = on[u] ? *reinterpret_cast<const uint4*>(x + row * N + 8 * (lane + 64 * u)) : make_uint4(0, 0, 0, 0);
+  }
+  for (; row < rows; row += stride) {
+    uint4 nxt[CPL];
+    if (row + stride < rows) {
+#pragma unroll
+      for (int u = 0; u < CPL; ++u)
+        nxt[u] = on[u] ? *reinterpret_cast<const uint4*>(x + (row + stride) * N + 8 * (lane + 64 * u)) : make_uint4(0, 0, 0, 0);
+    }
+    float v[CPL][8];
+    float m = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < CPL; ++u) {
+      unpack8(raw[u], v[u]);
+      if (on[u]) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) m = v[u][j] > m ? v[u][j] : m;
+      }
+    }
+    m = group_reduce<64>(m, OpMax());
+    float l = 0.f;
+#pragma unroll
+    for (int u = 0; u < CPL; ++u)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        v[u][j] = on[u] ? exp_fast(v[u][j] - m) : 0.f;
+        l += v[u][j];
+      }
+    l = wave_sum(l);
+    const float inv = 1.0f / l;
+    int kept = 0;
+#pragma unroll
+    for (int u = 0; u < CPL; ++u) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        v[u][j] = bfr(v[u][j] * inv);
+        kept += (v[u][j] > thr) ? 1 : 0;
+      }
+      if (on[u]) store_stream(y + row * N + 8 * (lane + 64 * u), pack8(v[u]));
+    }
+    if (counts) {
+      const float total = wave_sum((float)kept);
+      if (lane == 0) counts[row] = (int32_t)total;
+    }
+#pragma unroll
+    for (int u = 0; u < CPL; ++u) raw[u] = nxt[u];
+  }
+}
+
 // counts only, for probabilities computed elsewhere; one wave per row
 __global__ void __launch_bounds__(256)
 k_softmax_count(const uint16_t* __restrict__ y, int64_t rows, int64_t N, float thr, int32_t* __restrict__ counts) {
@@ -111,6 +178,53 @@ k_softmax_fill(const uint16_t* __restrict__ y, int64_t rows, int64_t N, float th
         cols[pos] = (int32_t)(8 * c + j);
         vals[pos] = f_to_bf(v[j]);
         ++pos;
+      }
+    }
+    running += __shfl(incl, 63, 64);
+  }
+}
+
+// the same for rows of up to 4096 entries with every load of the row issued up front (CPL chunks per lane)
+template <int CPL>
+__global__ void __launch_bounds__(256)
+k_softmax_fill_wave(const uint16_t* __restrict__ y, int64_t rows, int64_t N, float thr, const int32_t* __restrict__ row_ptr,
+                    int32_t* __restrict__ cols, uint16_t* __restrict__ vals) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const uint16_t* yr = y + row * N;
+  const int nch = (int)(N / 8);
+  uint4 raw[CPL];
+#pragma unroll
+  for (int u = 0; u < CPL; ++u)
+    raw[u] = lane + 64 * u < nch ? *reinterpret_cast<const uint4*>(yr + 8 * (lane + 64 * u)) : make_uint4(0, 0, 0, 0);
+  int running = row_ptr[row];
+#pragma unroll
+  for (int u = 0; u < CPL; ++u) {
+    const int c = lane + 64 * u;
+    float v[8];
+    unpack8(raw[u], v);
+    uint32_t m = 0;
+    if (c < nch) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) m |= (v[j] > thr) ? (1u << j) : 0u;
+    }
+    const int cnt = __popc(m);
+    int incl = cnt;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int t = __shfl_up(incl, d, 64);
+      if (lane >= d) incl += t;
+    }
+    int pos = running + incl - cnt;
+    if (m) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        if ((m >> j) & 1u) {
+          cols[pos] = (int32_t)(8 * c + j);
+          vals[pos] = f_to_bf(v[j]);
+          ++pos;
+        }
       }
     }
     running += __shfl(incl, 63, 64);
@@ -172,7 +286,16 @@ int hyc_softmax_fwd(const void* x, int64_t rows, int64_t N, float threshold, voi
   if ((x && !aligned16(x)) || !aligned16(y)) return fail(HYC_EINVAL, "hyc_softmax_fwd: x and y must be 16-byte aligned");
   hipStream_t st = begin_launch(stream);
   const float thr = round_to_bf16(threshold);
-  if (x) {
+  if (x && N <= 4096) {
+    const int cpl = (int)((N / 8 + 63) / 64);             // chunks per lane: 1..8
+    const int64_t blocks = (rows + 3) / 4, cap = 256 * 8;
+    const dim3 grid((unsigned)(blocks < cap ? blocks : cap));
+#define HYC_SMW(C_)                                                                                                \
+  hipLaunchKernelGGL((k_softmax_fwd_wave<C_>), grid, dim3(256), 0, st, static_cast<const uint16_t*>(x), rows, N, thr, \
+                     static_cast<uint16_t*>(y), counts)
+    if (cpl <= 1) HYC_SMW(1); else if (cpl <= 2) HYC_SMW(2); else if (cpl <= 4) HYC_SMW(4); else HYC_SMW(8);
+#undef HYC_SMW
+  } else if (x) {
     const int64_t cap = 256 * 8;
     hipLaunchKernelGGL(k_softmax_fwd, dim3((unsigned)(rows < cap ? rows : cap)), dim3(256), 0, st,
                        static_cast<const uint16_t*>(x), rows, N, thr, static_cast<uint16_t*>(y), counts);
@@ -191,9 +314,18 @@ int hyc_softmax_fill(const void* y, int64_t rows, int64_t N, float threshold, co
   if (rows == 0) return HYC_OK;
   if (!y || !row_ptr) return fail(HYC_EFAULT, "hyc_softmax_fill: null buffer");
   if (!aligned16(y)) return fail(HYC_EINVAL, "hyc_softmax_fill: y must be 16-byte aligned");
-  hipLaunchKernelGGL(k_softmax_fill, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, begin_launch(stream),
-                     static_cast<const uint16_t*>(y), rows, N, round_to_bf16(threshold), row_ptr, cols,
-                     static_cast<uint16_t*>(vals));
+  hipStream_t st = begin_launch(stream);
+  const dim3 grid((unsigned)((rows + 3) / 4));
+  const float thr = round_to_bf16(threshold);
+#define HYC_SMF(C_)                                                                                          \
+  hipLaunchKernelGGL((k_softmax_fill_wave<C_>), grid, dim3(256), 0, st, static_cast<const uint16_t*>(y), rows, N, thr, \
+                     row_ptr, cols, static_cast<uint16_t*>(vals))
+  const int cpl = (int)((N / 8 + 63) / 64);
+  if (cpl <= 1) HYC_SMF(1); else if (cpl <= 2) HYC_SMF(2); else if (cpl <= 4) HYC_SMF(4); else if (cpl <= 8) HYC_SMF(8);
+  else
+    hipLaunchKernelGGL(k_softmax_fill, grid, dim3(256), 0, st, static_cast<const uint16_t*>(y), rows, N, thr, row_ptr,
+                       cols, static_cast<uint16_t*>(vals));
+#undef HYC_SMF
   return check_launch("hyc_softmax_fill");
 }
 

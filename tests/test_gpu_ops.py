@@ -79,7 +79,8 @@ def test_gradw_config3_lora_a(K):
 
 
 # ------------------------------------------------------------------ softmax
-@pytest.mark.parametrize("shape", [(2, 4, 64, 64), (1, 2, 40, 2048), (3, 1, 7, 8)])
+@pytest.mark.parametrize("shape", [(2, 4, 64, 64), (1, 2, 40, 2048), (3, 1, 7, 8), (1, 1, 5, 4096), (1, 2, 9, 1024), (1, 1, 3, 8192),
+                                   (1, 4, 2100, 512), (1, 1, 11, 1096)])
 def test_softmax_kernels(K, shape):
     gen = torch.Generator().manual_seed(sum(shape))
     x = (3 * torch.randn(*shape, generator=gen)).bfloat16()
