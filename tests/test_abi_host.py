@@ -85,6 +85,25 @@ def test_argument_errors_without_a_gpu(abi):
     assert lib.hyc_softmax_fwd(null, 4, 12, 0.0, 0x10, null, null) == abi.ENOTSUP
     assert lib.hyc_low_rank_update(null, null, null, null, 4, 0, 64, 2, 1, null) == abi.EINVAL
     assert lib.hyc_select_channels(null, 4096, 5000, null, null, null) == abi.EINVAL
+    # the entry points added on top of the reference's operator set
+    D = ctypes.byref(d)
+    assert lib.hyc_gated_act_bwd(9, null, null, null, null, D, null, null, null, D, null, null, null, D, 4, 4096, null, null, null) == abi.EINVAL
+    assert lib.hyc_gated_act_bwd(abi.ACT_SILU, null, null, null, null, D, null, null, null, D, null, null, null, ctypes.byref(t),
+                                 4, 4096, null, null, null) == abi.ENOTSUP                                   # not channel-compressed
+    d2 = abi.HycDesc()
+    d2.mode, d2.bits, d2.group, d2.k, d2.chan_plan = abi.MODE_CHANNEL, 2, 64, 0, 0x1000
+    assert lib.hyc_gated_act_bwd(abi.ACT_SILU, null, null, null, null, D, null, null, null, ctypes.byref(d2), null, null, null, D,
+                                 4, 4096, null, null, null) == abi.ENOTSUP                                   # mixed code widths
+    assert lib.hyc_gated_act_bwd(abi.ACT_SILU, null, null, null, null, D, null, null, null, D, null, null, null, D,
+                                 4, 4096, null, null, null) == abi.EFAULT                                    # null buffers
+    assert lib.hyc_gated_act_bwd(abi.ACT_SILU, null, null, null, null, D, null, null, null, D, null, null, null, D,
+                                 0, 4096, null, null, null) == 0                                             # empty input
+    assert lib.hyc_layernorm_bwd(null, null, null, null, null, 0, null, null, 4, 4096, D, null, null, null, null) == abi.EFAULT
+    assert lib.hyc_layernorm_bwd(null, null, null, null, null, 0, null, null, 4, 4096, ctypes.byref(t), null, null, null, null) in (abi.EFAULT, abi.ENOTSUP)
+    assert lib.hyc_rmsnorm_bwd_partial_rows(0, 4096, D) == 0
+    rows = lib.hyc_rmsnorm_bwd_partial_rows(4096, 4096, D)
+    assert 1 <= rows <= lib.hyc_rmsnorm_bwd_partials(4096, 4096)
+    assert lib.hyc_gradw_workspace_bytes(4096, 16, 4096) >= 2 * 16 * 4096 * 4          # the LoRA-A shape splits the tokens
     with pytest.raises(NotImplementedError):
         abi.check(abi.ENOTSUP)
     with pytest.raises(ValueError):
