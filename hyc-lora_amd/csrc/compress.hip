@@ -348,8 +348,7 @@ k_outlier_fill(const uint16_t* __restrict__ x, int64_t M, int64_t H, ThrArgs a, 
 // ---- launch helpers -------------------------------------------------------------------------------
 static inline int row_grid(int64_t M, int threads) {
   // enough workgroups to keep 256 CUs busy with several rows in flight each
-  int per_cu = threads >= 512 ? 3 : 8;
-  if (const char* e = getenv("HYC_TUNE_ROW_GRID")) per_cu = atoi(e);   // tuning knob, not part of the interface
+  const int per_cu = threads >= 512 ? 3 : 8;
   const int64_t cap = (int64_t)256 * per_cu;
   return (int)(M < cap ? M : cap);
 }
