@@ -9,3 +9,6 @@ from .efficient_softmax import EfficientMemorySoftmax, EfficientMemorySoftmaxFun
 from .swap import replace_module_for_quantization  # noqa: F401
 from .efficient_rmsnorm_gemma import EfficientMemoryRMSNormGemma, EfficientMemoryRMSNormGemmaFunc  # noqa: F401
 from .efficient_layernorm import EfficientMemoryLayerNorm, EfficientMemoryLayerNormFunc  # noqa: F401
+from .efficient_gemm import (EfficientMemoryGEMM, EfficientMemoryGEMMFunc, EfficientMemoryGEMMWithSoftmax,  # noqa: F401
+                             EfficientMemoryGEMMWithSoftmaxFunc)
+from ._calibration import calibration_state, load_calibration_state  # noqa: F401

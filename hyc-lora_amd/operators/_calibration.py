@@ -5,7 +5,7 @@ Reference scheme ("ref" mode): `iteration` counts the calls; the first two calls
 (threshold, L, scale, R), compress with them, and fold them into the running mean
 `static = (iteration*static + fresh) / (iteration+1)`; from the third call on the stored values are used.
 `static_value` keeps the reference's order [threshold, L, scale, R].  Like in the reference these are plain
-Python attributes, not buffers.
+Python attributes, not buffers; `calibration_state` / `load_calibration_state` carry them across a restart.
 
 Channel scheme ("hyc" mode): the state is the running per-channel abs-max (elementwise max over the first two
 calls) and the outlier-channel plan selected from it; frozen from the third call on.
@@ -65,3 +65,64 @@ def as_rows(x):
     H = x.shape[-1]
     S = x.shape[-2] if x.dim() >= 2 else 1
     return x.contiguous().reshape(-1, H), S
+
+
+# ---- persistence ------------------------------------------------------------------------------------------
+# The reference keeps `iteration` / `static_value` as plain attributes (efficient_rmsnorm.py:293-294), so a resumed
+# run calibrates again on whatever two batches come first.  These two functions carry the state across a restart
+# without touching `state_dict()` (checkpoints stay loadable by code that knows nothing about it).
+def _site_state(site):
+    if site.plan is None:
+        return None
+    return {"amax": site.amax, "H": site.plan.H, "k": site.plan.k, "idx": site.plan.idx, "plan": site.plan.plan}
+
+
+def calibration_state(model):
+    """{qualified module name: state} for every memory-efficient module below `model` (tensors stay where they are;
+    the result can be handed to torch.save)"""
+    out = {}
+    for name, mod in model.named_modules():
+        if not hasattr(mod, "iteration") or not any(k.startswith("static_value") for k in vars(mod)):
+            continue
+        entry = {"iteration": int(mod.iteration)}
+        for key, val in vars(mod).items():
+            if key.startswith("static_value"):
+                entry[key] = list(val) if isinstance(val, (list, tuple)) else val
+            elif isinstance(val, CompressionSite):
+                entry[key] = _site_state(val)
+        out[name] = entry
+    return out
+
+
+def load_calibration_state(model, state, strict=True):
+    """inverse of calibration_state; tensors are moved to the device of the module's parameters when it has any.
+    Returns the names in `state` that matched no module."""
+    modules = dict(model.named_modules())
+    unknown = []
+    for name, entry in state.items():
+        mod = modules.get(name)
+        if mod is None or not hasattr(mod, "iteration"):
+            unknown.append(name)
+            continue
+        param = next(mod.parameters(), None)
+
+        def place(t):
+            if isinstance(t, torch.Tensor) and param is not None:
+                return t.to(param.device)
+            return t
+
+        for key, val in entry.items():
+            if key == "iteration":
+                mod.iteration = int(val)
+            elif key.startswith("static_value"):
+                setattr(mod, key, [place(v) for v in val] if isinstance(val, (list, tuple)) else place(val))
+            else:
+                site = getattr(mod, key)
+                if val is None:
+                    site.amax, site.plan = None, None
+                else:
+                    site.amax = place(val["amax"])
+                    site.plan = K.ChannelPlan(val["H"], val["k"], place(val["idx"]), place(val["plan"]))
+    if strict and unknown:
+        raise KeyError("no memory-efficient module named %s" % ", ".join(unknown))
+    return unknown

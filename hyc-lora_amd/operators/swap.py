@@ -2,13 +2,14 @@
 
 Mirrors `replace_module_for_quantization` of the reference's training scripts (train_gsm8k.py:426-592,
 train_glue.py:391-493): same selection rules, same constructor keywords taken from the same `compress_config`
-sections ("linear", "silu", "layernorm", "softmax", "hadamard"), weights re-pointed, recursion into everything else.
-Module kinds this package does not provide (Dropout, the attention GEMM wrappers) are
-left as they are and reported, or raise with `strict=True`.
+sections ("linear", "silu", "layernorm", "softmax", "hadamard", "gemm"), weights re-pointed, recursion into
+everything else.  The one module kind this package does not provide (Dropout) is left as it is and reported, or
+raises with `strict=True`.
 """
 import torch
 
 from .efficient_gelu import EfficientMemoryGELU
+from .efficient_gemm import EfficientMemoryGEMM, EfficientMemoryGEMMWithSoftmax
 from .efficient_hadamard import EfficientMemoryHadamard
 from .efficient_layernorm import EfficientMemoryLayerNorm
 from .efficient_linear import EfficientMemoryLinear
@@ -66,8 +67,23 @@ def replace_module_for_quantization(module, compress_config, model_args=None, *,
             if child.bias is not None:
                 new.bias.data = child.bias.data
             setattr(module, name, new)
-        elif isinstance(child, torch.nn.Dropout) or "GEMM" in cls:
+        elif isinstance(child, torch.nn.Dropout):
             unsupported(name, child)
+        elif "GEMM" in cls:
+            gm = compress_config["gemm"]
+            if "gemm1" in name:
+                new = EfficientMemoryGEMM(
+                    outlier_ratio_1=gm["outlier_ratio"], sub_outlier_ratio_1=gm["sub_outlier_ratio"],
+                    sub_outlier_bit_1=gm["sub_outlier_bit"], sub_outlier_quantize_method_1=gm["sub_outlier_quant_method"],
+                    outlier_ratio_2=gm["outlier_ratio"], sub_outlier_ratio_2=gm["sub_outlier_ratio"],
+                    sub_outlier_bit_2=gm["sub_outlier_bit"], sub_outlier_quantize_method_2=gm["sub_outlier_quant_method"],
+                    rank=gm["rank"], **extra)
+            else:
+                new = EfficientMemoryGEMMWithSoftmax(
+                    outlier_ratio_1=compress_config["softmax"]["outlier_ratio"], outlier_ratio_2=gm["outlier_ratio"],
+                    sub_outlier_ratio_2=gm["sub_outlier_ratio"], sub_outlier_bit_2=gm["sub_outlier_bit"],
+                    sub_outlier_quantize_method_2=gm["sub_outlier_quant_method"], rank=gm["rank"], **extra)
+            setattr(module, name, new)
         elif isinstance(child, torch.nn.Softmax):
             setattr(module, name, EfficientMemorySoftmax(outlier_ratio=compress_config["softmax"]["outlier_ratio"]))
         elif "Hadamard" in cls:

@@ -30,6 +30,7 @@ Pinning status (see tests/test_oracle_*.py):
 * layernorm_fwd / layernorm_bwd - torch's own layer norm + float64 torch.autograd (reference
                                  kernels are Triton): parity unpinned by reference outputs
 * linear_bwd                   - torch.matmul in fp32
+* gemm_bwd                     - torch.autograd of torch.matmul in float64
 * hyc_select_channels / hyc group scales - parity unpinned (no reference code)
 """
 import math
@@ -429,3 +430,14 @@ def linear_bwd(dy, x_hat, w, use_bias=False):
     dW_f32 = g2.reshape(-1, out_f).float().t() @ x_hat.reshape(-1, x_hat.shape[-1]).float()
     db = g2.reshape(-1, out_f).float().sum(0).to(w.dtype) if use_bias else None
     return dX, dW_lit, dW_f32, db
+
+
+# --------------------------------------------------------------------------------------
+# attention products                              operators/efficient_gemm.py:64-78, 232-240
+# --------------------------------------------------------------------------------------
+def gemm_bwd(g, x1_hat, x2_hat):
+    """y = x1 @ x2 with both operands restored from their compressed form:
+    d_x1 = g @ x2_hat^T, d_x2 = x1_hat^T @ g (operators/efficient_gemm.py:72-73, 238-239), in fp32 so that the
+    result carries no rounding of its own"""
+    gf = g.float()
+    return gf @ x2_hat.float().transpose(-2, -1), x1_hat.float().transpose(-2, -1) @ gf

@@ -181,10 +181,16 @@ def test_module_swap_follows_the_reference_rules(hyc):
             self.weight = torch.nn.Parameter(torch.ones(h))
             self.variance_epsilon = 1e-6
 
+    class PlainGEMM(torch.nn.Module):
+        def forward(self, a, b):
+            return a @ b
+
     class Block(torch.nn.Module):
         def __init__(self):
             super().__init__()
             self.norm = TinyRMSNorm(128)
+            self.gemm1 = PlainGEMM()
+            self.gemm2 = PlainGEMM()
             self.lora_A = torch.nn.Linear(128, 16, bias=False)
             self.lora_B = torch.nn.Linear(16, 128, bias=False)          # in_features <= 100: untouched
             self.base = torch.nn.Linear(128, 128)
@@ -196,7 +202,7 @@ def test_module_swap_follows_the_reference_rules(hyc):
 
     model = torch.nn.Sequential(Block(), Block())
     cfg = {k: dict(outlier_ratio=0.01, sub_outlier_ratio=1.0, rank=0, sub_outlier_bit=4, sub_outlier_quant_method="per-token")
-           for k in ("linear", "silu", "layernorm", "hadamard")}
+           for k in ("linear", "silu", "layernorm", "hadamard", "gemm")}
     cfg["softmax"] = dict(outlier_ratio=0.05)
     w_before = model[0].lora_A.weight.data_ptr()
     skipped = ops.replace_module_for_quantization(model, cfg, mode="hyc", group_size=64)
@@ -208,6 +214,8 @@ def test_module_swap_follows_the_reference_rules(hyc):
     assert isinstance(b.norm, ops.EfficientMemoryRMSNorm) and b.norm.eps == 1e-6 and b.norm.bias is None
     assert isinstance(b.act_fn, ops.EfficientMemorySiLU) and isinstance(b.softmax, ops.EfficientMemorySoftmax)
     assert b.softmax.outlier_ratio == 0.05
+    assert isinstance(b.gemm1, ops.EfficientMemoryGEMM) and b.gemm1.sub_outlier_bit_2 == 4 and b.gemm1.mode == "hyc"
+    assert isinstance(b.gemm2, ops.EfficientMemoryGEMMWithSoftmax) and b.gemm2.outlier_ratio_1 == 0.05
     assert sorted(skipped) == [("drop", "Dropout"), ("drop", "Dropout")]
 
     class Args:
@@ -221,3 +229,42 @@ def test_module_swap_follows_the_reference_rules(hyc):
     assert isinstance(ln[0], ops.EfficientMemoryLayerNorm) and ln[0].eps == 1e-12
     with pytest.raises(NotImplementedError):
         ops.replace_module_for_quantization(torch.nn.Sequential(torch.nn.Dropout(0.1)), cfg, strict=True)
+
+
+def test_calibration_state_round_trip(hyc, tmp_path):
+    """calibration_state / load_calibration_state: iteration, static values and the channel plan survive torch.save,
+    state_dict() is left alone, unknown names are reported"""
+    import pytest
+    import torch
+    ops = hyc.operators
+    K = hyc.kernels
+
+    def build():
+        return torch.nn.Sequential(ops.EfficientMemorySiLU(0.01, 1.0, 4, "per-token", 0, mode="hyc"),
+                                   ops.EfficientMemorySoftmax(0.05),
+                                   ops.EfficientMemoryHadamard(0.01, 1.0, 4, "per-token", 0.01, 1.0, 4, "per-token", 0),
+                                   torch.nn.Linear(8, 8))
+    src = build()
+    src[0].iteration = 5
+    src[0].site.amax = torch.arange(16, dtype=torch.float32)
+    src[0].site.plan = K.ChannelPlan(16, 1, torch.tensor([15], dtype=torch.int32), torch.tensor([0, 7], dtype=torch.int32))
+    src[1].iteration, src[1].static_value = 2, torch.tensor(0.25)
+    src[2].iteration = 2
+    src[2].static_value_1 = [torch.tensor(1.5), torch.zeros(4, 16).bfloat16(), torch.ones(1, 8).bfloat16(), torch.zeros(16, 8).bfloat16()]
+    state = ops.calibration_state(src)
+    assert sorted(state) == ["0", "1", "2"]
+    assert not any("static" in k or "extra" in k for k in src.state_dict())
+    path = tmp_path / "calib.pt"
+    torch.save(state, path)
+    state = torch.load(path, weights_only=True)
+    dst = build()
+    assert ops.load_calibration_state(dst, state) == []
+    assert dst[0].iteration == 5 and torch.equal(dst[0].site.amax, src[0].site.amax)
+    assert dst[0].site.plan.k == 1 and torch.equal(dst[0].site.plan.idx, src[0].site.plan.idx)
+    assert torch.equal(dst[0].site.plan.plan, src[0].site.plan.plan)
+    assert dst[1].iteration == 2 and float(dst[1].static_value) == 0.25
+    assert torch.equal(dst[2].static_value_1[2], src[2].static_value_1[2]) and dst[2].static_value_2 == [None] * 4
+    assert dst[2].site_1.plan is None
+    with pytest.raises(KeyError):
+        ops.load_calibration_state(dst, {"nope": {"iteration": 1}})
+    assert ops.load_calibration_state(dst, {"nope": {"iteration": 1}}, strict=False) == ["nope"]

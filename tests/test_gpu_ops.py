@@ -379,3 +379,95 @@ def test_gated_act_module_equals_silu_then_hadamard(ops):
         y1.backward(gout)
         y2.backward(gout)
         assert torch.equal(g1.grad, g2.grad) and torch.equal(u1.grad, u2.grad)
+
+
+# ------------------------------------------------------------------ attention products
+def _attention_operands(gen, B, nh, S, hd):
+    q = torch.randn(B, nh, S, hd, generator=gen)
+    k = torch.randn(B, nh, S, hd, generator=gen)
+    q[:, 1, :, 3] *= 12
+    k[:, 0, :, 5] *= 9
+    return q.bfloat16(), k.bfloat16()
+
+
+@pytest.mark.parametrize("mode,bits", [("ref", 4), ("ref", 8), ("hyc", 4), ("hyc", 2)])
+def test_gemm_module(ops, K, mode, bits):
+    """q @ kT: both operands are saved in the [B*S, nh*hd] layout (k through its transpose); the saved codes equal the
+    oracle's for the same statistics and the gradients equal the products with the restored operands"""
+    B, nh, S, hd = 2, 4, 48, 64
+    gen = torch.Generator().manual_seed(31)
+    mod = ops.EfficientMemoryGEMM(0.02, 1.0, bits, 'per-channel', 0.02, 1.0, bits, 'per-token', 0, mode=mode, group_size=64)
+    for call in range(3):
+        q, k = _attention_operands(gen, B, nh, S, hd)
+        g = (0.05 * torch.randn(B, nh, S, S, generator=gen)).bfloat16()
+        qd, ktd = q.cuda().requires_grad_(True), k.cuda().mT.contiguous().requires_grad_(True)
+        y = mod(qd, ktd)
+        assert torch.allclose(y.detach().cpu().float(), q.float() @ k.float().mT, rtol=2e-2, atol=0.3)
+        saved = y.grad_fn.saved
+        y.backward(g.cuda())
+        if mode == "ref":
+            c1, shape1, c2, shape2 = saved
+            assert shape1 == (B, S, nh * hd) and shape2 == (B, S, nh * hd)
+            sv = (mod.static_value_1, mod.static_value_2) if call == 0 else None
+            if sv is not None:                      # first call: the statistics used are the ones stored
+                for c, src, st in ((c1, q, sv[0]), (c2, k, sv[1])):
+                    _, stored_o, _ = O.ref_compress(O.head_to_hidden_shape(src), st[0].cpu(), st[2].cpu(), bits, 1.0, st[1].cpu(), st[3].cpu())
+                    assert torch.equal(c.stored.cpu().reshape(stored_o.shape).view(torch.uint8), stored_o.view(torch.uint8))
+            qh = K.decompress_threshold(c1).cpu().reshape(B, S, nh * hd)
+            kh = K.decompress_threshold(c2).cpu().reshape(B, S, nh * hd)
+        else:
+            qh = K.decompress_channel(saved[0]).cpu().reshape(B, S, nh * hd)
+            kh = K.decompress_channel(saved[1]).cpu().reshape(B, S, nh * hd)
+        qh, kh = O.hidden_to_head_shape(qh, nh), O.hidden_to_head_shape(kh, nh)
+        assert (qh.float() - q.float()).abs().max() < (2.0 if bits == 2 else 1.0)
+        d1, d2 = O.gemm_bwd(g, qh, kh.mT)
+        assert torch.allclose(qd.grad.cpu().float(), d1, rtol=1e-2, atol=1e-3 + 4e-3 * float(d1.abs().max()))
+        assert torch.allclose(ktd.grad.cpu().float(), d2, rtol=1e-2, atol=1e-3 + 4e-3 * float(d2.abs().max()))
+        assert mod.iteration == call + 1
+
+
+@pytest.mark.parametrize("mode", ["ref", "hyc"])
+def test_gemm_with_softmax_module(ops, K, mode):
+    """p @ v: p keeps the entries above the calibrated threshold (same set as the oracle's), v is saved as codes"""
+    B, nh, S, hd = 2, 4, 40, 64
+    gen = torch.Generator().manual_seed(32)
+    mod = ops.EfficientMemoryGEMMWithSoftmax(0.1, 0.02, 1.0, 4, 'per-channel', 0, mode=mode, group_size=64)
+    for call in range(3):
+        p = torch.softmax(2 * torch.randn(B, nh, S, S, generator=gen), -1).bfloat16()
+        v = torch.randn(B, nh, S, hd, generator=gen).bfloat16()
+        g = (0.05 * torch.randn(B, nh, S, hd, generator=gen)).bfloat16()
+        pd, vd = p.cuda().requires_grad_(True), v.cuda().requires_grad_(True)
+        y = mod(pd, vd)
+        assert torch.allclose(y.detach().cpu().float(), p.float() @ v.float(), rtol=2e-2, atol=2e-2)
+        fn = y.grad_fn
+        y.backward(g.cuda())
+        thr = O.get_statistics_softmax(p, call, 0.1) if call < 2 else mod.static_value_1.cpu()
+        ph = K.softmax_dense(fn.sparse).cpu()
+        assert bits_equal(ph, O.prune_softmax(p, thr))
+        c2 = fn.saved[0] if mode == "ref" else fn.saved
+        vh = (K.decompress_threshold(c2) if mode == "ref" else K.decompress_channel(c2)).cpu().reshape(B, S, nh * hd)
+        vh = O.hidden_to_head_shape(vh, nh)
+        d1, d2 = O.gemm_bwd(g, ph, vh)
+        assert torch.allclose(pd.grad.cpu().float(), d1, rtol=1e-2, atol=1e-3 + 4e-3 * float(d1.abs().max()))
+        assert torch.allclose(vd.grad.cpu().float(), d2, rtol=1e-2, atol=1e-3 + 4e-3 * float(d2.abs().max()))
+    assert mod.iteration == 3 and mod.static_value_1 is not None
+
+
+@pytest.mark.parametrize("mode", ["ref", "hyc"])
+def test_calibration_state_resume(ops, mode):
+    """a module restored with load_calibration_state continues exactly like the one that was calibrated"""
+    gen = torch.Generator().manual_seed(41)
+    kw = dict(outlier_ratio=0.02, sub_outlier_ratio=1.0, sub_outlier_bit=4, sub_outlier_quantize_method="per-channel", rank=0)
+    a = torch.nn.Sequential(ops.EfficientMemorySiLU(mode=mode, group_size=64, **kw))
+    xs = [torch.randn(2, 32, 512, generator=gen).bfloat16().cuda() for _ in range(3)]
+    for x in xs[:2]:
+        a(x.clone().requires_grad_(True))
+    b = torch.nn.Sequential(ops.EfficientMemorySiLU(mode=mode, group_size=64, **kw))
+    ops.load_calibration_state(b, ops.calibration_state(a))
+    g = torch.ones_like(xs[2])
+    grads = []
+    for m in (a, b):
+        x = xs[2].clone().requires_grad_(True)
+        m(x).backward(g)
+        grads.append(x.grad)
+    assert torch.equal(grads[0], grads[1]) and b[0].iteration == 3

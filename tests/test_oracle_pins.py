@@ -301,3 +301,18 @@ def test_layernorm_against_torch_and_autograd():
     y1, _, _ = O.layernorm_fwd(x.float(), w, b, 1e-5)
     y2, _, _ = O.layernorm_fwd(x.float() + 64, w, b, 1e-5)
     assert torch.allclose(y2, y1, rtol=1e-3, atol=1e-3)
+
+
+def test_gemm_bwd_autograd():
+    """gemm_bwd against float64 autograd of a batched matmul with non-square operands, so that a transposed operand
+    or swapped outputs cannot pass"""
+    gen = torch.Generator().manual_seed(8)
+    x1 = torch.randn(2, 3, 10, 6, generator=gen).bfloat16()
+    x2 = torch.randn(2, 3, 6, 14, generator=gen).bfloat16()
+    g = (0.1 * torch.randn(2, 3, 10, 14, generator=gen)).bfloat16()
+    a, b = x1.double().requires_grad_(True), x2.double().requires_grad_(True)
+    (a @ b).backward(g.double())
+    d1, d2 = O.gemm_bwd(g, x1, x2)
+    assert d1.shape == x1.shape and d2.shape == x2.shape
+    assert torch.allclose(d1.double(), a.grad, rtol=1e-5, atol=1e-6)
+    assert torch.allclose(d2.double(), b.grad, rtol=1e-5, atol=1e-6)
