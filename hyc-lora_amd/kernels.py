@@ -539,3 +539,34 @@ def low_rank_update(l, r, x, subtract, out=None):
         out = torch.empty_like(x)
     check(_abi.load().hyc_low_rank_update(_p(l), _p(r), _p(x), _p(out), M, S, H, l.shape[1], 1 if subtract else 0, _stream()))
     return out
+
+
+# ----------------------------------------------------------------------------------------------------
+# NF4 frozen base weights
+# ----------------------------------------------------------------------------------------------------
+@dataclass
+class NF4Weight:
+    """a frozen [out, in] bf16 weight held as 4-bit level indices + one fp32 abs-max per 64 consecutive weights"""
+    packed: torch.Tensor   # uint8 [out*in/2]
+    absmax: torch.Tensor   # fp32 [out*in/64]
+    shape: tuple
+
+    def nbytes(self):
+        return self.packed.numel() + 4 * self.absmax.numel()
+
+
+def nf4_quantize(w):
+    _need(w, BF16, "w")
+    n = w.numel()
+    packed = torch.empty(n // 2, dtype=torch.uint8, device=w.device)
+    absmax = torch.empty(n // 64, dtype=torch.float32, device=w.device)
+    check(_abi.load().hyc_nf4_quantize(_p(w), n, _p(packed), _p(absmax), _stream()))
+    return NF4Weight(packed, absmax, tuple(w.shape))
+
+
+def nf4_dequantize(q: NF4Weight, out=None):
+    n = q.packed.numel() * 2
+    if out is None:
+        out = torch.empty(q.shape, dtype=BF16, device=q.packed.device)
+    check(_abi.load().hyc_nf4_dequantize(_p(q.packed), _p(q.absmax), n, _p(out), _stream()))
+    return out

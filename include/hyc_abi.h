@@ -32,6 +32,9 @@
  *       grad_weight = grad_output^T @ decompress(x), operators/efficient_linear.py:56-67
  *   hyc_low_rank_update
  *       low_rank_extraction / low_rank_addition, operators/fused_compression.py:80-99, :184-210
+ *   hyc_nf4_dequantize / hyc_nf4_quantize
+ *       F.dequantize_4bit(B, quant_state) before each frozen-base matmul, bitsandbytes_fix/_function.py:509, :540
+ *       (the quantiser that wrote B is bitsandbytes' own and is not part of the reference tree)
  *
  * Compressed activation of a [M, H] bf16 matrix (M tokens, H channels), `bits` in {1,2,4,8}:
  *   stored   uint8 [M, H*bits/8]   (bits == 8: int8 [M, H], the signed code itself)
@@ -198,6 +201,14 @@ int hyc_gradw_gemm(const void* dy, int64_t ldy, const void* stored, const void* 
 /* out[m, :] = bf16(x[m, :] -/+ L[m mod S, :] @ R); L bf16 [S, rank], R bf16 [rank, H]; out may alias x */
 int hyc_low_rank_update(const void* L, const void* R, const void* x, void* out, int64_t M, int64_t S, int64_t H,
                         int32_t rank, int32_t subtract, void* stream);
+
+/* ---- NF4 frozen base weights ------------------------------------------------------------------- */
+/* Blocks of 64 consecutive weights: absmax[i] = max |w| of block i (fp32), packed byte j holds the level indices of
+ * weights 2j (high nibble) and 2j+1 (low nibble); level index = nearest of the 16 NormalFloat4 levels to w / absmax.
+ * n = number of weights, a multiple of 64.  w / out bf16 [n], packed uint8 [n/2], absmax fp32 [n/64].
+ * out = bf16(level * absmax). */
+int hyc_nf4_quantize(const void* w, int64_t n, void* packed, float* absmax, void* stream);
+int hyc_nf4_dequantize(const void* packed, const float* absmax, int64_t n, void* out, void* stream);
 
 #ifdef __cplusplus
 }

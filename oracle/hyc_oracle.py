@@ -32,6 +32,8 @@ Pinning status (see tests/test_oracle_*.py):
 * linear_bwd                   - torch.matmul in fp32
 * gemm_bwd                     - torch.autograd of torch.matmul in float64
 * hyc_select_channels / hyc group scales - parity unpinned (no reference code)
+* nf4_quantize / nf4_dequantize - parity unpinned (bitsandbytes is not in the reference tree); checked against
+                                 the published level table: nearest level by exact distance, round trips
 """
 import math
 
@@ -441,3 +443,32 @@ def gemm_bwd(g, x1_hat, x2_hat):
     result carries no rounding of its own"""
     gf = g.float()
     return gf @ x2_hat.float().transpose(-2, -1), x1_hat.float().transpose(-2, -1) @ gf
+
+
+# --------------------------------------------------------------------------------------
+# NF4 frozen base weights           call sites: bitsandbytes_fix/_function.py:509, :540
+# --------------------------------------------------------------------------------------
+# bitsandbytes (unpinned fork, README.md:37-49) is neither vendored by the reference nor installed, so this is a
+# restatement of its published NF4 block format: PARITY UNPINNED by reference outputs.
+NF4_LEVELS = torch.tensor([
+    -1.0, -0.6961928009986877, -0.5250730514526367, -0.39491748809814453, -0.28444138169288635,
+    -0.18477343022823334, -0.09105003625154495, 0.0, 0.07958029955625534, 0.16093020141124725,
+    0.24611230194568634, 0.33791524171829224, 0.44070982933044434, 0.5626170039176941, 0.7229568362236023,
+    1.0], dtype=torch.float32)
+
+
+def nf4_quantize(w, block=64):
+    """-> (packed uint8 [n/2], absmax fp32 [n/block]).  v = w * (1/absmax) in fp32; level index = number of
+    midpoints between neighbouring levels strictly below v; first weight of a pair in the high nibble."""
+    flat = w.float().reshape(-1, block)
+    absmax = flat.abs().amax(dim=1)
+    inv = torch.where(absmax > 0, 1.0 / absmax, torch.zeros_like(absmax))
+    v = flat * inv[:, None]
+    mids = 0.5 * (NF4_LEVELS[:-1] + NF4_LEVELS[1:])
+    codes = (v[..., None] > mids).sum(-1).to(torch.uint8).reshape(-1, 2)
+    return (codes[:, 0] << 4) | codes[:, 1], absmax
+
+
+def nf4_dequantize(packed, absmax, shape, block=64):
+    codes = torch.stack([packed >> 4, packed & 15], dim=1).reshape(-1, block).long()
+    return (NF4_LEVELS[codes] * absmax[:, None]).to(BF16).reshape(shape)

@@ -84,6 +84,11 @@ def test_argument_errors_without_a_gpu(abi):
     assert lib.hyc_gradw_gemm(null, 20, null, null, null, 4, 20, 4096, ctypes.byref(d), 1.0, 0.0, 0x10, 0, null, null) == abi.ENOTSUP
     assert lib.hyc_softmax_fwd(null, 4, 12, 0.0, 0x10, null, null) == abi.ENOTSUP
     assert lib.hyc_low_rank_update(null, null, null, null, 4, 0, 64, 2, 1, null) == abi.EINVAL
+    assert lib.hyc_nf4_quantize(null, 100, null, null, null) == abi.EINVAL            # not a multiple of 64
+    assert lib.hyc_nf4_quantize(null, 0, null, null, null) == 0
+    assert lib.hyc_nf4_quantize(null, 128, null, null, null) == abi.EFAULT
+    assert lib.hyc_nf4_dequantize(null, null, -64, null, null) == abi.EINVAL
+    assert lib.hyc_nf4_dequantize(null, null, 64, null, null) == abi.EFAULT
     assert lib.hyc_select_channels(null, 4096, 5000, null, null, null) == abi.EINVAL
     # the entry points added on top of the reference's operator set
     D = ctypes.byref(d)
@@ -157,6 +162,13 @@ def test_module_constructors_mirror_the_reference(hyc):
     assert s.static_value is None and s.outlier_ratio == 0.05
     h = ops.EfficientMemoryHadamard()
     assert h.static_value_1 == [None] * 4 and h.sub_outlier_bit_2 == 8
+    g1 = ops.EfficientMemoryGEMM(outlier_ratio_1=0.01, sub_outlier_ratio_1=0.2, sub_outlier_bit_1=8,
+                                 sub_outlier_quantize_method_1='per-tensor', outlier_ratio_2=0.01, sub_outlier_ratio_2=0.2,
+                                 sub_outlier_bit_2=4, sub_outlier_quantize_method_2='per-tensor', rank=16)
+    assert g1.static_value_1 == [None] * 4 and g1.static_value_2 == [None] * 4 and g1.sub_outlier_bit_2 == 4
+    g2 = ops.EfficientMemoryGEMMWithSoftmax(outlier_ratio_1=0.05, outlier_ratio_2=0.01, sub_outlier_ratio_2=0.2,
+                                            sub_outlier_bit_2=8, sub_outlier_quantize_method_2='per-tensor', rank=16)
+    assert g2.static_value_1 is None and g2.static_value_2 == [None] * 4 and g2.iteration == 0
     with pytest.raises(ValueError):
         ops.EfficientMemorySiLU(mode="bogus")
     cf = ops.compress_function

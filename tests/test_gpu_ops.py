@@ -471,3 +471,20 @@ def test_calibration_state_resume(ops, mode):
         m(x).backward(g)
         grads.append(x.grad)
     assert torch.equal(grads[0], grads[1]) and b[0].iteration == 3
+
+
+# ------------------------------------------------------------------ NF4 frozen base
+@pytest.mark.parametrize("shape", [(64,), (128, 192), (4096, 512)])
+def test_nf4_kernels(K, shape):
+    """level indices, packed bytes and abs-max bit-exact against the oracle; dequantised weights bit-exact"""
+    gen = torch.Generator().manual_seed(13)
+    w = (0.02 * torch.randn(*shape, generator=gen)).bfloat16()
+    w.view(-1)[5] = 0.25                                 # an extreme value
+    w.view(-1)[64 * (w.numel() // 64 - 1):] = 0          # an all-zero block
+    q = K.nf4_quantize(w.cuda())
+    packed_o, absmax_o = O.nf4_quantize(w)
+    assert torch.equal(q.absmax.cpu(), absmax_o)
+    assert torch.equal(q.packed.cpu(), packed_o)
+    back = K.nf4_dequantize(q)
+    assert back.shape == w.shape and bits_equal(back.cpu(), O.nf4_dequantize(packed_o, absmax_o, w.shape))
+    assert q.nbytes() == w.numel() // 2 + 4 * (w.numel() // 64)

@@ -316,3 +316,32 @@ def test_gemm_bwd_autograd():
     assert d1.shape == x1.shape and d2.shape == x2.shape
     assert torch.allclose(d1.double(), a.grad, rtol=1e-5, atol=1e-6)
     assert torch.allclose(d2.double(), b.grad, rtol=1e-5, atol=1e-6)
+
+
+def test_nf4_nearest_level_and_round_trip():
+    """the NF4 restatement against what the published format fixes: every weight maps to the level nearest to
+    w / absmax (exact float64 distances), a block's extreme weight maps to +-1 and comes back exactly, levels times a
+    power-of-two absmax round-trip exactly, the first weight of a pair sits in the high nibble"""
+    gen = torch.Generator().manual_seed(12)
+    w = (0.02 * torch.randn(64 * 50, generator=gen)).bfloat16()
+    packed, absmax = O.nf4_quantize(w)
+    assert packed.dtype == torch.uint8 and packed.numel() == w.numel() // 2 and absmax.numel() == 50
+    codes = torch.stack([packed >> 4, packed & 15], 1).reshape(-1).long()
+    v = (w.double().reshape(-1, 64) / absmax.double()[:, None]).reshape(-1)
+    dist = (v[:, None] - O.NF4_LEVELS.double()[None]).abs()
+    best = dist.argmin(1)
+    margin = dist.gather(1, codes[:, None])[:, 0] - dist.min(1).values
+    assert bool((margin < 1e-6).all()) and float((codes == best).float().mean()) > 0.999
+    back = O.nf4_dequantize(packed, absmax, w.shape)
+    assert float((back.float() - w.float()).abs().max()) <= 0.16 * float(absmax.max())     # half the widest gap
+    blk = w.float().reshape(-1, 64)
+    top = blk.abs().argmax(1)
+    assert torch.equal(back.float().reshape(-1, 64).gather(1, top[:, None]), blk.gather(1, top[:, None]))
+    exact = (O.NF4_LEVELS.repeat(4) * 0.5).bfloat16()            # 64 weights; not all levels are bf16 numbers
+    p2, a2 = O.nf4_quantize(exact)
+    assert float(a2[0]) == 0.5
+    assert torch.equal(torch.stack([p2 >> 4, p2 & 15], 1).reshape(-1).long(), torch.arange(16).repeat(4))
+    one = torch.zeros(64).bfloat16()
+    one[0] = 1.0
+    p3, _ = O.nf4_quantize(one)
+    assert int(p3[0]) == (15 << 4) | 7 and int(p3[1]) == (7 << 4) | 7
