@@ -293,7 +293,8 @@ __device__ __forceinline__ uint4 dequant8_fast(uint32_t lo, uint32_t hi, int seg
 }
 
 // e^x to about 2 ulp: v_exp_f32 on x*log2(e) with the rounding error of that product (and the low part of
-// log2(e)) applied as a first-order correction.  Arguments far below the fp32 range give 0, far above give inf.
+// log2(e)) applied as a first-order correction.  |x| must stay below 2^127 / log2(e) (about 2.3e38): beyond that
+// the product overflows and the correction term becomes inf * 0.
 __device__ __forceinline__ float exp_fast(float x) {
   const float L2E = 1.44269502162933349609375f, L2E_LO = 1.925963033500e-08f;
   const float t = x * L2E;

@@ -101,7 +101,8 @@ k_softmax_fwd_wave(const uint16_t* __restrict__ x, int64_t rows, int64_t N, floa
     for (int u = 0; u < CPL; ++u)
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        v[u][j] = on[u] ? exp_fast(v[u][j] - m) : 0.f;
+        // the clamp keeps x*log2(e) finite for mask values near the bottom of the bf16 range (e^-128 is 0 in fp32)
+        v[u][j] = on[u] ? exp_fast(fmaxf(v[u][j] - m, -128.f)) : 0.f;
         l += v[u][j];
       }
     l = wave_sum(l);

@@ -1,0 +1,317 @@
+"""One LLaMA-shaped decoder layer with a 4-bit NF4 frozen base, LoRA on all seven projections and every saved
+activation compressed: the harness for the full-layer configuration (peak activation memory and step time).
+
+What the reference assembles by swapping modules inside models/modeling_llama.py (attention :382-484, MLP
+:263-295) with peft LoRA around a bitsandbytes 4-bit base (bitsandbytes_fix/_function.py:509-540) is built here
+directly from this package's operators, with the savings a hand-assembled layer allows:
+
+* q/k/v (and gate/up) LoRA-A inputs are the same tensor: it is compressed once, not once per projection;
+* the attention probabilities are kept once (the reference keeps them in the softmax module and again in the
+  p @ v wrapper, efficient_gemm.py:222);
+* the frozen base saves nothing (as in the reference): W is dequantised again in the backward.
+
+Composite of one LoRA projection (peft `Linear.forward` around the swapped modules):
+    y  = x @ W^T + s * (x @ A^T) @ B^T          h = x @ A^T is kept exactly ([M, r])
+    dX = dY @ W + (s * dY @ B) @ A
+    dB = s * dY^T @ h
+    dA = (s * dY @ B)^T @ x_hat                 the only consumer of the compressed x (efficient_linear.py:56-67)
+"""
+import math
+from dataclasses import dataclass
+
+import torch
+
+from . import kernels as K
+from .operators._calibration import CompressionSite
+from .operators.compress_function import get_statistics_softmax
+from .operators.efficient_hadamard import EfficientMemoryGatedAct
+from .operators.efficient_rmsnorm import EfficientMemoryRMSNorm
+
+BF16 = torch.bfloat16
+
+
+@dataclass
+class LayerConfig:
+    hidden: int = 4096
+    heads: int = 32
+    head_dim: int = 128
+    intermediate: int = 11008
+    rope_theta: float = 10000.0
+    rms_eps: float = 1e-5
+    lora_r: int = 16
+    lora_alpha: float = 32.0
+    outlier_ratio: float = 0.01      # fraction of channels kept in bf16 at every compressed site
+    softmax_ratio: float = 0.01      # fraction of attention probabilities kept
+    linear_bits: int = 2             # LoRA-A inputs
+    linear_group: int = 64
+    act_bits: int = 4                # norm inputs, q / k / v, gate / act(gate) / up
+    act_group: int = 128
+    compress: bool = True            # False: the same functions keep their activations in bf16 (formula check)
+
+
+# ---- frozen base + LoRA -----------------------------------------------------------------------------------
+class LoRAProjections(torch.nn.Module):
+    """n projections of one input: frozen NF4 base W_i [out_i, in] plus trainable A_i [r, in], B_i [out_i, r]"""
+
+    def __init__(self, in_features, out_features, cfg: LayerConfig, device):
+        super().__init__()
+        gen = torch.Generator(device="cpu").manual_seed(in_features * 31 + sum(out_features))
+        self.in_features, self.out_features = in_features, list(out_features)
+        self.scaling = cfg.lora_alpha / cfg.lora_r
+        self.cfg = cfg
+        self.base = []
+        self.lora_A = torch.nn.ParameterList()
+        self.lora_B = torch.nn.ParameterList()
+        for out in self.out_features:
+            w = (0.02 * torch.randn(out, in_features, generator=gen)).to(BF16).to(device)
+            self.base.append(K.nf4_quantize(w))
+            a = torch.empty(cfg.lora_r, in_features)
+            torch.nn.init.kaiming_uniform_(a, a=math.sqrt(5), generator=gen)
+            self.lora_A.append(torch.nn.Parameter(a.to(BF16).to(device)))
+            # peft starts B at zero; a small random B keeps every gradient of the harness non-trivial
+            self.lora_B.append(torch.nn.Parameter((0.02 * torch.randn(out, cfg.lora_r, generator=gen)).to(BF16).to(device)))
+        self.site = CompressionSite(cfg.outlier_ratio, 1.0, cfg.linear_bits, "per-token", 0, "hyc", cfg.linear_group)
+        self.iteration = 0
+        self.record = None
+
+    def forward(self, x):
+        x2 = x.reshape(-1, self.in_features)
+        plan = self.site.channel_plan(x2, self.iteration) if self.cfg.compress else None
+        self.iteration += 1
+        n = len(self.out_features)
+        outs = _LoRAProjectionsFunc.apply(x, self, plan, *self.lora_A, *self.lora_B)
+        return outs if n > 1 else outs[0]
+
+
+class _LoRAProjectionsFunc(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, mod, plan, *ab):
+        n = len(mod.out_features)
+        A, B = ab[:n], ab[n:]
+        x2 = x.reshape(-1, mod.in_features)
+        if not x2.is_contiguous():
+            x2 = x2.contiguous()
+        s = mod.scaling
+        outs, hs = [], []
+        wbuf = None
+        for i in range(n):
+            wbuf = K.nf4_dequantize(mod.base[i], out=wbuf if wbuf is not None and wbuf.shape == mod.base[i].shape else None)
+            y = x2 @ wbuf.t()
+            h = x2 @ A[i].t()
+            y.addmm_(h, B[i].t(), alpha=s)
+            outs.append(y.reshape(x.shape[:-1] + (mod.out_features[i],)))
+            hs.append(h)
+        del wbuf
+        cfg = mod.cfg
+        ctx.saved_x = K.compress_channel(x2, plan, cfg.linear_bits, cfg.linear_group) if cfg.compress else x2
+        if mod.record is not None:
+            mod.record["x"], mod.record["saved"] = x2.detach().clone(), ctx.saved_x
+        ctx.mod, ctx.hs = mod, hs
+        ctx.save_for_backward(*ab)
+        return tuple(outs)
+
+    @staticmethod
+    def backward(ctx, *gs):
+        mod = ctx.mod
+        n = len(mod.out_features)
+        ab = ctx.saved_tensors
+        A, B = ab[:n], ab[n:]
+        s = mod.scaling
+        dx = None
+        dA, dB = [], []
+        wbuf = None
+        for i in range(n):
+            g = gs[i].reshape(-1, mod.out_features[i]).to(BF16)
+            if not g.is_contiguous():
+                g = g.contiguous()
+            wbuf = K.nf4_dequantize(mod.base[i], out=wbuf if wbuf is not None and wbuf.shape == mod.base[i].shape else None)
+            dx = g @ wbuf if dx is None else dx.addmm_(g, wbuf)
+            dh = (g @ B[i]) * s                                  # [M, r]
+            dx.addmm_(dh, A[i])
+            dB.append((g.t() @ ctx.hs[i]) * s)
+            dA.append(K.gradw_gemm(dh, ctx.saved_x, out_dtype=A[i].dtype))
+        ctx.hs = None
+        ctx.saved_x = None
+        return (dx.reshape(gs[0].shape[:-1] + (mod.in_features,)), None, None) + tuple(dA) + tuple(dB)
+
+
+# ---- attention -----------------------------------------------------------------------------------------------
+def rope_tables(S, head_dim, theta, device):
+    inv = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.float32, device=device) / head_dim))
+    freqs = torch.outer(torch.arange(S, dtype=torch.float32, device=device), inv)
+    emb = torch.cat((freqs, freqs), dim=-1)
+    return emb.cos().to(BF16), emb.sin().to(BF16)
+
+
+def rotate_half(x):
+    half = x.shape[-1] // 2
+    return torch.cat((-x[..., half:], x[..., :half]), dim=-1)
+
+
+def apply_rope(x, cos, sin):
+    """x [B, nh, S, hd]; cos / sin [S, hd] (models/modeling_llama.py:236-260)"""
+    return x * cos + rotate_half(x) * sin
+
+
+class CompressedAttention(torch.nn.Module):
+    """softmax(q @ k^T / sqrt(hd) + causal mask) @ v with q, k, v saved as codes in the [B*S, nh*hd] layout and the
+    probabilities saved once as the entries above a calibrated threshold.  Composition of the reference's gemm1,
+    softmax and gemm2 modules (models/modeling_llama.py:444-462, operators/efficient_gemm.py,
+    operators/efficient_softmax.py)."""
+
+    def __init__(self, cfg: LayerConfig):
+        super().__init__()
+        self.cfg = cfg
+        mk = lambda: CompressionSite(cfg.outlier_ratio, 1.0, cfg.act_bits, "per-token", 0, "hyc", cfg.act_group)
+        self.site_q, self.site_k, self.site_v = mk(), mk(), mk()
+        self.iteration = 0
+        self.static_value = None          # probability threshold, as in EfficientMemorySoftmax
+        self.record = None
+
+    def forward(self, q, k, v):
+        return _AttentionFunc.apply(q, k, v, self)
+
+
+def _heads_to_rows(x):
+    b, nh, s, hd = x.shape
+    return x.transpose(1, 2).reshape(b * s, nh * hd)
+
+
+def _rows_to_heads(x2d, b, nh, s, hd):
+    return x2d.reshape(b, s, nh, hd).transpose(1, 2)
+
+
+class _AttentionFunc(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, mod):
+        cfg = mod.cfg
+        b, nh, s, hd = q.shape
+        scale = 1.0 / math.sqrt(hd)
+        scores = q @ k.transpose(-2, -1)
+        scores.mul_(scale)
+        causal = torch.ones(s, s, dtype=torch.bool, device=q.device).triu_(1)
+        scores.masked_fill_(causal, torch.finfo(BF16).min)       # the additive mask of the reference, saturated
+        it = mod.iteration
+        if cfg.compress and it >= 2:
+            p, sparse = K.softmax_fwd(scores, float(mod.static_value))
+        else:
+            p, _ = K.softmax_fwd(scores)
+            if cfg.compress:
+                thr = get_statistics_softmax(p, it, cfg.softmax_ratio)
+                mod.static_value = thr if mod.static_value is None else (it * mod.static_value + thr) / (it + 1)
+            else:
+                thr = -1.0                                        # keep every entry
+            sparse = K.softmax_sparsify(p, float(thr))
+        del scores
+        out = p @ v
+        rows = [_heads_to_rows(t) for t in (q, k, v)]
+        if cfg.compress:
+            saved = []
+            for site, r in zip((mod.site_q, mod.site_k, mod.site_v), rows):
+                plan = site.channel_plan(r, it)
+                saved.append(K.compress_channel(r, plan, cfg.act_bits, cfg.act_group))
+        else:
+            saved = [r.contiguous() for r in rows]
+        mod.iteration += 1
+        if mod.record is not None:
+            mod.record.update(q=rows[0].detach().clone(), k=rows[1].detach().clone(), v=rows[2].detach().clone(),
+                              p=p.detach().clone(), saved=saved, sparse=sparse)
+        ctx.saved, ctx.sparse, ctx.geom, ctx.compress = saved, sparse, (b, nh, s, hd), cfg.compress
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        b, nh, s, hd = ctx.geom
+        restore = (lambda c: K.decompress_channel(c)) if ctx.compress else (lambda c: c)
+        g = g.to(BF16)
+        v = _rows_to_heads(restore(ctx.saved[2]), b, nh, s, hd)
+        p = K.softmax_dense(ctx.sparse)
+        dv = p.transpose(-2, -1) @ g
+        dp = g @ v.transpose(-2, -1)
+        del p, v
+        ds = K.softmax_bwd(dp.contiguous(), ctx.sparse)
+        del dp
+        ds.mul_(1.0 / math.sqrt(hd))
+        kk = _rows_to_heads(restore(ctx.saved[1]), b, nh, s, hd)
+        dq = ds @ kk
+        del kk
+        qq = _rows_to_heads(restore(ctx.saved[0]), b, nh, s, hd)
+        dk = ds.transpose(-2, -1) @ qq
+        ctx.saved = ctx.sparse = None
+        return dq, dk, dv, None
+
+
+# ---- the layer --------------------------------------------------------------------------------------------------
+class _PlainRMSNorm(torch.nn.Module):
+    def __init__(self, hidden, eps, device):
+        super().__init__()
+        self.weight = torch.nn.Parameter(torch.ones(hidden, dtype=BF16, device=device))
+        self.eps = eps
+
+    def forward(self, x):
+        xf = x.float()
+        return (self.weight.float() * (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.eps))).to(x.dtype)
+
+
+class DecoderLayer(torch.nn.Module):
+    def __init__(self, cfg: LayerConfig = None, device="cuda"):
+        super().__init__()
+        self.cfg = cfg = cfg or LayerConfig()
+        H, I = cfg.hidden, cfg.intermediate
+        if cfg.heads * cfg.head_dim != H:
+            raise ValueError("heads * head_dim must equal hidden")
+        if cfg.compress:
+            norm = lambda: EfficientMemoryRMSNorm(H, eps=cfg.rms_eps, elementwise_affine=True, bias=False,
+                                                  outlier_ratio=cfg.outlier_ratio, sub_outlier_ratio=1.0,
+                                                  sub_outlier_bit=cfg.act_bits, sub_outlier_quantize_method="per-token",
+                                                  rank=0, mode="hyc", group_size=cfg.act_group).to(device).to(BF16)
+        else:
+            norm = lambda: _PlainRMSNorm(H, cfg.rms_eps, device)
+        self.input_layernorm = norm()
+        self.post_attention_layernorm = norm()
+        self.qkv_proj = LoRAProjections(H, [H, H, H], cfg, device)
+        self.o_proj = LoRAProjections(H, [H], cfg, device)
+        self.gate_up_proj = LoRAProjections(H, [I, I], cfg, device)
+        self.down_proj = LoRAProjections(I, [H], cfg, device)
+        self.attention = CompressedAttention(cfg)
+        self.act = EfficientMemoryGatedAct("silu", cfg.outlier_ratio, 1.0, cfg.act_bits, "per-token", 0,
+                                           group_size=cfg.act_group) if cfg.compress else None
+        self._rope = None
+
+    def forward(self, x):
+        cfg = self.cfg
+        b, s, H = x.shape
+        if self._rope is None or self._rope[0].shape[0] != s:
+            self._rope = rope_tables(s, cfg.head_dim, cfg.rope_theta, x.device)
+        cos, sin = self._rope
+        h = self.input_layernorm(x)
+        q, k, v = self.qkv_proj(h)
+        heads = lambda t: t.view(b, s, cfg.heads, cfg.head_dim).transpose(1, 2)
+        q, k, v = apply_rope(heads(q), cos, sin), apply_rope(heads(k), cos, sin), heads(v)
+        a = self.attention(q, k, v)
+        a = a.transpose(1, 2).reshape(b, s, H)
+        x = x + self.o_proj(a)
+        h = self.post_attention_layernorm(x)
+        gate, up = self.gate_up_proj(h)
+        m = self.act(gate, up) if self.act is not None else torch.nn.functional.silu(gate) * up
+        return x + self.down_proj(m)
+
+    def saved_activation_bytes(self, batch, seq):
+        """analytic size of what one forward keeps for the backward (the probabilities' share is data dependent:
+        `softmax_ratio` of B*nh*S*S entries of 6 bytes plus row pointers)"""
+        cfg = self.cfg
+        M, H, I = batch * seq, cfg.hidden, cfg.intermediate
+
+        def site(width, bits, group):
+            k = K.num_outlier_channels(width, cfg.outlier_ratio)
+            return M * (width * bits // 8 + 2 * k + 2 * (width // group))
+
+        total = 2 * (site(H, cfg.act_bits, cfg.act_group) + 4 * M)                    # two norms: x + rstd
+        total += 2 * site(H, cfg.linear_bits, cfg.linear_group)                       # qkv input (once), o input
+        total += site(H, cfg.linear_bits, cfg.linear_group) + site(I, cfg.linear_bits, cfg.linear_group)  # gate/up, down
+        total += 3 * site(H, cfg.act_bits, cfg.act_group)                             # q, k, v
+        total += 3 * site(I, cfg.act_bits, cfg.act_group)                             # gate, act(gate), up
+        total += 7 * M * cfg.lora_r * 2                                               # h = x @ A^T, exact
+        rows = batch * cfg.heads * seq
+        total += int(cfg.softmax_ratio * rows * seq) * 6 + 4 * (rows + 1)
+        return total

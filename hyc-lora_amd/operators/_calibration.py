@@ -82,7 +82,8 @@ def calibration_state(model):
     the result can be handed to torch.save)"""
     out = {}
     for name, mod in model.named_modules():
-        if not hasattr(mod, "iteration") or not any(k.startswith("static_value") for k in vars(mod)):
+        if not hasattr(mod, "iteration") or not any(k.startswith("static_value") or isinstance(v, CompressionSite)
+                                                    for k, v in vars(mod).items()):
             continue
         entry = {"iteration": int(mod.iteration)}
         for key, val in vars(mod).items():

@@ -98,13 +98,11 @@ class _ChannelGatedActFunc(torch.autograd.Function):
     (gate; act(gate) and up), and one backward pass over them."""
 
     @staticmethod
-    def forward(ctx, gate, up, act, plan_a, plan_u, plan_g, bits, group):
+    def forward(ctx, gate, up, act, sites, iteration, bits, group):
         a = torch.nn.functional.silu(gate) if act == "silu" else torch.nn.functional.gelu(gate)
-        a2, _ = as_rows(a)
-        u2, _ = as_rows(up)
-        g2, _ = as_rows(gate)
-        ctx.saved = (K.compress_channel(a2, plan_a, bits, group), K.compress_channel(u2, plan_u, bits, group),
-                     K.compress_channel(g2, plan_g, bits, group))
+        rows = [as_rows(t)[0] for t in (a, up, gate)]
+        ctx.saved = tuple(K.compress_channel(r, site.channel_plan(r, iteration), bits, group)
+                          for r, site in zip(rows, sites))
         ctx.act = act
         return a * up
 
@@ -112,7 +110,7 @@ class _ChannelGatedActFunc(torch.autograd.Function):
     def backward(ctx, grad_output):
         g2, _ = as_rows(grad_output.to(torch.bfloat16))
         d_gate, d_up = K.gated_act_bwd(ctx.act, g2, *ctx.saved)
-        return d_gate.reshape(grad_output.shape), d_up.reshape(grad_output.shape), None, None, None, None, None, None
+        return d_gate.reshape(grad_output.shape), d_up.reshape(grad_output.shape), None, None, None, None, None
 
 
 class EfficientMemoryGatedAct(torch.nn.Module):
@@ -134,9 +132,7 @@ class EfficientMemoryGatedAct(torch.nn.Module):
         self.iteration = 0
 
     def forward(self, gate, up):
-        a = torch.nn.functional.silu(gate) if self.act == "silu" else torch.nn.functional.gelu(gate)
-        pa = self.site_act.channel_plan(as_rows(a)[0], self.iteration)
-        pu = self.site_up.channel_plan(as_rows(up)[0], self.iteration)
-        pg = self.site_gate.channel_plan(as_rows(gate)[0], self.iteration)
+        out = _ChannelGatedActFunc.apply(gate, up, self.act, (self.site_act, self.site_up, self.site_gate), self.iteration,
+                                         self.sub_outlier_bit, self.group_size)
         self.iteration += 1
-        return _ChannelGatedActFunc.apply(gate, up, self.act, pa, pu, pg, self.sub_outlier_bit, self.group_size)
+        return out

@@ -1,0 +1,182 @@
+"""GPU parity of the decoder-layer harness against the CPU layer oracle.
+
+Two links make the chain: every compressed site of the layer restores, bit for bit, what the oracle's compress /
+decompress gives for the activation the device saw; and the layer's gradients equal the oracle layer's evaluated at
+those restored activations."""
+import pytest
+import torch
+
+from conftest import bits_equal
+from oracle import hyc_oracle as O
+from oracle import layer_oracle as LO
+
+pytestmark = pytest.mark.gpu
+
+NAMES = ("q", "k", "v", "o", "gate", "up", "down")
+
+
+@pytest.fixture(scope="module")
+def DL(hyc):
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    import importlib
+    return importlib.import_module(hyc.__name__ + ".decoder_layer")
+
+
+def small_cfg(DL, **kw):
+    return DL.LayerConfig(hidden=256, heads=4, head_dim=64, intermediate=512, lora_r=16, lora_alpha=32.0,
+                          outlier_ratio=0.02, softmax_ratio=0.05, **kw)
+
+
+def oracle_params(K, layer):
+    groups = {"q": (layer.qkv_proj, 0), "k": (layer.qkv_proj, 1), "v": (layer.qkv_proj, 2), "o": (layer.o_proj, 0),
+              "gate": (layer.gate_up_proj, 0), "up": (layer.gate_up_proj, 1), "down": (layer.down_proj, 0)}
+    P = {"w_in": layer.input_layernorm.weight.detach().float().cpu().requires_grad_(True),
+         "w_post": layer.post_attention_layernorm.weight.detach().float().cpu().requires_grad_(True)}
+    for n, (mod, i) in groups.items():
+        P["W_" + n] = K.nf4_dequantize(mod.base[i]).float().cpu()
+        P["A_" + n] = mod.lora_A[i].detach().float().cpu().requires_grad_(True)
+        P["B_" + n] = mod.lora_B[i].detach().float().cpu().requires_grad_(True)
+    return P, groups
+
+
+def make_input(gen, B, S, H):
+    x = torch.randn(B, S, H, generator=gen)
+    x[..., 7] *= 15
+    x[..., 100] *= 8
+    return x.bfloat16()
+
+
+def rel_err(a, b):
+    return float((a.double() - b.double()).norm() / b.double().norm().clamp_min(1e-30))
+
+
+def check_grads(layer, groups, xg, P, xo, tol):
+    errs = {"dx": rel_err(xg.grad.cpu(), xo.grad)}
+    for n, (mod, i) in groups.items():
+        errs["A_" + n] = rel_err(mod.lora_A[i].grad.cpu(), P["A_" + n].grad)
+        errs["B_" + n] = rel_err(mod.lora_B[i].grad.cpu(), P["B_" + n].grad)
+    errs["w_in"] = rel_err(layer.input_layernorm.weight.grad.cpu(), P["w_in"].grad)
+    errs["w_post"] = rel_err(layer.post_attention_layernorm.weight.grad.cpu(), P["w_post"].grad)
+    bad = {k: v for k, v in errs.items() if not v < tol}
+    assert not bad, bad
+    return errs
+
+
+def test_layer_formulas_without_compression(DL, K):
+    """compress=False: the layer's own backward (LoRA composite, attention) against the oracle with exact activations,
+    whose gradients are pinned against plain float64 autograd"""
+    B, S = 2, 64
+    cfg = small_cfg(DL, compress=False)
+    layer = DL.DecoderLayer(cfg)
+    gen = torch.Generator().manual_seed(3)
+    x = make_input(gen, B, S, cfg.hidden)
+    g = (0.05 * torch.randn(B, S, cfg.hidden, generator=gen)).bfloat16()
+    xg = x.cuda().requires_grad_(True)
+    y = layer(xg)
+    y.backward(g.cuda())
+    P, groups = oracle_params(K, layer)
+    cos, sin = (t.float().cpu() for t in DL.rope_tables(S, cfg.head_dim, cfg.rope_theta, "cuda"))
+    xo = x.float().requires_grad_(True)
+    yo = LO.decoder_layer(xo, P, {}, cfg.heads, cfg.rms_eps, cfg.lora_alpha / cfg.lora_r, cos, sin, quirk=False)
+    yo.backward(g.float())
+    assert rel_err(y.detach().cpu(), yo.detach()) < 1e-2
+    check_grads(layer, groups, xg, P, xo, 2e-2)
+
+
+@pytest.fixture(scope="module")
+def K(hyc):
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    return hyc.kernels
+
+
+def test_layer_with_compression(DL, K):
+    """three steps (two calibrating, one steady); on each: every site restores what the oracle restores, the kept
+    probabilities are the oracle's set, and the gradients equal the oracle layer's at those restored activations
+    (relative error of each gradient tensor below 1e-2)"""
+    B, S = 2, 64
+    cfg = small_cfg(DL)
+    layer = DL.DecoderLayer(cfg)
+    H, I, nh = cfg.hidden, cfg.intermediate, cfg.heads
+    gen = torch.Generator().manual_seed(4)
+    P, groups = oracle_params(K, layer)
+    cos, sin = (t.float().cpu() for t in DL.rope_tables(S, cfg.head_dim, cfg.rope_theta, "cuda"))
+    rec = {"qkv": {}, "o": {}, "gate_up": {}, "down": {}, "attn": {}}
+    layer.qkv_proj.record, layer.o_proj.record = rec["qkv"], rec["o"]
+    layer.gate_up_proj.record, layer.down_proj.record = rec["gate_up"], rec["down"]
+    layer.attention.record = rec["attn"]
+    grabbed = {}
+    hooks = [layer.input_layernorm.register_forward_hook(lambda m, i, o: grabbed.__setitem__("norm_in", (i[0].detach().clone(), o.grad_fn.saved))),
+             layer.post_attention_layernorm.register_forward_hook(lambda m, i, o: grabbed.__setitem__("norm_post", (i[0].detach().clone(), o.grad_fn.saved))),
+             layer.act.register_forward_hook(lambda m, i, o: grabbed.__setitem__("act", (i[0].detach().clone(), i[1].detach().clone(), o.grad_fn.saved)))]
+
+    def restore_and_check(x2d, c, bits, group):
+        """device restore == oracle restore of the device's activation, bit for bit"""
+        xh = K.decompress_channel(c).cpu()
+        idx = c.plan.idx.cpu().long()
+        vals, stored, scales = O.hyc_compress(x2d.cpu(), idx, bits, group)
+        assert torch.equal(c.stored.cpu().view(torch.uint8), stored.view(torch.uint8))
+        assert bits_equal(xh, O.hyc_decompress(vals, stored, idx, scales, bits, group))
+        return xh
+
+    for step in range(3):
+        x = make_input(gen, B, S, H)
+        g = (0.05 * torch.randn(B, S, H, generator=gen)).bfloat16()
+        for p in layer.parameters():
+            p.grad = None
+        xg = x.cuda().requires_grad_(True)
+        y = layer(xg)
+        y.backward(g.cuda())
+
+        ab, ag, lb, lg = cfg.act_bits, cfg.act_group, cfg.linear_bits, cfg.linear_group
+        R = {}
+        for site in ("norm_in", "norm_post"):
+            xin, c = grabbed[site]
+            R[site] = restore_and_check(xin.reshape(-1, H), c, ab, ag).reshape(B, S, H)
+        for site, key in (("qkv_in", "qkv"), ("o_in", "o"), ("gate_up_in", "gate_up"), ("down_in", "down")):
+            xin, c = rec[key]["x"], rec[key]["saved"]
+            R[site] = restore_and_check(xin, c, lb, lg).reshape(B, S, -1)
+        for n, c in zip("qkv", rec["attn"]["saved"]):
+            R[n] = restore_and_check(rec["attn"][n].contiguous(), c, ab, ag).reshape(B, S, H)
+        gate, up, (c_act, c_up, c_gate) = grabbed["act"]
+        R["gate"] = restore_and_check(gate.reshape(-1, I), c_gate, ab, ag).reshape(B, S, I)
+        R["up"] = restore_and_check(up.reshape(-1, I), c_up, ab, ag).reshape(B, S, I)
+        R["act"] = restore_and_check(torch.nn.functional.silu(gate).reshape(-1, I), c_act, ab, ag).reshape(B, S, I)
+        p_dev = rec["attn"]["p"].cpu()
+        thr = O.get_statistics_softmax(p_dev, step, cfg.softmax_ratio) if step < 2 else layer.attention.static_value.cpu()
+        R["p"] = K.softmax_dense(rec["attn"]["sparse"]).cpu()
+        assert bits_equal(R["p"], O.prune_softmax(p_dev, thr))
+        kept = float((R["p"] > 0).float().mean())
+        assert 0.02 < kept < 0.08, kept
+
+        for t in P.values():
+            t.grad = None
+        xo = x.float().requires_grad_(True)
+        yo = LO.decoder_layer(xo, P, R, nh, cfg.rms_eps, cfg.lora_alpha / cfg.lora_r, cos, sin, quirk=True, probs=p_dev)
+        yo.backward(g.float())
+        assert rel_err(y.detach().cpu(), yo.detach()) < 1e-2
+        check_grads(layer, groups, xg, P, xo, 1e-2)
+    for h in hooks:
+        h.remove()
+    assert layer.attention.iteration == 3 and layer.qkv_proj.iteration == 3
+
+
+def test_saved_bytes_accounting(DL, K):
+    """what the forward keeps (allocator delta) matches the analytic count to within the allocator's rounding, and is
+    several times smaller than the bf16 activations of the uncompressed layer"""
+    B, S = 2, 128
+    cfg = small_cfg(DL)
+    layer = DL.DecoderLayer(cfg)
+    x = make_input(torch.Generator().manual_seed(5), B, S, cfg.hidden).cuda()
+    for _ in range(3):
+        layer(x.clone().requires_grad_(True)).sum().backward()
+    torch.cuda.synchronize()
+    xg = x.clone().requires_grad_(True)
+    before = torch.cuda.memory_allocated()
+    y = layer(xg)
+    torch.cuda.synchronize()
+    held = torch.cuda.memory_allocated() - before - y.numel() * 2
+    analytic = layer.saved_activation_bytes(B, S)
+    assert 0.7 * analytic < held < 1.6 * analytic, (held, analytic)
+    y.sum().backward()

@@ -488,3 +488,15 @@ def test_nf4_kernels(K, shape):
     back = K.nf4_dequantize(q)
     assert back.shape == w.shape and bits_equal(back.cpu(), O.nf4_dequantize(packed_o, absmax_o, w.shape))
     assert q.nbytes() == w.numel() // 2 + 4 * (w.numel() // 64)
+
+
+def test_softmax_with_saturated_mask(K):
+    """additive masks at the bottom of the bf16 range (what the reference's attention adds) give exact zeros, not NaN"""
+    gen = torch.Generator().manual_seed(14)
+    x = torch.randn(2, 3, 64, 64, generator=gen).bfloat16()
+    x.masked_fill_(torch.ones(64, 64, dtype=torch.bool).triu(1), torch.finfo(torch.bfloat16).min)
+    y, _ = K.softmax_fwd(x.cuda())
+    want = torch.softmax(x.float(), -1)
+    assert not torch.isnan(y).any()
+    assert torch.equal(y.cpu().triu(1), torch.zeros_like(x))
+    assert bf16_ulp_diff(y.cpu(), want.bfloat16()).max() <= 1

@@ -345,3 +345,65 @@ def test_nf4_nearest_level_and_round_trip():
     one[0] = 1.0
     p3, _ = O.nf4_quantize(one)
     assert int(p3[0]) == (15 << 4) | 7 and int(p3[1]) == (7 << 4) | 7
+
+
+def _tiny_layer_params(gen, H, I, r):
+    P = {"w_in": 1 + 0.1 * torch.randn(H, generator=gen), "w_post": 1 + 0.1 * torch.randn(H, generator=gen)}
+    for name, (out, inp) in dict(q=(H, H), k=(H, H), v=(H, H), o=(H, H), gate=(I, H), up=(I, H), down=(H, I)).items():
+        P["W_" + name] = 0.1 * torch.randn(out, inp, generator=gen)
+        P["A_" + name] = 0.2 * torch.randn(r, inp, generator=gen)
+        P["B_" + name] = 0.2 * torch.randn(out, r, generator=gen)
+    return P
+
+
+def test_layer_oracle_against_plain_autograd():
+    """with every restored activation equal to the exact one, the layer oracle must give the true gradients: compared
+    with float64 autograd of an independently written layer (merged weights W + s*B@A, F.rms_norm,
+    F.scaled_dot_product_attention)"""
+    from oracle import layer_oracle as LO
+    F = torch.nn.functional
+    gen = torch.Generator().manual_seed(17)
+    B, S, H, nh, I, r, s, eps = 2, 12, 32, 4, 48, 4, 2.0, 1e-5
+    hd = H // nh
+    P = _tiny_layer_params(gen, H, I, r)
+    x = torch.randn(B, S, H, generator=gen).bfloat16().float()
+    g = 0.1 * torch.randn(B, S, H, generator=gen)
+    inv = 1.0 / (10000.0 ** (torch.arange(0, hd, 2).float() / hd))
+    emb = torch.cat([torch.outer(torch.arange(S).float(), inv)] * 2, -1)
+    cos, sin = emb.cos(), emb.sin()
+
+    xo = x.clone().requires_grad_(True)
+    Po = {k: v.clone().requires_grad_(not k.startswith("W_")) for k, v in P.items()}
+    cap = {}
+    y = LO.decoder_layer(xo, Po, {}, nh, eps, s, cos, sin, quirk=False, capture=cap)
+    y.backward(g)
+    assert set(cap) == {"norm_in", "qkv_in", "q", "k", "v", "p", "o_in", "norm_post", "gate_up_in", "gate", "act", "up", "down_in"}
+
+    xd = x.double().requires_grad_(True)
+    Pd = {k: v.double().requires_grad_(not k.startswith("W_")) for k, v in P.items()}
+    merged = lambda n: Pd["W_" + n] + s * Pd["B_" + n] @ Pd["A_" + n]
+    split = lambda t: t.view(B, S, nh, hd).transpose(1, 2)
+    rot = lambda t: t * cos.double() + torch.cat((-t[..., hd // 2:], t[..., :hd // 2]), -1) * sin.double()
+    h = F.rms_norm(xd, (H,), Pd["w_in"], eps)
+    q, k, v = (split(F.linear(h, merged(n))) for n in "qkv")
+    a = F.scaled_dot_product_attention(rot(q), rot(k), v, is_causal=True).transpose(1, 2).reshape(B, S, H)
+    x1 = xd + F.linear(a, merged("o"))
+    h2 = F.rms_norm(x1, (H,), Pd["w_post"], eps)
+    yd = x1 + F.linear(F.silu(F.linear(h2, merged("gate"))) * F.linear(h2, merged("up")), merged("down"))
+    yd.backward(g.double())
+
+    def close(a, b, what):
+        err = float((a.double() - b).abs().max()) / float(b.abs().max())
+        assert err < 2e-2, (what, err)
+    close(y.detach(), yd.detach(), "y")
+    close(xo.grad, xd.grad, "dx")
+    for name in Po:
+        if not name.startswith("W_"):
+            close(Po[name].grad, Pd[name].grad, name)
+    # the substitution really is used: a wrong restored activation changes exactly the gradients that read it
+    xo2 = x.clone().requires_grad_(True)
+    Po2 = {k: v.clone().requires_grad_(not k.startswith("W_")) for k, v in P.items()}
+    LO.decoder_layer(xo2, Po2, {"qkv_in": 2 * cap["qkv_in"]}, nh, eps, s, cos, sin, quirk=False).backward(g)
+    assert torch.allclose(Po2["A_q"].grad, 2 * Po["A_q"].grad, rtol=1e-4, atol=1e-6)
+    assert torch.allclose(Po2["B_q"].grad, Po["B_q"].grad, rtol=1e-4, atol=1e-6)
+    assert torch.allclose(Po2["A_o"].grad, Po["A_o"].grad, rtol=1e-4, atol=1e-6)
