@@ -173,6 +173,60 @@ def kernel_tour(pkg, torch, reps=5):
     print(json.dumps({"kernel_tour": True}))
 
 
+def layer_report(pkg, torch, steps=6):
+    """full LLaMA-2-7B-shaped decoder layer (hidden 4096, 32 x 128 heads, intermediate 11008, NF4 base, LoRA r=16 on
+    all seven projections), forward + backward, at batch 1 x seq 2048 and batch 4 x seq 1024: what the forward keeps
+    for the backward, the peak above the resident weights, and the step time - with every saved activation compressed
+    (1 % outlier channels, INT2 for linear inputs, INT4 elsewhere) and with the same layer keeping bf16."""
+    DL = importlib.import_module("hyc-lora_amd.decoder_layer")
+    out = []
+    for compress in (True, False):
+        layer = DL.DecoderLayer(DL.LayerConfig(compress=compress))
+        torch.cuda.synchronize()
+        for (B, S) in ((1, 2048), (4, 1024)):
+            gen = torch.Generator(device="cuda").manual_seed(B * 7 + S)
+            x = torch.randn(B, S, 4096, generator=gen, device="cuda")
+            x[..., torch.randperm(4096, generator=gen, device="cuda")[:20]] *= 30
+            x = x.bfloat16()
+            g = (0.01 * torch.randn(B, S, 4096, generator=gen, device="cuda")).bfloat16()
+            for mod in layer.modules():                      # a new sequence length calibrates again
+                if hasattr(mod, "iteration"):
+                    mod.iteration = 0
+            layer.attention.static_value = None
+            times, held, peak = [], 0, 0
+            for it in range(3 + steps):
+                for p in layer.parameters():
+                    p.grad = None
+                xg = x.clone().requires_grad_(True)
+                torch.cuda.synchronize()
+                torch.cuda.reset_peak_memory_stats()
+                base = torch.cuda.memory_allocated()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                y = layer(xg)
+                if it == 3 + steps - 1:
+                    torch.cuda.synchronize()
+                    held = torch.cuda.memory_allocated() - base - y.numel() * 2
+                y.backward(g)
+                e1.record()
+                torch.cuda.synchronize()
+                if it >= 3:
+                    times.append(e0.elapsed_time(e1))
+                    peak = max(peak, torch.cuda.max_memory_allocated() - base)
+                del y, xg
+            times.sort()
+            rec = {"layer_report": True, "compress": compress, "batch": B, "seq": S,
+                   "saved_for_backward_bytes": int(held), "peak_above_weights_bytes": int(peak),
+                   "step_ms": round(times[len(times) // 2], 3)}
+            if compress:
+                rec["saved_analytic_bytes"] = int(layer.saved_activation_bytes(B, S))
+            out.append(rec)
+            print(json.dumps(rec), flush=True)
+        del layer
+        torch.cuda.empty_cache()
+    return out
+
+
 def cpu_baseline(torch, wl, rows, seconds):
     """the oracle (CPU PyTorch restatement of the path) on the host cores, bounded sample of the same workload"""
     from oracle import hyc_oracle as O
@@ -214,6 +268,8 @@ def main():
                     help="for rocprofv3 --kernel-trace: run every kernel of the path a few times at the config shapes, then exit")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="for rocprofv3 --pmc: 5x a plain 32 MiB device copy, 5x fwd, 5x bwd, then exit")
+    ap.add_argument("--layer-report", action="store_true",
+                    help="full decoder layer (the fifth BASELINE configuration): saved bytes, peak memory, step time; then exit")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this path runs on ONE GPU (no sharding, no collectives); run with --gpus 1")
@@ -232,6 +288,10 @@ def main():
 
     if args.kernel_tour:
         kernel_tour(pkg, torch)
+        return
+    if args.layer_report:
+        del wl
+        layer_report(pkg, torch)
         return
     if args.pmc_probe:
         dst = torch.empty_like(wl.x)

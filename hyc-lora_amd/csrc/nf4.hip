@@ -51,29 +51,38 @@ k_nf4_quantize(const uint16_t* __restrict__ w, int64_t nblocks, uint8_t* __restr
   }
 }
 
-// One lane expands 16 bytes (32 weights, half a block) into four 16-byte stores.
+// One lane expands 4 bytes (8 weights) into one 16-byte store, so that a wave reads 256 and writes 1024 contiguous
+// bytes per step; four independent steps per trip keep enough loads in flight.
 __global__ void __launch_bounds__(256)
-k_nf4_dequantize(const uint8_t* __restrict__ packed, const float* __restrict__ absmax, int64_t nblocks,
+k_nf4_dequantize(const uint8_t* __restrict__ packed, const float* __restrict__ absmax, int64_t nwords,
                  uint16_t* __restrict__ out) {
   __shared__ float lut[16];
   if (threadIdx.x < 16) lut[threadIdx.x] = kNF4[threadIdx.x];
   __syncthreads();
-  const int64_t halves = nblocks * 2;
-  for (int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x; t < halves; t += (int64_t)gridDim.x * 256) {
-    const uint4 p = *reinterpret_cast<const uint4*>(packed + 16 * t);
-    const float s = absmax[t >> 1];
-    const uint32_t words[4] = {p.x, p.y, p.z, p.w};
-    uint16_t* o = out + 32 * t;
+  const uint32_t* words = reinterpret_cast<const uint32_t*>(packed);
+  const int64_t step = (int64_t)gridDim.x * 256;
+  for (int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x; t < nwords; t += 4 * step) {
+    uint32_t w[4];
+    float s[4];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
+    for (int u = 0; u < 4; ++u) {
+      const int64_t i = t + u * step;
+      const bool on = i < nwords;
+      w[u] = on ? words[i] : 0u;
+      s[u] = on ? absmax[i >> 3] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int64_t i = t + u * step;
+      if (i >= nwords) break;
       float v[8];
 #pragma unroll
       for (int b = 0; b < 4; ++b) {
-        const uint32_t byte = (words[q] >> (8 * b)) & 0xFFu;
-        v[2 * b] = lut[byte >> 4] * s;
-        v[2 * b + 1] = lut[byte & 15u] * s;
+        const uint32_t byte = (w[u] >> (8 * b)) & 0xFFu;
+        v[2 * b] = lut[byte >> 4] * s[u];
+        v[2 * b + 1] = lut[byte & 15u] * s[u];
       }
-      *reinterpret_cast<uint4*>(o + 8 * q) = pack8(v);
+      *reinterpret_cast<uint4*>(out + 8 * i) = pack8(v);
     }
   }
 }
@@ -115,7 +124,7 @@ int hyc_nf4_dequantize(const void* packed, const float* absmax, int64_t n, void*
     return fail(HYC_EINVAL, "hyc_nf4_dequantize: packed and out must be 16-byte aligned");
   const int64_t nblocks = n / 64;
   hipLaunchKernelGGL(k_nf4_dequantize, dim3(stream_grid(nblocks * 2)), dim3(256), 0, begin_launch(stream),
-                     static_cast<const uint8_t*>(packed), absmax, nblocks, static_cast<uint16_t*>(out));
+                     static_cast<const uint8_t*>(packed), absmax, nblocks * 8, static_cast<uint16_t*>(out));
   return check_launch("hyc_nf4_dequantize");
 }
 

@@ -192,15 +192,15 @@ class _AttentionFunc(torch.autograd.Function):
         causal = torch.ones(s, s, dtype=torch.bool, device=q.device).triu_(1)
         scores.masked_fill_(causal, torch.finfo(BF16).min)       # the additive mask of the reference, saturated
         it = mod.iteration
-        if cfg.compress and it >= 2:
+        if not cfg.compress:
+            p, _ = K.softmax_fwd(scores)
+            sparse = p                                             # kept whole, in bf16
+        elif it >= 2:
             p, sparse = K.softmax_fwd(scores, float(mod.static_value))
         else:
             p, _ = K.softmax_fwd(scores)
-            if cfg.compress:
-                thr = get_statistics_softmax(p, it, cfg.softmax_ratio)
-                mod.static_value = thr if mod.static_value is None else (it * mod.static_value + thr) / (it + 1)
-            else:
-                thr = -1.0                                        # keep every entry
+            thr = get_statistics_softmax(p, it, cfg.softmax_ratio)
+            mod.static_value = thr if mod.static_value is None else (it * mod.static_value + thr) / (it + 1)
             sparse = K.softmax_sparsify(p, float(thr))
         del scores
         out = p @ v
@@ -225,11 +225,15 @@ class _AttentionFunc(torch.autograd.Function):
         restore = (lambda c: K.decompress_channel(c)) if ctx.compress else (lambda c: c)
         g = g.to(BF16)
         v = _rows_to_heads(restore(ctx.saved[2]), b, nh, s, hd)
-        p = K.softmax_dense(ctx.sparse)
+        p = K.softmax_dense(ctx.sparse) if ctx.compress else ctx.sparse
         dv = p.transpose(-2, -1) @ g
         dp = g @ v.transpose(-2, -1)
-        del p, v
-        ds = K.softmax_bwd(dp.contiguous(), ctx.sparse)
+        if ctx.compress:
+            del p, v
+            ds = K.softmax_bwd(dp.contiguous(), ctx.sparse)
+        else:
+            ds = torch._softmax_backward_data(dp, p, -1, BF16)
+            del p, v
         del dp
         ds.mul_(1.0 / math.sqrt(hd))
         kk = _rows_to_heads(restore(ctx.saved[1]), b, nh, s, hd)

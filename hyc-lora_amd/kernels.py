@@ -51,6 +51,22 @@ class ChannelPlan:
     plan: torch.Tensor   # int32 [H/8] (bit pattern of the uint32 lookup words)
 
 
+def kth_value(x, k):
+    """the k-th smallest (1-based) of all elements of x (bf16 or fp32) as a 0-d fp32 tensor; the value
+    `torch.kthvalue(x.flatten().float(), k).values` gives, without a sort and without a host round trip"""
+    if x.dtype not in (BF16, torch.float32):
+        raise ValueError("x must be bfloat16 or float32, got %s" % x.dtype)
+    if not x.is_cuda:
+        raise ValueError("x must live on the GPU")
+    x = x.contiguous()
+    lib = _abi.load()
+    out = torch.empty((), dtype=torch.float32, device=x.device)
+    ws = torch.empty(lib.hyc_kth_value_workspace_bytes() // 4, dtype=torch.int32, device=x.device)
+    code = _abi.DTYPE_BF16 if x.dtype == BF16 else _abi.DTYPE_F32
+    check(lib.hyc_kth_value(_p(x), code, x.numel(), int(k), _p(out), _p(ws), _stream()))
+    return out
+
+
 def channel_absmax(x2d, amax=None):
     """running per-channel max |x| (fp32 [H]); pass the previous result to accumulate"""
     _need(x2d, BF16, "x")

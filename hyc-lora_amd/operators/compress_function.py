@@ -46,7 +46,7 @@ def get_statistics(x: torch.Tensor, iteration: int, outlier_ratio: float, sub_ou
         R = torch.zeros((16, H), dtype=x.dtype, device=x.device)
     x0 = x[0]
     kth = int(x0.numel() * (1 - outlier_ratio))
-    outlier = torch.kthvalue(x0.flatten().to(torch.float32), kth).values
+    outlier = K.kth_value(x0, kth)
     x = x - (x0 * (x0.abs() > outlier)).to(BF16)
     if sub_outlier_ratio > 0 and sub_outlier_bit != 16:
         z = x[0]
@@ -67,7 +67,7 @@ def get_statistics(x: torch.Tensor, iteration: int, outlier_ratio: float, sub_ou
 @torch.no_grad()
 def get_statistics_softmax(x: torch.Tensor, iteration: int, outlier_ratio: float):
     x0 = x[0]
-    return torch.kthvalue(x0.float().flatten(), int(x0.numel() * (1 - outlier_ratio))).values
+    return K.kth_value(x0, int(x0.numel() * (1 - outlier_ratio)))
 
 
 # ---- compress / decompress (reference :136-261) --------------------------------------------------------------

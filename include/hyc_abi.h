@@ -16,6 +16,9 @@
  *   hyc_channel_absmax / hyc_select_channels
  *       the calibration statistics, operators/compress_function.py:292-340 (get_statistics), for the
  *       channel-structured outlier rule
+ *   hyc_kth_value
+ *       torch.kthvalue(x[0].flatten().float(), k).values, the calibration quantile of
+ *       operators/compress_function.py:319 (get_statistics) and :345 (get_statistics_softmax)
  *   hyc_rmsnorm_fwd_compress
  *       EfficientMemoryRMSNormFunc.forward + _rms_norm_fwd_fused, operators/efficient_rmsnorm.py:147-212, :15-60
  *   hyc_rmsnorm_bwd
@@ -119,6 +122,13 @@ int64_t hyc_rmsnorm_bwd_partial_rows(int64_t M, int64_t H, const hyc_desc* d);
 int hyc_channel_absmax(const void* x, int64_t M, int64_t H, float* amax, void* stream);
 /* the k largest amax, ties to the lower channel, written ascending to idx [k]; plan [H/8] as described above. */
 int hyc_select_channels(const float* amax, int64_t H, int32_t k, int32_t* idx, uint32_t* plan, void* stream);
+
+/* ---- calibration quantile ---------------------------------------------------------------------- */
+/* out[0] = the k-th smallest (k = 1..n) of the n values of x (bf16 or fp32, HYC_DTYPE_*), as fp32; NaN sorts last,
+ * -0 before +0.  workspace: hyc_kth_value_workspace_bytes() bytes of device memory, 16-byte aligned, any contents.
+ * n < 2^31. */
+int64_t hyc_kth_value_workspace_bytes(void);
+int hyc_kth_value(const void* x, int32_t x_dtype, int64_t n, int64_t k, float* out, void* workspace, void* stream);
 
 /* ---- standalone compress / decompress -------------------------------------------------------- */
 /* x bf16 [M,H] -> stored; channel mode also writes vals [M,k] and scales [M,H/group];

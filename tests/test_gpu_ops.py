@@ -500,3 +500,29 @@ def test_softmax_with_saturated_mask(K):
     assert not torch.isnan(y).any()
     assert torch.equal(y.cpu().triu(1), torch.zeros_like(x))
     assert bf16_ulp_diff(y.cpu(), want.bfloat16()).max() <= 1
+
+
+# ------------------------------------------------------------------ calibration quantile
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n", [1, 5, 1000, 4099, 1 << 20])
+def test_kth_value_matches_torch(K, dtype, n):
+    """hyc_kth_value against torch.kthvalue on the CPU (a library routine): random values, a block of exact zeros,
+    repeated values and negatives; ranks at both ends, around the zero block and in the bulk"""
+    gen = torch.Generator().manual_seed(n)
+    x = torch.randn(n, generator=gen)
+    x[: n // 3] = 0
+    x[n // 3: n // 2] = x[n // 3: n // 2].round()
+    x = x[torch.randperm(n, generator=gen)].to(dtype)
+    xd = x.cuda()
+    for k in sorted({1, n, max(1, n // 3), max(1, n // 2), max(1, int(n * 0.99)), max(1, n // 7)}):
+        want = torch.kthvalue(x.float(), k).values
+        got = K.kth_value(xd, k).cpu()
+        assert got.dtype == torch.float32 and float(got) == float(want), (n, k, float(got), float(want))
+
+
+def test_kth_value_softmax_shape(K):
+    gen = torch.Generator().manual_seed(3)
+    p = torch.softmax(3 * torch.randn(2, 4, 96, 96, generator=gen), -1).bfloat16()
+    k = int(p[0].numel() * 0.95)
+    want = torch.kthvalue(p[0].float().flatten(), k).values
+    assert float(K.kth_value(p[0].cuda(), k)) == float(want)
