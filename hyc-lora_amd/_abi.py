@@ -58,6 +58,7 @@ SIGNATURES = {
     "hyc_gated_act_bwd": (c_i32, [c_i32, c_ptr, c_ptr, c_ptr, c_ptr, ctypes.POINTER(HycDesc), c_ptr, c_ptr, c_ptr, ctypes.POINTER(HycDesc),
                                   c_ptr, c_ptr, c_ptr, ctypes.POINTER(HycDesc), c_i64, c_i64, c_ptr, c_ptr, c_ptr]),
     "hyc_softmax_fwd": (c_i32, [c_ptr, c_i64, c_i64, c_f32, c_ptr, c_ptr, c_ptr]),
+    "hyc_softmax_causal_fwd": (c_i32, [c_ptr, c_i64, c_i64, c_i64, c_f32, c_ptr, c_ptr, c_ptr]),
     "hyc_softmax_fill": (c_i32, [c_ptr, c_i64, c_i64, c_f32, c_ptr, c_ptr, c_ptr, c_ptr]),
     "hyc_softmax_bwd": (c_i32, [c_ptr, c_i64, c_i64, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr]),
     "hyc_softmax_dense": (c_i32, [c_i64, c_i64, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr]),

@@ -60,10 +60,12 @@ k_softmax_fwd(const uint16_t* __restrict__ x, int64_t rows, int64_t N, float thr
 
 // Rows of up to 4096 entries: one wave per row, the row stays in registers (CPL chunks of 8 per lane), wave-level
 // reductions only (no barrier), exp evaluated once per element, the next row requested before this one is processed.
-template <int CPL>
+// CAUSAL: row r belongs to query position r % period and sees columns 0..position only; the rest of the row is
+// neither read (x may hold anything there) nor exponentiated, and comes out as exact zeros.
+template <int CPL, bool CAUSAL>
 __global__ void __launch_bounds__(256)
 k_softmax_fwd_wave(const uint16_t* __restrict__ x, int64_t rows, int64_t N, float thr, uint16_t* __restrict__ y,
-                   int32_t* __restrict__ counts) {
+                   int32_t* __restrict__ counts, int64_t period) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
   const int nch = (int)(N / 8);
@@ -72,24 +74,35 @@ k_softmax_fwd_wave(const uint16_t* __restrict__ x, int64_t rows, int64_t N, floa
   bool on[CPL];
 #pragma unroll
   for (int u = 0; u < CPL; ++u) on[u] = lane + 64 * u < nch;
+  // last visible column of a row (everything when not causal)
+  auto last_col = [&](int64_t r) __attribute__((always_inline)) { return CAUSAL ? (int)(r % period) : (int)N - 1; };
   uint4 raw[CPL];
   if (row < rows) {
+    const int lc = last_col(row);
 #pragma unroll
     for (int u = 0; u < CPL; ++u)
-      raw[u] = on[u] ? *reinterpret_cast<const uint4*>(x + row * N + 8 * (lane + 64 * u)) : make_uint4(0, 0, 0, 0);
+      raw[u] = on[u] && 8 * (lane + 64 * u) <= lc ? *reinterpret_cast<const uint4*>(x + row * N + 8 * (lane + 64 * u))
+                                                  : make_uint4(0, 0, 0, 0);
   }
   for (; row < rows; row += stride) {
     uint4 nxt[CPL];
     if (row + stride < rows) {
+      const int lc = last_col(row + stride);
 #pragma unroll
       for (int u = 0; u < CPL; ++u)
-        nxt[u] = on[u] ? *reinterpret_cast<const uint4*>(x + (row + stride) * N + 8 * (lane + 64 * u)) : make_uint4(0, 0, 0, 0);
+        nxt[u] = on[u] && 8 * (lane + 64 * u) <= lc
+                     ? *reinterpret_cast<const uint4*>(x + (row + stride) * N + 8 * (lane + 64 * u)) : make_uint4(0, 0, 0, 0);
     }
     float v[CPL][8];
     float m = -INFINITY;
+    const int lc = last_col(row);
 #pragma unroll
     for (int u = 0; u < CPL; ++u) {
       unpack8(raw[u], v[u]);
+      if (CAUSAL) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[u][j] = 8 * (lane + 64 * u) + j <= lc ? v[u][j] : -INFINITY;
+      }
       if (on[u]) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) m = v[u][j] > m ? v[u][j] : m;
@@ -292,8 +305,8 @@ int hyc_softmax_fwd(const void* x, int64_t rows, int64_t N, float threshold, voi
     const int64_t blocks = (rows + 3) / 4, cap = 256 * 8;
     const dim3 grid((unsigned)(blocks < cap ? blocks : cap));
 #define HYC_SMW(C_)                                                                                                \
-  hipLaunchKernelGGL((k_softmax_fwd_wave<C_>), grid, dim3(256), 0, st, static_cast<const uint16_t*>(x), rows, N, thr, \
-                     static_cast<uint16_t*>(y), counts)
+  hipLaunchKernelGGL((k_softmax_fwd_wave<C_, false>), grid, dim3(256), 0, st, static_cast<const uint16_t*>(x), rows, N, \
+                     thr, static_cast<uint16_t*>(y), counts, (int64_t)1)
     if (cpl <= 1) HYC_SMW(1); else if (cpl <= 2) HYC_SMW(2); else if (cpl <= 4) HYC_SMW(4); else HYC_SMW(8);
 #undef HYC_SMW
   } else if (x) {
@@ -306,6 +319,29 @@ int hyc_softmax_fwd(const void* x, int64_t rows, int64_t N, float threshold, voi
                        static_cast<const uint16_t*>(y), rows, N, thr, counts);
   }
   return check_launch("hyc_softmax_fwd");
+}
+
+int hyc_softmax_causal_fwd(const void* x, int64_t rows, int64_t N, int64_t period, float threshold, void* y,
+                           int32_t* counts, void* stream) {
+  int rc = softmax_shape("hyc_softmax_causal_fwd", rows, N);
+  if (rc) return rc;
+  if (N > 4096) return fail(HYC_ENOTSUP, "hyc_softmax_causal_fwd: N=%lld (rows of at most 4096 entries)", (long long)N);
+  if (period <= 0 || period > N)
+    return fail(HYC_EINVAL, "hyc_softmax_causal_fwd: period=%lld must be in 1..N=%lld", (long long)period, (long long)N);
+  if (rows == 0) return HYC_OK;
+  if (!x || !y) return fail(HYC_EFAULT, "hyc_softmax_causal_fwd: null buffer");
+  if (!aligned16(x) || !aligned16(y)) return fail(HYC_EINVAL, "hyc_softmax_causal_fwd: x and y must be 16-byte aligned");
+  hipStream_t st = begin_launch(stream);
+  const float thr = round_to_bf16(threshold);
+  const int cpl = (int)((N / 8 + 63) / 64);
+  const int64_t blocks = (rows + 3) / 4, cap = 256 * 8;
+  const dim3 grid((unsigned)(blocks < cap ? blocks : cap));
+#define HYC_SMC(C_)                                                                                               \
+  hipLaunchKernelGGL((k_softmax_fwd_wave<C_, true>), grid, dim3(256), 0, st, static_cast<const uint16_t*>(x), rows, N, \
+                     thr, static_cast<uint16_t*>(y), counts, period)
+  if (cpl <= 1) HYC_SMC(1); else if (cpl <= 2) HYC_SMC(2); else if (cpl <= 4) HYC_SMC(4); else HYC_SMC(8);
+#undef HYC_SMC
+  return check_launch("hyc_softmax_causal_fwd");
 }
 
 int hyc_softmax_fill(const void* y, int64_t rows, int64_t N, float threshold, const int32_t* row_ptr, int32_t* cols,

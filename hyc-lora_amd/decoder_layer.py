@@ -187,18 +187,19 @@ class _AttentionFunc(torch.autograd.Function):
         cfg = mod.cfg
         b, nh, s, hd = q.shape
         scale = 1.0 / math.sqrt(hd)
-        scores = q @ k.transpose(-2, -1)
-        scores.mul_(scale)
-        causal = torch.ones(s, s, dtype=torch.bool, device=q.device).triu_(1)
-        scores.masked_fill_(causal, torch.finfo(BF16).min)       # the additive mask of the reference, saturated
+        # scores = (q @ k^T) / sqrt(hd) as one library GEMM; the causal mask is applied inside the softmax kernel,
+        # which never reads the masked half
+        q3, k3 = q.reshape(b * nh, s, hd), k.reshape(b * nh, s, hd)
+        scores = torch.baddbmm(q.new_zeros(1), q3, k3.transpose(1, 2), beta=0.0,
+                               alpha=scale).view(b, nh, s, s)
         it = mod.iteration
         if not cfg.compress:
-            p, _ = K.softmax_fwd(scores)
+            p, _ = K.softmax_fwd(scores, causal_period=s)
             sparse = p                                             # kept whole, in bf16
         elif it >= 2:
-            p, sparse = K.softmax_fwd(scores, float(mod.static_value))
+            p, sparse = K.softmax_fwd(scores, float(mod.static_value), causal_period=s)
         else:
-            p, _ = K.softmax_fwd(scores)
+            p, _ = K.softmax_fwd(scores, causal_period=s)
             thr = get_statistics_softmax(p, it, cfg.softmax_ratio)
             mod.static_value = thr if mod.static_value is None else (it * mod.static_value + thr) / (it + 1)
             sparse = K.softmax_sparsify(p, float(thr))
@@ -235,12 +236,14 @@ class _AttentionFunc(torch.autograd.Function):
             ds = torch._softmax_backward_data(dp, p, -1, BF16)
             del p, v
         del dp
-        ds.mul_(1.0 / math.sqrt(hd))
-        kk = _rows_to_heads(restore(ctx.saved[1]), b, nh, s, hd)
-        dq = ds @ kk
+        scale = 1.0 / math.sqrt(hd)
+        empty = g.new_zeros(1)                                   # ignored (beta = 0), only has to broadcast
+        ds3 = ds.view(b * nh, s, s)
+        kk = _rows_to_heads(restore(ctx.saved[1]), b, nh, s, hd).reshape(b * nh, s, hd)
+        dq = torch.baddbmm(empty, ds3, kk, beta=0.0, alpha=scale).view(b, nh, s, hd)
         del kk
-        qq = _rows_to_heads(restore(ctx.saved[0]), b, nh, s, hd)
-        dk = ds.transpose(-2, -1) @ qq
+        qq = _rows_to_heads(restore(ctx.saved[0]), b, nh, s, hd).reshape(b * nh, s, hd)
+        dk = torch.baddbmm(empty, ds3.transpose(1, 2), qq, beta=0.0, alpha=scale).view(b, nh, s, hd)
         ctx.saved = ctx.sparse = None
         return dq, dk, dv, None
 

@@ -451,19 +451,23 @@ def _csr_from_counts(lib, y2d, threshold, counts):
     return row_ptr, cols, vals
 
 
-def softmax_fwd(x, threshold=None):
-    """y = softmax(x, -1) bf16; with a threshold also the kept entries (y > bf16(threshold)) as SparseRows"""
+def softmax_fwd(x, threshold=None, causal_period=None):
+    """y = softmax(x, -1) bf16; with a threshold also the kept entries (y > bf16(threshold)) as SparseRows.
+    causal_period = S applies the causal mask of S query positions inside the kernel (row r is position r % S)."""
     _need(x, BF16, "x")
     N = x.shape[-1]
     x2 = x.reshape(-1, N)
     rows = x2.shape[0]
     lib = _abi.load()
     y = torch.empty_like(x2)
+    counts = None if threshold is None else torch.empty(rows, dtype=torch.int32, device=x.device)
+    thr = 0.0 if threshold is None else float(threshold)
+    if causal_period is None:
+        check(lib.hyc_softmax_fwd(_p(x2), rows, N, thr, _p(y), _p(counts), _stream()))
+    else:
+        check(lib.hyc_softmax_causal_fwd(_p(x2), rows, N, int(causal_period), thr, _p(y), _p(counts), _stream()))
     if threshold is None:
-        check(lib.hyc_softmax_fwd(_p(x2), rows, N, 0.0, _p(y), None, _stream()))
         return y.reshape(x.shape), None
-    counts = torch.empty(rows, dtype=torch.int32, device=x.device)
-    check(lib.hyc_softmax_fwd(_p(x2), rows, N, float(threshold), _p(y), _p(counts), _stream()))
     row_ptr, cols, vals = _csr_from_counts(lib, y, threshold, counts)
     return y.reshape(x.shape), SparseRows(row_ptr, cols, vals, tuple(x.shape))
 

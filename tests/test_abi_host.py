@@ -84,6 +84,10 @@ def test_argument_errors_without_a_gpu(abi):
     assert lib.hyc_gradw_gemm(null, 20, null, null, null, 4, 20, 4096, ctypes.byref(d), 1.0, 0.0, 0x10, 0, null, null) == abi.ENOTSUP
     assert lib.hyc_softmax_fwd(null, 4, 12, 0.0, 0x10, null, null) == abi.ENOTSUP
     assert lib.hyc_low_rank_update(null, null, null, null, 4, 0, 64, 2, 1, null) == abi.EINVAL
+    assert lib.hyc_softmax_causal_fwd(null, 4, 8192, 4, 0.0, null, null, null) == abi.ENOTSUP
+    assert lib.hyc_softmax_causal_fwd(null, 4, 64, 0, 0.0, null, null, null) == abi.EINVAL
+    assert lib.hyc_softmax_causal_fwd(null, 4, 64, 65, 0.0, null, null, null) == abi.EINVAL
+    assert lib.hyc_softmax_causal_fwd(null, 4, 64, 4, 0.0, null, null, null) == abi.EFAULT
     assert lib.hyc_kth_value_workspace_bytes() >= 1024 + 12
     assert lib.hyc_kth_value(null, 7, 10, 1, null, null, null) == abi.ENOTSUP
     assert lib.hyc_kth_value(null, abi.DTYPE_F32, 0, 1, null, null, null) == abi.EINVAL

@@ -526,3 +526,24 @@ def test_kth_value_softmax_shape(K):
     k = int(p[0].numel() * 0.95)
     want = torch.kthvalue(p[0].float().flatten(), k).values
     assert float(K.kth_value(p[0].cuda(), k)) == float(want)
+
+
+@pytest.mark.parametrize("shape,period", [((2, 3, 64, 64), 64), ((1, 2, 40, 1024), 40), ((1, 1, 24, 4096), 24), ((3, 50, 72), 50)])
+def test_softmax_causal(K, shape, period):
+    """the causal variant equals the plain kernel fed with explicitly masked scores, bit for bit, whatever the
+    masked positions of its own input hold; masked outputs are exact zeros and the counts agree"""
+    gen = torch.Generator().manual_seed(15)
+    x = (2 * torch.randn(*shape, generator=gen)).bfloat16()
+    N = shape[-1]
+    rows = x.reshape(-1, N).shape[0]
+    pos = torch.arange(rows) % period
+    hidden = (torch.arange(N)[None, :] > pos[:, None]).reshape(shape)
+    masked = x.masked_fill(hidden, torch.finfo(torch.bfloat16).min)
+    garbage = torch.where(hidden, torch.full_like(x, float("nan")), x)
+    want, sp_want = K.softmax_fwd(masked.cuda(), 0.01)
+    got, sp_got = K.softmax_fwd(garbage.cuda(), 0.01, causal_period=period)
+    assert bits_equal(got.cpu(), want.cpu())
+    assert torch.equal(got.cpu()[hidden], torch.zeros(int(hidden.sum()), dtype=torch.bfloat16))
+    assert torch.equal(sp_got.row_ptr, sp_want.row_ptr) and torch.equal(sp_got.cols, sp_want.cols)
+    ref = torch.softmax(masked.float(), -1).bfloat16()
+    assert bf16_ulp_diff(got.cpu(), ref).max() <= 1
