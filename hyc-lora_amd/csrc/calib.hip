@@ -29,30 +29,45 @@ k_channel_absmax(const uint16_t* __restrict__ x, int64_t M, int64_t H, unsigned 
   for (int j = 0; j < 8; ++j) atomicMax(amax_bits + 8 * cc + j, m[j] << 16);   // non-negative floats order as uints
 }
 
-// selected(c) <=> #{c' : s[c'] > s[c] or (s[c'] == s[c] and c' < c)} < k ; mask byte per chunk into plan's low byte
+// selected(c) <=> #{c' : s[c'] > s[c] or (s[c'] == s[c] and c' < c)} < k ; mask byte per chunk into plan's low byte.
+// A workgroup ranks 32 channels; its 8 sub-groups of 32 threads each count over one eighth of every tile of scores,
+// and the eight partial ranks of a channel are added through LDS.
+constexpr int RANK_CH = 32, RANK_SUB = 8, RANK_TILE = 4096;
 __global__ void __launch_bounds__(256)
 k_select_rank(const float* __restrict__ amax, int H, int k, uint32_t* __restrict__ plan) {
-  __shared__ float tile[1024];
-  const int c = blockIdx.x * 256 + threadIdx.x;
+  __shared__ float tile[RANK_TILE];
+  __shared__ int part[RANK_SUB][RANK_CH];
+  const int ch = threadIdx.x & (RANK_CH - 1), sub = threadIdx.x / RANK_CH;
+  const int c = blockIdx.x * RANK_CH + ch;
   const float my = c < H ? amax[c] : 0.f;
   int rank = 0;
-  for (int base = 0; base < H; base += 1024) {
+  constexpr int SPAN = RANK_TILE / RANK_SUB;
+  for (int base = 0; base < H; base += RANK_TILE) {
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < RANK_TILE / 256; ++u) {
       const int i = base + u * 256 + threadIdx.x;
       tile[u * 256 + threadIdx.x] = i < H ? amax[i] : -1.f;
     }
     __syncthreads();
-    for (int i = 0; i < 1024; ++i) {
-      const float s = tile[i];
-      rank += (s > my || (s == my && base + i < c)) ? 1 : 0;
+    const int first = sub * SPAN;
+#pragma unroll 8
+    for (int i = 0; i < SPAN; ++i) {
+      const float s = tile[first + i];
+      rank += (s > my || (s == my && base + first + i < c)) ? 1 : 0;
     }
     __syncthreads();
   }
-  const bool sel = (c < H) && (rank < k);
-  const unsigned long long ballot = __ballot(sel);
-  const int lane = threadIdx.x & 63;
-  if ((lane & 7) == 0 && c < H) plan[c >> 3] = (uint32_t)((ballot >> lane) & 0xFFull);
+  part[sub][ch] = rank;
+  __syncthreads();
+  if (threadIdx.x < RANK_CH) {
+    int total = 0;
+#pragma unroll
+    for (int u = 0; u < RANK_SUB; ++u) total += part[u][threadIdx.x];
+    const bool sel = (c < H) && (total < k);
+    const unsigned long long ballot = __ballot(sel);
+    const int lane = threadIdx.x & 63;
+    if ((lane & 7) == 0 && c < H) plan[c >> 3] = (uint32_t)((ballot >> lane) & 0xFFull);
+  }
 }
 
 // one workgroup: prefix counts into plan's high half, ascending channel list into idx
@@ -111,7 +126,7 @@ int hyc_select_channels(const float* amax, int64_t H, int32_t k, int32_t* idx, u
   if (k < 0 || k > H || k > 65535) return fail(HYC_EINVAL, "hyc_select_channels: k=%d", k);
   if (!amax || !plan || (k > 0 && !idx)) return fail(HYC_EFAULT, "hyc_select_channels: null buffer");
   hipStream_t st = begin_launch(stream);
-  hipLaunchKernelGGL(k_select_rank, dim3((unsigned)((H + 255) / 256)), dim3(256), 0, st, amax, (int)H, (int)k, plan);
+  hipLaunchKernelGGL(k_select_rank, dim3((unsigned)((H + RANK_CH - 1) / RANK_CH)), dim3(256), 0, st, amax, (int)H, (int)k, plan);
   hipLaunchKernelGGL(k_select_finish, dim3(1), dim3(1024), 0, st, (int)H, plan, idx);
   return check_launch("hyc_select_channels");
 }

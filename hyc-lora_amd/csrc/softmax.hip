@@ -74,11 +74,15 @@ k_softmax_fwd_wave(const uint16_t* __restrict__ x, int64_t rows, int64_t N, floa
   bool on[CPL];
 #pragma unroll
   for (int u = 0; u < CPL; ++u) on[u] = lane + 64 * u < nch;
-  // last visible column of a row (everything when not causal)
-  auto last_col = [&](int64_t r) __attribute__((always_inline)) { return CAUSAL ? (int)(r % period) : (int)N - 1; };
+  // last visible column of the current row (everything when not causal); rows advance by a fixed stride, so the
+  // position advances by stride mod period with one conditional subtraction
+  const int per = CAUSAL ? (int)period : 1;
+  const int step = CAUSAL ? (int)(stride % period) : 0;
+  int pos = CAUSAL && row < rows ? (int)(row % period) : 0;
+  auto wrap = [&](int p) __attribute__((always_inline)) { return p >= per ? p - per : p; };
   uint4 raw[CPL];
   if (row < rows) {
-    const int lc = last_col(row);
+    const int lc = CAUSAL ? pos : (int)N - 1;
 #pragma unroll
     for (int u = 0; u < CPL; ++u)
       raw[u] = on[u] && 8 * (lane + 64 * u) <= lc ? *reinterpret_cast<const uint4*>(x + row * N + 8 * (lane + 64 * u))
@@ -86,8 +90,9 @@ k_softmax_fwd_wave(const uint16_t* __restrict__ x, int64_t rows, int64_t N, floa
   }
   for (; row < rows; row += stride) {
     uint4 nxt[CPL];
+    const int pos_next = wrap(pos + step);
     if (row + stride < rows) {
-      const int lc = last_col(row + stride);
+      const int lc = CAUSAL ? pos_next : (int)N - 1;
 #pragma unroll
       for (int u = 0; u < CPL; ++u)
         nxt[u] = on[u] && 8 * (lane + 64 * u) <= lc
@@ -95,9 +100,16 @@ k_softmax_fwd_wave(const uint16_t* __restrict__ x, int64_t rows, int64_t N, floa
     }
     float v[CPL][8];
     float m = -INFINITY;
-    const int lc = last_col(row);
+    const int lc = CAUSAL ? pos : (int)N - 1;
+    pos = pos_next;
+    // a 512-column slice of the row (one chunk per lane) that lies wholly beyond the position is skipped by the
+    // whole wave: no max, no exp, zeros stored
+    bool live[CPL];
+#pragma unroll
+    for (int u = 0; u < CPL; ++u) live[u] = !CAUSAL || 512 * u <= lc;
 #pragma unroll
     for (int u = 0; u < CPL; ++u) {
+      if (!live[u]) continue;
       unpack8(raw[u], v[u]);
       if (CAUSAL) {
 #pragma unroll
@@ -111,24 +123,31 @@ k_softmax_fwd_wave(const uint16_t* __restrict__ x, int64_t rows, int64_t N, floa
     m = group_reduce<64>(m, OpMax());
     float l = 0.f;
 #pragma unroll
-    for (int u = 0; u < CPL; ++u)
+    for (int u = 0; u < CPL; ++u) {
+      if (!live[u]) continue;
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         // the clamp keeps x*log2(e) finite for mask values near the bottom of the bf16 range (e^-128 is 0 in fp32)
         v[u][j] = on[u] ? exp_fast(fmaxf(v[u][j] - m, -128.f)) : 0.f;
         l += v[u][j];
       }
+    }
     l = wave_sum(l);
     const float inv = 1.0f / l;
     int kept = 0;
 #pragma unroll
     for (int u = 0; u < CPL; ++u) {
+      if (live[u]) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        v[u][j] = bfr(v[u][j] * inv);
-        kept += (v[u][j] > thr) ? 1 : 0;
+        for (int j = 0; j < 8; ++j) {
+          v[u][j] = bfr(v[u][j] * inv);
+          kept += (v[u][j] > thr) ? 1 : 0;
+        }
+        if (on[u]) store_stream(y + row * N + 8 * (lane + 64 * u), pack8(v[u]));
+      } else if (on[u]) {
+        kept += 0.f > thr ? 8 : 0;
+        store_stream(y + row * N + 8 * (lane + 64 * u), make_uint4(0, 0, 0, 0));
       }
-      if (on[u]) store_stream(y + row * N + 8 * (lane + 64 * u), pack8(v[u]));
     }
     if (counts) {
       const float total = wave_sum((float)kept);
