@@ -22,7 +22,7 @@ from dataclasses import dataclass
 import torch
 
 from . import kernels as K
-from .operators._calibration import CompressionSite
+from .operators._calibration import CompressionSite, running_mean
 from .operators.compress_function import get_statistics_softmax
 from .operators.efficient_hadamard import EfficientMemoryGatedAct
 from .operators.efficient_rmsnorm import EfficientMemoryRMSNorm
@@ -201,7 +201,7 @@ class _AttentionFunc(torch.autograd.Function):
         else:
             p, _ = K.softmax_fwd(scores, causal_period=s)
             thr = get_statistics_softmax(p, it, cfg.softmax_ratio)
-            mod.static_value = thr if mod.static_value is None else (it * mod.static_value + thr) / (it + 1)
+            mod.static_value = running_mean(mod.static_value, thr, it)
             sparse = K.softmax_sparsify(p, float(thr))
         del scores
         out = p @ v

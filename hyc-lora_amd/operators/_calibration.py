@@ -18,6 +18,13 @@ from .compress_function import pad_cut_L
 MODES = ("ref", "hyc")
 
 
+def running_mean(previous, fresh, iteration):
+    """mean over the calibration calls so far: `fresh` on the first call, (iteration*previous + fresh)/(iteration+1) after"""
+    if previous is None:
+        return fresh
+    return (iteration * previous + fresh) / (iteration + 1)
+
+
 def fold_statistics(static_value, iteration, outlier, L, scale, R):
     """one step of the running mean over the calibration calls; returns the new list"""
     fresh = [outlier, L, scale, R]

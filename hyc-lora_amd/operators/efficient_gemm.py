@@ -9,7 +9,7 @@ compress / decompress / sparsify work around them goes through the HIP kernels.
 import torch
 
 from .. import kernels as K
-from ._calibration import CompressionSite, fold_statistics
+from ._calibration import CompressionSite, fold_statistics, running_mean
 from .compress_function import (compress_to_csr, get_statistics, get_statistics_softmax, head_to_hidden_shape,
                                 hidden_to_head_shape)
 
@@ -194,8 +194,7 @@ class EfficientMemoryGEMMWithSoftmax(torch.nn.Module):
             # the probabilities keep the reference's threshold rule; only v uses the channel scheme
             if self.iteration < 2:
                 o1 = get_statistics_softmax(x1, self.iteration, self.outlier_ratio_1)
-                self.static_value_1 = o1 if self.static_value_1 is None else \
-                    (self.iteration * self.static_value_1 + o1) / (self.iteration + 1)
+                self.static_value_1 = running_mean(self.static_value_1, o1, self.iteration)
             else:
                 o1 = self.static_value_1
             r2, _ = _as_hidden_rows(x2)
@@ -207,8 +206,7 @@ class EfficientMemoryGEMMWithSoftmax(torch.nn.Module):
             x1, x2, self.outlier_ratio_1, self.outlier_ratio_2, self.sub_outlier_ratio_2, self.sub_outlier_bit_2,
             self.sub_outlier_quantize_method_2, self.rank, self.iteration, self.static_value_1, self.static_value_2)
         if self.iteration < 2:
-            self.static_value_1 = o1 if self.static_value_1 is None else \
-                (self.iteration * self.static_value_1 + o1) / (self.iteration + 1)
+            self.static_value_1 = running_mean(self.static_value_1, o1, self.iteration)
             self.static_value_2 = fold_statistics(self.static_value_2, self.iteration, o2, L2, s2, R2)
         self.iteration += 1
         return result

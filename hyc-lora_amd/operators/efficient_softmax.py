@@ -1,44 +1,51 @@
-"""Softmax that keeps only the probabilities above a calibrated threshold for its backward.
-Reference: operators/efficient_softmax.py:10-75."""
+"""Softmax over the last dimension whose backward runs from the few probabilities above a calibrated threshold.
+
+Mirror of the reference's operators/efficient_softmax.py:10-75 (same class names, `apply` signature, `iteration` /
+`static_value` attributes).  Steady state is one kernel for y plus the per-row counts of kept entries and one kernel
+that writes them as CSR (int32 column, bf16 value); the backward reads the incoming gradient once:
+dx = (g - sum_j g_j * p_j) * p with p zero outside the kept set.
+"""
 import torch
 
 from .. import kernels as K
+from ._calibration import running_mean
 from .compress_function import get_statistics_softmax
+
+_CALIBRATION_CALLS = 2      # the threshold is measured on the first two calls and frozen afterwards
 
 
 class EfficientMemorySoftmaxFunc(torch.autograd.Function):
-    """apply(x, outlier_ratio, iteration, static_value) -> (softmax(x, -1), outlier)"""
+    """apply(x, outlier_ratio, iteration, static_value) -> (softmax(x, -1), threshold)"""
 
     @staticmethod
     def forward(ctx, x, outlier_ratio, iteration, static_value):
-        x = x.contiguous()
-        if iteration < 2:
-            y, _ = K.softmax_fwd(x)
-            outlier = get_statistics_softmax(y, iteration, outlier_ratio)
-            ctx.y_sparse = K.softmax_sparsify(y, float(outlier))
+        scores = x.contiguous()
+        if iteration >= _CALIBRATION_CALLS:
+            threshold = static_value
+            probs, ctx.kept = K.softmax_fwd(scores, float(threshold))
         else:
-            outlier = static_value
-            y, ctx.y_sparse = K.softmax_fwd(x, float(outlier))
-        ctx.mark_non_differentiable(outlier)
-        return y, outlier
+            # the threshold of this call comes from its own probabilities, so they are needed before the pruning
+            probs, _ = K.softmax_fwd(scores)
+            threshold = get_statistics_softmax(probs, iteration, outlier_ratio)
+            ctx.kept = K.softmax_sparsify(probs, float(threshold))
+        ctx.mark_non_differentiable(threshold)
+        return probs, threshold
 
     @staticmethod
-    def backward(ctx, grad_output, grad_outlier):
-        g = grad_output.to(torch.bfloat16).contiguous()
-        return K.softmax_bwd(g, ctx.y_sparse), None, None, None
+    def backward(ctx, grad_probs, _grad_threshold):
+        return K.softmax_bwd(grad_probs.to(torch.bfloat16).contiguous(), ctx.kept), None, None, None
 
 
 class EfficientMemorySoftmax(torch.nn.Module):
     def __init__(self, outlier_ratio: float = 0.01):
-        super(EfficientMemorySoftmax, self).__init__()
+        super().__init__()
         self.outlier_ratio = outlier_ratio
         self.iteration = 0
         self.static_value = None
 
     def forward(self, x):
-        result, outlier = EfficientMemorySoftmaxFunc.apply(x, self.outlier_ratio, self.iteration, self.static_value)
-        if self.iteration < 2:
-            self.static_value = (outlier if self.static_value is None
-                                 else (self.iteration * self.static_value + outlier) / (self.iteration + 1))
+        probs, threshold = EfficientMemorySoftmaxFunc.apply(x, self.outlier_ratio, self.iteration, self.static_value)
+        if self.iteration < _CALIBRATION_CALLS:
+            self.static_value = running_mean(self.static_value, threshold, self.iteration)
         self.iteration += 1
-        return result
+        return probs
