@@ -68,6 +68,8 @@ SIGNATURES = {
     "hyc_low_rank_update": (c_i32, [c_ptr, c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_i64, c_i32, c_i32, c_ptr]),
     "hyc_kth_value_workspace_bytes": (c_i64, []),
     "hyc_kth_value": (c_i32, [c_ptr, c_i32, c_i64, c_i64, c_ptr, c_ptr, c_ptr]),
+    "hyc_rope_to_heads": (c_i32, [c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_i64, c_i64, c_ptr, c_ptr, c_ptr]),
+    "hyc_rope_from_heads": (c_i32, [c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_i64, c_i64, c_ptr, c_ptr]),
     "hyc_nf4_quantize": (c_i32, [c_ptr, c_i64, c_ptr, c_ptr, c_ptr]),
     "hyc_nf4_dequantize": (c_i32, [c_ptr, c_ptr, c_i64, c_ptr, c_ptr]),
 }

@@ -143,21 +143,11 @@ def rope_tables(S, head_dim, theta, device):
     return emb.cos().to(BF16), emb.sin().to(BF16)
 
 
-def rotate_half(x):
-    half = x.shape[-1] // 2
-    return torch.cat((-x[..., half:], x[..., :half]), dim=-1)
-
-
-def apply_rope(x, cos, sin):
-    """x [B, nh, S, hd]; cos / sin [S, hd] (models/modeling_llama.py:236-260)"""
-    return x * cos + rotate_half(x) * sin
-
-
 class CompressedAttention(torch.nn.Module):
-    """softmax(q @ k^T / sqrt(hd) + causal mask) @ v with q, k, v saved as codes in the [B*S, nh*hd] layout and the
-    probabilities saved once as the entries above a calibrated threshold.  Composition of the reference's gemm1,
-    softmax and gemm2 modules (models/modeling_llama.py:444-462, operators/efficient_gemm.py,
-    operators/efficient_softmax.py)."""
+    """RoPE, softmax(q @ k^T / sqrt(hd) + causal mask) @ v on the [B, S, H] projections, with q, k (after RoPE) and v
+    saved as codes in the [B*S, nh*hd] layout and the probabilities saved once as the entries above a calibrated
+    threshold.  Composition of apply_rotary_pos_emb and the reference's gemm1, softmax and gemm2 modules
+    (models/modeling_llama.py:423-462, operators/efficient_gemm.py, operators/efficient_softmax.py)."""
 
     def __init__(self, cfg: LayerConfig):
         super().__init__()
@@ -168,30 +158,28 @@ class CompressedAttention(torch.nn.Module):
         self.static_value = None          # probability threshold, as in EfficientMemorySoftmax
         self.record = None
 
-    def forward(self, q, k, v):
-        return _AttentionFunc.apply(q, k, v, self)
-
-
-def _heads_to_rows(x):
-    b, nh, s, hd = x.shape
-    return x.transpose(1, 2).reshape(b * s, nh * hd)
-
-
-def _rows_to_heads(x2d, b, nh, s, hd):
-    return x2d.reshape(b, s, nh, hd).transpose(1, 2)
+    def forward(self, q, k, v, cos, sin):
+        return _AttentionFunc.apply(q, k, v, cos, sin, self)
 
 
 class _AttentionFunc(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, q, k, v, mod):
+    def forward(ctx, q, k, v, cos, sin, mod):
         cfg = mod.cfg
-        b, nh, s, hd = q.shape
+        b, s, H = q.shape
+        nh, hd = cfg.heads, cfg.head_dim
         scale = 1.0 / math.sqrt(hd)
+        # one pass per tensor: rotate, and write both the head-major copy the batched GEMMs need and the rows that
+        # are compressed
+        qh, q_rows = K.rope_to_heads(q.contiguous(), nh, cos, sin, want_rows=True)
+        kh, k_rows = K.rope_to_heads(k.contiguous(), nh, cos, sin, want_rows=True)
+        v_rows = v.contiguous()
+        vh = K.rope_to_heads(v_rows, nh)
         # scores = (q @ k^T) / sqrt(hd) as one library GEMM; the causal mask is applied inside the softmax kernel,
         # which never reads the masked half
-        q3, k3 = q.reshape(b * nh, s, hd), k.reshape(b * nh, s, hd)
-        scores = torch.baddbmm(q.new_zeros(1), q3, k3.transpose(1, 2), beta=0.0,
+        scores = torch.baddbmm(q.new_zeros(1), qh.view(b * nh, s, hd), kh.view(b * nh, s, hd).transpose(1, 2), beta=0.0,
                                alpha=scale).view(b, nh, s, s)
+        del qh, kh
         it = mod.iteration
         if not cfg.compress:
             p, _ = K.softmax_fwd(scores, causal_period=s)
@@ -204,48 +192,57 @@ class _AttentionFunc(torch.autograd.Function):
             mod.static_value = running_mean(mod.static_value, thr, it)
             sparse = K.softmax_sparsify(p, float(thr))
         del scores
-        out = p @ v
-        rows = [_heads_to_rows(t) for t in (q, k, v)]
+        out = K.rope_from_heads(torch.bmm(p.view(b * nh, s, s), vh.view(b * nh, s, hd)).view(b, nh, s, hd))   # [B, S, H]
+        del vh
+        rows = [t.view(b * s, H) for t in (q_rows, k_rows, v_rows)]
         if cfg.compress:
             saved = []
             for site, r in zip((mod.site_q, mod.site_k, mod.site_v), rows):
                 plan = site.channel_plan(r, it)
                 saved.append(K.compress_channel(r, plan, cfg.act_bits, cfg.act_group))
         else:
-            saved = [r.contiguous() for r in rows]
+            saved = rows
         mod.iteration += 1
         if mod.record is not None:
             mod.record.update(q=rows[0].detach().clone(), k=rows[1].detach().clone(), v=rows[2].detach().clone(),
                               p=p.detach().clone(), saved=saved, sparse=sparse)
         ctx.saved, ctx.sparse, ctx.geom, ctx.compress = saved, sparse, (b, nh, s, hd), cfg.compress
+        ctx.save_for_backward(cos, sin)
         return out
 
     @staticmethod
     def backward(ctx, g):
         b, nh, s, hd = ctx.geom
+        cos, sin = ctx.saved_tensors
         restore = (lambda c: K.decompress_channel(c)) if ctx.compress else (lambda c: c)
-        g = g.to(BF16)
-        v = _rows_to_heads(restore(ctx.saved[2]), b, nh, s, hd)
-        p = K.softmax_dense(ctx.sparse) if ctx.compress else ctx.sparse
-        dv = p.transpose(-2, -1) @ g
-        dp = g @ v.transpose(-2, -1)
+        to_heads = lambda rows: K.rope_to_heads(rows.view(b, s, nh * hd), nh).view(b * nh, s, hd)
+        gh = K.rope_to_heads(g.to(BF16).contiguous(), nh).view(b * nh, s, hd)
+        v = to_heads(restore(ctx.saved[2]))
+        p = (K.softmax_dense(ctx.sparse) if ctx.compress else ctx.sparse).view(b * nh, s, s)
+        dv = torch.bmm(p.transpose(1, 2), gh)
+        dp = torch.bmm(gh, v.transpose(1, 2))
+        del v, gh
         if ctx.compress:
-            del p, v
-            ds = K.softmax_bwd(dp.contiguous(), ctx.sparse)
+            del p
+            ds = K.softmax_bwd(dp.view(b, nh, s, s), ctx.sparse)
         else:
             ds = torch._softmax_backward_data(dp, p, -1, BF16)
-            del p, v
+            del p
         del dp
         scale = 1.0 / math.sqrt(hd)
-        empty = g.new_zeros(1)                                   # ignored (beta = 0), only has to broadcast
+        zero = g.new_zeros(1).to(BF16)                           # ignored (beta = 0), only has to broadcast
         ds3 = ds.view(b * nh, s, s)
-        kk = _rows_to_heads(restore(ctx.saved[1]), b, nh, s, hd).reshape(b * nh, s, hd)
-        dq = torch.baddbmm(empty, ds3, kk, beta=0.0, alpha=scale).view(b, nh, s, hd)
+        kk = to_heads(restore(ctx.saved[1]))
+        dq = torch.baddbmm(zero, ds3, kk, beta=0.0, alpha=scale)
         del kk
-        qq = _rows_to_heads(restore(ctx.saved[0]), b, nh, s, hd).reshape(b * nh, s, hd)
-        dk = torch.baddbmm(empty, ds3.transpose(1, 2), qq, beta=0.0, alpha=scale).view(b, nh, s, hd)
+        qq = to_heads(restore(ctx.saved[0]))
+        dk = torch.baddbmm(zero, ds3.transpose(1, 2), qq, beta=0.0, alpha=scale)
+        del qq, ds, ds3
         ctx.saved = ctx.sparse = None
-        return dq, dk, dv, None
+        dq = K.rope_from_heads(dq.view(b, nh, s, hd), cos, sin)
+        dk = K.rope_from_heads(dk.view(b, nh, s, hd), cos, sin)
+        dv = K.rope_from_heads(dv.view(b, nh, s, hd))
+        return dq, dk, dv, None, None, None
 
 
 # ---- the layer --------------------------------------------------------------------------------------------------
@@ -293,11 +290,7 @@ class DecoderLayer(torch.nn.Module):
         cos, sin = self._rope
         h = self.input_layernorm(x)
         q, k, v = self.qkv_proj(h)
-        heads = lambda t: t.view(b, s, cfg.heads, cfg.head_dim).transpose(1, 2)
-        q, k, v = apply_rope(heads(q), cos, sin), apply_rope(heads(k), cos, sin), heads(v)
-        a = self.attention(q, k, v)
-        a = a.transpose(1, 2).reshape(b, s, H)
-        x = x + self.o_proj(a)
+        x = x + self.o_proj(self.attention(q, k, v, cos, sin))
         h = self.post_attention_layernorm(x)
         gate, up = self.gate_up_proj(h)
         m = self.act(gate, up) if self.act is not None else torch.nn.functional.silu(gate) * up

@@ -590,3 +590,27 @@ def nf4_dequantize(q: NF4Weight, out=None):
         out = torch.empty(q.shape, dtype=BF16, device=q.packed.device)
     check(_abi.load().hyc_nf4_dequantize(_p(q.packed), _p(q.absmax), n, _p(out), _stream()))
     return out
+
+
+# ----------------------------------------------------------------------------------------------------
+# rotary embedding + attention layout
+# ----------------------------------------------------------------------------------------------------
+def rope_to_heads(x, heads, cos=None, sin=None, want_rows=False):
+    """x bf16 [B, S, heads*hd] -> rotated [B, heads, S, hd] contiguous (and, with want_rows, also [B, S, heads*hd]);
+    cos / sin bf16 [S, hd]; without them only the layout changes"""
+    _need(x, BF16, "x")
+    B, S, H = x.shape
+    hd = H // heads
+    out_heads = torch.empty((B, heads, S, hd), dtype=BF16, device=x.device)
+    out_rows = torch.empty_like(x) if want_rows else None
+    check(_abi.load().hyc_rope_to_heads(_p(x), _p(cos), _p(sin), B, S, heads, hd, _p(out_heads), _p(out_rows), _stream()))
+    return (out_heads, out_rows) if want_rows else out_heads
+
+
+def rope_from_heads(g, cos=None, sin=None):
+    """gradient bf16 [B, heads, S, hd] -> [B, S, heads*hd] through the transposed rotation"""
+    _need(g, BF16, "g")
+    B, heads, S, hd = g.shape
+    out = torch.empty((B, S, heads * hd), dtype=BF16, device=g.device)
+    check(_abi.load().hyc_rope_from_heads(_p(g), _p(cos), _p(sin), B, S, heads, hd, _p(out), _stream()))
+    return out

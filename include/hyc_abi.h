@@ -35,6 +35,8 @@
  *       grad_weight = grad_output^T @ decompress(x), operators/efficient_linear.py:56-67
  *   hyc_low_rank_update
  *       low_rank_extraction / low_rank_addition, operators/fused_compression.py:80-99, :184-210
+ *   hyc_rope_to_heads / hyc_rope_from_heads
+ *       apply_rotary_pos_emb and the head-major transposition around it, models/modeling_llama.py:236-260, :423-425
  *   hyc_nf4_dequantize / hyc_nf4_quantize
  *       F.dequantize_4bit(B, quant_state) before each frozen-base matmul, bitsandbytes_fix/_function.py:509, :540
  *       (the quantiser that wrote B is bitsandbytes' own and is not part of the reference tree)
@@ -216,6 +218,20 @@ int hyc_gradw_gemm(const void* dy, int64_t ldy, const void* stored, const void* 
 /* out[m, :] = bf16(x[m, :] -/+ L[m mod S, :] @ R); L bf16 [S, rank], R bf16 [rank, H]; out may alias x */
 int hyc_low_rank_update(const void* L, const void* R, const void* x, void* out, int64_t M, int64_t S, int64_t H,
                         int32_t rank, int32_t subtract, void* stream);
+
+/* ---- rotary embedding + attention layout ----------------------------------------------------- */
+/* x bf16 [B, S, heads, head_dim] (what the projections produce) -> the rotated tensor as [B, heads, S, head_dim] in
+ * out_heads (what the batched attention GEMMs consume) and, when out_rows is not NULL, also in the input's layout
+ * (apply_rotary_pos_emb, models/modeling_llama.py:236-260, with the .view().transpose(1, 2) of :423-425).
+ *   y[i] = x[i] cos[i] - x[i+h] sin[i],  y[i+h] = x[i+h] cos[i+h] + x[i] sin[i+h],  h = head_dim / 2
+ * cos / sin bf16 [S, head_dim]; both NULL = layout change only (the value tensor).  fp32 arithmetic, one rounding.
+ * hyc_rope_from_heads is the transpose: gradients [B, heads, S, head_dim] -> [B, S, heads, head_dim],
+ *   dx[i] = g[i] cos[i] + g[i+h] sin[i+h],  dx[i+h] = g[i+h] cos[i+h] - g[i] sin[i].
+ * head_dim a multiple of 16. */
+int hyc_rope_to_heads(const void* x, const void* cosv, const void* sinv, int64_t B, int64_t S, int64_t heads,
+                      int64_t head_dim, void* out_heads, void* out_rows, void* stream);
+int hyc_rope_from_heads(const void* g, const void* cosv, const void* sinv, int64_t B, int64_t S, int64_t heads,
+                        int64_t head_dim, void* out_rows, void* stream);
 
 /* ---- NF4 frozen base weights ------------------------------------------------------------------- */
 /* Blocks of 64 consecutive weights: absmax[i] = max |w| of block i (fp32), packed byte j holds the level indices of

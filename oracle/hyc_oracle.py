@@ -31,6 +31,7 @@ Pinning status (see tests/test_oracle_*.py):
                                  kernels are Triton): parity unpinned by reference outputs
 * linear_bwd                   - torch.matmul in fp32
 * gemm_bwd                     - torch.autograd of torch.matmul in float64
+* rope_fwd / rope_bwd          - complex-number form of the rotation; float64 torch.autograd
 * hyc_select_channels / hyc group scales - parity unpinned (no reference code)
 * nf4_quantize / nf4_dequantize - parity unpinned (bitsandbytes is not in the reference tree); checked against
                                  the published level table: nearest level by exact distance, round trips
@@ -472,3 +473,25 @@ def nf4_quantize(w, block=64):
 def nf4_dequantize(packed, absmax, shape, block=64):
     codes = torch.stack([packed >> 4, packed & 15], dim=1).reshape(-1, block).long()
     return (NF4_LEVELS[codes] * absmax[:, None]).to(BF16).reshape(shape)
+
+
+# --------------------------------------------------------------------------------------
+# rotary position embedding                       models/modeling_llama.py:229-260
+# --------------------------------------------------------------------------------------
+def rotate_half(x):
+    """models/modeling_llama.py:229-233"""
+    half = x.shape[-1] // 2
+    return torch.cat((-x[..., half:], x[..., :half]), dim=-1)
+
+
+def rope_fwd(x, cos, sin):
+    """x [B, nh, S, hd], cos / sin [S, hd] -> x*cos + rotate_half(x)*sin (models/modeling_llama.py:258-259), in fp32
+    with one rounding to x's dtype (the reference rounds each of its three bf16 steps)"""
+    xf = x.float()
+    return (xf * cos.float() + rotate_half(xf) * sin.float()).to(x.dtype)
+
+
+def rope_bwd(g, cos, sin):
+    """transpose of rope_fwd: d/dx of sum(g * rope_fwd(x))"""
+    gf = g.float()
+    return (gf * cos.float() - rotate_half(gf * sin.float())).to(g.dtype)

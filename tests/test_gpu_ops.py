@@ -547,3 +547,28 @@ def test_softmax_causal(K, shape, period):
     assert torch.equal(sp_got.row_ptr, sp_want.row_ptr) and torch.equal(sp_got.cols, sp_want.cols)
     ref = torch.softmax(masked.float(), -1).bfloat16()
     assert bf16_ulp_diff(got.cpu(), ref).max() <= 1
+
+
+# ------------------------------------------------------------------ rotary embedding + layout
+@pytest.mark.parametrize("B,S,nh,hd", [(2, 64, 4, 64), (1, 100, 3, 32), (2, 33, 32, 128), (1, 7, 5, 16)])
+def test_rope_kernels(K, B, S, nh, hd):
+    """rotation within 1 bf16 ulp of the oracle in both layouts (the two outputs bit-identical to each other), its
+    transpose likewise, and the table-free form a bit-exact transposition; general tables (halves differ)"""
+    gen = torch.Generator().manual_seed(S)
+    x = torch.randn(B, S, nh * hd, generator=gen).bfloat16()
+    cos = torch.randn(S, hd, generator=gen).bfloat16()
+    sin = torch.randn(S, hd, generator=gen).bfloat16()
+    heads = lambda t: t.view(B, S, nh, hd).transpose(1, 2)
+    y_heads, y_rows = K.rope_to_heads(x.cuda(), nh, cos.cuda(), sin.cuda(), want_rows=True)
+    want = O.rope_fwd(heads(x), cos, sin)
+    assert y_heads.shape == (B, nh, S, hd) and y_heads.is_contiguous()
+    assert bf16_ulp_diff(y_heads.cpu(), want).max() <= 1
+    assert bits_equal(heads(y_rows.cpu()).contiguous(), y_heads.cpu())
+    only = K.rope_to_heads(x.cuda(), nh, cos.cuda(), sin.cuda())
+    assert bits_equal(only.cpu(), y_heads.cpu())
+    g = torch.randn(B, nh, S, hd, generator=gen).bfloat16()
+    dx = K.rope_from_heads(g.cuda(), cos.cuda(), sin.cuda())
+    want_dx = O.rope_bwd(g, cos, sin).transpose(1, 2).reshape(B, S, nh * hd)
+    assert bf16_ulp_diff(dx.cpu(), want_dx).max() <= 1
+    assert bits_equal(K.rope_to_heads(x.cuda(), nh).cpu(), heads(x).contiguous())
+    assert bits_equal(K.rope_from_heads(g.cuda()).cpu(), g.transpose(1, 2).reshape(B, S, nh * hd))

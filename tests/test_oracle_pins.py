@@ -407,3 +407,25 @@ def test_layer_oracle_against_plain_autograd():
     assert torch.allclose(Po2["A_q"].grad, 2 * Po["A_q"].grad, rtol=1e-4, atol=1e-6)
     assert torch.allclose(Po2["B_q"].grad, Po["B_q"].grad, rtol=1e-4, atol=1e-6)
     assert torch.allclose(Po2["A_o"].grad, Po["A_o"].grad, rtol=1e-4, atol=1e-6)
+
+
+def test_rope_against_complex_rotation_and_autograd():
+    """rope_fwd is the rotation of the pairs (x[i], x[i+h]) by the angle of (cos[i], sin[i]): checked as a complex
+    multiplication with independently built angles; rope_bwd against float64 autograd.  Distinct tables for the two
+    halves make a swapped half or a wrong sign fail."""
+    gen = torch.Generator().manual_seed(19)
+    B, nh, S, hd = 2, 3, 10, 16
+    h = hd // 2
+    x = torch.randn(B, nh, S, hd, generator=gen, dtype=torch.float64)
+    theta = torch.rand(S, h, generator=gen, dtype=torch.float64) * 6.28
+    cos, sin = torch.cat([theta.cos()] * 2, -1), torch.cat([theta.sin()] * 2, -1)
+    z = torch.complex(x[..., :h], x[..., h:]) * torch.polar(torch.ones_like(theta), theta)
+    want = torch.cat([z.real, z.imag], -1)
+    assert torch.allclose(O.rope_fwd(x, cos, sin), want, rtol=1e-5, atol=1e-5)
+    # general tables (the two halves differ): autograd of the reference expression
+    cos2, sin2 = torch.randn(S, hd, generator=gen, dtype=torch.float64), torch.randn(S, hd, generator=gen, dtype=torch.float64)
+    g = torch.randn(B, nh, S, hd, generator=gen, dtype=torch.float64)
+    xa = x.clone().requires_grad_(True)
+    (xa * cos2 + O.rotate_half(xa) * sin2).backward(g)
+    assert torch.allclose(O.rope_bwd(g, cos2, sin2), xa.grad, rtol=1e-5, atol=1e-5)
+    assert torch.allclose(O.rope_fwd(x, cos2, sin2), x * cos2 + O.rotate_half(x) * sin2, rtol=1e-5, atol=1e-5)
