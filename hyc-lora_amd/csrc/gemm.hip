@@ -9,6 +9,8 @@
 //
 // Because of the segment packing, one packed tile [tokens, 8c bytes] feeds NSEG separate ranges of output
 // columns; a workgroup owns all of them so the packed bytes are read once.
+#include <algorithm>
+
 #include "abi_util.hpp"
 #include "row_kernels.hpp"
 
@@ -224,7 +226,6 @@ __device__ __forceinline__ void gradw_direct_tile(const DirectArgs& A, float* re
   const int seg = MAINT ? hy / c_tiles : 0;
   const int c = MAINT ? (hy - seg * c_tiles) * 16 + l16 : 0;                     // chunk inside the segment
   const int q = MAINT ? 0 : hy * 16 + l16;                                       // outlier number
-  const bool lane_ok = MAINT ? c < CPS : q < ca.k;
   const int shs = (BITS == 8) ? 0 : seg * BITS;
   const int64_t m_begin = (int64_t)blockIdx.z * A.tokens_per_split;
   const int64_t m_end = m_begin + A.tokens_per_split < A.M ? m_begin + A.tokens_per_split : A.M;
@@ -444,6 +445,25 @@ constexpr int WK = 32;      // tokens per stage
 constexpr int WN = 128;     // dY features per workgroup: WN (four waves) or 2*WN (eight waves)
 constexpr int WH = 256;     // channels per workgroup
 
+// Buffer loads: a resource is (base, bytes); an offset at or beyond `bytes` reads as zero instead of faulting.
+typedef __amdgpu_buffer_rsrc_t BufferRsrc;
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ BufferRsrc make_rsrc(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ uint4 load_b128(BufferRsrc r, uint32_t off) {
+  const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, 0);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ uint2 load_b64(BufferRsrc r, uint32_t off) {
+  const u32x2_t v = __builtin_amdgcn_raw_buffer_load_b64(r, (int)off, 0, 0);
+  return make_uint2(v.x, v.y);
+}
+__device__ __forceinline__ uint32_t load_b16(BufferRsrc r, uint32_t off) {
+  return (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(r, (int)off, 0, 0);
+}
+
 template <int NSEG, int A_PER, int B_PER>
 struct WideRegs {            // one stage of global data per thread
   uint4 a[A_PER];            // dY chunks
@@ -506,33 +526,61 @@ k_gradw_wide(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_
     co.init(pw);
   }
 
-  // Loads past the token range re-read the last token with the dY operand zeroed; nothing is conditional.
-  auto fetch = [&](Regs& R, int64_t m0) __attribute__((always_inline)) {
+  // Every operand of the token loop is read through a buffer resource that spans exactly this workgroup's token
+  // range: the hardware drops what lies beyond it (rows past m_end, features past N_out, outlier slots a chunk
+  // does not have) and returns zeros, so nothing is clamped, predicated or branched on, and the address of a load
+  // is a per-thread constant.
+  const uint32_t gpr = (uint32_t)ca.groups_per_row, kk2 = 2u * (uint32_t)ca.k;
+  const uint32_t b_pitch = (SRC == 0) ? (uint32_t)SEG : 2u * (uint32_t)H;          // bytes per token of the x operand
+  constexpr uint32_t NOWHERE = 0x80000000u;              // beyond any resource of at most 2 GiB
+  uint32_t va[A_PER], vb[B_PER], vs[B_PER][NST], vo0[B_PER][NST], vo1[B_PER][NST];
 #pragma unroll
-    for (int u = 0; u < A_PER; ++u) {
-      const int idx = tid + u * THREADS;
-      const int row = idx / (WNT / 8), cc = idx % (WNT / 8);
-      const int64_t m = m0 + row, n = n0 + 8 * cc;
-      const bool ok = m < m_end && n < N_out;
-      const uint4 v = *reinterpret_cast<const uint4*>(dy + (m < m_end ? m : m_end - 1) * ldy + (n < N_out ? n : 0));
-      R.a[u] = ok ? v : make_uint4(0, 0, 0, 0);
+  for (int u = 0; u < A_PER; ++u) {
+    const int idx = tid + u * THREADS;
+    const int row = idx / (WNT / 8), cc = idx % (WNT / 8);
+    va[u] = n0 + 8 * cc < N_out ? 2u * ((uint32_t)row * (uint32_t)ldy + (uint32_t)n0 + 8u * cc) : NOWHERE;
+  }
+#pragma unroll
+  for (int u = 0; u < B_PER; ++u) {
+    const int idx = item0 + u * THREADS;
+    const int row = idx / CPR, cc = idx % CPR;
+    if (SRC == 0) {
+      const int c = (int)(j0 / 8) + cc;
+      vb[u] = (uint32_t)row * b_pitch + 8u * c;
+#pragma unroll
+      for (int i = 0; i < NST; ++i) {
+        vs[u][i] = 2u * ((uint32_t)row * gpr + (uint32_t)(((seg0 + i) * CPS + c) >> ca.chunk_to_group_shift));
+        vo0[u][i] = co.has0[i] ? (uint32_t)row * kk2 + co.vb[i] : NOWHERE;
+        vo1[u][i] = co.has1[i] ? (uint32_t)row * kk2 + co.vb[i] + 2u : NOWHERE;
+      }
+    } else {
+      vb[u] = (uint32_t)row * b_pitch + 2u * ((uint32_t)j0 + 8u * cc);
     }
+  }
+  auto fetch = [&](Regs& R, int64_t m0) __attribute__((always_inline)) {
+    // the resources of a stage start at its first token (scalar arithmetic), so the per-thread offsets never change
+    const uint32_t left = (uint32_t)(m_end - m0);
+    const BufferRsrc rs_a = make_rsrc(dy + m0 * ldy, left * 2u * (uint32_t)ldy);
+    const BufferRsrc rs_b = make_rsrc(stored + m0 * (int64_t)b_pitch, left * b_pitch);
 #pragma unroll
-    for (int u = 0; u < B_PER; ++u) {
-      const int idx = item0 + u * THREADS;
-      const int row = idx / CPR, cc = idx % CPR;
-      const int64_t m = m0 + row < m_end ? m0 + row : m_end - 1;
-      if (SRC == 0) {
-        const int c = (int)(j0 / 8) + cc;
-        const uint2 pk = *reinterpret_cast<const uint2*>(stored + m * SEG + 8 * c);
+    for (int u = 0; u < A_PER; ++u) R.a[u] = load_b128(rs_a, va[u]);
+    if (SRC == 0) {
+      const BufferRsrc rs_s = make_rsrc(scales + m0 * (int64_t)gpr, left * 2u * gpr);
+      const BufferRsrc rs_o = make_rsrc(ca.k ? vals + m0 * (int64_t)ca.k : nullptr, left * kk2);
+#pragma unroll
+      for (int u = 0; u < B_PER; ++u) {
+        const uint2 pk = load_b64(rs_b, vb[u]);
         R.b[u] = make_uint4(pk.x, pk.y, 0, 0);
 #pragma unroll
-        for (int i = 0; i < NST; ++i)
-          R.s[u][i] = scales[m * ca.groups_per_row + (((seg0 + i) * CPS + c) >> ca.chunk_to_group_shift)];
-        co.request(vals + m * ca.k, R.o0[u], R.o1[u]);
-      } else {
-        R.b[u] = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(stored) + m * H + j0 + 8 * cc);
+        for (int i = 0; i < NST; ++i) {
+          R.s[u][i] = load_b16(rs_s, vs[u][i]);
+          R.o0[u][i] = load_b16(rs_o, vo0[u][i]);
+          R.o1[u][i] = load_b16(rs_o, vo1[u][i]);
+        }
       }
+    } else {
+#pragma unroll
+      for (int u = 0; u < B_PER; ++u) R.b[u] = load_b128(rs_b, vb[u]);
     }
   };
   // (chunks with more than two outlier channels: the remaining pairs, rare, loaded in place)
@@ -558,8 +606,8 @@ k_gradw_wide(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_
 #pragma unroll
           for (int i = 0; i < NST; ++i)
             *reinterpret_cast<uint4*>(&Bs[buf][row * BP + (seg0 + i) * HS + 8 * cc]) = finish_chunk(
-                co.splice(i, dequant8_fast<BITS>(R.b[u].x, R.b[u].y, seg0 + i, bf_to_f((uint16_t)R.s[u][i])), R.o0[u][i],
-                          R.o1[u][i], 1.f), i, cc, mb + row);
+                co.splice_value(i, dequant8_fast<BITS>(R.b[u].x, R.b[u].y, seg0 + i, bf_to_f((uint16_t)R.s[u][i])), R.o0[u][i],
+                                R.o1[u][i]), i, cc, mb + row);
         } else {
           *reinterpret_cast<uint4*>(&Bs[buf][row * BP + 8 * cc]) = R.b[u];
         }
@@ -654,7 +702,7 @@ k_gradw_wide(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_
 #pragma unroll
           for (int i = 0; i < NST; ++i)
             *reinterpret_cast<uint4*>(&Bs[buf ^ 1][row * BP + (seg0 + i) * HS + 8 * cc]) = finish_chunk(
-                co.splice(i, make_uint4(res[u][i][0], res[u][i][1], res[u][i][2], res[u][i][3]), R.o0[u][i], R.o1[u][i], 1.f),
+                co.splice_value(i, make_uint4(res[u][i][0], res[u][i][1], res[u][i][2], res[u][i][3]), R.o0[u][i], R.o1[u][i]),
                 i, cc, mb + row);
         }
       }
@@ -842,7 +890,11 @@ int hyc_gradw_gemm(const void* dy, int64_t ldy, const void* stored, const void* 
   float* partial = splits > 1 ? static_cast<float*>(workspace) : nullptr;
   const dim3 grid((unsigned)n_tiles, (unsigned)h_tiles, (unsigned)splits);
   const int of32 = out_dtype == HYC_DTYPE_F32;
-  if (wide) {
+  // the wide kernel addresses a workgroup's token range with 32-bit offsets: each operand's share must stay under 2 GiB
+  const int64_t pitch_max = std::max<int64_t>(std::max<int64_t>(2 * ldy, chan ? g.seg : 2 * H),
+                                              chan ? std::max<int64_t>(2 * (H / d->group), 2 * (int64_t)d->k) : 0);
+  const bool fits32 = (tps + WK) * pitch_max < ((int64_t)1 << 31);
+  if (wide && fits32) {
     // eight waves (256 features per workgroup) halve the decode work per MFMA; four waves fill the chip better
     // when the output is small
     const int wnt = chan || (N_out >= 2 * WN && ((N_out + 2 * WN - 1) / (2 * WN)) * (H / WH) >= 128) ? 2 * WN : WN;

@@ -131,9 +131,14 @@ __device__ __forceinline__ void splice_selectors(bool has0, int j0, bool has1, i
 }
 // The reconstruction is (0 + outlier) + dequant(zero code): a -0 outlier comes out as +0, and a group whose scale
 // is inf/NaN is NaN at the outlier channels too.
+// SIGNED_ZERO = false leaves a -0 outlier as it is: for consumers that only multiply and add the restored value
+// (the weight gradient) the sign of a zero cannot reach the result.
+template <bool SIGNED_ZERO = true>
 __device__ __forceinline__ uint4 splice_pair(const uint4& r, const uint32_t (&sel)[4], uint32_t o0, uint32_t o1, float s) {
-  o0 = o0 == 0x8000u ? 0u : o0;
-  o1 = o1 == 0x8000u ? 0u : o1;
+  if (SIGNED_ZERO) {
+    o0 = o0 == 0x8000u ? 0u : o0;
+    o1 = o1 == 0x8000u ? 0u : o1;
+  }
   uint32_t oo = o0 | (o1 << 16);
   oo = (0.f * s == 0.f) ? oo : 0x7FC07FC0u;
   return make_uint4(__builtin_amdgcn_perm(oo, r.x, sel[0]), __builtin_amdgcn_perm(oo, r.y, sel[1]),
@@ -182,6 +187,10 @@ struct ChunkOutliers {
   }
   __device__ __forceinline__ uint4 splice(int i, const uint4& r, uint32_t o0, uint32_t o1, float s) const {
     return splice_pair(r, sel[i], o0, o1, s);
+  }
+  // the same for consumers that are indifferent to the sign of a zero
+  __device__ __forceinline__ uint4 splice_value(int i, const uint4& r, uint32_t o0, uint32_t o1) const {
+    return splice_pair<false>(r, sel[i], o0, o1, 1.f);
   }
 };
 
