@@ -180,3 +180,36 @@ def test_saved_bytes_accounting(DL, K):
     analytic = layer.saved_activation_bytes(B, S)
     assert 0.7 * analytic < held < 1.6 * analytic, (held, analytic)
     y.sum().backward()
+
+
+def test_training_tracks_the_uncompressed_layer(DL, K):
+    """two small layers trained for 40 AdamW steps on a fixed regression task, once with every saved activation
+    compressed and once keeping bf16: the compressed run must learn (loss falls by a third) and stay close to the
+    uncompressed loss curve (INT2 / INT4 gradients are noisy estimates of the same gradients)"""
+    B, S = 2, 64
+    losses = {}
+    for compress in (True, False):
+        torch.manual_seed(0)
+        cfg = small_cfg(DL, compress=compress)
+        layers = torch.nn.ModuleList([DL.DecoderLayer(cfg), DL.DecoderLayer(cfg)])
+        params = [p for p in layers.parameters() if p.requires_grad]
+        opt = torch.optim.AdamW(params, lr=2e-3, weight_decay=0.0)
+        gen = torch.Generator().manual_seed(9)
+        x = make_input(gen, B, S, cfg.hidden).cuda()
+        target = (0.5 * torch.randn(B, S, cfg.hidden, generator=gen)).bfloat16().cuda()
+        curve = []
+        for step in range(40):
+            opt.zero_grad(set_to_none=True)
+            h = x
+            for layer in layers:
+                h = layer(h)
+            loss = torch.nn.functional.mse_loss(h.float(), x.float() + target.float())
+            loss.backward()
+            opt.step()
+            curve.append(float(loss.detach()))
+        losses[compress] = curve
+    c, u = losses[True], losses[False]
+    assert all(v == v for v in c), "NaN in the compressed run"
+    assert c[-1] < 0.67 * c[0], (c[0], c[-1])
+    assert u[-1] < 0.67 * u[0], (u[0], u[-1])
+    assert abs(c[-1] - u[-1]) < 0.15 * u[0], (c[-1], u[-1], u[0])
