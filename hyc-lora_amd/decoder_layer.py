@@ -47,6 +47,7 @@ class LayerConfig:
     act_bits: int = 4                # norm inputs, q / k / v, gate / act(gate) / up
     act_group: int = 128
     compress: bool = True            # False: the same functions keep their activations in bf16 (formula check)
+    attn_group_bytes: int = 128 << 20  # attention is walked in groups of [S, S] score matrices of about this size
 
 
 # ---- frozen base + LoRA -----------------------------------------------------------------------------------
@@ -162,6 +163,13 @@ class CompressedAttention(torch.nn.Module):
         return _AttentionFunc.apply(q, k, v, cos, sin, self)
 
 
+def _matrices_per_group(total, s, budget_bytes):
+    """[S, S] bf16 score matrices per group: within the budget, and the groups of equal size"""
+    most = max(1, min(total, budget_bytes // (2 * s * s)))
+    groups = -(-total // most)
+    return -(-total // groups)
+
+
 class _AttentionFunc(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, cos, sin, mod):
@@ -175,25 +183,40 @@ class _AttentionFunc(torch.autograd.Function):
         kh, k_rows = K.rope_to_heads(k.contiguous(), nh, cos, sin, want_rows=True)
         v_rows = v.contiguous()
         vh = K.rope_to_heads(v_rows, nh)
-        # scores = (q @ k^T) / sqrt(hd) as one library GEMM; the causal mask is applied inside the softmax kernel,
-        # which never reads the masked half
-        scores = torch.baddbmm(q.new_zeros(1), qh.view(b * nh, s, hd), kh.view(b * nh, s, hd).transpose(1, 2), beta=0.0,
-                               alpha=scale).view(b, nh, s, s)
-        del qh, kh
+        # The [S, S] score matrices are processed in groups that keep the transient tensors near 128 MB (they stay in
+        # the last-level cache and the peak memory no longer grows with B * heads): per group one library GEMM for
+        # scores = (q @ k^T) / sqrt(hd), the softmax kernel with the causal mask built in (the masked half is never
+        # read), one GEMM for p @ v.
+        q3, k3, v3 = qh.view(b * nh, s, hd), kh.view(b * nh, s, hd), vh.view(b * nh, s, hd)
+        group = _matrices_per_group(b * nh, s, cfg.attn_group_bytes)
         it = mod.iteration
-        if not cfg.compress:
-            p, _ = K.softmax_fwd(scores, causal_period=s)
-            sparse = p                                             # kept whole, in bf16
-        elif it >= 2:
-            p, sparse = K.softmax_fwd(scores, float(mod.static_value), causal_period=s)
-        else:
-            p, _ = K.softmax_fwd(scores, causal_period=s)
-            thr = get_statistics_softmax(p, it, cfg.softmax_ratio)
-            mod.static_value = running_mean(mod.static_value, thr, it)
-            sparse = K.softmax_sparsify(p, float(thr))
-        del scores
-        out = K.rope_from_heads(torch.bmm(p.view(b * nh, s, s), vh.view(b * nh, s, hd)).view(b, nh, s, hd))   # [B, S, H]
-        del vh
+        calibrating = cfg.compress and it < 2
+        if calibrating:
+            group = b * nh                 # the threshold is a quantile over batch element 0: all of it is needed
+        zero = q.new_zeros(1)
+        out3 = torch.empty_like(q3)
+        kept, p_all = [], None
+        for c0 in range(0, b * nh, group):
+            c1 = min(c0 + group, b * nh)
+            scores = torch.baddbmm(zero, q3[c0:c1], k3[c0:c1].transpose(1, 2), beta=0.0, alpha=scale)
+            if not cfg.compress:
+                p, _ = K.softmax_fwd(scores, causal_period=s)
+                kept.append(p)                                     # kept whole, in bf16
+            elif not calibrating:
+                p, sp = K.softmax_fwd(scores, float(mod.static_value), causal_period=s)
+                kept.append(sp)
+            else:
+                p, _ = K.softmax_fwd(scores, causal_period=s)
+                thr = get_statistics_softmax(p.view(b, nh, s, s), it, cfg.softmax_ratio)
+                mod.static_value = running_mean(mod.static_value, thr, it)
+                kept.append(K.softmax_sparsify(p, float(thr)))
+            del scores
+            torch.bmm(p, v3[c0:c1], out=out3[c0:c1])
+            if mod.record is not None:
+                p_all = p if p_all is None else torch.cat([p_all, p])
+            del p
+        out = K.rope_from_heads(out3.view(b, nh, s, hd))            # [B, S, H]
+        del qh, kh, vh, q3, k3, v3, out3
         rows = [t.view(b * s, H) for t in (q_rows, k_rows, v_rows)]
         if cfg.compress:
             saved = []
@@ -205,8 +228,8 @@ class _AttentionFunc(torch.autograd.Function):
         mod.iteration += 1
         if mod.record is not None:
             mod.record.update(q=rows[0].detach().clone(), k=rows[1].detach().clone(), v=rows[2].detach().clone(),
-                              p=p.detach().clone(), saved=saved, sparse=sparse)
-        ctx.saved, ctx.sparse, ctx.geom, ctx.compress = saved, sparse, (b, nh, s, hd), cfg.compress
+                              p=p_all.view(b, nh, s, s), saved=saved, sparse=list(kept))
+        ctx.saved, ctx.kept, ctx.group, ctx.geom, ctx.compress = saved, kept, group, (b, nh, s, hd), cfg.compress
         ctx.save_for_backward(cos, sin)
         return out
 
@@ -218,27 +241,30 @@ class _AttentionFunc(torch.autograd.Function):
         to_heads = lambda rows: K.rope_to_heads(rows.view(b, s, nh * hd), nh).view(b * nh, s, hd)
         gh = K.rope_to_heads(g.to(BF16).contiguous(), nh).view(b * nh, s, hd)
         v = to_heads(restore(ctx.saved[2]))
-        p = (K.softmax_dense(ctx.sparse) if ctx.compress else ctx.sparse).view(b * nh, s, s)
-        dv = torch.bmm(p.transpose(1, 2), gh)
-        dp = torch.bmm(gh, v.transpose(1, 2))
-        del v, gh
-        if ctx.compress:
-            del p
-            ds = K.softmax_bwd(dp.view(b, nh, s, s), ctx.sparse)
-        else:
-            ds = torch._softmax_backward_data(dp, p, -1, BF16)
-            del p
-        del dp
-        scale = 1.0 / math.sqrt(hd)
-        zero = g.new_zeros(1).to(BF16)                           # ignored (beta = 0), only has to broadcast
-        ds3 = ds.view(b * nh, s, s)
         kk = to_heads(restore(ctx.saved[1]))
-        dq = torch.baddbmm(zero, ds3, kk, beta=0.0, alpha=scale)
-        del kk
         qq = to_heads(restore(ctx.saved[0]))
-        dk = torch.baddbmm(zero, ds3.transpose(1, 2), qq, beta=0.0, alpha=scale)
-        del qq, ds, ds3
-        ctx.saved = ctx.sparse = None
+        dq, dk, dv = torch.empty_like(qq), torch.empty_like(qq), torch.empty_like(qq)
+        scale = 1.0 / math.sqrt(hd)
+        zero = gh.new_zeros(1)                                     # ignored (beta = 0), only has to broadcast
+        for i, c0 in enumerate(range(0, b * nh, ctx.group)):
+            c1 = min(c0 + ctx.group, b * nh)
+            item = ctx.kept[i]
+            p = K.softmax_dense(item) if ctx.compress else item
+            torch.bmm(p.transpose(1, 2), gh[c0:c1], out=dv[c0:c1])
+            dp = torch.bmm(gh[c0:c1], v[c0:c1].transpose(1, 2))
+            if ctx.compress:
+                del p
+                ds = K.softmax_bwd(dp, item)
+            else:
+                ds = torch._softmax_backward_data(dp, p, -1, BF16)
+                del p
+            del dp
+            torch.baddbmm(zero, ds, kk[c0:c1], beta=0.0, alpha=scale, out=dq[c0:c1])
+            torch.baddbmm(zero, ds.transpose(1, 2), qq[c0:c1], beta=0.0, alpha=scale, out=dk[c0:c1])
+            del ds
+            ctx.kept[i] = None
+        del v, kk, qq, gh
+        ctx.saved = ctx.kept = None
         dq = K.rope_from_heads(dq.view(b, nh, s, hd), cos, sin)
         dk = K.rope_from_heads(dk.view(b, nh, s, hd), cos, sin)
         dv = K.rope_from_heads(dv.view(b, nh, s, hd))
