@@ -70,6 +70,7 @@ SIGNATURES = {
     "hyc_kth_value": (c_i32, [c_ptr, c_i32, c_i64, c_i64, c_ptr, c_ptr, c_ptr]),
     "hyc_rope_to_heads": (c_i32, [c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_i64, c_i64, c_ptr, c_ptr, c_ptr]),
     "hyc_rope_from_heads": (c_i32, [c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_i64, c_i64, c_ptr, c_ptr]),
+    "hyc_dropout": (c_i32, [c_ptr, c_ptr, c_i64, c_f32, ctypes.c_uint64, c_i32, c_ptr]),
     "hyc_nf4_quantize": (c_i32, [c_ptr, c_i64, c_ptr, c_ptr, c_ptr]),
     "hyc_nf4_dequantize": (c_i32, [c_ptr, c_ptr, c_i64, c_ptr, c_ptr]),
 }

@@ -614,3 +614,15 @@ def rope_from_heads(g, cos=None, sin=None):
     out = torch.empty((B, S, heads * hd), dtype=BF16, device=g.device)
     check(_abi.load().hyc_rope_from_heads(_p(g), _p(cos), _p(sin), B, S, heads, hd, _p(out), _stream()))
     return out
+
+
+# ----------------------------------------------------------------------------------------------------
+# seeded dropout
+# ----------------------------------------------------------------------------------------------------
+def dropout(x, p, seed, backward=False):
+    """forward: keep ? x / (1 - p) : 0; backward: keep ? x : 0; keep is a pure function of (seed, element index)"""
+    _need(x, BF16, "x")
+    out = torch.empty_like(x)
+    check(_abi.load().hyc_dropout(_p(x), _p(out), x.numel(), float(p), int(seed) & 0xFFFFFFFFFFFFFFFF,
+                                  1 if backward else 0, _stream()))
+    return out

@@ -12,3 +12,4 @@ from .efficient_layernorm import EfficientMemoryLayerNorm, EfficientMemoryLayerN
 from .efficient_gemm import (EfficientMemoryGEMM, EfficientMemoryGEMMFunc, EfficientMemoryGEMMWithSoftmax,  # noqa: F401
                              EfficientMemoryGEMMWithSoftmaxFunc)
 from ._calibration import calibration_state, load_calibration_state  # noqa: F401
+from .efficient_dropout import EfficientMemoryDropout, EfficientMemoryDropoutFunc  # noqa: F401

@@ -3,11 +3,11 @@
 Mirrors `replace_module_for_quantization` of the reference's training scripts (train_gsm8k.py:426-592,
 train_glue.py:391-493): same selection rules, same constructor keywords taken from the same `compress_config`
 sections ("linear", "silu", "layernorm", "softmax", "hadamard", "gemm"), weights re-pointed, recursion into
-everything else.  The one module kind this package does not provide (Dropout) is left as it is and reported, or
-raises with `strict=True`.
+everything else.  Every kind the reference swaps has a counterpart here.
 """
 import torch
 
+from .efficient_dropout import EfficientMemoryDropout
 from .efficient_gelu import EfficientMemoryGELU
 from .efficient_gemm import EfficientMemoryGEMM, EfficientMemoryGEMMWithSoftmax
 from .efficient_hadamard import EfficientMemoryHadamard
@@ -25,19 +25,11 @@ def _knobs(section):
                 sub_outlier_quantize_method=section["sub_outlier_quant_method"])
 
 
-def replace_module_for_quantization(module, compress_config, model_args=None, *, mode="ref", group_size=128,
-                                    strict=False, _skipped=None):
-    """In place.  Returns the list of (qualified name, class name) of modules the reference would have swapped but this
-    package has no counterpart for.  `model_args` is accepted for signature compatibility (the reference reads
-    `model_name_or_path` from it to pick the Gemma RMSNorm)."""
-    skipped = [] if _skipped is None else _skipped
+def replace_module_for_quantization(module, compress_config, model_args=None, *, mode="ref", group_size=128):
+    """In place, like the reference's.  `model_args` is read for `model_name_or_path` only (a name containing "gemma"
+    selects the Gemma RMSNorm)."""
     extra = dict(mode=mode, group_size=group_size)
     gemma = model_args is not None and "gemma" in str(getattr(model_args, "model_name_or_path", ""))
-
-    def unsupported(name, child):
-        if strict:
-            raise NotImplementedError("no memory-efficient counterpart for %s (%s)" % (name, child.__class__.__name__))
-        skipped.append((name, child.__class__.__name__))
 
     for name, child in module.named_children():
         cls = child.__class__.__name__
@@ -68,7 +60,7 @@ def replace_module_for_quantization(module, compress_config, model_args=None, *,
                 new.bias.data = child.bias.data
             setattr(module, name, new)
         elif isinstance(child, torch.nn.Dropout):
-            unsupported(name, child)
+            setattr(module, name, EfficientMemoryDropout(0.0))        # sic: the reference swaps in p = 0 (train_gsm8k.py:540-541)
         elif "GEMM" in cls:
             gm = compress_config["gemm"]
             if "gemm1" in name:
@@ -95,6 +87,4 @@ def replace_module_for_quantization(module, compress_config, model_args=None, *,
                 sub_outlier_bit_2=h["sub_outlier_bit"], sub_outlier_quantize_method_2=h["sub_outlier_quant_method"],
                 rank=h["rank"], **extra))
         else:
-            replace_module_for_quantization(child, compress_config, model_args, mode=mode, group_size=group_size,
-                                            strict=strict, _skipped=skipped)
-    return skipped
+            replace_module_for_quantization(child, compress_config, model_args, mode=mode, group_size=group_size)

@@ -37,6 +37,8 @@
  *       low_rank_extraction / low_rank_addition, operators/fused_compression.py:80-99, :184-210
  *   hyc_rope_to_heads / hyc_rope_from_heads
  *       apply_rotary_pos_emb and the head-major transposition around it, models/modeling_llama.py:236-260, :423-425
+ *   hyc_dropout
+ *       EfficientMemoryDropoutFunc (_seeded_dropout / _seeded_dropout_backward), operators/efficient_dropout.py:7-79
  *   hyc_nf4_dequantize / hyc_nf4_quantize
  *       F.dequantize_4bit(B, quant_state) before each frozen-base matmul, bitsandbytes_fix/_function.py:509, :540
  *       (the quantiser that wrote B is bitsandbytes' own and is not part of the reference tree)
@@ -232,6 +234,13 @@ int hyc_rope_to_heads(const void* x, const void* cosv, const void* sinv, int64_t
                       int64_t head_dim, void* out_heads, void* out_rows, void* stream);
 int hyc_rope_from_heads(const void* g, const void* cosv, const void* sinv, int64_t B, int64_t S, int64_t heads,
                         int64_t head_dim, void* out_rows, void* stream);
+
+/* ---- seeded dropout ----------------------------------------------------------------------------- */
+/* EfficientMemoryDropoutFunc, operators/efficient_dropout.py:56-79: the keep mask of element i is
+ * tl.rand(seed, i) > p (Philox4x32-10, counter (i,0,0,0), key = the two words of seed), so nothing is saved.
+ * backward == 0: out = keep ? bf16(x / (1-p)) : 0;  backward != 0: out = keep ? x : 0 (the reference's backward does
+ * not rescale).  x, out bf16 [n], n < 2^31, 0 <= p < 1. */
+int hyc_dropout(const void* x, void* out, int64_t n, float p, uint64_t seed, int32_t backward, void* stream);
 
 /* ---- NF4 frozen base weights ------------------------------------------------------------------- */
 /* Blocks of 64 consecutive weights: absmax[i] = max |w| of block i (fp32), packed byte j holds the level indices of

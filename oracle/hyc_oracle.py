@@ -32,6 +32,8 @@ Pinning status (see tests/test_oracle_*.py):
 * linear_bwd                   - torch.matmul in fp32
 * gemm_bwd                     - torch.autograd of torch.matmul in float64
 * rope_fwd / rope_bwd          - complex-number form of the rotation; float64 torch.autograd
+* philox4x32_10 / dropout_*    - Random123 known-answer vectors for the generator; keep fraction; the mask
+                                 mapping itself restates triton 3.6.0's tl.rand: parity unpinned by reference outputs
 * hyc_select_channels / hyc group scales - parity unpinned (no reference code)
 * nf4_quantize / nf4_dequantize - parity unpinned (bitsandbytes is not in the reference tree); checked against
                                  the published level table: nearest level by exact distance, round trips
@@ -495,3 +497,49 @@ def rope_bwd(g, cos, sin):
     """transpose of rope_fwd: d/dx of sum(g * rope_fwd(x))"""
     gf = g.float()
     return (gf * cos.float() - rotate_half(gf * sin.float())).to(g.dtype)
+
+
+# --------------------------------------------------------------------------------------
+# seeded dropout                                  operators/efficient_dropout.py:7-79
+# --------------------------------------------------------------------------------------
+# The reference's kernels are Triton (cannot run without a GPU) and draw their mask with tl.rand; this restates
+# triton/language/random.py of the installed triton 3.6.0 (the reference pins no version): Philox4x32-10 with counter
+# (index, 0, 0, 0) and key (seed & 0xffffffff, seed >> 32), first output word, folded to a non-negative int32 and
+# scaled by 4.6566127342e-10.  PARITY UNPINNED by reference outputs; the generator is pinned by the Random123
+# known-answer vectors.
+def philox4x32_10(counter, key):
+    """counter: four uint32 arrays (or ints), key: two -> four uint32 arrays; numpy uint64 arithmetic"""
+    import numpy as np
+    c0, c1, c2, c3 = (np.asarray(c, dtype=np.uint64) for c in counter)
+    k0, k1 = (np.uint64(k) for k in key)
+    A, B, M = np.uint64(0xD2511F53), np.uint64(0xCD9E8D57), np.uint64(0xFFFFFFFF)
+    for _ in range(10):
+        pa, pb = A * c0, B * c2
+        c0, c1, c2, c3 = ((pb >> np.uint64(32)) ^ c1 ^ k0) & M, pb & M, ((pa >> np.uint64(32)) ^ c3 ^ k1) & M, pa & M
+        k0, k1 = (k0 + np.uint64(0x9E3779B9)) & M, (k1 + np.uint64(0xBB67AE85)) & M
+    return c0, c1, c2, c3
+
+
+def dropout_keep_mask(n, p, seed):
+    """bool [n]: tl.rand(seed, i) > p for i in 0..n-1 (operators/efficient_dropout.py:24-25)"""
+    import numpy as np
+    idx = np.arange(n, dtype=np.uint64)
+    zero = np.zeros(n, dtype=np.uint64)
+    word = philox4x32_10((idx, zero, zero, zero), (seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF))[0].astype(np.uint32)
+    v = word.view(np.int32).astype(np.int64)
+    v = np.where(v < 0, -v - 1, v)
+    u = v.astype(np.float32) * np.float32(4.6566127342e-10)
+    return torch.from_numpy(u > np.float32(p))
+
+
+def dropout_fwd(x, p, seed):
+    """where(keep, x / (1 - p), 0) (:27): fp32 division, rounded to x's dtype"""
+    keep = dropout_keep_mask(x.numel(), p, seed).reshape(x.shape)
+    scaled = (x.float() / torch.tensor(1.0, dtype=torch.float32).sub(torch.tensor(p, dtype=torch.float32))).to(x.dtype)
+    return torch.where(keep, scaled, torch.zeros_like(x))
+
+
+def dropout_bwd(g, p, seed):
+    """where(keep, g, 0) (:52): the reference does not rescale the gradient"""
+    keep = dropout_keep_mask(g.numel(), p, seed).reshape(g.shape)
+    return torch.where(keep, g, torch.zeros_like(g))

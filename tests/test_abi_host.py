@@ -93,6 +93,10 @@ def test_argument_errors_without_a_gpu(abi):
     assert lib.hyc_rope_to_heads(null, null, null, 2, 8, 4, 32, null, null, null) == abi.EFAULT
     assert lib.hyc_rope_from_heads(null, null, null, 2, 8, 0, 32, null, null) == abi.EINVAL
     assert lib.hyc_rope_from_heads(null, null, null, 1 << 20, 1 << 12, 64, 128, null, null) == abi.EINVAL   # 2^32 items
+    assert lib.hyc_dropout(null, null, 16, 1.0, 5, 0, null) == abi.EINVAL              # p must be below 1
+    assert lib.hyc_dropout(null, null, 1 << 31, 0.1, 5, 0, null) == abi.EINVAL
+    assert lib.hyc_dropout(null, null, 0, 0.1, 5, 0, null) == 0
+    assert lib.hyc_dropout(null, null, 16, 0.1, 5, 0, null) == abi.EFAULT
     assert lib.hyc_kth_value_workspace_bytes() >= 1024 + 12
     assert lib.hyc_kth_value(null, 7, 10, 1, null, null, null) == abi.ENOTSUP
     assert lib.hyc_kth_value(null, abi.DTYPE_F32, 0, 1, null, null, null) == abi.EINVAL
@@ -175,6 +179,8 @@ def test_module_constructors_mirror_the_reference(hyc):
         assert a.iteration == 0 and a.static_value == [None] * 4
     s = ops.EfficientMemorySoftmax(outlier_ratio=0.05)
     assert s.static_value is None and s.outlier_ratio == 0.05
+    dr = ops.EfficientMemoryDropout(0.1)
+    assert dr.p == 0.1 and 0 <= dr.seed < 2 ** 32 and dr.training
     h = ops.EfficientMemoryHadamard()
     assert h.static_value_1 == [None] * 4 and h.sub_outlier_bit_2 == 8
     g1 = ops.EfficientMemoryGEMM(outlier_ratio_1=0.01, sub_outlier_ratio_1=0.2, sub_outlier_bit_1=8,
@@ -198,7 +204,7 @@ def test_module_constructors_mirror_the_reference(hyc):
 
 def test_module_swap_follows_the_reference_rules(hyc):
     """replace_module_for_quantization (train_gsm8k.py:426-592): trainable wide Linear, SiLU, RMSNorm, Softmax are
-    swapped with their weights shared; frozen / narrow Linear, lm_head, unsupported kinds are not"""
+    swapped with their weights shared; frozen / narrow Linear and lm_head are not"""
     import torch
     ops = hyc.operators
 
@@ -232,7 +238,7 @@ def test_module_swap_follows_the_reference_rules(hyc):
            for k in ("linear", "silu", "layernorm", "hadamard", "gemm")}
     cfg["softmax"] = dict(outlier_ratio=0.05)
     w_before = model[0].lora_A.weight.data_ptr()
-    skipped = ops.replace_module_for_quantization(model, cfg, mode="hyc", group_size=64)
+    ops.replace_module_for_quantization(model, cfg, mode="hyc", group_size=64)
     b = model[1]
     assert isinstance(b.lora_A, ops.EfficientMemoryLinear) and b.lora_A.mode == "hyc" and b.lora_A.group_size == 64
     assert b.lora_A.sub_outlier_bit == 4 and b.lora_A.rank == 0
@@ -243,7 +249,7 @@ def test_module_swap_follows_the_reference_rules(hyc):
     assert b.softmax.outlier_ratio == 0.05
     assert isinstance(b.gemm1, ops.EfficientMemoryGEMM) and b.gemm1.sub_outlier_bit_2 == 4 and b.gemm1.mode == "hyc"
     assert isinstance(b.gemm2, ops.EfficientMemoryGEMMWithSoftmax) and b.gemm2.outlier_ratio_1 == 0.05
-    assert sorted(skipped) == [("drop", "Dropout"), ("drop", "Dropout")]
+    assert isinstance(b.drop, ops.EfficientMemoryDropout) and b.drop.p == 0.0          # sic: the reference swaps in p = 0
 
     class Args:
         model_name_or_path = "google/gemma-7b"
@@ -254,8 +260,6 @@ def test_module_swap_follows_the_reference_rules(hyc):
     ln = torch.nn.Sequential(torch.nn.LayerNorm(128, eps=1e-12))
     ops.replace_module_for_quantization(ln, cfg)
     assert isinstance(ln[0], ops.EfficientMemoryLayerNorm) and ln[0].eps == 1e-12
-    with pytest.raises(NotImplementedError):
-        ops.replace_module_for_quantization(torch.nn.Sequential(torch.nn.Dropout(0.1)), cfg, strict=True)
 
 
 def test_calibration_state_round_trip(hyc, tmp_path):

@@ -572,3 +572,30 @@ def test_rope_kernels(K, B, S, nh, hd):
     assert bf16_ulp_diff(dx.cpu(), want_dx).max() <= 1
     assert bits_equal(K.rope_to_heads(x.cuda(), nh).cpu(), heads(x).contiguous())
     assert bits_equal(K.rope_from_heads(g.cuda()).cpu(), g.transpose(1, 2).reshape(B, S, nh * hd))
+
+
+# ------------------------------------------------------------------ seeded dropout
+@pytest.mark.parametrize("n,p,seed", [(8 * 1000, 0.1, 12345), (8 * 513 + 5, 0.5, (1 << 32) + 77), (3, 0.25, 1), (1 << 20, 0.0, 4242)])
+def test_dropout_kernel(K, n, p, seed):
+    """mask, scaled values and the (unscaled) backward bit-exact against the oracle"""
+    gen = torch.Generator().manual_seed(n)
+    x = torch.randn(n, generator=gen).bfloat16()
+    y = K.dropout(x.cuda(), p, seed).cpu()
+    assert bits_equal(y, O.dropout_fwd(x, p, seed))
+    g = K.dropout(x.cuda(), p, seed, backward=True).cpu()
+    assert bits_equal(g, O.dropout_bwd(x, p, seed))
+    if p == 0.0:
+        assert bits_equal(y, x)
+
+
+def test_dropout_module(ops):
+    mod = ops.EfficientMemoryDropout(0.2).cuda()
+    x = torch.randn(4, 64, 96).bfloat16().cuda().requires_grad_(True)
+    y = mod(x)
+    assert y.grad_fn.saved_tensors == ()                                # nothing is kept for the backward
+    y.backward(torch.ones_like(y))
+    keep = O.dropout_keep_mask(x.numel(), 0.2, mod.seed).reshape(x.shape)
+    assert torch.equal((y != 0).cpu() | (x.detach() == 0).cpu(), keep | (x.detach() == 0).cpu())
+    assert torch.equal(x.grad.cpu(), keep.to(torch.bfloat16))           # the reference's backward masks, it does not rescale
+    mod.eval()
+    assert mod(x) is x

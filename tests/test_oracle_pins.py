@@ -429,3 +429,30 @@ def test_rope_against_complex_rotation_and_autograd():
     (xa * cos2 + O.rotate_half(xa) * sin2).backward(g)
     assert torch.allclose(O.rope_bwd(g, cos2, sin2), xa.grad, rtol=1e-5, atol=1e-5)
     assert torch.allclose(O.rope_fwd(x, cos2, sin2), x * cos2 + O.rotate_half(x) * sin2, rtol=1e-5, atol=1e-5)
+
+
+def test_philox_known_answers_and_dropout_mask():
+    """the generator against the three published Random123 Philox4x32-10 known-answer vectors; the mask: a pure
+    function of (seed, index), keeps everything at p = 0 and about 1 - p otherwise, differs between seeds"""
+    kat = [((0, 0, 0, 0), (0, 0), (0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8)),
+           ((0xffffffff,) * 4, (0xffffffff, 0xffffffff), (0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd)),
+           ((0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344), (0xa4093822, 0x299f31d0),
+            (0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1))]
+    for counter, key, want in kat:
+        got = O.philox4x32_10(counter, key)
+        assert tuple(int(g) for g in got) == want
+    n = 200000
+    m1 = O.dropout_keep_mask(n, 0.3, 1234567)
+    assert torch.equal(m1, O.dropout_keep_mask(n, 0.3, 1234567))
+    assert abs(float(m1.float().mean()) - 0.7) < 0.005
+    assert bool(O.dropout_keep_mask(n, 0.0, 99).all())
+    assert not torch.equal(m1, O.dropout_keep_mask(n, 0.3, 1234568))
+    assert torch.equal(O.dropout_keep_mask(1000, 0.3, 1234567), m1[:1000])          # index-addressed, not stateful
+    big = (1 << 32) + 5                                                              # the high seed word reaches the key
+    assert not torch.equal(O.dropout_keep_mask(n, 0.3, big), O.dropout_keep_mask(n, 0.3, 5))
+    x = torch.randn(64, 33).bfloat16()
+    y = O.dropout_fwd(x, 0.25, 7)
+    keep = O.dropout_keep_mask(x.numel(), 0.25, 7).reshape(x.shape)
+    assert torch.equal(y[~keep], torch.zeros(int((~keep).sum()), dtype=torch.bfloat16))
+    assert torch.allclose(y[keep].float(), x[keep].float() / 0.75, rtol=2 ** -8)
+    assert bits_equal(O.dropout_bwd(x, 0.25, 7), torch.where(keep, x, torch.zeros_like(x)))
