@@ -64,7 +64,7 @@ k_softmax_fwd(const uint16_t* __restrict__ x, int64_t rows, int64_t N, float thr
 // neither read (x may hold anything there) nor exponentiated, and comes out as exact zeros.
 template <int CPL, bool CAUSAL>
 __global__ void __launch_bounds__(256)
-k_softmax_fwd_wave(const uint16_t* __restrict__ x, int64_t rows, int64_t N, float thr, uint16_t* __restrict__ y,
+k_softmax_fwd_wave(const uint16_t* x, int64_t rows, int64_t N, float thr, uint16_t* y,   // y may be x (in place)
                    int32_t* __restrict__ counts, int64_t period) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
@@ -268,8 +268,8 @@ k_softmax_fill_wave(const uint16_t* __restrict__ y, int64_t rows, int64_t N, flo
 // BWD: dx = (g - s) * yh with s = bf16(sum_j bf16(g_j * yh_j)), every product rounded to bf16 as torch does.
 template <bool BWD>
 __global__ void __launch_bounds__(256)
-k_softmax_rows(const uint16_t* __restrict__ g, int64_t rows, int64_t N, const int32_t* __restrict__ row_ptr,
-               const int32_t* __restrict__ cols, const uint16_t* __restrict__ vals, uint16_t* __restrict__ out) {
+k_softmax_rows(const uint16_t* g, int64_t rows, int64_t N, const int32_t* __restrict__ row_ptr,
+               const int32_t* __restrict__ cols, const uint16_t* __restrict__ vals, uint16_t* out) {   // out may be g
   extern __shared__ __align__(16) uint16_t lds[];          // [4][N]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int64_t row = (int64_t)blockIdx.x * 4 + wave;

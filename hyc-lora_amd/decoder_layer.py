@@ -47,7 +47,7 @@ class LayerConfig:
     act_bits: int = 4                # norm inputs, q / k / v, gate / act(gate) / up
     act_group: int = 128
     compress: bool = True            # False: the same functions keep their activations in bf16 (formula check)
-    attn_group_bytes: int = 128 << 20  # attention is walked in groups of [S, S] score matrices of about this size
+    attn_group_bytes: int = 128 << 20  # attention is walked in groups of [S, S] score matrices of at most this size
 
 
 # ---- frozen base + LoRA -----------------------------------------------------------------------------------
@@ -183,10 +183,10 @@ class _AttentionFunc(torch.autograd.Function):
         kh, k_rows = K.rope_to_heads(k.contiguous(), nh, cos, sin, want_rows=True)
         v_rows = v.contiguous()
         vh = K.rope_to_heads(v_rows, nh)
-        # The [S, S] score matrices are processed in groups that keep the transient tensors near 128 MB (they stay in
+        # The [S, S] score matrices are processed in groups that bound the transient tensors (they stay in
         # the last-level cache and the peak memory no longer grows with B * heads): per group one library GEMM for
         # scores = (q @ k^T) / sqrt(hd), the softmax kernel with the causal mask built in (the masked half is never
-        # read), one GEMM for p @ v.
+        # read; the probabilities overwrite the scores), one GEMM for p @ v.
         q3, k3, v3 = qh.view(b * nh, s, hd), kh.view(b * nh, s, hd), vh.view(b * nh, s, hd)
         group = _matrices_per_group(b * nh, s, cfg.attn_group_bytes)
         it = mod.iteration
@@ -200,13 +200,13 @@ class _AttentionFunc(torch.autograd.Function):
             c1 = min(c0 + group, b * nh)
             scores = torch.baddbmm(zero, q3[c0:c1], k3[c0:c1].transpose(1, 2), beta=0.0, alpha=scale)
             if not cfg.compress:
-                p, _ = K.softmax_fwd(scores, causal_period=s)
+                p, _ = K.softmax_fwd(scores, causal_period=s, inplace=True)
                 kept.append(p)                                     # kept whole, in bf16
             elif not calibrating:
-                p, sp = K.softmax_fwd(scores, float(mod.static_value), causal_period=s)
+                p, sp = K.softmax_fwd(scores, float(mod.static_value), causal_period=s, inplace=True)
                 kept.append(sp)
             else:
-                p, _ = K.softmax_fwd(scores, causal_period=s)
+                p, _ = K.softmax_fwd(scores, causal_period=s, inplace=True)
                 thr = get_statistics_softmax(p.view(b, nh, s, s), it, cfg.softmax_ratio)
                 mod.static_value = running_mean(mod.static_value, thr, it)
                 kept.append(K.softmax_sparsify(p, float(thr)))
@@ -254,7 +254,7 @@ class _AttentionFunc(torch.autograd.Function):
             dp = torch.bmm(gh[c0:c1], v[c0:c1].transpose(1, 2))
             if ctx.compress:
                 del p
-                ds = K.softmax_bwd(dp, item)
+                ds = K.softmax_bwd(dp, item, inplace=True)
             else:
                 ds = torch._softmax_backward_data(dp, p, -1, BF16)
                 del p
@@ -314,13 +314,14 @@ class DecoderLayer(torch.nn.Module):
         if self._rope is None or self._rope[0].shape[0] != s:
             self._rope = rope_tables(s, cfg.head_dim, cfg.rope_theta, x.device)
         cos, sin = self._rope
-        h = self.input_layernorm(x)
-        q, k, v = self.qkv_proj(h)
-        x = x + self.o_proj(self.attention(q, k, v, cos, sin))
-        h = self.post_attention_layernorm(x)
-        gate, up = self.gate_up_proj(h)
-        m = self.act(gate, up) if self.act is not None else torch.nn.functional.silu(gate) * up
-        return x + self.down_proj(m)
+        # no names for the wide intermediates: each is released as soon as its consumer has run
+        x = x + self.o_proj(self.attention(*self.qkv_proj(self.input_layernorm(x)), cos, sin))
+        return x + self.down_proj(self._gated(*self.gate_up_proj(self.post_attention_layernorm(x))))
+
+    def _gated(self, gate, up):
+        if self.act is not None:
+            return self.act(gate, up)
+        return torch.nn.functional.silu(gate) * up
 
     def saved_activation_bytes(self, batch, seq):
         """analytic size of what one forward keeps for the backward (the probabilities' share is data dependent:

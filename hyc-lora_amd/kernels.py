@@ -451,15 +451,18 @@ def _csr_from_counts(lib, y2d, threshold, counts):
     return row_ptr, cols, vals
 
 
-def softmax_fwd(x, threshold=None, causal_period=None):
+def softmax_fwd(x, threshold=None, causal_period=None, inplace=False):
     """y = softmax(x, -1) bf16; with a threshold also the kept entries (y > bf16(threshold)) as SparseRows.
-    causal_period = S applies the causal mask of S query positions inside the kernel (row r is position r % S)."""
+    causal_period = S applies the causal mask of S query positions inside the kernel (row r is position r % S).
+    inplace: y overwrites x (rows of at most 4096 entries: a row is held in registers before anything is written)."""
     _need(x, BF16, "x")
     N = x.shape[-1]
     x2 = x.reshape(-1, N)
     rows = x2.shape[0]
     lib = _abi.load()
-    y = torch.empty_like(x2)
+    if inplace and N > 4096:
+        raise ValueError("in-place softmax needs rows of at most 4096 entries")
+    y = x2 if inplace else torch.empty_like(x2)
     counts = None if threshold is None else torch.empty(rows, dtype=torch.int32, device=x.device)
     thr = 0.0 if threshold is None else float(threshold)
     if causal_period is None:
@@ -484,11 +487,12 @@ def softmax_sparsify(y, threshold):
     return SparseRows(row_ptr, cols, vals, tuple(y.shape))
 
 
-def softmax_bwd(g, sp: SparseRows):
+def softmax_bwd(g, sp: SparseRows, inplace=False):
+    """dx = (g - sum(g * p_hat)) * p_hat; with inplace, dx overwrites g"""
     _need(g, BF16, "grad_output")
     N = g.shape[-1]
     g2 = g.reshape(-1, N)
-    dx = torch.empty_like(g2)
+    dx = g2 if inplace else torch.empty_like(g2)
     check(_abi.load().hyc_softmax_bwd(_p(g2), g2.shape[0], N, _p(sp.row_ptr), _p(sp.cols) if sp.cols.numel() else None,
                                       _p(sp.vals) if sp.vals.numel() else None, _p(dx), _stream()))
     return dx.reshape(g.shape)

@@ -190,7 +190,8 @@ int hyc_gated_act_bwd(int32_t act, const void* g, const void* stored_a, const vo
 
 /* ---- softmax -------------------------------------------------------------------------------- */
 /* x bf16 [rows, N] -> y = softmax(x, -1) bf16 and counts[r] = #{j : y[r,j] > bf16(threshold)} (counts may be
- * NULL).  With x == NULL, y is taken as given and only the counts are produced. */
+ * NULL).  With x == NULL, y is taken as given and only the counts are produced.  For N <= 4096 y may be x itself
+ * (in place: a row is held in registers before any of it is written); the same holds for the causal form. */
 int hyc_softmax_fwd(const void* x, int64_t rows, int64_t N, float threshold, void* y, int32_t* counts, void* stream);
 /* the same with the causal attention mask built in (models/modeling_llama.py:452-459 adds it to the scores before the
  * softmax): row r is query position r % period and sees columns 0..position; columns beyond are not read and come
@@ -200,7 +201,7 @@ int hyc_softmax_causal_fwd(const void* x, int64_t rows, int64_t N, int64_t perio
 /* the kept probabilities as CSR: row_ptr int32 [rows+1] (exclusive prefix sums of counts), cols ascending per row */
 int hyc_softmax_fill(const void* y, int64_t rows, int64_t N, float threshold, const int32_t* row_ptr, int32_t* cols,
                      void* vals, void* stream);
-/* dx = (g - sum_j g_j*yh_j) * yh, yh = the CSR probabilities (zero elsewhere) */
+/* dx = (g - sum_j g_j*yh_j) * yh, yh = the CSR probabilities (zero elsewhere); dx may be g itself (in place) */
 int hyc_softmax_bwd(const void* g, int64_t rows, int64_t N, const int32_t* row_ptr, const int32_t* cols,
                     const void* vals, void* dx, void* stream);
 /* yh as a dense bf16 [rows, N] matrix */

@@ -599,3 +599,20 @@ def test_dropout_module(ops):
     assert torch.equal(x.grad.cpu(), keep.to(torch.bfloat16))           # the reference's backward masks, it does not rescale
     mod.eval()
     assert mod(x) is x
+
+
+def test_softmax_in_place(K):
+    """y written over x (plain and causal) and dx written over g give the same bits as the out-of-place calls"""
+    gen = torch.Generator().manual_seed(16)
+    x = (2 * torch.randn(3, 5, 96, 1024, generator=gen)).bfloat16().cuda()
+    g = (0.1 * torch.randn(3, 5, 96, 1024, generator=gen)).bfloat16().cuda()
+    for period in (None, 96):
+        want, sp_want = K.softmax_fwd(x, 0.01, causal_period=period)
+        buf = x.clone()
+        got, sp_got = K.softmax_fwd(buf, 0.01, causal_period=period, inplace=True)
+        assert got.data_ptr() == buf.data_ptr() and torch.equal(got, want)
+        assert torch.equal(sp_got.row_ptr, sp_want.row_ptr) and torch.equal(sp_got.vals, sp_want.vals)
+        dx = K.softmax_bwd(g, sp_want)
+        gb = g.clone()
+        dx2 = K.softmax_bwd(gb, sp_want, inplace=True)
+        assert dx2.data_ptr() == gb.data_ptr() and torch.equal(dx2, dx)
