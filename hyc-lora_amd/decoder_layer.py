@@ -95,11 +95,14 @@ class _LoRAProjectionsFunc(torch.autograd.Function):
         s = mod.scaling
         outs, hs = [], []
         wbuf = None
+        zero = x2.new_zeros(1)                                   # ignored (beta = 0), only has to broadcast
         for i in range(n):
             wbuf = K.nf4_dequantize(mod.base[i], out=wbuf if wbuf is not None and wbuf.shape == mod.base[i].shape else None)
-            y = x2 @ wbuf.t()
+            # the rank-r term first, the base GEMM accumulates onto it (its epilogue reads y once; the other order
+            # costs a separate read-modify-write pass over y)
             h = x2 @ A[i].t()
-            y.addmm_(h, B[i].t(), alpha=s)
+            y = torch.addmm(zero, h, B[i].t(), beta=0.0, alpha=s)
+            y.addmm_(x2, wbuf.t())
             outs.append(y.reshape(x.shape[:-1] + (mod.out_features[i],)))
             hs.append(h)
         del wbuf
@@ -118,19 +121,24 @@ class _LoRAProjectionsFunc(torch.autograd.Function):
         ab = ctx.saved_tensors
         A, B = ab[:n], ab[n:]
         s = mod.scaling
-        dx = None
-        dA, dB = [], []
-        wbuf = None
+        dA, dB, dhs, grads = [], [], [], []
+        zero = ab[0].new_zeros(1)
         for i in range(n):
             g = gs[i].reshape(-1, mod.out_features[i]).to(BF16)
             if not g.is_contiguous():
                 g = g.contiguous()
-            wbuf = K.nf4_dequantize(mod.base[i], out=wbuf if wbuf is not None and wbuf.shape == mod.base[i].shape else None)
-            dx = g @ wbuf if dx is None else dx.addmm_(g, wbuf)
-            dh = (g @ B[i]) * s                                  # [M, r]
-            dx.addmm_(dh, A[i])
-            dB.append((g.t() @ ctx.hs[i]) * s)
+            grads.append(g)
+            dh = torch.addmm(zero, g, B[i], beta=0.0, alpha=s)    # [M, r]
+            dhs.append(dh)
+            dB.append(torch.addmm(zero, g.t(), ctx.hs[i], beta=0.0, alpha=s))
             dA.append(K.gradw_gemm(dh, ctx.saved_x, out_dtype=A[i].dtype))
+        # dX: all rank-r terms as one thin GEMM, then each base GEMM accumulates onto it in its epilogue
+        dx = (dhs[0] @ A[0]) if n == 1 else (torch.cat(dhs, dim=1) @ torch.cat(list(A), dim=0))
+        wbuf = None
+        for i in range(n):
+            wbuf = K.nf4_dequantize(mod.base[i], out=wbuf if wbuf is not None and wbuf.shape == mod.base[i].shape else None)
+            dx.addmm_(grads[i], wbuf)
+        del wbuf, grads, dhs
         ctx.hs = None
         ctx.saved_x = None
         return (dx.reshape(gs[0].shape[:-1] + (mod.in_features,)), None, None) + tuple(dA) + tuple(dB)
