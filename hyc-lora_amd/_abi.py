@@ -43,6 +43,7 @@ SIGNATURES = {
     "hyc_channel_absmax": (c_i32, [c_ptr, c_i64, c_i64, c_ptr, c_ptr]),
     "hyc_select_channels": (c_i32, [c_ptr, c_i64, c_i32, c_ptr, c_ptr, c_ptr]),
     "hyc_compress": (c_i32, [c_ptr, c_i64, c_i64, ctypes.POINTER(HycDesc), c_ptr, c_ptr, c_ptr, c_ptr, c_ptr]),
+    "hyc_compress_rows": (c_i32, [c_ptr, c_i64, c_i64, c_i64, ctypes.POINTER(HycDesc), c_ptr, c_ptr, c_ptr, c_ptr, c_ptr]),
     "hyc_decompress": (c_i32, [c_ptr, c_ptr, c_ptr, c_i64, c_i64, ctypes.POINTER(HycDesc), c_ptr, c_ptr]),
     "hyc_ref_outlier_count": (c_i32, [c_ptr, c_i64, c_i64, ctypes.POINTER(HycDesc), c_ptr, c_ptr]),
     "hyc_ref_outlier_fill": (c_i32, [c_ptr, c_i64, c_i64, ctypes.POINTER(HycDesc), c_ptr, c_ptr, c_ptr, c_ptr]),
@@ -68,7 +69,7 @@ SIGNATURES = {
     "hyc_low_rank_update": (c_i32, [c_ptr, c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_i64, c_i32, c_i32, c_ptr]),
     "hyc_kth_value_workspace_bytes": (c_i64, []),
     "hyc_kth_value": (c_i32, [c_ptr, c_i32, c_i64, c_i64, c_ptr, c_ptr, c_ptr]),
-    "hyc_rope_to_heads": (c_i32, [c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_i64, c_i64, c_ptr, c_ptr, c_ptr]),
+    "hyc_rope_to_heads": (c_i32, [c_ptr, c_i64, c_ptr, c_ptr, c_i64, c_i64, c_i64, c_i64, c_ptr, c_ptr, c_ptr]),
     "hyc_rope_from_heads": (c_i32, [c_ptr, c_ptr, c_ptr, c_i64, c_i64, c_i64, c_i64, c_ptr, c_ptr]),
     "hyc_dropout": (c_i32, [c_ptr, c_ptr, c_i64, c_f32, ctypes.c_uint64, c_i32, c_ptr]),
     "hyc_nf4_quantize": (c_i32, [c_ptr, c_i64, c_ptr, c_ptr, c_ptr]),

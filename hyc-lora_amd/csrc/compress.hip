@@ -12,7 +12,7 @@ namespace hyc {
 // ------------------------------------------------------------------------------------------------
 template <int BITS>
 __global__ void __launch_bounds__(1024)
-k_compress_chan(const uint16_t* __restrict__ x, int64_t M, int64_t H, int CPS, int iters, int lpg, ChanArgs a,
+k_compress_chan(const uint16_t* __restrict__ x, int64_t M, int64_t H /* row pitch of x */, int CPS, int iters, int lpg, ChanArgs a,
                 uint8_t* __restrict__ stored, uint16_t* __restrict__ vals, uint16_t* __restrict__ scales) {
   constexpr int NSEG = Q<BITS>::NSEG;
   const int64_t SEG = (int64_t)CPS * 8;
@@ -65,7 +65,7 @@ k_decompress_chan(const uint8_t* __restrict__ stored, const uint16_t* __restrict
 // current one is processed.
 template <int BITS, int LPGT, int MAXT>
 __global__ void __launch_bounds__(MAXT)
-k_compress_chan_fast(const uint16_t* __restrict__ x, int64_t M, int64_t H, int CPS, ChanArgs a,
+k_compress_chan_fast(const uint16_t* __restrict__ x, int64_t M, int64_t H /* row pitch of x */, int CPS, ChanArgs a,
                      uint8_t* __restrict__ stored, uint16_t* __restrict__ vals, uint16_t* __restrict__ scales) {
   constexpr int NSEG = Q<BITS>::NSEG;
   const int c = threadIdx.x;
@@ -368,8 +368,16 @@ extern "C" {
 
 int hyc_compress(const void* x, int64_t M, int64_t H, const hyc_desc* d, void* stored, void* vals, void* scales,
                  int32_t* row_counts, void* stream) {
+  return hyc_compress_rows(x, H, M, H, d, stored, vals, scales, row_counts, stream);
+}
+
+int hyc_compress_rows(const void* x, int64_t ldx, int64_t M, int64_t H, const hyc_desc* d, void* stored, void* vals,
+                      void* scales, int32_t* row_counts, void* stream) {
   if (!d) return fail(HYC_EFAULT, "hyc_compress: null descriptor");
   if (M < 0) return fail(HYC_EINVAL, "hyc_compress: M=%lld", (long long)M);
+  if (ldx < H || ldx % 8 != 0 || (d->mode != HYC_MODE_CHANNEL && ldx != H))
+    return fail(HYC_EINVAL, "hyc_compress: row pitch %lld (at least H=%lld, a multiple of 8; equal to H outside the channel scheme)",
+                (long long)ldx, (long long)H);
   RowGeom g;
   int rc = row_geom(H, d->bits, &g);
   if (rc) return rc;
@@ -386,11 +394,11 @@ int hyc_compress(const void* x, int64_t M, int64_t H, const hyc_desc* d, void* s
   do {                                                                                                             \
     if (g.threads <= 256)                                                                                          \
       hipLaunchKernelGGL((k_compress_chan_fast<B_, L_, 256>), dim3(grid), dim3(g.threads), 0, st,                  \
-                         static_cast<const uint16_t*>(x), M, H, g.cps, a, static_cast<uint8_t*>(stored),                 \
+                         static_cast<const uint16_t*>(x), M, ldx, g.cps, a, static_cast<uint8_t*>(stored),               \
                          static_cast<uint16_t*>(vals), static_cast<uint16_t*>(scales));                            \
     else                                                                                                           \
       hipLaunchKernelGGL((k_compress_chan_fast<B_, L_, 1024>), dim3(grid), dim3(g.threads), 0, st,                 \
-                         static_cast<const uint16_t*>(x), M, H, g.cps, a, static_cast<uint8_t*>(stored),                 \
+                         static_cast<const uint16_t*>(x), M, ldx, g.cps, a, static_cast<uint8_t*>(stored),               \
                          static_cast<uint16_t*>(vals), static_cast<uint16_t*>(scales));                            \
   } while (0)
       switch (d->bits * 100 + lpg) {
@@ -406,7 +414,7 @@ int hyc_compress(const void* x, int64_t M, int64_t H, const hyc_desc* d, void* s
     }
     HYC_DISPATCH_BITS(d->bits,
       hipLaunchKernelGGL((k_compress_chan<B>), dim3(grid), dim3(g.threads), 0, st,
-                         static_cast<const uint16_t*>(x), M, H, g.cps, g.iters, lpg, a, static_cast<uint8_t*>(stored),
+                         static_cast<const uint16_t*>(x), M, ldx, g.cps, g.iters, lpg, a, static_cast<uint8_t*>(stored),
                          static_cast<uint16_t*>(vals), static_cast<uint16_t*>(scales)));
     return check_launch("hyc_compress");
   }

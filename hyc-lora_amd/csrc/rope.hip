@@ -31,8 +31,8 @@ static Divisor make_divisor(int64_t d) {
 template <bool TO_HEADS, bool ROTATE>
 __global__ void __launch_bounds__(256)
 k_rope(const uint16_t* __restrict__ in, const uint16_t* __restrict__ cosv, const uint16_t* __restrict__ sinv,
-       uint32_t items, Divisor per_head, Divisor heads, Divisor seq, int hd, uint16_t* __restrict__ out_heads,
-       uint16_t* __restrict__ out_rows) {
+       uint32_t items, Divisor per_head, Divisor heads, Divisor seq, int hd, int64_t in_pitch,
+       uint16_t* __restrict__ out_heads, uint16_t* __restrict__ out_rows) {
   const int half = hd / 2;
   const uint32_t step = gridDim.x * 256u;
   for (uint32_t t = blockIdx.x * 256u + threadIdx.x; t < items; t += step) {
@@ -41,7 +41,8 @@ k_rope(const uint16_t* __restrict__ in, const uint16_t* __restrict__ cosv, const
     const uint32_t b = seq.div(bs), s = bs - b * seq.d;
     const int64_t rows_off = (int64_t)bsh * hd + 8 * sub;                                              // [b, s, h, d]
     const int64_t heads_off = (((int64_t)b * heads.d + h) * seq.d + s) * hd + 8 * sub;               // [b, h, s, d]
-    const int64_t in_off = TO_HEADS ? rows_off : heads_off;
+    // a row-major input may be a column slice of a wider matrix: its tokens are in_pitch elements apart
+    const int64_t in_off = TO_HEADS ? (int64_t)bs * in_pitch + (int64_t)h * hd + 8 * sub : heads_off;
     float lo[8], hi[8];
     const uint4 rlo = *reinterpret_cast<const uint4*>(in + in_off);
     const uint4 rhi = *reinterpret_cast<const uint4*>(in + in_off + half);
@@ -104,10 +105,12 @@ using namespace hyc;
 
 extern "C" {
 
-int hyc_rope_to_heads(const void* x, const void* cosv, const void* sinv, int64_t B, int64_t S, int64_t heads,
-                      int64_t head_dim, void* out_heads, void* out_rows, void* stream) {
+int hyc_rope_to_heads(const void* x, int64_t x_pitch, const void* cosv, const void* sinv, int64_t B, int64_t S,
+                      int64_t heads, int64_t head_dim, void* out_heads, void* out_rows, void* stream) {
   int rc = rope_args("hyc_rope_to_heads", B, S, heads, head_dim);
   if (rc) return rc;
+  if (x_pitch < heads * head_dim || x_pitch % 8 != 0)
+    return fail(HYC_EINVAL, "hyc_rope_to_heads: token pitch %lld (at least heads*head_dim, a multiple of 8)", (long long)x_pitch);
   if (B == 0 || S == 0) return HYC_OK;
   if (!x || !out_heads || ((cosv == nullptr) != (sinv == nullptr))) return fail(HYC_EFAULT, "hyc_rope_to_heads: null buffer");
   if (!aligned16(x) || !aligned16(out_heads) || !aligned16(out_rows) || !aligned16(cosv) || !aligned16(sinv))
@@ -118,12 +121,12 @@ int hyc_rope_to_heads(const void* x, const void* cosv, const void* sinv, int64_t
   if (cosv)
     hipLaunchKernelGGL((k_rope<true, true>), grid, dim3(256), 0, st, static_cast<const uint16_t*>(x),
                        static_cast<const uint16_t*>(cosv), static_cast<const uint16_t*>(sinv), (uint32_t)items,
-                       make_divisor(head_dim / 16), make_divisor(heads), make_divisor(S), (int)head_dim,
+                       make_divisor(head_dim / 16), make_divisor(heads), make_divisor(S), (int)head_dim, x_pitch,
                        static_cast<uint16_t*>(out_heads), static_cast<uint16_t*>(out_rows));
   else
     hipLaunchKernelGGL((k_rope<true, false>), grid, dim3(256), 0, st, static_cast<const uint16_t*>(x),
                        static_cast<const uint16_t*>(nullptr), static_cast<const uint16_t*>(nullptr), (uint32_t)items,
-                       make_divisor(head_dim / 16), make_divisor(heads), make_divisor(S), (int)head_dim,
+                       make_divisor(head_dim / 16), make_divisor(heads), make_divisor(S), (int)head_dim, x_pitch,
                        static_cast<uint16_t*>(out_heads), static_cast<uint16_t*>(out_rows));
   return check_launch("hyc_rope_to_heads");
 }
@@ -142,12 +145,12 @@ int hyc_rope_from_heads(const void* g, const void* cosv, const void* sinv, int64
   if (cosv)
     hipLaunchKernelGGL((k_rope<false, true>), grid, dim3(256), 0, st, static_cast<const uint16_t*>(g),
                        static_cast<const uint16_t*>(cosv), static_cast<const uint16_t*>(sinv), (uint32_t)items,
-                       make_divisor(head_dim / 16), make_divisor(heads), make_divisor(S), (int)head_dim,
+                       make_divisor(head_dim / 16), make_divisor(heads), make_divisor(S), (int)head_dim, (int64_t)0,
                        static_cast<uint16_t*>(nullptr), static_cast<uint16_t*>(out_rows));
   else
     hipLaunchKernelGGL((k_rope<false, false>), grid, dim3(256), 0, st, static_cast<const uint16_t*>(g),
                        static_cast<const uint16_t*>(nullptr), static_cast<const uint16_t*>(nullptr), (uint32_t)items,
-                       make_divisor(head_dim / 16), make_divisor(heads), make_divisor(S), (int)head_dim,
+                       make_divisor(head_dim / 16), make_divisor(heads), make_divisor(S), (int)head_dim, (int64_t)0,
                        static_cast<uint16_t*>(nullptr), static_cast<uint16_t*>(out_rows));
   return check_launch("hyc_rope_from_heads");
 }

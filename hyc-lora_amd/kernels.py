@@ -69,6 +69,8 @@ def kth_value(x, k):
 
 def channel_absmax(x2d, amax=None):
     """running per-channel max |x| (fp32 [H]); pass the previous result to accumulate"""
+    if isinstance(x2d, torch.Tensor) and x2d.is_cuda and not x2d.is_contiguous():
+        x2d = x2d.contiguous()                     # calibration only (twice per site): a copy is acceptable
     _need(x2d, BF16, "x")
     M, H = x2d.shape
     if amax is None:
@@ -126,14 +128,25 @@ def alloc_channel(M, H, plan, bits, group, device):
     return ChannelCompressed(stored, vals, scales, plan, bits, group, M, H)
 
 
+def _need_rows(t, name):
+    """a bf16 [M, H] matrix whose rows are contiguous; the rows themselves may be further apart (a column slice)"""
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise ValueError("%s must be a CUDA (ROCm) tensor: the hot path runs on the GPU only" % name)
+    if t.dtype != BF16 or t.dim() != 2 or (t.shape[1] > 1 and t.stride(1) != 1):
+        raise ValueError("%s must be a bfloat16 matrix with contiguous rows" % name)
+    return t
+
+
 def compress_channel(x2d, plan, bits, group):
-    _need(x2d, BF16, "x")
+    _need_rows(x2d, "x")
     M, H = x2d.shape
     lib = _abi.load()
     check(lib.hyc_check_shape(H, bits, group, _abi.MODE_CHANNEL))
     out = alloc_channel(M, H, plan, bits, group, x2d.device)
     d = out.desc()
-    check(lib.hyc_compress(_p(x2d), M, H, ctypes.byref(d), _p(out.stored), _p(out.vals), _p(out.scales), None, _stream()))
+    pitch = x2d.stride(0) if M > 1 else H
+    check(lib.hyc_compress_rows(_p(x2d), pitch, M, H, ctypes.byref(d), _p(out.stored), _p(out.vals), _p(out.scales), None,
+                                _stream()))
     return out
 
 
@@ -601,13 +614,19 @@ def nf4_dequantize(q: NF4Weight, out=None):
 # ----------------------------------------------------------------------------------------------------
 def rope_to_heads(x, heads, cos=None, sin=None, want_rows=False):
     """x bf16 [B, S, heads*hd] -> rotated [B, heads, S, hd] contiguous (and, with want_rows, also [B, S, heads*hd]);
-    cos / sin bf16 [S, hd]; without them only the layout changes"""
-    _need(x, BF16, "x")
+    cos / sin bf16 [S, hd]; without them only the layout changes.  x may be a column slice of a wider [B, S, *]
+    tensor (tokens a fixed pitch apart)."""
+    if not isinstance(x, torch.Tensor) or not x.is_cuda or x.dtype != BF16 or x.dim() != 3:
+        raise ValueError("x must be a bfloat16 [B, S, H] tensor on the GPU")
     B, S, H = x.shape
+    pitch = x.stride(1) if S > 1 else H
+    if x.stride(2) != 1 or (B > 1 and x.stride(0) != S * pitch):
+        raise ValueError("x must have contiguous channels and evenly spaced tokens")
     hd = H // heads
     out_heads = torch.empty((B, heads, S, hd), dtype=BF16, device=x.device)
-    out_rows = torch.empty_like(x) if want_rows else None
-    check(_abi.load().hyc_rope_to_heads(_p(x), _p(cos), _p(sin), B, S, heads, hd, _p(out_heads), _p(out_rows), _stream()))
+    out_rows = torch.empty((B, S, H), dtype=BF16, device=x.device) if want_rows else None
+    check(_abi.load().hyc_rope_to_heads(_p(x), pitch, _p(cos), _p(sin), B, S, heads, hd, _p(out_heads), _p(out_rows),
+                                        _stream()))
     return (out_heads, out_rows) if want_rows else out_heads
 
 

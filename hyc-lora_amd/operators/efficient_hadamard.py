@@ -93,6 +93,17 @@ class EfficientMemoryHadamard(torch.nn.Module):
         return result
 
 
+def _row_view(t):
+    """[..., H] -> [M, H] without a copy when the rows are evenly spaced (e.g. a column slice of a fused projection)"""
+    H = t.shape[-1]
+    if t.stride(-1) != 1:
+        t = t.contiguous()
+    try:
+        return t.view(-1, H)
+    except RuntimeError:
+        return t.reshape(-1, H)
+
+
 class _ChannelGatedActFunc(torch.autograd.Function):
     """h = act(gate) * up with the three activations EfficientMemorySiLU/GELU and EfficientMemoryHadamard would save
     (gate; act(gate) and up), and one backward pass over them."""
@@ -100,7 +111,7 @@ class _ChannelGatedActFunc(torch.autograd.Function):
     @staticmethod
     def forward(ctx, gate, up, act, sites, iteration, bits, group):
         a = torch.nn.functional.silu(gate) if act == "silu" else torch.nn.functional.gelu(gate)
-        rows = [as_rows(t)[0] for t in (a, up, gate)]
+        rows = [_row_view(t) for t in (a, up, gate)]
         ctx.saved = tuple(K.compress_channel(r, site.channel_plan(r, iteration), bits, group)
                           for r, site in zip(rows, sites))
         ctx.act = act

@@ -139,6 +139,10 @@ int hyc_kth_value(const void* x, int32_t x_dtype, int64_t n, int64_t k, float* o
  * threshold mode writes per-row outlier counts to row_counts (int32 [M], may be NULL). */
 int hyc_compress(const void* x, int64_t M, int64_t H, const hyc_desc* d, void* stored, void* vals, void* scales,
                  int32_t* row_counts, void* stream);
+/* the same for x whose rows are ldx >= H elements apart (a column slice of a wider matrix, e.g. one projection out
+ * of a fused q/k/v GEMM); ldx a multiple of 8; channel scheme only (otherwise ldx must equal H) */
+int hyc_compress_rows(const void* x, int64_t ldx, int64_t M, int64_t H, const hyc_desc* d, void* stored, void* vals,
+                      void* scales, int32_t* row_counts, void* stream);
 /* -> xhat bf16 [M,H]; channel mode reads vals/scales, threshold mode reads the CSR in the descriptor. */
 int hyc_decompress(const void* stored, const void* vals, const void* scales, int64_t M, int64_t H, const hyc_desc* d,
                    void* xhat, void* stream);
@@ -228,11 +232,13 @@ int hyc_low_rank_update(const void* L, const void* R, const void* x, void* out, 
  * (apply_rotary_pos_emb, models/modeling_llama.py:236-260, with the .view().transpose(1, 2) of :423-425).
  *   y[i] = x[i] cos[i] - x[i+h] sin[i],  y[i+h] = x[i+h] cos[i+h] + x[i] sin[i+h],  h = head_dim / 2
  * cos / sin bf16 [S, head_dim]; both NULL = layout change only (the value tensor).  fp32 arithmetic, one rounding.
+ * x_pitch = elements between consecutive tokens of x (heads*head_dim when x is contiguous; larger when x is a column
+ * slice of a fused q/k/v projection).
  * hyc_rope_from_heads is the transpose: gradients [B, heads, S, head_dim] -> [B, S, heads, head_dim],
  *   dx[i] = g[i] cos[i] + g[i+h] sin[i+h],  dx[i+h] = g[i+h] cos[i+h] - g[i] sin[i].
  * head_dim a multiple of 16. */
-int hyc_rope_to_heads(const void* x, const void* cosv, const void* sinv, int64_t B, int64_t S, int64_t heads,
-                      int64_t head_dim, void* out_heads, void* out_rows, void* stream);
+int hyc_rope_to_heads(const void* x, int64_t x_pitch, const void* cosv, const void* sinv, int64_t B, int64_t S,
+                      int64_t heads, int64_t head_dim, void* out_heads, void* out_rows, void* stream);
 int hyc_rope_from_heads(const void* g, const void* cosv, const void* sinv, int64_t B, int64_t S, int64_t heads,
                         int64_t head_dim, void* out_rows, void* stream);
 

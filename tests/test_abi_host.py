@@ -88,15 +88,20 @@ def test_argument_errors_without_a_gpu(abi):
     assert lib.hyc_softmax_causal_fwd(null, 4, 64, 0, 0.0, null, null, null) == abi.EINVAL
     assert lib.hyc_softmax_causal_fwd(null, 4, 64, 65, 0.0, null, null, null) == abi.EINVAL
     assert lib.hyc_softmax_causal_fwd(null, 4, 64, 4, 0.0, null, null, null) == abi.EFAULT
-    assert lib.hyc_rope_to_heads(null, null, null, 2, 8, 4, 24, null, null, null) == abi.EINVAL      # head_dim % 16
-    assert lib.hyc_rope_to_heads(null, null, null, 0, 8, 4, 32, null, null, null) == 0
-    assert lib.hyc_rope_to_heads(null, null, null, 2, 8, 4, 32, null, null, null) == abi.EFAULT
+    assert lib.hyc_rope_to_heads(null, 96, null, null, 2, 8, 4, 24, null, null, null) == abi.EINVAL      # head_dim % 16
+    assert lib.hyc_rope_to_heads(null, 128, null, null, 0, 8, 4, 32, null, null, null) == 0
+    assert lib.hyc_rope_to_heads(null, 120, null, null, 2, 8, 4, 32, null, null, null) == abi.EINVAL     # pitch < heads*head_dim
+    assert lib.hyc_rope_to_heads(null, 128, null, null, 2, 8, 4, 32, null, null, null) == abi.EFAULT
     assert lib.hyc_rope_from_heads(null, null, null, 2, 8, 0, 32, null, null) == abi.EINVAL
     assert lib.hyc_rope_from_heads(null, null, null, 1 << 20, 1 << 12, 64, 128, null, null) == abi.EINVAL   # 2^32 items
     assert lib.hyc_dropout(null, null, 16, 1.0, 5, 0, null) == abi.EINVAL              # p must be below 1
     assert lib.hyc_dropout(null, null, 1 << 31, 0.1, 5, 0, null) == abi.EINVAL
     assert lib.hyc_dropout(null, null, 0, 0.1, 5, 0, null) == 0
     assert lib.hyc_dropout(null, null, 16, 0.1, 5, 0, null) == abi.EFAULT
+    assert lib.hyc_compress_rows(null, 4000, 4, 4096, ctypes.byref(d), null, null, null, null, null) == abi.EINVAL       # pitch < H
+    assert lib.hyc_compress_rows(null, 4100, 4, 4096, ctypes.byref(d), null, null, null, null, null) == abi.EINVAL       # pitch % 8
+    assert lib.hyc_compress_rows(null, 8192, 4, 4096, ctypes.byref(t), null, null, null, null, null) == abi.EINVAL  # threshold scheme
+    assert lib.hyc_compress_rows(null, 8192, 4, 4096, ctypes.byref(d), null, null, null, null, null) == abi.EFAULT
     assert lib.hyc_kth_value_workspace_bytes() >= 1024 + 12
     assert lib.hyc_kth_value(null, 7, 10, 1, null, null, null) == abi.ENOTSUP
     assert lib.hyc_kth_value(null, abi.DTYPE_F32, 0, 1, null, null, null) == abi.EINVAL

@@ -616,3 +616,28 @@ def test_softmax_in_place(K):
         gb = g.clone()
         dx2 = K.softmax_bwd(gb, sp_want, inplace=True)
         assert dx2.data_ptr() == gb.data_ptr() and torch.equal(dx2, dx)
+
+
+def test_column_slices_need_no_copy(K):
+    """compress and the rotary kernel take a column slice of a wider matrix (rows a fixed pitch apart) and give the
+    bits they give for a contiguous copy of it"""
+    gen = torch.Generator().manual_seed(17)
+    B, S, nh, hd = 2, 40, 4, 64
+    H = nh * hd
+    wide = torch.randn(B, S, 3 * H, generator=gen).bfloat16().cuda()
+    wide[..., H + 3] *= 20
+    part = wide[..., H:2 * H]
+    assert not part.is_contiguous()
+    rows = part.reshape(B * S, H)
+    assert rows.data_ptr() == part.data_ptr()                      # a view: nothing was copied
+    plan = K.select_channels(K.channel_absmax(rows), 3)
+    a = K.compress_channel(rows, plan, 4, 64)
+    b = K.compress_channel(rows.contiguous(), plan, 4, 64)
+    assert torch.equal(a.stored, b.stored) and torch.equal(a.vals, b.vals) and torch.equal(a.scales, b.scales)
+    cos = torch.randn(S, hd, generator=gen).bfloat16().cuda()
+    sin = torch.randn(S, hd, generator=gen).bfloat16().cuda()
+    h1, r1 = K.rope_to_heads(part, nh, cos, sin, want_rows=True)
+    h2, r2 = K.rope_to_heads(part.contiguous(), nh, cos, sin, want_rows=True)
+    assert torch.equal(h1, h2) and torch.equal(r1, r2) and r1.is_contiguous()
+    with pytest.raises(ValueError):
+        K.rope_to_heads(wide[..., ::2], nh)                        # channels not contiguous
