@@ -156,3 +156,22 @@ def true_compress_softmax(x: torch.Tensor, outlier: float):
 @torch.no_grad()
 def true_decompress_softmax(x_sparse: torch.Tensor):
     return K.sparse_coo_to_dense(x_sparse)
+
+
+# ---- small helpers other code may import (reference :71-95, :284-290) -------------------------------------
+def convert_coo_to_tuple(x_coo):
+    """identity, as in the reference (its int16 tuple form sits unreachable behind an early return)"""
+    return x_coo
+
+
+def convert_tuple_to_coo(x_coo_tuple):
+    return x_coo_tuple
+
+
+def profile_memory(name):
+    """debug print of the allocator state in MiB"""
+    mib = 1024 * 1024
+    print("%s %s %s" % ("-" * 21, name, "-" * 21))
+    print("allocated: %.2f MB" % (torch.cuda.memory_allocated() / mib), flush=True)
+    print("reserved:  %.2f MB" % (torch.cuda.memory_reserved() / mib), flush=True)
+    print("-" * 50)

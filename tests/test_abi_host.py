@@ -200,7 +200,8 @@ def test_module_constructors_mirror_the_reference(hyc):
     cf = ops.compress_function
     for name in ("true_divide_outlier_suboutlier_svd_compress", "true_divide_outlier_suboutlier_svd_decompress",
                  "true_compress_softmax", "true_decompress_softmax", "prune_softmax", "get_statistics",
-                 "get_statistics_softmax", "pad_cut_L", "hidden_to_head_shape", "head_to_hidden_shape"):
+                 "get_statistics_softmax", "pad_cut_L", "hidden_to_head_shape", "head_to_hidden_shape",
+                 "convert_coo_to_tuple", "convert_tuple_to_coo", "profile_memory"):
         assert callable(getattr(cf, name))
     assert callable(ops.fused_compression.low_rank_extraction) and callable(ops.fused_compression.low_rank_addition)
     x = torch.arange(2 * 3 * 8, dtype=torch.float32).reshape(2, 3, 8)
