@@ -444,6 +444,7 @@ static int direct_splits(int64_t M, int64_t N_out, int64_t H) {
 constexpr int WK = 32;      // tokens per stage
 constexpr int WN = 128;     // dY features per workgroup: WN (four waves) or 2*WN (eight waves)
 constexpr int WH = 256;     // channels per workgroup
+constexpr int WPAD = 32;    // row padding of the wide kernel's LDS tiles, in elements
 
 // Buffer loads: a resource is (base, bytes); an offset at or beyond `bytes` reads as zero instead of faulting.
 typedef __amdgpu_buffer_rsrc_t BufferRsrc;
@@ -482,7 +483,7 @@ k_gradw_wide(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_
   constexpr int HS = WH / NSEG;               // columns of the tile that come from one segment
   constexpr int CPR = HS / 8;                 // packed 8-byte chunks (channel scheme) / 16-byte chunks (dense) per token row and segment
   constexpr int THREADS = 2 * WNT;            // waves: WNT/64 along n x 2 along h, 64 x 128 each
-  constexpr int AP = WNT + GPAD, BP = WH + GPAD;
+  constexpr int AP = WNT + WPAD, BP = WH + WPAD;
   __shared__ __align__(16) uint16_t As[2][WK * AP];
   __shared__ __align__(16) uint16_t Bs[2][WK * BP];
 
