@@ -123,8 +123,11 @@ def gradw_extra(pkg, torch, wl):
         ms = time_events(torch, fn, iters, 3)
         xh = K.decompress_channel(wl.c)
         ms_lib = time_events(torch, lambda: torch.matmul(dy.t(), xh), iters, 3)
+        # the same library's other route: decompress into a scratch matrix, then this kernel on the dense operand
+        ms_staged = time_events(torch, lambda: K.gradw_gemm(dy, wl.c, staged=True), iters, 3)
         out[name] = {"M": M, "N_out": N, "H": H, "ms": round(ms, 5), "TFLOPs": round(2 * M * N * H / ms / 1e9, 1),
                      "frac_of_bf16_mfma_peak": round(2 * M * N * H / ms / 1e9 / 2500.0, 4),
+                     "staged_ms": round(ms_staged, 5), "staged_TFLOPs": round(2 * M * N * H / ms_staged / 1e9, 1),
                      "library_gemm_on_decompressed_ms": round(ms_lib, 5)}
         del dy, dw, ws, xh
     return out

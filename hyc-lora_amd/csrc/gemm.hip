@@ -616,10 +616,10 @@ k_gradw_wide(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_
     }
   };
   // The 16 MFMAs of a stage run as 8 pairs (k sub-step t/4, column tile t%4; both row tiles of the wave).  Operand
-  // fragments are fetched two pairs ahead of their use (a ring of three B fragments, the A fragments of the second
+  // fragments are fetched two pairs ahead of their use (a ring of four B fragments, the A fragments of the second
   // sub-step during the first), so the LDS latency sits under the MFMAs already issued.
   auto mfma_stage = [&](int buf) __attribute__((always_inline)) {
-    bf16x8_t af[2][2], bq[3];
+    bf16x8_t af[2][2], bq[4];
     af[0][0] = frag32(As[buf], AP, wn, 0);
     af[0][1] = frag32(As[buf], AP, wn + 32, 0);
     bq[0] = frag32(Bs[buf], BP, wh, 0);
@@ -627,7 +627,7 @@ k_gradw_wide(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_
 #pragma unroll
     for (int t = 0; t < 8; ++t) {
       __builtin_amdgcn_sched_barrier(0);
-      if (t + 2 < 8) bq[(t + 2) % 3] = frag32(Bs[buf], BP, wh + 32 * ((t + 2) & 3), 16 * ((t + 2) >> 2));
+      if (t + 2 < 8) bq[(t + 2) & 3] = frag32(Bs[buf], BP, wh + 32 * ((t + 2) & 3), 16 * ((t + 2) >> 2));
       if (t == 1) {
         af[1][0] = frag32(As[buf], AP, wn, 16);
         af[1][1] = frag32(As[buf], AP, wn + 32, 16);
@@ -635,7 +635,7 @@ k_gradw_wide(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int a = 0; a < 2; ++a)
-        acc[a][t & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[t >> 2][a], bq[t % 3], acc[a][t & 3], 0, 0, 0);
+        acc[a][t & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[t >> 2][a], bq[t & 3], acc[a][t & 3], 0, 0, 0);
     }
   };
 
@@ -674,7 +674,7 @@ k_gradw_wide(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_
           }
         // the pair schedule of mfma_stage, with one decode piece after every (EVERY-th) MFMA
         int piece = 0;
-        bf16x8_t af[2][2], bq[3];
+        bf16x8_t af[2][2], bq[4];
         af[0][0] = frag32(As[buf], AP, wn, 0);
         af[0][1] = frag32(As[buf], AP, wn + 32, 0);
         bq[0] = frag32(Bs[buf], BP, wh, 0);
@@ -683,7 +683,7 @@ k_gradw_wide(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_
         for (int t = 0; t < 8; ++t) {
           const int k = t >> 2, b = t & 3;
           __builtin_amdgcn_sched_barrier(0);
-          if (t + 2 < 8) bq[(t + 2) % 3] = frag32(Bs[buf], BP, wh + 32 * ((t + 2) & 3), 16 * ((t + 2) >> 2));
+          if (t + 2 < 8) bq[(t + 2) & 3] = frag32(Bs[buf], BP, wh + 32 * ((t + 2) & 3), 16 * ((t + 2) >> 2));
           if (t == 1) {
             af[1][0] = frag32(As[buf], AP, wn, 16);
             af[1][1] = frag32(As[buf], AP, wn + 32, 16);
@@ -691,7 +691,7 @@ k_gradw_wide(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_
 #pragma unroll
           for (int a = 0; a < 2; ++a) {
             __builtin_amdgcn_sched_barrier(0);
-            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[k][a], bq[t % 3], acc[a][b], 0, 0, 0);
+            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[k][a], bq[t & 3], acc[a][b], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
             if ((2 * t + a) % EVERY == 0) {
               const int u = piece / (4 * NST), i = (piece / 4) % NST, w = piece % 4;

@@ -418,10 +418,21 @@ def gated_act_bwd(act, g2d, src_act, src_up, src_gate):
 # ----------------------------------------------------------------------------------------------------
 # weight gradient
 # ----------------------------------------------------------------------------------------------------
-def gradw_gemm(dy2d, src, out_dtype=BF16, alpha=1.0, out=None, beta=0.0):
-    """dW [N_out, H] = alpha * dy^T @ x_hat (+ beta * out); src as for rmsnorm_bwd"""
+STAGED_GRADW_MIN_FEATURES = 2048
+
+
+def gradw_gemm(dy2d, src, out_dtype=BF16, alpha=1.0, out=None, beta=0.0, staged=None):
+    """dW [N_out, H] = alpha * dy^T @ x_hat (+ beta * out); src as for rmsnorm_bwd.
+
+    A compressed src is decoded inside the GEMM.  Every 256 output features decode the same activation tile again, so
+    for wide outputs (N_out >= 2048; not a shape LoRA training has) it is cheaper to restore x_hat once into a
+    transient matrix and run the same kernel on the dense operand (`staged`; None = by that rule)."""
     _need(dy2d, BF16, "grad_output")
     M, N_out = dy2d.shape
+    if staged is None:
+        staged = N_out >= STAGED_GRADW_MIN_FEATURES
+    if staged and isinstance(src, ChannelCompressed):
+        src = decompress_channel(src)
     stored, vals, scales, d = _source(src)
     H = src.H if isinstance(src, (ChannelCompressed, ThresholdCompressed)) else stored.shape[-1]
     lib = _abi.load()

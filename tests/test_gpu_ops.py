@@ -45,16 +45,19 @@ def test_gradw_channel(K, bits, group, M, H, N, k):
     c = K.compress_channel(xd, plan, bits, group)
     xh = K.decompress_channel(c)
     want = dy.float().t() @ xh.cpu().float()
-    got32 = K.gradw_gemm(dy.cuda(), c, out_dtype=torch.float32).cpu()
+    got32 = K.gradw_gemm(dy.cuda(), c, out_dtype=torch.float32, staged=False).cpu()      # decoded inside the GEMM
     assert torch.allclose(got32, want, rtol=1e-3, atol=1e-3 * float(want.abs().max()) + 1e-6)
-    got16 = K.gradw_gemm(dy.cuda(), c, out_dtype=torch.bfloat16).cpu()
+    got16 = K.gradw_gemm(dy.cuda(), c, out_dtype=torch.bfloat16, staged=False).cpu()
     assert torch.allclose(got16.float(), want, rtol=1e-2, atol=1e-3 * float(want.abs().max()) + 1e-3)
     if H % 128 == 0:
         dense = K.gradw_gemm(dy.cuda(), xh, out_dtype=torch.float32).cpu()
         assert torch.allclose(dense, got32, rtol=1e-5, atol=1e-5 * float(want.abs().max()))
+        # the staged route (restore once, then the same kernel on the dense operand) is what wide outputs default to
+        assert torch.equal(K.gradw_gemm(dy.cuda(), c, out_dtype=torch.float32, staged=True).cpu(), dense)
+        assert torch.equal(K.gradw_gemm(dy.cuda(), c, out_dtype=torch.float32).cpu(), dense if N >= 2048 else got32)
     # alpha / beta
     base = torch.ones(N, H, dtype=torch.float32, device="cuda")
-    out = K.gradw_gemm(dy.cuda(), c, alpha=2.0, out=base, beta=0.5).cpu()
+    out = K.gradw_gemm(dy.cuda(), c, alpha=2.0, out=base, beta=0.5, staged=False).cpu()
     assert torch.allclose(out, 2.0 * want + 0.5, rtol=1e-3, atol=2e-3 * float(want.abs().max()) + 1e-6)
 
 
