@@ -26,7 +26,7 @@ static Divisor make_divisor(int64_t d) {
   return r;
 }
 
-// An item is 8 channels of the low half and the matching 8 of the high half of one (b, s, head); fewer than 2^32 items.
+// An item is 8 channels of the low half and the matching 8 of the high half of one (b, s, head); fewer than 2^31 items.
 // TO_HEADS: in = rows layout, out_heads (and optionally out_rows); else in = heads layout, out = rows layout.
 template <bool TO_HEADS, bool ROTATE>
 __global__ void __launch_bounds__(256)
@@ -88,8 +88,8 @@ static int rope_args(const char* who, int64_t B, int64_t S, int64_t nh, int64_t 
   if (B < 0 || S < 0 || nh <= 0 || hd <= 0 || hd % 16 != 0 || hd > 1024 || nh > 65536)
     return fail(HYC_EINVAL, "%s: B=%lld S=%lld heads=%lld head_dim=%lld (head_dim must be a multiple of 16, at most 1024)",
                 who, (long long)B, (long long)S, (long long)nh, (long long)hd);
-  if (S > 0 && B * S * nh > (((int64_t)1 << 32) - 1) / (hd / 16))
-    return fail(HYC_EINVAL, "%s: B*S*heads*head_dim/16 must stay below 2^32", who);
+  if (S > 0 && B * S * nh > (((int64_t)1 << 31) - 1) / (hd / 16))      // 32-bit item counter with room for its stride
+    return fail(HYC_EINVAL, "%s: B*S*heads*head_dim/16 must stay below 2^31", who);
   return HYC_OK;
 }
 

@@ -93,7 +93,7 @@ def test_argument_errors_without_a_gpu(abi):
     assert lib.hyc_rope_to_heads(null, 120, null, null, 2, 8, 4, 32, null, null, null) == abi.EINVAL     # pitch < heads*head_dim
     assert lib.hyc_rope_to_heads(null, 128, null, null, 2, 8, 4, 32, null, null, null) == abi.EFAULT
     assert lib.hyc_rope_from_heads(null, null, null, 2, 8, 0, 32, null, null) == abi.EINVAL
-    assert lib.hyc_rope_from_heads(null, null, null, 1 << 20, 1 << 12, 64, 128, null, null) == abi.EINVAL   # 2^32 items
+    assert lib.hyc_rope_from_heads(null, null, null, 1 << 20, 1 << 12, 64, 128, null, null) == abi.EINVAL   # 2^31 items
     assert lib.hyc_dropout(null, null, 16, 1.0, 5, 0, null) == abi.EINVAL              # p must be below 1
     assert lib.hyc_dropout(null, null, 1 << 31, 0.1, 5, 0, null) == abi.EINVAL
     assert lib.hyc_dropout(null, null, 0, 0.1, 5, 0, null) == 0
