@@ -161,7 +161,8 @@ def kernel_tour(pkg, torch, reps=5):
             K.hadamard_bwd(g, cs[2], cs[1])
             K.gated_act_bwd("silu", g, cs[2], cs[1], cs[0])
             K.gradw_gemm(dy16, cs[0])
-            K.gradw_gemm(dyN, cs[0])
+            K.gradw_gemm(dyN, cs[0], staged=False)        # x_hat decoded inside the GEMM
+            K.gradw_gemm(dyN, cs[0], staged=True)         # x_hat restored once, then the dense form of the kernel
         torch.cuda.synchronize()
         del x, up, a, g, cs
     # softmax at config 5's shape: probabilities [1, 32, 2048, 2048], 5 % kept
