@@ -27,7 +27,9 @@ TRAFFIC_BWD = int((21039.0 * 1.9986 + 36888.7) * 1024)
 
 
 def algorithmic_bytes(M, H, bits, group, k):
-    """per-launch bytes a perfect kernel must move (no re-reads): see DESIGN.md for the derivation"""
+    """per-launch bytes a perfect kernel must move (every tensor read or written once): per token the forward reads x
+    and writes y, the packed codes, the outlier values, the group scales and rstd; the backward reads dy and that side
+    data and writes dx"""
     side = H * bits // 8 + 2 * k + 2 * (H // group)          # packed codes + outlier values + group scales
     fwd = M * (2 * H + 2 * H + side + 4)                       # read x, write y, side data, rstd
     bwd = M * (2 * H + side + 4 + 2 * H)                       # read dy, side data, rstd; write dx
