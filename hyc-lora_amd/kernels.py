@@ -33,6 +33,20 @@ def _need(t, dtype, name):
     return t
 
 
+def _need_vec(t, dtype, n, name):
+    """a contiguous device vector of exactly n elements (the kernels index it without further checks)"""
+    _need(t, dtype, name)
+    if t.numel() != n:
+        raise ValueError("%s must hold %d elements, got %d" % (name, n, t.numel()))
+    return t
+
+
+def _need_weight(w, H):
+    if not isinstance(w, torch.Tensor) or not w.is_cuda or not w.is_contiguous() or w.numel() != H:
+        raise ValueError("weight must be a contiguous CUDA tensor of %d elements" % H)
+    return w
+
+
 def num_outlier_channels(H, ratio):
     """k = floor(ratio*H + 1/2)"""
     import math
@@ -75,6 +89,7 @@ def channel_absmax(x2d, amax=None):
     M, H = x2d.shape
     if amax is None:
         amax = torch.zeros(H, dtype=torch.float32, device=x2d.device)
+    _need_vec(amax, torch.float32, H, "amax")
     check(_abi.load().hyc_channel_absmax(_p(x2d), M, H, _p(amax), _stream()))
     return amax
 
@@ -82,6 +97,8 @@ def channel_absmax(x2d, amax=None):
 def select_channels(amax, k):
     _need(amax, torch.float32, "amax")
     H = amax.numel()
+    if H % 8 or not 0 <= k <= H:
+        raise ValueError("select_channels: H=%d must be a multiple of 8 and 0 <= k=%d <= H" % (H, k))
     idx = torch.empty(max(k, 1), dtype=torch.int32, device=amax.device)[:k]
     plan = torch.empty(H // 8, dtype=torch.int32, device=amax.device)
     check(_abi.load().hyc_select_channels(_p(amax), H, k, _p(idx), _p(plan), _stream()))
@@ -122,6 +139,8 @@ class ChannelCompressed:
 
 
 def alloc_channel(M, H, plan, bits, group, device):
+    if plan.H != H:
+        raise ValueError("the outlier-channel plan was made for %d channels, the activation has %d" % (plan.H, H))
     stored = torch.empty((M, H * bits // 8), dtype=torch.int8 if bits == 8 else torch.uint8, device=device)
     vals = torch.empty((M, plan.k), dtype=BF16, device=device)
     scales = torch.empty((M, H // group), dtype=BF16, device=device)
@@ -282,9 +301,8 @@ def _wdtype(w):
 def rmsnorm_fwd_compress_channel(x2d, w, eps, plan, bits, group):
     """-> (y bf16 [M,H], rstd fp32 [M], ChannelCompressed of x)"""
     _need(x2d, BF16, "x")
-    if not (w.is_cuda and w.is_contiguous()):
-        raise ValueError("weight must be a contiguous CUDA tensor")
     M, H = x2d.shape
+    _need_weight(w, H)
     lib = _abi.load()
     check(lib.hyc_check_shape(H, bits, group, _abi.MODE_CHANNEL))
     y = torch.empty_like(x2d)
@@ -301,6 +319,7 @@ def rmsnorm_fwd_compress_threshold(x2d, w, eps, S, threshold, scale, bits, L=Non
     _need(x2d, BF16, "x")
     _need(scale, BF16, "scale")
     M, H = x2d.shape
+    _need_weight(w, H)
     lib = _abi.load()
     dev = x2d.device
     if L is not None:
@@ -323,13 +342,17 @@ def rmsnorm_fwd_compress_threshold(x2d, w, eps, S, threshold, scale, bits, L=Non
     return y, rstd, ThresholdCompressed(stored, row_ptr, cols, vals, float(threshold), scale, L, R, bits, M, H, S)
 
 
-def _source(c):
-    """(stored, vals, scales, desc) of a ChannelCompressed, or of a dense bf16 x_hat"""
+def _source(c, M, H):
+    """(stored, vals, scales, desc) of a ChannelCompressed, or of a dense bf16 x_hat, that holds an [M, H] activation"""
+    if isinstance(c, (ChannelCompressed, ThresholdCompressed)) and (c.M, c.H) != (M, H):
+        raise ValueError("the saved activation is [%d, %d], the gradient is [%d, %d]" % (c.M, c.H, M, H))
     if isinstance(c, ChannelCompressed):
         return c.stored, c.vals, c.scales, c.desc()
     if isinstance(c, ThresholdCompressed):
         c = decompress_threshold(c)
     _need(c, BF16, "x_hat")
+    if c.numel() != M * H or c.shape[-1] != H:
+        raise ValueError("the saved activation is %s, the gradient is [%d, %d]" % (tuple(c.shape), M, H))
     return c, None, None, dense_desc()
 
 
@@ -337,8 +360,10 @@ def rmsnorm_bwd(dy2d, src, w, rstd, c2_quirk=True):
     """-> (dx bf16 [M,H], dw in w's dtype [H]); src is a ChannelCompressed, ThresholdCompressed or dense x_hat"""
     _need(dy2d, BF16, "dy")
     M, H = dy2d.shape
+    _need_weight(w, H)
+    _need_vec(rstd, torch.float32, M, "rstd")
     lib = _abi.load()
-    stored, vals, scales, d = _source(src)
+    stored, vals, scales, d = _source(src, M, H)
     P = lib.hyc_rmsnorm_bwd_partials(M, H)
     partials = torch.empty((max(P, 1), H), dtype=torch.float32, device=dy2d.device)
     dx = torch.empty_like(dy2d)
@@ -352,8 +377,11 @@ def layernorm_bwd(dy2d, src, w, mean, rstd):
     """-> (dx bf16 [M,H], dw in w's dtype [H]) with xn = (x_hat - mean) * rstd; db = dy.sum(0) is the caller's"""
     _need(dy2d, BF16, "dy")
     M, H = dy2d.shape
+    _need_weight(w, H)
+    _need_vec(mean, torch.float32, M, "mean")
+    _need_vec(rstd, torch.float32, M, "rstd")
     lib = _abi.load()
-    stored, vals, scales, d = _source(src)
+    stored, vals, scales, d = _source(src, M, H)
     P = lib.hyc_rmsnorm_bwd_partials(M, H)
     partials = torch.empty((max(P, 1), H), dtype=torch.float32, device=dy2d.device)
     dx = torch.empty_like(dy2d)
@@ -367,8 +395,10 @@ def rmsnorm_bwd_partial(dy2d, src, w, rstd, c2_quirk=True):
     """-> (dx bf16 [M,H], fp32 partial rows [P,H] whose column sum is dw); the caller does the last reduction"""
     _need(dy2d, BF16, "dy")
     M, H = dy2d.shape
+    _need_weight(w, H)
+    _need_vec(rstd, torch.float32, M, "rstd")
     lib = _abi.load()
-    stored, vals, scales, d = _source(src)
+    stored, vals, scales, d = _source(src, M, H)
     P = lib.hyc_rmsnorm_bwd_partials(M, H)
     partials = torch.empty((max(P, 1), H), dtype=torch.float32, device=dy2d.device)
     dx = torch.empty_like(dy2d)
@@ -381,7 +411,7 @@ def act_bwd(act, g2d, src):
     """act in {'silu', 'gelu'} -> dx bf16 [M,H]"""
     _need(g2d, BF16, "grad_output")
     M, H = g2d.shape
-    stored, vals, scales, d = _source(src)
+    stored, vals, scales, d = _source(src, M, H)
     dx = torch.empty_like(g2d)
     code = {"silu": _abi.ACT_SILU, "gelu": _abi.ACT_GELU_TANH}[act]
     check(_abi.load().hyc_act_bwd(code, _p(g2d), _p(stored), _p(vals), _p(scales), M, H, ctypes.byref(d), _p(dx), _stream()))
@@ -392,8 +422,8 @@ def hadamard_bwd(g2d, src1, src2):
     """-> (g * x2_hat, x1_hat * g)"""
     _need(g2d, BF16, "grad_output")
     M, H = g2d.shape
-    s1, v1, c1, d1 = _source(src1)
-    s2, v2, c2, d2 = _source(src2)
+    s1, v1, c1, d1 = _source(src1, M, H)
+    s2, v2, c2, d2 = _source(src2, M, H)
     dx1, dx2 = torch.empty_like(g2d), torch.empty_like(g2d)
     check(_abi.load().hyc_hadamard_bwd(_p(g2d), _p(s1), _p(v1), _p(c1), ctypes.byref(d1), _p(s2), _p(v2), _p(c2),
                                        ctypes.byref(d2), M, H, _p(dx1), _p(dx2), _stream()))
@@ -404,9 +434,9 @@ def gated_act_bwd(act, g2d, src_act, src_up, src_gate):
     """backward of act(gate) * up in one pass -> (d_gate, d_up); the three sources are ChannelCompressed"""
     _need(g2d, BF16, "grad_output")
     M, H = g2d.shape
-    sa, va, ca, da = _source(src_act)
-    su, vu, cu, du = _source(src_up)
-    sg, vg, cg, dg = _source(src_gate)
+    sa, va, ca, da = _source(src_act, M, H)
+    su, vu, cu, du = _source(src_up, M, H)
+    sg, vg, cg, dg = _source(src_gate, M, H)
     d_gate, d_up = torch.empty_like(g2d), torch.empty_like(g2d)
     code = {"silu": _abi.ACT_SILU, "gelu": _abi.ACT_GELU_TANH}[act]
     check(_abi.load().hyc_gated_act_bwd(code, _p(g2d), _p(sa), _p(va), _p(ca), ctypes.byref(da), _p(su), _p(vu), _p(cu),
@@ -433,11 +463,14 @@ def gradw_gemm(dy2d, src, out_dtype=BF16, alpha=1.0, out=None, beta=0.0, staged=
         staged = N_out >= STAGED_GRADW_MIN_FEATURES
     if staged and isinstance(src, ChannelCompressed):
         src = decompress_channel(src)
-    stored, vals, scales, d = _source(src)
-    H = src.H if isinstance(src, (ChannelCompressed, ThresholdCompressed)) else stored.shape[-1]
+    H = src.H if isinstance(src, (ChannelCompressed, ThresholdCompressed)) else src.shape[-1]
+    stored, vals, scales, d = _source(src, M, H)
     lib = _abi.load()
     if out is None:
         out = torch.empty((N_out, H), dtype=out_dtype, device=dy2d.device)
+    elif (not out.is_cuda or not out.is_contiguous() or tuple(out.shape) != (N_out, H)
+          or out.dtype not in (BF16, torch.float32)):
+        raise ValueError("out must be a contiguous bf16 or fp32 [%d, %d] CUDA tensor" % (N_out, H))
     ws_bytes = lib.hyc_gradw_workspace_bytes(M, N_out, H)
     ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=dy2d.device) if ws_bytes else None
     code = _abi.DTYPE_F32 if out.dtype == torch.float32 else _abi.DTYPE_BF16
@@ -516,6 +549,8 @@ def softmax_bwd(g, sp: SparseRows, inplace=False):
     _need(g, BF16, "grad_output")
     N = g.shape[-1]
     g2 = g.reshape(-1, N)
+    if sp.rows != g2.shape[0] or sp.shape[-1] != N:
+        raise ValueError("the kept probabilities are %s, the gradient is %s" % (tuple(sp.shape), tuple(g.shape)))
     dx = g2 if inplace else torch.empty_like(g2)
     check(_abi.load().hyc_softmax_bwd(_p(g2), g2.shape[0], N, _p(sp.row_ptr), _p(sp.cols) if sp.cols.numel() else None,
                                       _p(sp.vals) if sp.vals.numel() else None, _p(dx), _stream()))
@@ -585,6 +620,8 @@ def low_rank_update(l, r, x, subtract, out=None):
         raise ValueError("Incompatible dimensions")
     if out is None:
         out = torch.empty_like(x)
+    elif _need(out, BF16, "out").shape != x.shape:
+        raise ValueError("out must have x's shape")
     check(_abi.load().hyc_low_rank_update(_p(l), _p(r), _p(x), _p(out), M, S, H, l.shape[1], 1 if subtract else 0, _stream()))
     return out
 
@@ -606,6 +643,8 @@ class NF4Weight:
 def nf4_quantize(w):
     _need(w, BF16, "w")
     n = w.numel()
+    if n % 64:
+        raise ValueError("NF4 blocks hold 64 weights: %d is not a multiple of 64" % n)
     packed = torch.empty(n // 2, dtype=torch.uint8, device=w.device)
     absmax = torch.empty(n // 64, dtype=torch.float32, device=w.device)
     check(_abi.load().hyc_nf4_quantize(_p(w), n, _p(packed), _p(absmax), _stream()))
@@ -616,6 +655,8 @@ def nf4_dequantize(q: NF4Weight, out=None):
     n = q.packed.numel() * 2
     if out is None:
         out = torch.empty(q.shape, dtype=BF16, device=q.packed.device)
+    elif _need(out, BF16, "out").numel() != n:
+        raise ValueError("out must hold %d weights" % n)
     check(_abi.load().hyc_nf4_dequantize(_p(q.packed), _p(q.absmax), n, _p(out), _stream()))
     return out
 
@@ -623,6 +664,14 @@ def nf4_dequantize(q: NF4Weight, out=None):
 # ----------------------------------------------------------------------------------------------------
 # rotary embedding + attention layout
 # ----------------------------------------------------------------------------------------------------
+def _need_tables(cos, sin, S, hd):
+    if (cos is None) != (sin is None):
+        raise ValueError("cos and sin go together")
+    if cos is not None:
+        _need_vec(cos, BF16, S * hd, "cos")
+        _need_vec(sin, BF16, S * hd, "sin")
+
+
 def rope_to_heads(x, heads, cos=None, sin=None, want_rows=False):
     """x bf16 [B, S, heads*hd] -> rotated [B, heads, S, hd] contiguous (and, with want_rows, also [B, S, heads*hd]);
     cos / sin bf16 [S, hd]; without them only the layout changes.  x may be a column slice of a wider [B, S, *]
@@ -633,7 +682,10 @@ def rope_to_heads(x, heads, cos=None, sin=None, want_rows=False):
     pitch = x.stride(1) if S > 1 else H
     if x.stride(2) != 1 or (B > 1 and x.stride(0) != S * pitch):
         raise ValueError("x must have contiguous channels and evenly spaced tokens")
+    if heads <= 0 or H % heads:
+        raise ValueError("%d channels do not split into %d heads" % (H, heads))
     hd = H // heads
+    _need_tables(cos, sin, S, hd)
     out_heads = torch.empty((B, heads, S, hd), dtype=BF16, device=x.device)
     out_rows = torch.empty((B, S, H), dtype=BF16, device=x.device) if want_rows else None
     check(_abi.load().hyc_rope_to_heads(_p(x), pitch, _p(cos), _p(sin), B, S, heads, hd, _p(out_heads), _p(out_rows),
@@ -645,6 +697,7 @@ def rope_from_heads(g, cos=None, sin=None):
     """gradient bf16 [B, heads, S, hd] -> [B, S, heads*hd] through the transposed rotation"""
     _need(g, BF16, "g")
     B, heads, S, hd = g.shape
+    _need_tables(cos, sin, S, hd)
     out = torch.empty((B, S, heads * hd), dtype=BF16, device=g.device)
     check(_abi.load().hyc_rope_from_heads(_p(g), _p(cos), _p(sin), B, S, heads, hd, _p(out), _stream()))
     return out

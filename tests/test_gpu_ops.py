@@ -644,3 +644,40 @@ def test_column_slices_need_no_copy(K):
     assert torch.equal(h1, h2) and torch.equal(r1, r2) and r1.is_contiguous()
     with pytest.raises(ValueError):
         K.rope_to_heads(wide[..., ::2], nh)                        # channels not contiguous
+
+
+def test_launchers_reject_operands_that_do_not_fit(K):
+    """Shapes are checked on the host: a kernel indexes its operands by the shape of the gradient alone."""
+    x, gen = make_x(0, 64, 512, 5, 20)
+    xd = x.cuda()
+    plan = K.select_channels(K.channel_absmax(xd), 5)
+    c = K.compress_channel(xd, plan, 4, 128)
+    w = torch.ones(512, device="cuda")
+    _, rstd, _ = K.rmsnorm_fwd_compress_channel(xd, w, 1e-6, plan, 4, 128)
+    g = torch.zeros(64, 512, dtype=torch.bfloat16, device="cuda")
+    wide = torch.zeros(64, 1024, dtype=torch.bfloat16, device="cuda")
+    tall = torch.zeros(128, 512, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ValueError):
+        K.compress_channel(wide, plan, 4, 128)                 # a plan made for another width
+    with pytest.raises(ValueError):
+        K.act_bwd("silu", tall, c)                             # more gradient rows than saved rows
+    with pytest.raises(ValueError):
+        K.hadamard_bwd(g, c, wide)
+    with pytest.raises(ValueError):
+        K.rmsnorm_bwd(g, c, w[:256].contiguous(), rstd)
+    with pytest.raises(ValueError):
+        K.rmsnorm_bwd(g, c, w, rstd[:32].contiguous())
+    with pytest.raises(ValueError):
+        K.gradw_gemm(tall[:, :16].contiguous(), c)
+    with pytest.raises(ValueError):
+        K.gradw_gemm(g[:, :16].contiguous(), c, out=torch.empty(16, 256, dtype=torch.bfloat16, device="cuda"))
+    y, sp = K.softmax_fwd(g, threshold=0.01)
+    with pytest.raises(ValueError):
+        K.softmax_bwd(tall, sp)
+    with pytest.raises(ValueError):
+        K.rope_to_heads(g.view(1, 64, 512), 4, cos=torch.zeros(64, 64, dtype=torch.bfloat16, device="cuda"),
+                        sin=torch.zeros(64, 128, dtype=torch.bfloat16, device="cuda"))
+    with pytest.raises(ValueError):
+        K.nf4_quantize(torch.zeros(100, dtype=torch.bfloat16, device="cuda"))
+    with pytest.raises(ValueError):
+        K.select_channels(torch.zeros(512, device="cuda"), 600)
