@@ -7,15 +7,20 @@ from ._calibration import CompressionSite, as_rows, fold_statistics
 from .compress_function import compress_to_csr, get_statistics
 
 
-def _linear_backward(grad_output, w, saved, use_bias):
+def _linear_backward(grad_output, w, saved, use_bias, needs):
+    """(dX, dW, db); `needs` = ctx.needs_input_grad[:3]: a gradient nobody asked for is not computed (a frozen weight
+    has no dW, and its input was not saved)"""
     g = grad_output.to(w.dtype)
-    grad_input = g @ w
+    grad_input = g @ w if needs[0] else None
     g2, _ = as_rows(g.to(torch.bfloat16))
-    # the reference forms [B, out, in] per batch element and lets autograd sum it; here the sum over all tokens is
-    # accumulated in fp32 inside the kernel and rounded once
-    grad_weight = K.gradw_gemm(g2, saved, out_dtype=torch.float32 if w.dtype == torch.float32 else torch.bfloat16)
-    grad_bias = g2.sum(0).to(w.dtype) if use_bias else None
-    return grad_input, grad_weight.to(w.dtype), grad_bias
+    grad_weight = None
+    if needs[1]:
+        # the reference forms [B, out, in] per batch element and lets autograd sum it; here the sum over all tokens
+        # is accumulated in fp32 inside the kernel and rounded once
+        grad_weight = K.gradw_gemm(g2, saved, out_dtype=torch.float32 if w.dtype == torch.float32 else torch.bfloat16)
+        grad_weight = grad_weight.to(w.dtype)
+    grad_bias = g2.sum(0).to(w.dtype) if use_bias and needs[2] else None
+    return grad_input, grad_weight, grad_bias
 
 
 class EfficientMemoryLinearFunc(torch.autograd.Function):
@@ -34,15 +39,17 @@ class EfficientMemoryLinearFunc(torch.autograd.Function):
                                                   sub_outlier_quantize_method, rank)
         else:
             outlier, L, scale, R = static_value[0], static_value[1], static_value[2], static_value[3]
-        ctx.saved, _ = compress_to_csr(x, outlier, scale, sub_outlier_bit, sub_outlier_ratio,
-                                       L if rank > 0 else None, R if rank > 0 else None)
+        ctx.saved = None
+        if ctx.needs_input_grad[1]:                  # x is kept for dW only
+            ctx.saved, _ = compress_to_csr(x, outlier, scale, sub_outlier_bit, sub_outlier_ratio,
+                                           L if rank > 0 else None, R if rank > 0 else None)
         ctx.w = w
         ctx.mark_non_differentiable(outlier, L, R, scale)
         return output, outlier, L, R, scale
 
     @staticmethod
     def backward(ctx, grad_output, grad_outlier, grad_L, grad_R, grad_scale):
-        gi, gw, gb = _linear_backward(grad_output, ctx.w.detach(), ctx.saved, ctx.use_bias)
+        gi, gw, gb = _linear_backward(grad_output, ctx.w.detach(), ctx.saved, ctx.use_bias, ctx.needs_input_grad[:3])
         return gi, gw, gb, None, None, None, None, None, None, None, None
 
 
@@ -52,14 +59,16 @@ class _ChannelLinearFunc(torch.autograd.Function):
         output = x @ w.transpose(0, 1)
         if b is not None:
             output = output + b[None, ...]
-        x2, _ = as_rows(x)
-        ctx.saved = K.compress_channel(x2, plan, bits, group)
+        ctx.saved = None
+        if ctx.needs_input_grad[1]:                  # x is kept for dW only
+            x2, _ = as_rows(x)
+            ctx.saved = K.compress_channel(x2, plan, bits, group)
         ctx.w, ctx.use_bias = w, b is not None
         return output
 
     @staticmethod
     def backward(ctx, grad_output):
-        gi, gw, gb = _linear_backward(grad_output, ctx.w.detach(), ctx.saved, ctx.use_bias)
+        gi, gw, gb = _linear_backward(grad_output, ctx.w.detach(), ctx.saved, ctx.use_bias, ctx.needs_input_grad[:3])
         return gi, gw, gb, None, None, None
 
 

@@ -41,6 +41,7 @@ class EfficientMemoryRMSNormFunc(torch.autograd.Function):
         ctx.saved = c
         ctx.rstd = rstd
         ctx.weight = weight
+        ctx.c2_quirk = cls.c2_quirk            # as set for this call: modules with different settings share the class
         ctx.mark_non_differentiable(outlier, L, R, scale)
         return y.reshape(x.shape), outlier, L, R, scale
 
@@ -48,7 +49,7 @@ class EfficientMemoryRMSNormFunc(torch.autograd.Function):
     def backward(cls, ctx, dy, grad_outlier, grad_L, grad_R, grad_scale):
         dy2, _ = as_rows(dy.to(torch.bfloat16))
         dx, dw = K.rmsnorm_bwd(dy2, ctx.saved, _effective_weight(ctx.weight, cls.weight_offset), ctx.rstd,
-                               c2_quirk=cls.c2_quirk)
+                               c2_quirk=ctx.c2_quirk)
         return dx.reshape(dy.shape), None, None, None, None, None, None, dw.to(ctx.weight.dtype), None, None, None, None
 
 

@@ -681,3 +681,22 @@ def test_launchers_reject_operands_that_do_not_fit(K):
         K.nf4_quantize(torch.zeros(100, dtype=torch.bfloat16, device="cuda"))
     with pytest.raises(ValueError):
         K.select_channels(torch.zeros(512, device="cuda"), 600)
+
+
+@pytest.mark.parametrize("mode", ["ref", "hyc"])
+def test_linear_with_frozen_weight_saves_nothing(ops, mode):
+    """x is kept for dW only: with a frozen weight nothing is compressed and only dX comes back"""
+    gen = torch.Generator().manual_seed(5)
+    lin = ops.EfficientMemoryLinear(256, 64, bias=False, outlier_ratio=0.01, sub_outlier_ratio=1.0, sub_outlier_bit=4,
+                                    sub_outlier_quantize_method="per-channel", rank=0, mode=mode).cuda().bfloat16()
+    lin.weight.requires_grad_(False)
+    x = torch.randn(2, 32, 256, generator=gen).bfloat16().cuda().requires_grad_(True)
+    y = lin(x)
+    assert y.grad_fn is not None and getattr(y.grad_fn, "saved", None) is None
+    g = torch.randn(2, 32, 64, generator=gen).bfloat16().cuda()
+    y.backward(g)
+    assert lin.weight.grad is None
+    want = g.float() @ lin.weight.float()
+    assert torch.allclose(x.grad.float(), want, rtol=1e-2, atol=1e-2)
+    with torch.no_grad():
+        assert lin(x).shape == (2, 32, 64)
