@@ -305,3 +305,43 @@ def test_calibration_state_round_trip(hyc, tmp_path):
     with pytest.raises(KeyError):
         ops.load_calibration_state(dst, {"nope": {"iteration": 1}})
     assert ops.load_calibration_state(dst, {"nope": {"iteration": 1}}, strict=False) == ["nope"]
+
+
+def test_header_is_plain_c_and_links_from_a_c_program(abi, tmp_path):
+    """The boundary is a C ABI: a C99 translation unit that includes only include/hyc_abi.h references every
+    declared entry point, links against the library and gets the documented codes back (host-only calls)."""
+    import shutil
+    import subprocess
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc")
+    names = declared_symbols()
+    src = tmp_path / "host.c"
+    src.write_text(
+        '#include <stdio.h>\n#include <string.h>\n#include "hyc_abi.h"\n'
+        "typedef void (*entry)(void);\n"
+        "static const entry table[] = {\n" + "".join("  (entry)%s,\n" % n for n in names) + "};\n"
+        "int main(void) {\n"
+        "  hyc_desc d;\n"
+        "  memset(&d, 0, sizeof d);\n"
+        "  if (sizeof table / sizeof table[0] != %d) return 10;\n" % len(names) +
+        "  if (hyc_abi_version() != HYC_ABI_VERSION) return 11;\n"
+        "  if (hyc_check_shape(4096, 4, 128, HYC_MODE_CHANNEL) != HYC_OK) return 12;\n"
+        "  if (hyc_check_shape(4100, 4, 128, HYC_MODE_CHANNEL) != HYC_ENOTSUP) return 13;\n"
+        "  if (!strstr(hyc_last_error(), \"multiple of 16\")) return 14;\n"
+        "  if (hyc_compress(0, 8, 4096, 0, 0, 0, 0, 0, 0) != HYC_EFAULT) return 15;\n"
+        "  d.mode = HYC_MODE_CHANNEL; d.bits = 3; d.group = 128;\n"
+        "  if (hyc_compress(0, 8, 4096, &d, 0, 0, 0, 0, 0) != HYC_ENOTSUP) return 16;\n"
+        "  printf(\"%d entry points\\n\", (int)(sizeof table / sizeof table[0]));\n"
+        "  return 0;\n}\n")
+    exe = tmp_path / "host"
+    libdir = os.path.dirname(abi.LIB_PATH)
+    libname = os.path.basename(abi.LIB_PATH)[3:-3]
+    cmd = [gcc, "-std=c99", "-Wall", "-Werror", "-pedantic", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe),
+           "-L", libdir, "-l" + libname, "-Wl,-rpath," + libdir, "-Wl,-rpath,/opt/rocm/lib", "-L/opt/rocm/lib",
+           "-Wl,--allow-shlib-undefined"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    r = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, (r.returncode, r.stdout, r.stderr)
+    assert "%d entry points" % len(names) in r.stdout
