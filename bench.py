@@ -179,15 +179,17 @@ def kernel_tour(pkg, torch, reps=5):
     print(json.dumps({"kernel_tour": True}))
 
 
-def layer_report(pkg, torch, steps=6):
+def layer_report(pkg, torch, steps=6, attentions=("eager", "flash")):
     """full LLaMA-2-7B-shaped decoder layer (hidden 4096, 32 x 128 heads, intermediate 11008, NF4 base, LoRA r=16 on
     all seven projections), forward + backward, at batch 1 x seq 2048 and batch 4 x seq 1024: what the forward keeps
     for the backward, the peak above the resident weights, and the step time - with every saved activation compressed
-    (1 % outlier channels, INT2 for linear inputs, INT4 elsewhere) and with the same layer keeping bf16."""
+    (1 % outlier channels, INT2 for linear inputs, INT4 elsewhere) and with the same layer keeping bf16; each with the
+    attention the reference wires into its models (scores, softmax, kept probabilities) and with the library's fused
+    attention kernel around compressed q, k, v and output."""
     DL = importlib.import_module("hyc-lora_amd.decoder_layer")
     out = []
-    for compress in (True, False):
-        layer = DL.DecoderLayer(DL.LayerConfig(compress=compress))
+    for compress, attention in [(c, a) for c in (True, False) for a in attentions]:
+        layer = DL.DecoderLayer(DL.LayerConfig(compress=compress, attention=attention))
         torch.cuda.synchronize()
         for (B, S) in ((1, 2048), (4, 1024)):
             gen = torch.Generator(device="cuda").manual_seed(B * 7 + S)
@@ -221,7 +223,7 @@ def layer_report(pkg, torch, steps=6):
                     peak = max(peak, torch.cuda.max_memory_allocated() - base)
                 del y, xg
             times.sort()
-            rec = {"layer_report": True, "compress": compress, "batch": B, "seq": S,
+            rec = {"layer_report": True, "compress": compress, "attention": attention, "batch": B, "seq": S,
                    "saved_for_backward_bytes": int(held), "peak_above_weights_bytes": int(peak),
                    "step_ms": round(times[len(times) // 2], 3)}
             if compress:
@@ -276,6 +278,8 @@ def main():
                     help="for rocprofv3 --pmc: 5x a plain 32 MiB device copy, 5x fwd, 5x bwd, then exit")
     ap.add_argument("--layer-report", action="store_true",
                     help="full decoder layer (the fifth BASELINE configuration): saved bytes, peak memory, step time; then exit")
+    ap.add_argument("--layer-attention", choices=["eager", "flash", "both"], default="both",
+                    help="with --layer-report: which attention form(s) of the layer to run")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this path runs on ONE GPU (no sharding, no collectives); run with --gpus 1")
@@ -297,7 +301,7 @@ def main():
         return
     if args.layer_report:
         del wl
-        layer_report(pkg, torch)
+        layer_report(pkg, torch, attentions=("eager", "flash") if args.layer_attention == "both" else (args.layer_attention,))
         return
     if args.pmc_probe:
         dst = torch.empty_like(wl.x)

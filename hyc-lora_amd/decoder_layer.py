@@ -47,6 +47,9 @@ class LayerConfig:
     act_bits: int = 4                # norm inputs, q / k / v, gate / act(gate) / up
     act_group: int = 128
     compress: bool = True            # False: the same functions keep their activations in bf16 (formula check)
+    attention: str = "eager"         # "eager": scores, softmax, p @ v with the kept probabilities (the path the
+                                     # reference wires into its models); "flash": the library's fused attention with
+                                     # q, k, v and the output saved as codes (operators/efficient_flashattention.py)
     attn_group_bytes: int = 128 << 20  # attention is walked in groups of [S, S] score matrices of at most this size
 
 
@@ -215,15 +218,18 @@ class CompressedAttention(torch.nn.Module):
 
     def __init__(self, cfg: LayerConfig):
         super().__init__()
+        if cfg.attention not in ("eager", "flash"):
+            raise ValueError("attention must be 'eager' or 'flash', got %r" % (cfg.attention,))
         self.cfg = cfg
         mk = lambda: CompressionSite(cfg.outlier_ratio, 1.0, cfg.act_bits, "per-token", 0, "hyc", cfg.act_group)
-        self.site_q, self.site_k, self.site_v = mk(), mk(), mk()
+        self.site_q, self.site_k, self.site_v, self.site_o = mk(), mk(), mk(), mk()
         self.iteration = 0
         self.static_value = None          # probability threshold, as in EfficientMemorySoftmax
         self.record = None
 
     def forward(self, q, k, v, cos, sin):
-        return _AttentionFunc.apply(q, k, v, cos, sin, self)
+        func = _FlashAttentionFunc if self.cfg.attention == "flash" else _AttentionFunc
+        return func.apply(q, k, v, cos, sin, self)
 
 
 def _matrices_per_group(total, s, budget_bytes):
@@ -334,6 +340,61 @@ class _AttentionFunc(torch.autograd.Function):
         return dq, dk, dv, None, None, None
 
 
+class _FlashAttentionFunc(torch.autograd.Function):
+    """The design of the reference's flash-attention operator (operators/efficient_flashattention.py:10-135): the
+    fused attention kernel of the library runs the forward, what is kept is q, k (after RoPE), v and the attention
+    output as codes plus the fp32 log-sum-exp of every row, and the library's backward kernel runs on the restored
+    tensors.  No [S, S] matrix exists at any time.  The backward kernel rebuilds the probabilities from the restored
+    q and k with the exact log-sum-exp, and takes its row term sum(dO * O) from the restored output."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, cos, sin, mod):
+        cfg = mod.cfg
+        b, s, H = q.shape
+        nh, hd = cfg.heads, cfg.head_dim
+        scale = 1.0 / math.sqrt(hd)
+        qh, q_rows = K.rope_to_heads(q, nh, cos, sin, want_rows=True)
+        kh, k_rows = K.rope_to_heads(k, nh, cos, sin, want_rows=True)
+        vh = K.rope_to_heads(v, nh)
+        out_h, lse, _, _, _, _, seed, offset, _ = torch.ops.aten._scaled_dot_product_flash_attention(
+            qh, kh, vh, 0.0, True, False, scale=scale)
+        del qh, kh, vh
+        out = K.rope_from_heads(out_h)                              # [B, S, H]
+        del out_h
+        rows = [t.reshape(b * s, H) for t in (q_rows, k_rows, v, out)]
+        it = mod.iteration
+        if cfg.compress:
+            saved = []
+            for site, r in zip((mod.site_q, mod.site_k, mod.site_v, mod.site_o), rows):
+                saved.append(K.compress_channel(r, site.channel_plan(r, it), cfg.act_bits, cfg.act_group))
+        else:
+            saved = [r.contiguous() for r in rows]
+        mod.iteration += 1
+        if mod.record is not None:
+            mod.record.update(q=rows[0].detach().clone(), k=rows[1].detach().clone(), v=rows[2].detach().clone(),
+                              o=rows[3].detach().clone(), saved=saved, lse=lse)
+        ctx.saved, ctx.geom, ctx.compress, ctx.rng = saved, (b, nh, s, hd), cfg.compress, (seed, offset)
+        ctx.save_for_backward(cos, sin, lse)
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        b, nh, s, hd = ctx.geom
+        cos, sin, lse = ctx.saved_tensors
+        restore = (lambda c: K.decompress_channel(c)) if ctx.compress else (lambda c: c)
+        to_heads = lambda rows: K.rope_to_heads(rows.view(b, s, nh * hd), nh)
+        gh = K.rope_to_heads(g.to(BF16).contiguous(), nh)
+        qq, kk, vv, oo = (to_heads(restore(c)) for c in ctx.saved)
+        ctx.saved = None
+        dq, dk, dv = torch.ops.aten._scaled_dot_product_flash_attention_backward(
+            gh, qq, kk, vv, oo, lse, None, None, s, s, 0.0, True, ctx.rng[0], ctx.rng[1], scale=1.0 / math.sqrt(hd))
+        del gh, qq, kk, vv, oo
+        dq = K.rope_from_heads(dq.contiguous(), cos, sin)
+        dk = K.rope_from_heads(dk.contiguous(), cos, sin)
+        dv = K.rope_from_heads(dv.contiguous())
+        return dq, dk, dv, None, None, None
+
+
 # ---- the layer --------------------------------------------------------------------------------------------------
 class _PlainRMSNorm(torch.nn.Module):
     def __init__(self, hidden, eps, device):
@@ -388,7 +449,8 @@ class DecoderLayer(torch.nn.Module):
 
     def saved_activation_bytes(self, batch, seq):
         """analytic size of what one forward keeps for the backward (the probabilities' share is data dependent:
-        `softmax_ratio` of B*nh*S*S entries of 6 bytes plus row pointers)"""
+        `softmax_ratio` of B*nh*S*S entries of 6 bytes plus row pointers; the fused attention keeps its output and
+        one fp32 log-sum-exp per row instead)"""
         cfg = self.cfg
         M, H, I = batch * seq, cfg.hidden, cfg.intermediate
 
@@ -403,5 +465,8 @@ class DecoderLayer(torch.nn.Module):
         total += 3 * site(I, cfg.act_bits, cfg.act_group)                             # gate, act(gate), up
         total += 7 * M * cfg.lora_r * 2                                               # h = x @ A^T, exact
         rows = batch * cfg.heads * seq
-        total += int(cfg.softmax_ratio * rows * seq) * 6 + 4 * (rows + 1)
+        if cfg.attention == "flash":
+            total += site(H, cfg.act_bits, cfg.act_group) + 4 * rows                  # attention output, log-sum-exp
+        else:
+            total += int(cfg.softmax_ratio * rows * seq) * 6 + 4 * (rows + 1)
         return total

@@ -13,3 +13,5 @@ from .efficient_gemm import (EfficientMemoryGEMM, EfficientMemoryGEMMFunc, Effic
                              EfficientMemoryGEMMWithSoftmaxFunc)
 from ._calibration import calibration_state, load_calibration_state  # noqa: F401
 from .efficient_dropout import EfficientMemoryDropout, EfficientMemoryDropoutFunc  # noqa: F401
+from .efficient_flashattention import (EfficientFlashAttnVarlenQKVPacked,  # noqa: F401
+                                       EfficientFlashAttnVarlenQKVPackedFunc)

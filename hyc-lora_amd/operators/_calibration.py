@@ -89,12 +89,12 @@ def calibration_state(model):
     the result can be handed to torch.save)"""
     out = {}
     for name, mod in model.named_modules():
-        if not hasattr(mod, "iteration") or not any(k.startswith("static_value") or isinstance(v, CompressionSite)
+        if not hasattr(mod, "iteration") or not any("static_value" in k or isinstance(v, CompressionSite)
                                                     for k, v in vars(mod).items()):
             continue
         entry = {"iteration": int(mod.iteration)}
         for key, val in vars(mod).items():
-            if key.startswith("static_value"):
+            if "static_value" in key:
                 entry[key] = list(val) if isinstance(val, (list, tuple)) else val
             elif isinstance(val, CompressionSite):
                 entry[key] = _site_state(val)
@@ -122,7 +122,7 @@ def load_calibration_state(model, state, strict=True):
         for key, val in entry.items():
             if key == "iteration":
                 mod.iteration = int(val)
-            elif key.startswith("static_value"):
+            elif "static_value" in key:
                 setattr(mod, key, [place(v) for v in val] if isinstance(val, (list, tuple)) else place(val))
             else:
                 site = getattr(mod, key)

@@ -195,6 +195,9 @@ def test_module_constructors_mirror_the_reference(hyc):
     g2 = ops.EfficientMemoryGEMMWithSoftmax(outlier_ratio_1=0.05, outlier_ratio_2=0.01, sub_outlier_ratio_2=0.2,
                                             sub_outlier_bit_2=8, sub_outlier_quantize_method_2='per-tensor', rank=16)
     assert g2.static_value_1 is None and g2.static_value_2 == [None] * 4 and g2.iteration == 0
+    fa = ops.EfficientFlashAttnVarlenQKVPacked(outlier_ratio=0.01, sub_outlier_ratio=0.2, sub_outlier_bit=8,
+                                               sub_outlier_quantize_method='per-tensor', rank=16)
+    assert fa.iteration == 0 and all(getattr(fa, n + "_static_value") == [None] * 4 for n in "qkvo")
     with pytest.raises(ValueError):
         ops.EfficientMemorySiLU(mode="bogus")
     cf = ops.compress_function

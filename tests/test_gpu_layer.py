@@ -63,11 +63,12 @@ def check_grads(layer, groups, xg, P, xo, tol):
     return errs
 
 
-def test_layer_formulas_without_compression(DL, K):
+@pytest.mark.parametrize("attention", ["eager", "flash"])
+def test_layer_formulas_without_compression(DL, K, attention):
     """compress=False: the layer's own backward (LoRA composite, attention) against the oracle with exact activations,
     whose gradients are pinned against plain float64 autograd"""
     B, S = 2, 64
-    cfg = small_cfg(DL, compress=False, attn_group_bytes=5 * 2 * 64 * 64)
+    cfg = small_cfg(DL, compress=False, attn_group_bytes=5 * 2 * 64 * 64, attention=attention)
     layer = DL.DecoderLayer(cfg)
     gen = torch.Generator().manual_seed(3)
     x = make_input(gen, B, S, cfg.hidden)
@@ -78,7 +79,8 @@ def test_layer_formulas_without_compression(DL, K):
     P, groups = oracle_params(K, layer)
     cos, sin = (t.float().cpu() for t in DL.rope_tables(S, cfg.head_dim, cfg.rope_theta, "cuda"))
     xo = x.float().requires_grad_(True)
-    yo = LO.decoder_layer(xo, P, {}, cfg.heads, cfg.rms_eps, cfg.lora_alpha / cfg.lora_r, cos, sin, quirk=False)
+    yo = LO.decoder_layer(xo, P, {}, cfg.heads, cfg.rms_eps, cfg.lora_alpha / cfg.lora_r, cos, sin, quirk=False,
+                          attention=attention)
     yo.backward(g.float())
     assert rel_err(y.detach().cpu(), yo.detach()) < 1e-2
     check_grads(layer, groups, xg, P, xo, 2e-2)
@@ -91,12 +93,14 @@ def K(hyc):
     return hyc.kernels
 
 
-def test_layer_with_compression(DL, K):
+@pytest.mark.parametrize("attention", ["eager", "flash"])
+def test_layer_with_compression(DL, K, attention):
     """three steps (two calibrating, one steady); on each: every site restores what the oracle restores, the kept
-    probabilities are the oracle's set, and the gradients equal the oracle layer's at those restored activations
-    (relative error of each gradient tensor below 1e-2)"""
+    probabilities are the oracle's set (eager attention; the fused attention keeps its output instead), and the
+    gradients equal the oracle layer's at those restored activations (relative error of each gradient tensor below
+    1e-2)"""
     B, S = 2, 64
-    cfg = small_cfg(DL, attn_group_bytes=3 * 2 * 64 * 64)       # 8 score matrices walked as groups of 3, 3, 2
+    cfg = small_cfg(DL, attn_group_bytes=3 * 2 * 64 * 64, attention=attention)   # 8 score matrices in groups of 3, 3, 2
     layer = DL.DecoderLayer(cfg)
     H, I, nh = cfg.hidden, cfg.intermediate, cfg.heads
     gen = torch.Generator().manual_seed(4)
@@ -143,17 +147,22 @@ def test_layer_with_compression(DL, K):
         R["gate"] = restore_and_check(gate.reshape(-1, I), c_gate, ab, ag).reshape(B, S, I)
         R["up"] = restore_and_check(up.reshape(-1, I), c_up, ab, ag).reshape(B, S, I)
         R["act"] = restore_and_check(torch.nn.functional.silu(gate).reshape(-1, I), c_act, ab, ag).reshape(B, S, I)
-        p_dev = rec["attn"]["p"].cpu()
-        thr = O.get_statistics_softmax(p_dev, step, cfg.softmax_ratio) if step < 2 else layer.attention.static_value.cpu()
-        R["p"] = torch.cat([K.softmax_dense(sp) for sp in rec["attn"]["sparse"]]).cpu().reshape(p_dev.shape)
-        assert bits_equal(R["p"], O.prune_softmax(p_dev, thr))
-        kept = float((R["p"] > 0).float().mean())
-        assert 0.02 < kept < 0.08, kept
+        p_dev = None
+        if attention == "flash":
+            R["o"] = restore_and_check(rec["attn"]["o"].contiguous(), rec["attn"]["saved"][3], ab, ag).reshape(B, S, H)
+        else:
+            p_dev = rec["attn"]["p"].cpu()
+            thr = O.get_statistics_softmax(p_dev, step, cfg.softmax_ratio) if step < 2 else layer.attention.static_value.cpu()
+            R["p"] = torch.cat([K.softmax_dense(sp) for sp in rec["attn"]["sparse"]]).cpu().reshape(p_dev.shape)
+            assert bits_equal(R["p"], O.prune_softmax(p_dev, thr))
+            kept = float((R["p"] > 0).float().mean())
+            assert 0.02 < kept < 0.08, kept
 
         for t in P.values():
             t.grad = None
         xo = x.float().requires_grad_(True)
-        yo = LO.decoder_layer(xo, P, R, nh, cfg.rms_eps, cfg.lora_alpha / cfg.lora_r, cos, sin, quirk=True, probs=p_dev)
+        yo = LO.decoder_layer(xo, P, R, nh, cfg.rms_eps, cfg.lora_alpha / cfg.lora_r, cos, sin, quirk=True, probs=p_dev,
+                              attention=attention)
         yo.backward(g.float())
         assert rel_err(y.detach().cpu(), yo.detach()) < 1e-2
         check_grads(layer, groups, xg, P, xo, 1e-2)
@@ -162,11 +171,12 @@ def test_layer_with_compression(DL, K):
     assert layer.attention.iteration == 3 and layer.qkv_proj.iteration == 3
 
 
-def test_saved_bytes_accounting(DL, K):
+@pytest.mark.parametrize("attention", ["eager", "flash"])
+def test_saved_bytes_accounting(DL, K, attention):
     """what the forward keeps (allocator delta) matches the analytic count to within the allocator's rounding, and is
     several times smaller than the bf16 activations of the uncompressed layer"""
     B, S = 2, 128
-    cfg = small_cfg(DL)
+    cfg = small_cfg(DL, attention=attention)
     layer = DL.DecoderLayer(cfg)
     x = make_input(torch.Generator().manual_seed(5), B, S, cfg.hidden).cuda()
     for _ in range(3):

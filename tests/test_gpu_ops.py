@@ -700,3 +700,69 @@ def test_linear_with_frozen_weight_saves_nothing(ops, mode):
     assert torch.allclose(x.grad.float(), want, rtol=1e-2, atol=1e-2)
     with torch.no_grad():
         assert lin(x).shape == (2, 32, 64)
+
+
+# ------------------------------------------------------------------ fused attention over packed sequences
+def _attention_oracle(qkv, bounds, restored, causal, dout):
+    """per sequence: exact forward, flash backward at the restored q, k, v, out (oracle/layer_oracle.py)"""
+    from oracle import layer_oracle as LO
+    total, _, nh, hd = qkv.shape
+    x = qkv.float().requires_grad_(True)
+    outs = []
+    for a, b in zip(bounds, bounds[1:]):
+        heads = lambda t: t[a:b].transpose(0, 1).unsqueeze(0)               # [1, nh, S, hd]
+        hats = [heads(r.float().view(total, nh, hd)) for r in restored]
+        o = LO._FlashAttentionAt.apply(heads(x[:, 0]), heads(x[:, 1]), heads(x[:, 2]), *hats, hd ** -0.5, causal)
+        outs.append(o.squeeze(0).transpose(0, 1))
+    out = torch.cat(outs)
+    out.backward(dout.float())
+    return out.detach(), x.grad
+
+
+@pytest.mark.parametrize("mode", ["hyc", "ref"])
+@pytest.mark.parametrize("lens,causal", [([64, 64], True), ([40, 64, 24], True), ([48, 80], False)])
+def test_flash_attention_module(ops, K, mode, lens, causal):
+    """out is the attention output; the saved q, k, v, out restore what the oracle's codec restores; dqkv equals the
+    flash backward evaluated at those restored tensors; calibration runs for five calls in the reference scheme"""
+    nh, hd = 4, 64
+    H = nh * hd
+    total = sum(lens)
+    bounds = [0]
+    for n in lens:
+        bounds.append(bounds[-1] + n)
+    gen = torch.Generator().manual_seed(31 + total)
+    mod = ops.EfficientFlashAttnVarlenQKVPacked(outlier_ratio=0.02, sub_outlier_ratio=1.0, sub_outlier_bit=4,
+                                                sub_outlier_quantize_method="per-channel", rank=0, mode=mode)
+    cu = torch.tensor(bounds, dtype=torch.int32, device="cuda")
+    calls = 6 if mode == "ref" else 3
+    for call in range(calls):
+        qkv = torch.randn(total, 3, nh, hd, generator=gen)
+        qkv[:, :, 1, 5] *= 12
+        qkv = qkv.bfloat16()
+        dout = (0.1 * torch.randn(total, nh, hd, generator=gen)).bfloat16()
+        xg = qkv.cuda().requires_grad_(True)
+        out = mod(xg, cu, max(lens), causal=causal)
+        saved = out.grad_fn.saved
+        if mode == "hyc":
+            restored = [K.decompress_channel(c).cpu() for c in saved]
+            rows = [qkv[:, i].reshape(total, H) for i in range(3)] + [out.detach().cpu().view(total, H)]
+            for r, c, xh in zip(rows, saved, restored):                     # the codec link, bit for bit
+                idx = c.plan.idx.cpu().long()
+                vals, stored, scales = O.hyc_compress(r, idx, 4, 128)
+                assert bits_equal(xh, O.hyc_decompress(vals, stored, idx, scales, 4, 128))
+        else:
+            restored = [K.decompress_threshold(c).cpu() for c in saved]
+        out.backward(dout.cuda())
+        out_o, dqkv_o = _attention_oracle(qkv, bounds, restored, causal, dout)
+        assert torch.allclose(out.detach().cpu().float(), out_o, rtol=2e-2, atol=2e-2)
+        err = float((xg.grad.cpu().float() - dqkv_o).norm() / dqkv_o.norm())
+        assert err < 1e-2, (call, err)
+    assert mod.iteration == calls
+    if mode == "ref":
+        assert all(v is not None for v in mod.q_static_value + mod.o_static_value)
+        state = ops.calibration_state(torch.nn.ModuleDict({"attn": mod}))
+        assert state["attn"]["iteration"] == calls and "k_static_value" in state["attn"]
+    with pytest.raises(NotImplementedError):
+        mod(xg, cu, max(lens), window_size=(128, 0))
+    with pytest.raises(ValueError):
+        mod(xg, torch.tensor([0, total + 1], dtype=torch.int32, device="cuda"), total)

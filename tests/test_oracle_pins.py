@@ -409,6 +409,78 @@ def test_layer_oracle_against_plain_autograd():
     assert torch.allclose(Po2["A_o"].grad, Po["A_o"].grad, rtol=1e-4, atol=1e-6)
 
 
+def test_flash_attention_backward_oracle():
+    """the fused-attention backward of the layer oracle: the true derivative when nothing was lossy (float64 autograd
+    of scaled_dot_product_attention), and the three properties of the flash backward pass that a restatement could get
+    wrong: the row term comes from the restored OUTPUT (dV does not read it), dV does not read v_hat, and the
+    probabilities are rebuilt against the forward's exact log-sum-exp without renormalising."""
+    from oracle import layer_oracle as LO
+    F = torch.nn.functional
+    gen = torch.Generator().manual_seed(23)
+    B, nh, S, hd = 2, 3, 9, 8
+    q, k, v, g = (torch.randn(B, nh, S, hd, generator=gen, dtype=torch.float64) for _ in range(4))
+    scale = hd ** -0.5
+    qa, ka, va = (t.clone().requires_grad_(True) for t in (q, k, v))
+    o = F.scaled_dot_product_attention(qa, ka, va, is_causal=True)
+    o.backward(g)
+
+    def run(q_hat, k_hat, v_hat, o_hat):
+        qb, kb, vb = (t.clone().requires_grad_(True) for t in (q, k, v))
+        out = LO._FlashAttentionAt.apply(qb, kb, vb, q_hat, k_hat, v_hat, o_hat, scale)
+        out.backward(g)
+        return out.detach(), qb.grad, kb.grad, vb.grad
+
+    out, dq, dk, dv = run(q, k, v, o.detach())
+    for got, want in ((out, o.detach()), (dq, qa.grad), (dk, ka.grad), (dv, va.grad)):
+        assert torch.allclose(got, want, rtol=1e-10, atol=1e-12)
+    # a wrong restored output moves dq and dk through the row term, and nothing else
+    _, dq2, dk2, dv2 = run(q, k, v, 1.5 * o.detach())
+    assert torch.equal(dv2, dv) and not torch.allclose(dq2, dq) and not torch.allclose(dk2, dk)
+    d = (g * o.detach()).sum(-1, keepdim=True)
+    p = torch.softmax((q @ k.transpose(-2, -1) * scale).masked_fill(torch.ones(S, S, dtype=torch.bool).triu(1), -1e300), -1)
+    assert torch.allclose(dq2 - dq, -0.5 * scale * ((p * d) @ k), rtol=1e-9, atol=1e-12)
+    # dV = P_hat^T dO does not read v_hat
+    _, _, _, dv3 = run(q, k, 3.0 * v, o.detach())
+    assert torch.equal(dv3, dv)
+    # q_hat = 0: every rebuilt probability of row i is exp(-lse_i), with lse the forward's; no renormalisation
+    _, _, _, dv4 = run(torch.zeros_like(q), k, v, o.detach())
+    sc = (q @ k.transpose(-2, -1) * scale).masked_fill(torch.ones(S, S, dtype=torch.bool).triu(1), float("-inf"))
+    w = torch.exp(-torch.logsumexp(sc, -1, keepdim=True))                  # [B,nh,S,1]
+    want = torch.flip(torch.cumsum(torch.flip(w * g, [-2]), -2), [-2])     # row j gets the rows i >= j
+    assert torch.allclose(dv4, want, rtol=1e-10, atol=1e-12)
+
+
+def test_layer_oracle_with_fused_attention_against_plain_autograd():
+    """attention="flash" with exact restored activations gives the true gradients of the layer"""
+    from oracle import layer_oracle as LO
+    gen = torch.Generator().manual_seed(19)
+    B, S, H, nh, I, r, s, eps = 2, 10, 32, 4, 48, 4, 2.0, 1e-5
+    hd = H // nh
+    P = _tiny_layer_params(gen, H, I, r)
+    x = torch.randn(B, S, H, generator=gen).bfloat16().float()
+    g = 0.1 * torch.randn(B, S, H, generator=gen)
+    inv = 1.0 / (10000.0 ** (torch.arange(0, hd, 2).float() / hd))
+    emb = torch.cat([torch.outer(torch.arange(S).float(), inv)] * 2, -1)
+    cos, sin = emb.cos(), emb.sin()
+    grads = {}
+    for attention in ("eager", "flash"):
+        xo = x.clone().requires_grad_(True)
+        Po = {k: v.clone().requires_grad_(not k.startswith("W_")) for k, v in P.items()}
+        cap = {}
+        y = LO.decoder_layer(xo, Po, {}, nh, eps, s, cos, sin, quirk=False, capture=cap, attention=attention)
+        y.backward(g)
+        grads[attention] = [y.detach(), xo.grad] + [Po[n].grad for n in sorted(Po) if not n.startswith("W_")]
+        assert ("o" in cap) == (attention == "flash") and ("p" in cap) == (attention == "eager")
+    for a, b in zip(grads["eager"], grads["flash"]):        # the eager form is pinned against float64 autograd above
+        assert float((a - b).abs().max()) <= 1e-4 * float(b.abs().max()) + 1e-7
+    # the restored output is what the backward reads
+    xo = x.clone().requires_grad_(True)
+    Po = {k: v.clone().requires_grad_(not k.startswith("W_")) for k, v in P.items()}
+    LO.decoder_layer(xo, Po, {"o": 2 * cap["o"]}, nh, eps, s, cos, sin, quirk=False, attention="flash").backward(g)
+    assert not torch.allclose(Po["A_q"].grad, grads["flash"][2 + sorted(n for n in Po if not n.startswith("W_")).index("A_q")])
+    assert torch.allclose(Po["A_o"].grad, grads["flash"][2 + sorted(n for n in Po if not n.startswith("W_")).index("A_o")])
+
+
 def test_rope_against_complex_rotation_and_autograd():
     """rope_fwd is the rotation of the pairs (x[i], x[i+h]) by the angle of (cos[i], sin[i]): checked as a complex
     multiplication with independently built angles; rope_bwd against float64 autograd.  Distinct tables for the two
