@@ -263,3 +263,50 @@ def test_golden_cases_on_gpu(K, golden_compress):
         assert bits_equal(got, want), i
         checked += 1
     assert checked >= 40
+
+
+# ------------------------------------------------------------------ the configurations at their full size
+FULL_SIZE = [  # (name, M, H, bits, group, hot channels, gain)
+    ("config 1: [4,512,4096], 41 channels x50, INT4 G128", 2048, 4096, 4, 128, 41, 50.0),
+    ("config 3: [4,1024,4096], INT2 G64", 4096, 4096, 2, 64, 41, 30.0),
+    ("config 4: [4,1024,11008], 110 channels x20, INT4 G128", 4096, 11008, 4, 128, 110, 20.0),
+]
+
+
+@pytest.mark.parametrize("name,M,H,bits,group,n_hot,gain", FULL_SIZE)
+def test_full_size_configurations(K, name, M, H, bits, group, n_hot, gain):
+    """At the configurations' own sizes: the channel choice equals the oracle's; rows are independent, so the packed
+    bytes, scales, outlier values and the reconstruction of a seeded sample of 96 rows must equal, bit for bit, the
+    oracle run on those rows alone; and over ALL rows the properties the scheme guarantees hold: outlier channels
+    come back exactly, every other element is within half a quantisation step (one bf16 ulp of slack) of the
+    original unless its code sits on the clamp, and the scale of each group is bf16(bf16(max - min) / levels)."""
+    x, hot = make_x(len(name), M, H, n_hot, gain)
+    k = K.num_outlier_channels(H, 0.01)
+    xd = x.cuda()
+    plan = K.select_channels(K.channel_absmax(xd), k)
+    idx = O.hyc_select_channels(O.hyc_channel_scores(x), k)
+    assert torch.equal(plan.idx.cpu(), idx)
+    assert set(hot.tolist()) <= set(idx.tolist()) or n_hot > k
+    c = K.compress_channel(xd, plan, bits, group)
+    xh = K.decompress_channel(c)
+    rows = torch.randperm(M, generator=torch.Generator().manual_seed(M + H))[:96].sort().values
+    vals, stored, scales = O.hyc_compress(x[rows], idx, bits, group)
+    assert torch.equal(c.stored.cpu()[rows].view(torch.uint8), stored.view(torch.uint8))
+    assert bits_equal(c.scales.cpu()[rows], scales) and bits_equal(c.vals.cpu()[rows], vals)
+    assert bits_equal(xh.cpu()[rows], O.hyc_decompress(vals, stored, idx, scales, bits, group))
+    # whole-tensor properties, evaluated on the device in fp32
+    xf, hf = xd.float(), xh.float()
+    keep = torch.ones(H, dtype=torch.bool, device="cuda")
+    keep[plan.idx.long()] = False
+    assert torch.equal(xd[:, ~keep], xh[:, ~keep])
+    inl = torch.where(keep, xf, torch.zeros((), device="cuda")).view(M, H // group, group)
+    span = (inl.amax(-1) - inl.amin(-1)).bfloat16().float()
+    levels = float(2 ** bits - 1)
+    assert bits_equal((span / levels).bfloat16().cpu(), c.scales.cpu())
+    s = c.scales.float().repeat_interleave(group, dim=1)
+    err = (hf - xf).abs()
+    off = float(2 ** (bits - 1))
+    clamped = (xf / s.clamp_min(1e-30)).abs() >= off - 0.5              # the code sits on (or next to) a clamp bound
+    slack = hf.abs() * 2.0 ** -7 + 1e-30                                # one bf16 rounding of the product
+    bad = keep[None, :] & ~clamped & (err > 0.5 * s + slack)
+    assert int(bad.sum()) == 0

@@ -81,6 +81,33 @@ def test_gradw_config3_lora_a(K):
     assert torch.allclose(got.float(), dW_lit.float(), rtol=2e-2, atol=2e-2 * float(dW_f32.abs().max()))
 
 
+@pytest.mark.parametrize("name,M,N,H,bits,group,k,gain", [
+    ("config 3 full W: dY [4096, 4096], x INT2 G64", 4096, 4096, 4096, 2, 64, 41, 30.0),
+    ("config 4 down_proj: dY [4096, 4096], x [4096, 11008] INT4 G128", 4096, 4096, 11008, 4, 128, 110, 20.0)])
+def test_gradw_full_size(K, name, M, N, H, bits, group, k, gain):
+    """The wide weight gradients at the configurations' own sizes (137 and 369 GFLOP), checked on the device: against
+    an fp32 library product with the restored activation (whose bits the codec tests tie to the oracle), both routes;
+    and through linearity in dY, which the fused decode must not break."""
+    x, gen = make_x(len(name), M, H, k, gain)
+    dy1 = (0.01 * torch.randn(M, N, generator=gen)).bfloat16().cuda()
+    dy2 = (0.01 * torch.randn(M, N, generator=gen)).bfloat16().cuda()
+    xd = x.cuda()
+    c = K.compress_channel(xd, K.select_channels(K.channel_absmax(xd), k), bits, group)
+    xh = K.decompress_channel(c).float()
+    want = dy1.float().t() @ xh
+    scale = float(want.abs().max())
+    for staged in (False, True):
+        got = K.gradw_gemm(dy1, c, out_dtype=torch.float32, staged=staged)
+        assert torch.allclose(got, want, rtol=1e-2, atol=1e-3 * scale), (staged, float((got - want).abs().max()), scale)
+    a = K.gradw_gemm(dy1, c, out_dtype=torch.float32, staged=False)
+    b = K.gradw_gemm(dy2, c, out_dtype=torch.float32, staged=False)
+    both = K.gradw_gemm((dy1.float() + dy2.float()).bfloat16(), c, out_dtype=torch.float32, staged=False)
+    # dy1 + dy2 is rounded to bf16 once more: 2^-9 relative per element, averaged down over 4096 tokens
+    assert float((both - (a + b)).abs().max()) < 2e-3 * float((a + b).abs().max())
+    half = K.gradw_gemm(dy1, c, out_dtype=torch.float32, alpha=0.5, staged=False)
+    assert torch.allclose(half, 0.5 * a, rtol=1e-6, atol=1e-6 * scale)
+
+
 # ------------------------------------------------------------------ softmax
 @pytest.mark.parametrize("shape", [(2, 4, 64, 64), (1, 2, 40, 2048), (3, 1, 7, 8), (1, 1, 5, 4096), (1, 2, 9, 1024), (1, 1, 3, 8192),
                                    (1, 4, 2100, 512), (1, 1, 11, 1096)])
