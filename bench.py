@@ -137,7 +137,7 @@ def gradw_extra(pkg, torch, wl):
 
 def kernel_tour(pkg, torch, reps=5):
     """every kernel of the path at the BASELINE config shapes (INT4 / group 128 and INT2 / group 64, 1 % outlier
-    channels): compress, decompress, activation / Hadamard / gated backward at H = 11008, weight gradient"""
+    channels): compress, decompress, activation / Hadamard / gated backward and forward, weight gradient"""
     K = pkg.kernels
     gen = torch.Generator(device="cuda").manual_seed(0)
 
@@ -162,6 +162,7 @@ def kernel_tour(pkg, torch, reps=5):
             K.act_bwd("gelu", g, cs[0])
             K.hadamard_bwd(g, cs[2], cs[1])
             K.gated_act_bwd("silu", g, cs[2], cs[1], cs[0])
+            K.gated_act_fwd("silu", x, up, cs[2].plan, cs[1].plan, cs[0].plan, bits, G)
             K.gradw_gemm(dy16, cs[0])
             K.gradw_gemm(dyN, cs[0], staged=False)        # x_hat decoded inside the GEMM
             K.gradw_gemm(dyN, cs[0], staged=True)         # x_hat restored once, then the dense form of the kernel

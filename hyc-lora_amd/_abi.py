@@ -58,6 +58,8 @@ SIGNATURES = {
                                  ctypes.POINTER(HycDesc), c_i64, c_i64, c_ptr, c_ptr, c_ptr]),
     "hyc_gated_act_bwd": (c_i32, [c_i32, c_ptr, c_ptr, c_ptr, c_ptr, ctypes.POINTER(HycDesc), c_ptr, c_ptr, c_ptr, ctypes.POINTER(HycDesc),
                                   c_ptr, c_ptr, c_ptr, ctypes.POINTER(HycDesc), c_i64, c_i64, c_ptr, c_ptr, c_ptr]),
+    "hyc_gated_act_fwd": (c_i32, [c_i32, c_ptr, c_i64, c_ptr, c_i64, c_i64, c_i64, ctypes.POINTER(HycDesc), ctypes.POINTER(HycDesc),
+                                  ctypes.POINTER(HycDesc), c_ptr] + [c_ptr] * 9 + [c_ptr]),
     "hyc_softmax_fwd": (c_i32, [c_ptr, c_i64, c_i64, c_f32, c_ptr, c_ptr, c_ptr]),
     "hyc_softmax_causal_fwd": (c_i32, [c_ptr, c_i64, c_i64, c_i64, c_f32, c_ptr, c_ptr, c_ptr]),
     "hyc_softmax_fill": (c_i32, [c_ptr, c_i64, c_i64, c_f32, c_ptr, c_ptr, c_ptr, c_ptr]),

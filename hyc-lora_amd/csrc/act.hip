@@ -361,6 +361,122 @@ k_gated_act_bwd_fast(const uint16_t* __restrict__ g, const uint8_t* __restrict__
   }
 }
 
+// ---- forward of h = act(gate) * up with the three saves fused in ----------------------------------------------
+// The activation value as the framework computes it for a bf16 tensor: fp32 arithmetic with the accurate library
+// exp / erf, one rounding to bf16 (operators/efficient_silu.py:16 F.silu, operators/efficient_gelu.py:16 F.gelu).
+template <int ACT>
+__device__ __forceinline__ float act_value(float x) {
+  if (ACT == HYC_ACT_SILU) return x / (1.0f + expf(-x));
+  return (x * 0.5f) * (1.0f + erff(x * 0.70710678118654752440f));
+}
+
+struct GatedFwdSite {       // one compressed output
+  ChanArgs ca;
+  uint8_t* stored;
+  uint16_t* vals;
+  uint16_t* scales;
+};
+
+// One pass: reads gate and up (row pitches ldg, ldu: they may be column slices of one projection output), writes
+// h = bf16(bf16(act(gate)) * up) and the channel-compressed forms of act(gate), up and gate - what F.silu,
+// three hyc_compress calls and a multiply write and re-read through memory.  act(gate) itself is never stored.
+template <int BITS, int LPGT, int ACT, int MAXT>
+__global__ void __launch_bounds__(MAXT)
+k_gated_act_fwd_fast(const uint16_t* __restrict__ gate, int64_t ldg, const uint16_t* __restrict__ up, int64_t ldu, int64_t M,
+                     int64_t H, int CPS, GatedFwdSite sa, GatedFwdSite su, GatedFwdSite sg, uint16_t* __restrict__ h) {
+  constexpr int NSEG = Q<BITS>::NSEG;
+  const int c = threadIdx.x;
+  if (c >= CPS) return;                                 // tail of the last wave; scale groups never straddle it
+  const int64_t SEG = (int64_t)CPS * 8;
+  const bool leader = (c & (LPGT - 1)) == 0;
+  const int shift = sa.ca.chunk_to_group_shift;         // the three sites share the group width
+  const int seg_groups = CPS >> shift;
+  const int gpr = sa.ca.groups_per_row;
+  uint32_t km_a[NSEG][4], km_u[NSEG][4], km_g[NSEG][4];
+  {
+    uint32_t plan[NSEG];
+    ChunkOutliers<NSEG> co;
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) plan[i] = sa.ca.plan[i * CPS + c];
+    co.init(plan);
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) co.keep_masks(i, km_a[i]);
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) plan[i] = su.ca.plan[i * CPS + c];
+    co.init(plan);
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) co.keep_masks(i, km_u[i]);
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) plan[i] = sg.ca.plan[i * CPS + c];
+    co.init(plan);
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) co.keep_masks(i, km_g[i]);
+  }
+  const int64_t stride = gridDim.x;
+  int64_t row = blockIdx.x;
+  const uint16_t* grow = gate + row * ldg;
+  const uint16_t* urow = up + row * ldu;
+  uint16_t* hp = h + row * H + 8 * c;
+  const int64_t gstep = stride * ldg, ustep = stride * ldu, hstep = stride * H, sstep = stride * SEG, scstep = stride * gpr;
+  int64_t soff = row * SEG + 8 * c, scoff = row * gpr + (c >> shift);
+  uint4 graw[NSEG], uraw[NSEG];
+  if (row < M) {
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) {
+      graw[i] = *reinterpret_cast<const uint4*>(grow + i * SEG + 8 * c);
+      uraw[i] = *reinterpret_cast<const uint4*>(urow + i * SEG + 8 * c);
+    }
+  }
+  for (; row < M; row += stride) {
+    uint4 g_n[NSEG], u_n[NSEG];
+    if (row + stride < M) {
+#pragma unroll
+      for (int i = 0; i < NSEG; ++i) {
+        g_n[i] = *reinterpret_cast<const uint4*>(grow + gstep + i * SEG + 8 * c);
+        u_n[i] = *reinterpret_cast<const uint4*>(urow + ustep + i * SEG + 8 * c);
+      }
+    }
+    uint32_t lo_a = 0, hi_a = 0, lo_u = 0, hi_u = 0, lo_g = 0, hi_g = 0;
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) {
+      float gv[8], uv[8], av[8], v[8];
+      unpack8(graw[i], gv);
+      unpack8(uraw[i], uv);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) av[j] = act_value<ACT>(gv[j]);
+      const uint4 araw = pack8(av);                     // act(gate) as the bf16 tensor the framework would hold
+      unpack8(araw, av);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = av[j] * uv[j];
+      store_stream(hp + i * SEG, pack8(v));
+      uint32_t cl, ch;
+      unpack8(make_uint4(araw.x & km_a[i][0], araw.y & km_a[i][1], araw.z & km_a[i][2], araw.w & km_a[i][3]), v);
+      float s = quant_seg<BITS, LPGT>(v, LPGT, cl, ch);
+      if (leader) sa.scales[scoff + i * seg_groups] = f_to_bf(s);
+      if (BITS == 8) { lo_a = cl; hi_a = ch; } else { lo_a |= cl << (i * BITS); hi_a |= ch << (i * BITS); }
+      unpack8(make_uint4(uraw[i].x & km_u[i][0], uraw[i].y & km_u[i][1], uraw[i].z & km_u[i][2], uraw[i].w & km_u[i][3]), v);
+      s = quant_seg<BITS, LPGT>(v, LPGT, cl, ch);
+      if (leader) su.scales[scoff + i * seg_groups] = f_to_bf(s);
+      if (BITS == 8) { lo_u = cl; hi_u = ch; } else { lo_u |= cl << (i * BITS); hi_u |= ch << (i * BITS); }
+      unpack8(make_uint4(graw[i].x & km_g[i][0], graw[i].y & km_g[i][1], graw[i].z & km_g[i][2], graw[i].w & km_g[i][3]), v);
+      s = quant_seg<BITS, LPGT>(v, LPGT, cl, ch);
+      if (leader) sg.scales[scoff + i * seg_groups] = f_to_bf(s);
+      if (BITS == 8) { lo_g = cl; hi_g = ch; } else { lo_g |= cl << (i * BITS); hi_g |= ch << (i * BITS); }
+    }
+    *reinterpret_cast<uint2*>(sa.stored + soff) = make_uint2(lo_a, hi_a);
+    *reinterpret_cast<uint2*>(su.stored + soff) = make_uint2(lo_u, hi_u);
+    *reinterpret_cast<uint2*>(sg.stored + soff) = make_uint2(lo_g, hi_g);
+    // outlier channels, kept verbatim: thread t copies channel idx[t] (+ CPS, ...) of each site
+    for (int t = c; t < sa.ca.k; t += CPS)
+      sa.vals[row * sa.ca.k + t] = f_to_bf(act_value<ACT>(bf_to_f(grow[sa.ca.idx[t]])));
+    for (int t = c; t < su.ca.k; t += CPS) su.vals[row * su.ca.k + t] = urow[su.ca.idx[t]];
+    for (int t = c; t < sg.ca.k; t += CPS) sg.vals[row * sg.ca.k + t] = grow[sg.ca.idx[t]];
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) { graw[i] = g_n[i]; uraw[i] = u_n[i]; }
+    grow += gstep; urow += ustep; hp += hstep; soff += sstep; scoff += scstep;
+  }
+}
+
 // SRC 0 = channel-compressed, 2 = dense bf16
 template <int BITS, int SRC, int ACT>
 __global__ void __launch_bounds__(1024)
@@ -564,6 +680,66 @@ int hyc_gated_act_bwd(int32_t act, const void* g, const void* stored_a, const vo
 #undef HYC_GATED_T
 #undef HYC_GATED
   return check_launch("hyc_gated_act_bwd");
+}
+
+int hyc_gated_act_fwd(int32_t act, const void* gate, int64_t ld_gate, const void* up, int64_t ld_up, int64_t M, int64_t H,
+                      const hyc_desc* d_a, const hyc_desc* d_u, const hyc_desc* d_g, void* h, void* stored_a, void* vals_a,
+                      void* scales_a, void* stored_u, void* vals_u, void* scales_u, void* stored_g, void* vals_g,
+                      void* scales_g, void* stream) {
+  if (act != HYC_ACT_SILU && act != HYC_ACT_GELU_TANH) return fail(HYC_EINVAL, "hyc_gated_act_fwd: act=%d", act);
+  if (!d_a || !d_u || !d_g) return fail(HYC_EFAULT, "hyc_gated_act_fwd: null descriptor");
+  if (M < 0) return fail(HYC_EINVAL, "hyc_gated_act_fwd: M=%lld", (long long)M);
+  if (d_a->mode != HYC_MODE_CHANNEL || d_u->mode != HYC_MODE_CHANNEL || d_g->mode != HYC_MODE_CHANNEL)
+    return fail(HYC_ENOTSUP, "hyc_gated_act_fwd: channel scheme only");
+  if (d_a->bits != d_u->bits || d_a->bits != d_g->bits || d_a->group != d_u->group || d_a->group != d_g->group)
+    return fail(HYC_ENOTSUP, "hyc_gated_act_fwd: one code width and one group size for the three activations");
+  if (ld_gate < H || ld_up < H || ld_gate % 8 != 0 || ld_up % 8 != 0)
+    return fail(HYC_EINVAL, "hyc_gated_act_fwd: row pitches %lld, %lld (at least H=%lld, multiples of 8)",
+                (long long)ld_gate, (long long)ld_up, (long long)H);
+  RowGeom geo;
+  int rc = row_geom(H, d_a->bits, &geo);
+  if (rc) return rc;
+  ChanArgs c_a = {}, c_u = {}, c_g = {};
+  int lpg = 16;
+  if ((rc = make_chan_args(d_a, geo, &c_a, &lpg)) || (rc = make_chan_args(d_u, geo, &c_u, &lpg)) ||
+      (rc = make_chan_args(d_g, geo, &c_g, &lpg)))
+    return rc;
+  if (geo.iters != 1 || d_a->bits == 1 || (lpg != 8 && lpg != 16))
+    return fail(HYC_ENOTSUP, "hyc_gated_act_fwd: needs 2-, 4- or 8-bit codes, groups of 64 or 128 channels and rows of at "
+                             "most 1024 chunks per segment (use the activation, hyc_compress and a product otherwise)");
+  if (M == 0) return HYC_OK;
+  if (!gate || !up || !h || !stored_a || !stored_u || !stored_g || !scales_a || !scales_u || !scales_g ||
+      (d_a->k > 0 && !vals_a) || (d_u->k > 0 && !vals_u) || (d_g->k > 0 && !vals_g))
+    return fail(HYC_EFAULT, "hyc_gated_act_fwd: null buffer");
+  if (!aligned16(gate) || !aligned16(up) || !aligned16(h) || !aligned8(stored_a) || !aligned8(stored_u) || !aligned8(stored_g))
+    return fail(HYC_EINVAL, "hyc_gated_act_fwd: gate, up, h must be 16-byte aligned, stored 8-byte");
+  const GatedFwdSite sa = {c_a, static_cast<uint8_t*>(stored_a), static_cast<uint16_t*>(vals_a), static_cast<uint16_t*>(scales_a)};
+  const GatedFwdSite su = {c_u, static_cast<uint8_t*>(stored_u), static_cast<uint16_t*>(vals_u), static_cast<uint16_t*>(scales_u)};
+  const GatedFwdSite sg = {c_g, static_cast<uint8_t*>(stored_g), static_cast<uint16_t*>(vals_g), static_cast<uint16_t*>(scales_g)};
+  const int64_t cap = 256 * (geo.threads >= 512 ? 3 : 8);
+  const int grid = (int)(M < cap ? M : cap);
+  hipStream_t st = begin_launch(stream);
+#define HYC_GFWD(B_, L_, A_, MT_)                                                                                  \
+  hipLaunchKernelGGL((k_gated_act_fwd_fast<B_, L_, A_, MT_>), dim3(grid), dim3(geo.threads), 0, st,                \
+                     static_cast<const uint16_t*>(gate), ld_gate, static_cast<const uint16_t*>(up), ld_up, M, H,   \
+                     geo.cps, sa, su, sg, static_cast<uint16_t*>(h))
+#define HYC_GFWD_T(B_, L_, A_)                                                    \
+  do {                                                                            \
+    if (geo.threads <= 256) HYC_GFWD(B_, L_, A_, 256);                            \
+    else if (geo.threads <= 768) HYC_GFWD(B_, L_, A_, 768); /* H = 11008: 704 threads; 1024 would cap the registers at 128 */ \
+    else HYC_GFWD(B_, L_, A_, 1024);                                              \
+  } while (0)
+#define HYC_GFWD_L(B_, A_) do { if (lpg == 8) HYC_GFWD_T(B_, 8, A_); else HYC_GFWD_T(B_, 16, A_); } while (0)
+#define HYC_GFWD_B(A_)                                                                                             \
+  do {                                                                                                             \
+    if (d_a->bits == 2) HYC_GFWD_L(2, A_); else if (d_a->bits == 4) HYC_GFWD_L(4, A_); else HYC_GFWD_L(8, A_);     \
+  } while (0)
+  if (act == HYC_ACT_SILU) HYC_GFWD_B(HYC_ACT_SILU); else HYC_GFWD_B(HYC_ACT_GELU_TANH);
+#undef HYC_GFWD_B
+#undef HYC_GFWD_L
+#undef HYC_GFWD_T
+#undef HYC_GFWD
+  return check_launch("hyc_gated_act_fwd");
 }
 
 }  // extern "C"

@@ -445,6 +445,34 @@ def gated_act_bwd(act, g2d, src_act, src_up, src_gate):
     return d_gate, d_up
 
 
+def gated_act_fwd_supported(H, bits, group):
+    """shapes the one-pass forward covers (the rest takes the activation, three compress calls and a product)"""
+    return bits in (2, 4, 8) and group in (64, 128) and H * bits // 64 <= 1024 and H % (64 // bits) == 0
+
+
+def gated_act_fwd(act, gate2d, up2d, plan_act, plan_up, plan_gate, bits, group):
+    """h = act(gate) * up and the compressed act(gate), up, gate in one pass -> (h, c_act, c_up, c_gate).
+    gate and up are bf16 [M, H] matrices with contiguous rows (column slices of one projection output are fine);
+    the plans are the outlier-channel sets of the three sites."""
+    _need_rows(gate2d, "gate")
+    _need_rows(up2d, "up")
+    if gate2d.shape != up2d.shape:
+        raise ValueError("gate %s and up %s differ in shape" % (tuple(gate2d.shape), tuple(up2d.shape)))
+    M, H = gate2d.shape
+    dev = gate2d.device
+    outs = [alloc_channel(M, H, p, bits, group, dev) for p in (plan_act, plan_up, plan_gate)]
+    descs = [o.desc() for o in outs]
+    h = torch.empty((M, H), dtype=BF16, device=dev)
+    code = {"silu": _abi.ACT_SILU, "gelu": _abi.ACT_GELU_TANH}[act]
+    flat = []
+    for o in outs:
+        flat += [_p(o.stored), _p(o.vals), _p(o.scales)]
+    check(_abi.load().hyc_gated_act_fwd(code, _p(gate2d), gate2d.stride(0) if M > 1 else H, _p(up2d),
+                                        up2d.stride(0) if M > 1 else H, M, H, ctypes.byref(descs[0]), ctypes.byref(descs[1]),
+                                        ctypes.byref(descs[2]), _p(h), *flat, _stream()))
+    return (h,) + tuple(outs)
+
+
 # ----------------------------------------------------------------------------------------------------
 # weight gradient
 # ----------------------------------------------------------------------------------------------------

@@ -110,11 +110,20 @@ class _ChannelGatedActFunc(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, gate, up, act, sites, iteration, bits, group):
+        ctx.act = act
+        calibrated = iteration >= 2 and all(site.plan is not None for site in sites)
+        if calibrated and K.gated_act_fwd_supported(gate.shape[-1], bits, group):
+            # steady state: one pass over gate and up writes the product and the three compressed activations;
+            # act(gate) is never held in memory
+            h, c_act, c_up, c_gate = K.gated_act_fwd(act, _row_view(gate), _row_view(up), sites[0].plan, sites[1].plan,
+                                                     sites[2].plan, bits, group)
+            ctx.saved = (c_act, c_up, c_gate)
+            return h.view(gate.shape)
+        # calibration calls need act(gate) as a tensor (its channel maxima choose the outlier channels)
         a = torch.nn.functional.silu(gate) if act == "silu" else torch.nn.functional.gelu(gate)
         rows = [_row_view(t) for t in (a, up, gate)]
         ctx.saved = tuple(K.compress_channel(r, site.channel_plan(r, iteration), bits, group)
                           for r, site in zip(rows, sites))
-        ctx.act = act
         return a * up
 
     @staticmethod

@@ -192,6 +192,17 @@ int hyc_gated_act_bwd(int32_t act, const void* g, const void* stored_a, const vo
                       const hyc_desc* d_u, const void* stored_g, const void* vals_g, const void* scales_g,
                       const hyc_desc* d_g, int64_t M, int64_t H, void* d_gate, void* d_up, void* stream);
 
+/* Forward of the same product with its three saves fused in: h = bf16(bf16(act(gate)) * up), plus the channel-compressed
+ * forms of act(gate), up and gate (what EfficientMemorySiLU/GELU.forward, efficient_silu.py:13-40 / efficient_gelu.py:13-40,
+ * and EfficientMemoryHadamard.forward, efficient_hadamard.py:11-53, compute and save), in one pass over gate and up;
+ * act(gate) is never written to memory.  gate and up are bf16 [M, H] with row pitches ld_gate, ld_up (elements).  act:
+ * HYC_ACT_SILU = F.silu; HYC_ACT_GELU_TANH = the GELU module, whose forward is the erf form (F.gelu) and whose backward
+ * is the tanh form.  Same bytes as the separate calls; channel scheme, one code width and group size for the three. */
+int hyc_gated_act_fwd(int32_t act, const void* gate, int64_t ld_gate, const void* up, int64_t ld_up, int64_t M, int64_t H,
+                      const hyc_desc* d_a, const hyc_desc* d_u, const hyc_desc* d_g, void* h, void* stored_a, void* vals_a,
+                      void* scales_a, void* stored_u, void* vals_u, void* scales_u, void* stored_g, void* vals_g,
+                      void* scales_g, void* stream);
+
 /* ---- softmax -------------------------------------------------------------------------------- */
 /* x bf16 [rows, N] -> y = softmax(x, -1) bf16 and counts[r] = #{j : y[r,j] > bf16(threshold)} (counts may be
  * NULL).  With x == NULL, y is taken as given and only the counts are produced.  For N <= 4096 y may be x itself

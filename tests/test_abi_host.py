@@ -127,6 +127,15 @@ def test_argument_errors_without_a_gpu(abi):
                                  4, 4096, null, null, null) == abi.EFAULT                                    # null buffers
     assert lib.hyc_gated_act_bwd(abi.ACT_SILU, null, null, null, null, D, null, null, null, D, null, null, null, D,
                                  0, 4096, null, null, null) == 0                                             # empty input
+    nine = [null] * 9
+    assert lib.hyc_gated_act_fwd(9, null, 4096, null, 4096, 4, 4096, D, D, D, null, *nine, null) == abi.EINVAL
+    assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 4096, null, 4096, 4, 4096, D, D, ctypes.byref(t), null, *nine, null) == abi.ENOTSUP
+    assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 4096, null, 4096, 4, 4096, D, ctypes.byref(d2), D, null, *nine, null) == abi.ENOTSUP
+    assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 4000, null, 4096, 4, 4096, D, D, D, null, *nine, null) == abi.EINVAL   # pitch < H
+    assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 8192, null, 4100, 4, 4096, D, D, D, null, *nine, null) == abi.EINVAL   # pitch % 8
+    assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 8192, null, 8192, 4, 4096, D, D, D, null, *nine, null) == abi.EFAULT
+    assert lib.hyc_gated_act_fwd(abi.ACT_GELU_TANH, null, 8192, null, 8192, 0, 4096, D, D, D, null, *nine, null) == 0
+    assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 65536, null, 65536, 4, 65536, D, D, D, null, *nine, null) == abi.ENOTSUP  # row too long
     assert lib.hyc_layernorm_bwd(null, null, null, null, null, 0, null, null, 4, 4096, D, null, null, null, null) == abi.EFAULT
     assert lib.hyc_layernorm_bwd(null, null, null, null, null, 0, null, null, 4, 4096, ctypes.byref(t), null, null, null, null) in (abi.EFAULT, abi.ENOTSUP)
     assert lib.hyc_rmsnorm_bwd_partial_rows(0, 4096, D) == 0

@@ -209,3 +209,41 @@ def test_config2_shape(K):
     dx_o, dw_o = O.rmsnorm_bwd(dy, xh, w, rstd_o)
     assert torch.allclose(dx.cpu().float(), dx_o.float(), rtol=1e-2, atol=1e-3)
     assert torch.allclose(dw.cpu(), dw_o, rtol=1e-2, atol=1e-3)
+
+
+@pytest.mark.parametrize("act", ["silu", "gelu"])
+def test_gated_forward_activation_matches_the_framework_for_every_bf16_value(K, act):
+    """h = act(gate) * 1 from the one-pass forward against F.silu / F.gelu on all 65 536 bf16 patterns (NaN aside):
+    the compressed act(gate) is only the framework's if every value is"""
+    H = 512
+    bits16 = torch.arange(65536, dtype=torch.int32)
+    gate = bits16.to(torch.int16).view(torch.bfloat16).view(-1, H).cuda()
+    up = torch.ones_like(gate)
+    M = gate.shape[0]
+    plan = K.select_channels(torch.zeros(H, device="cuda"), 0)
+    h, _, _, _ = K.gated_act_fwd(act, gate, up, plan, plan, plan, 4, 128)
+    want = torch.nn.functional.silu(gate) if act == "silu" else torch.nn.functional.gelu(gate)
+    ok = torch.isnan(want) & torch.isnan(h) | (h.view(torch.int16) == want.view(torch.int16))
+    assert bool(ok.all()), [(hex(int(b) & 0xFFFF)) for b in gate.view(torch.int16)[~ok][:8].cpu()]
+
+
+@pytest.mark.parametrize("act,M,H,bits,group,k", [("silu", 333, 11008, 4, 128, 110), ("gelu", 64, 4096, 4, 128, 41),
+                                                  ("silu", 2100, 4096, 2, 64, 41), ("silu", 40, 512, 8, 64, 5),
+                                                  ("gelu", 130, 2048, 2, 128, 300)])
+def test_gated_forward_equals_the_separate_calls(K, act, M, H, bits, group, k):
+    """one pass = F.silu / F.gelu, three hyc_compress calls and a product, bit for bit; gate and up are column slices of
+    one wider matrix, as a fused gate/up projection hands them over"""
+    gen = torch.Generator().manual_seed(M + H + bits)
+    both = torch.randn(M, 2 * H, generator=gen)
+    both[:, torch.randperm(2 * H, generator=gen)[:2 * k]] *= 15
+    both = both.bfloat16().cuda()
+    gate, up = both[:, :H], both[:, H:]
+    a = torch.nn.functional.silu(gate) if act == "silu" else torch.nn.functional.gelu(gate)
+    plans = [K.select_channels(K.channel_absmax(t), k) for t in (a, up, gate)]
+    want = [K.compress_channel(t, p, bits, group) for t, p in zip((a, up, gate), plans)]
+    h, c_a, c_u, c_g = K.gated_act_fwd(act, gate, up, plans[0], plans[1], plans[2], bits, group)
+    assert bits_equal(h, a * up)
+    for got, ref in zip((c_a, c_u, c_g), want):
+        assert torch.equal(got.stored.view(torch.uint8), ref.stored.view(torch.uint8))
+        assert bits_equal(got.scales, ref.scales) and bits_equal(got.vals, ref.vals)
+    assert not K.gated_act_fwd_supported(4096, 1, 128) and K.gated_act_fwd_supported(11008, 4, 128)
