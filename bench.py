@@ -162,7 +162,8 @@ def kernel_tour(pkg, torch, reps=5):
             K.act_bwd("gelu", g, cs[0])
             K.hadamard_bwd(g, cs[2], cs[1])
             K.gated_act_bwd("silu", g, cs[2], cs[1], cs[0])
-            K.gated_act_fwd("silu", x, up, cs[2].plan, cs[1].plan, cs[0].plan, bits, G)
+            if K.gated_act_fwd_supported(H, bits, G):
+                K.gated_act_fwd("silu", x, up, cs[2].plan, cs[1].plan, cs[0].plan, bits, G)
             K.gradw_gemm(dy16, cs[0])
             K.gradw_gemm(dyN, cs[0], staged=False)        # x_hat decoded inside the GEMM
             K.gradw_gemm(dyN, cs[0], staged=True)         # x_hat restored once, then the dense form of the kernel

@@ -704,9 +704,11 @@ int hyc_gated_act_fwd(int32_t act, const void* gate, int64_t ld_gate, const void
   if ((rc = make_chan_args(d_a, geo, &c_a, &lpg)) || (rc = make_chan_args(d_u, geo, &c_u, &lpg)) ||
       (rc = make_chan_args(d_g, geo, &c_g, &lpg)))
     return rc;
-  if (geo.iters != 1 || d_a->bits == 1 || (lpg != 8 && lpg != 16))
-    return fail(HYC_ENOTSUP, "hyc_gated_act_fwd: needs 2-, 4- or 8-bit codes, groups of 64 or 128 channels and rows of at "
-                             "most 1024 chunks per segment (use the activation, hyc_compress and a product otherwise)");
+  // Three encoders side by side: with four segments per thread (2-bit codes) or more than 768 threads per row the
+  // kernel would not fit the register file, so those shapes are left to the separate calls.
+  if (geo.iters != 1 || geo.threads > 768 || (d_a->bits != 4 && d_a->bits != 8) || (lpg != 8 && lpg != 16))
+    return fail(HYC_ENOTSUP, "hyc_gated_act_fwd: needs 4- or 8-bit codes, groups of 64 or 128 channels and rows of at "
+                             "most 768 chunks per segment (use the activation, hyc_compress and a product otherwise)");
   if (M == 0) return HYC_OK;
   if (!gate || !up || !h || !stored_a || !stored_u || !stored_g || !scales_a || !scales_u || !scales_g ||
       (d_a->k > 0 && !vals_a) || (d_u->k > 0 && !vals_u) || (d_g->k > 0 && !vals_g))
@@ -723,16 +725,12 @@ int hyc_gated_act_fwd(int32_t act, const void* gate, int64_t ld_gate, const void
   hipLaunchKernelGGL((k_gated_act_fwd_fast<B_, L_, A_, MT_>), dim3(grid), dim3(geo.threads), 0, st,                \
                      static_cast<const uint16_t*>(gate), ld_gate, static_cast<const uint16_t*>(up), ld_up, M, H,   \
                      geo.cps, sa, su, sg, static_cast<uint16_t*>(h))
-#define HYC_GFWD_T(B_, L_, A_)                                                    \
-  do {                                                                            \
-    if (geo.threads <= 256) HYC_GFWD(B_, L_, A_, 256);                            \
-    else if (geo.threads <= 768) HYC_GFWD(B_, L_, A_, 768); /* H = 11008: 704 threads; 1024 would cap the registers at 128 */ \
-    else HYC_GFWD(B_, L_, A_, 1024);                                              \
-  } while (0)
+#define HYC_GFWD_T(B_, L_, A_) /* H = 11008: 704 threads, up to 168 registers each */ \
+  do { if (geo.threads <= 256) HYC_GFWD(B_, L_, A_, 256); else HYC_GFWD(B_, L_, A_, 768); } while (0)
 #define HYC_GFWD_L(B_, A_) do { if (lpg == 8) HYC_GFWD_T(B_, 8, A_); else HYC_GFWD_T(B_, 16, A_); } while (0)
 #define HYC_GFWD_B(A_)                                                                                             \
   do {                                                                                                             \
-    if (d_a->bits == 2) HYC_GFWD_L(2, A_); else if (d_a->bits == 4) HYC_GFWD_L(4, A_); else HYC_GFWD_L(8, A_);     \
+    if (d_a->bits == 4) HYC_GFWD_L(4, A_); else HYC_GFWD_L(8, A_);                                                \
   } while (0)
   if (act == HYC_ACT_SILU) HYC_GFWD_B(HYC_ACT_SILU); else HYC_GFWD_B(HYC_ACT_GELU_TANH);
 #undef HYC_GFWD_B

@@ -447,7 +447,7 @@ def gated_act_bwd(act, g2d, src_act, src_up, src_gate):
 
 def gated_act_fwd_supported(H, bits, group):
     """shapes the one-pass forward covers (the rest takes the activation, three compress calls and a product)"""
-    return bits in (2, 4, 8) and group in (64, 128) and H * bits // 64 <= 1024 and H % (64 // bits) == 0
+    return bits in (4, 8) and group in (64, 128) and H * bits // 64 <= 768 and H % (64 // bits) == 0
 
 
 def gated_act_fwd(act, gate2d, up2d, plan_act, plan_up, plan_gate, bits, group):

@@ -131,6 +131,9 @@ def test_argument_errors_without_a_gpu(abi):
     assert lib.hyc_gated_act_fwd(9, null, 4096, null, 4096, 4, 4096, D, D, D, null, *nine, null) == abi.EINVAL
     assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 4096, null, 4096, 4, 4096, D, D, ctypes.byref(t), null, *nine, null) == abi.ENOTSUP
     assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 4096, null, 4096, 4, 4096, D, ctypes.byref(d2), D, null, *nine, null) == abi.ENOTSUP
+    d2b = ctypes.byref(d2)
+    assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 4096, null, 4096, 4, 4096, d2b, d2b, d2b, null, *nine, null) == abi.ENOTSUP  # 2-bit codes
+    assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 14336, null, 14336, 4, 14336, D, D, D, null, *nine, null) == abi.ENOTSUP    # 896 chunks
     assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 4000, null, 4096, 4, 4096, D, D, D, null, *nine, null) == abi.EINVAL   # pitch < H
     assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 8192, null, 4100, 4, 4096, D, D, D, null, *nine, null) == abi.EINVAL   # pitch % 8
     assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 8192, null, 8192, 4, 4096, D, D, D, null, *nine, null) == abi.EFAULT

@@ -228,8 +228,8 @@ def test_gated_forward_activation_matches_the_framework_for_every_bf16_value(K, 
 
 
 @pytest.mark.parametrize("act,M,H,bits,group,k", [("silu", 333, 11008, 4, 128, 110), ("gelu", 64, 4096, 4, 128, 41),
-                                                  ("silu", 2100, 4096, 2, 64, 41), ("silu", 40, 512, 8, 64, 5),
-                                                  ("gelu", 130, 2048, 2, 128, 300)])
+                                                  ("silu", 2100, 4096, 4, 64, 41), ("silu", 40, 512, 8, 64, 5),
+                                                  ("gelu", 130, 2048, 8, 128, 300)])
 def test_gated_forward_equals_the_separate_calls(K, act, M, H, bits, group, k):
     """one pass = F.silu / F.gelu, three hyc_compress calls and a product, bit for bit; gate and up are column slices of
     one wider matrix, as a fused gate/up projection hands them over"""
@@ -246,4 +246,5 @@ def test_gated_forward_equals_the_separate_calls(K, act, M, H, bits, group, k):
     for got, ref in zip((c_a, c_u, c_g), want):
         assert torch.equal(got.stored.view(torch.uint8), ref.stored.view(torch.uint8))
         assert bits_equal(got.scales, ref.scales) and bits_equal(got.vals, ref.vals)
-    assert not K.gated_act_fwd_supported(4096, 1, 128) and K.gated_act_fwd_supported(11008, 4, 128)
+    assert not K.gated_act_fwd_supported(4096, 2, 64) and K.gated_act_fwd_supported(11008, 4, 128)
+    assert not K.gated_act_fwd_supported(14336, 4, 128)          # 896 chunks per segment: left to the separate calls
