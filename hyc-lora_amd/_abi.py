@@ -49,6 +49,8 @@ SIGNATURES = {
     "hyc_ref_outlier_fill": (c_i32, [c_ptr, c_i64, c_i64, ctypes.POINTER(HycDesc), c_ptr, c_ptr, c_ptr, c_ptr]),
     "hyc_rmsnorm_fwd_compress": (c_i32, [c_ptr, c_ptr, c_i32, c_f32, c_i64, c_i64, ctypes.POINTER(HycDesc),
                                          c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr]),
+    "hyc_layernorm_fwd_compress": (c_i32, [c_ptr, c_ptr, c_ptr, c_i32, c_f32, c_i64, c_i64, ctypes.POINTER(HycDesc),
+                                           c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr]),
     "hyc_rmsnorm_bwd": (c_i32, [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_i32, c_ptr, c_i64, c_i64,
                                 ctypes.POINTER(HycDesc), c_i32, c_ptr, c_ptr, c_ptr, c_ptr]),
     "hyc_layernorm_bwd": (c_i32, [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_i32, c_ptr, c_ptr, c_i64, c_i64,

@@ -348,13 +348,17 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
 
 // ------------------------------------------------------------------------------------------------
 // forward: y, rstd, and x compressed.  MODE 0 = channel, 1 = threshold.  One workgroup = one row at a time.
+// LN: LayerNorm instead of RMSNorm, with the two-pass statistics of operators/efficient_layernorm.py:15-61
+// (mean = sum(x)/H, var = sum((x - mean)^2)/H, y = ((x - mean)*rstd)*w + b); the row is in registers, so the
+// second pass costs one more workgroup reduction and no memory traffic.
 // ------------------------------------------------------------------------------------------------
-template <int BITS, int ITERS, int MAXT, int MODE>
+template <int BITS, int ITERS, int MAXT, int MODE, bool LN = false>
 __global__ void __launch_bounds__(MAXT)
-k_rmsnorm_fwd(const uint16_t* __restrict__ x, const void* __restrict__ w, bool wf32, float eps, int64_t M, int64_t H,
+k_rmsnorm_fwd(const uint16_t* __restrict__ x, const void* __restrict__ w, const void* __restrict__ bias, bool wf32,
+              float eps, int64_t M, int64_t H,
               int CPS, ChanArgs ca, int lpg, ThrArgs ta, bool perchan, uint16_t* __restrict__ y,
-              float* __restrict__ rstd_out, uint8_t* __restrict__ stored, uint16_t* __restrict__ vals,
-              uint16_t* __restrict__ scales, int32_t* __restrict__ row_counts) {
+              float* __restrict__ mean_out, float* __restrict__ rstd_out, uint8_t* __restrict__ stored,
+              uint16_t* __restrict__ vals, uint16_t* __restrict__ scales, int32_t* __restrict__ row_counts) {
   constexpr int NSEG = Q<BITS>::NSEG;
   __shared__ float red[2 * 16 * 2];
   const int64_t SEG = (int64_t)CPS * 8;
@@ -405,7 +409,7 @@ k_rmsnorm_fwd(const uint16_t* __restrict__ x, const void* __restrict__ w, bool w
           float v[8];
           unpack8(raw[it][i], v);
 #pragma unroll
-          for (int j = 0; j < 8; ++j) ss = __builtin_fmaf(v[j], v[j], ss);
+          for (int j = 0; j < 8; ++j) ss = LN ? ss + v[j] : __builtin_fmaf(v[j], v[j], ss);
           uint32_t cl, ch;
           const float s = encode_seg<BITS>(raw[it][i], v, plan[it][i], lpg, vals + row * ca.k, cl, ch);
           if (act[it] && (c & (lpg - 1)) == 0)
@@ -419,7 +423,7 @@ k_rmsnorm_fwd(const uint16_t* __restrict__ x, const void* __restrict__ w, bool w
           float v[8];
           unpack8(raw[it][i], v);
 #pragma unroll
-          for (int j = 0; j < 8; ++j) ss = __builtin_fmaf(v[j], v[j], ss);
+          for (int j = 0; j < 8; ++j) ss = LN ? ss + v[j] : __builtin_fmaf(v[j], v[j], ss);
         }
         if (act[it]) {
           hot += (float)(perchan ? encode_thr<BITS, true>(raw[it], c, CPS, H, row % ta.S, ta, lo, hi)
@@ -429,9 +433,30 @@ k_rmsnorm_fwd(const uint16_t* __restrict__ x, const void* __restrict__ w, bool w
       if (act[it]) *reinterpret_cast<uint2*>(stored + row * SEG + 8 * c) = make_uint2(lo, hi);
     }
     slot_sum2(ss, hot, red, parity, 0, 1, wave, nw);
+    float mean = 0.f;
+    if (LN) {
+      mean = ss * invH;
+      float var = 0.f, unused = 0.f;
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) {
+        if (act[it]) {                                  // lanes past the row hold zeros, not x - mean
+#pragma unroll
+          for (int i = 0; i < NSEG; ++i) {
+            float v[8];
+            unpack8(raw[it][i], v);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) { const float dlt = v[j] - mean; var = __builtin_fmaf(dlt, dlt, var); }
+          }
+        }
+      }
+      parity ^= 1;                                      // the other buffer: see slot_sum2
+      slot_sum2(var, unused, red, parity, 0, 1, wave, nw);
+      ss = var;
+    }
     const float rstd = 1.0f / __builtin_sqrtf(ss * invH + eps);
     if (threadIdx.x == 0) {
       rstd_out[row] = rstd;
+      if (LN) mean_out[row] = mean;
       if (MODE == 1 && row_counts) row_counts[row] = (int32_t)hot;
     }
     uint16_t* yr = y + row * H;
@@ -444,8 +469,17 @@ k_rmsnorm_fwd(const uint16_t* __restrict__ x, const void* __restrict__ w, bool w
           float v[8], wv[8];
           unpack8(raw[it][i], v);
           load_w8(w, wf32, col, wv);
+          if (LN) {
+            float bv[8];
 #pragma unroll
-          for (int j = 0; j < 8; ++j) v[j] = (v[j] * rstd) * wv[j];
+            for (int j = 0; j < 8; ++j) bv[j] = 0.f;
+            if (bias) load_w8(bias, wf32, col, bv);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = ((v[j] - mean) * rstd) * wv[j] + bv[j];
+          } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = (v[j] * rstd) * wv[j];
+          }
           *reinterpret_cast<uint4*>(yr + col) = pack8(v);
         }
       }
@@ -752,9 +786,9 @@ int64_t hyc_rmsnorm_bwd_partial_rows(int64_t M, int64_t H, const hyc_desc* d) {
   return (d->mode == HYC_MODE_CHANNEL && b.fast_ok) ? b.fast_P : b.P;
 }
 
-int hyc_rmsnorm_fwd_compress(const void* x, const void* w, int32_t w_dtype, float eps, int64_t M, int64_t H,
-                             const hyc_desc* d, void* y, float* rstd, void* stored, void* vals, void* scales,
-                             int32_t* row_counts, void* stream) {
+static int norm_fwd_impl(const void* x, const void* w, const void* bias, int32_t w_dtype, float eps, int64_t M, int64_t H,
+                         const hyc_desc* d, void* y, float* mean, float* rstd, void* stored, void* vals, void* scales,
+                         int32_t* row_counts, void* stream, bool ln) {
   if (!d) return fail(HYC_EFAULT, "hyc_rmsnorm_fwd_compress: null descriptor");
   if (M < 0) return fail(HYC_EINVAL, "hyc_rmsnorm_fwd_compress: M=%lld", (long long)M);
   if (w_dtype != HYC_DTYPE_BF16 && w_dtype != HYC_DTYPE_F32) return fail(HYC_EINVAL, "hyc_rmsnorm_fwd_compress: w_dtype=%d", w_dtype);
@@ -768,7 +802,10 @@ int hyc_rmsnorm_fwd_compress(const void* x, const void* w, int32_t w_dtype, floa
   NormGeom n;
   if ((rc = norm_geom(g.cps, &n))) return rc;
   if (M == 0) return HYC_OK;
-  if (!x || !w || !y || !rstd || !stored) return fail(HYC_EFAULT, "hyc_rmsnorm_fwd_compress: null buffer");
+  if (!x || !w || !y || !rstd || !stored || (ln && !mean)) return fail(HYC_EFAULT, "hyc_rmsnorm_fwd_compress: null buffer");
+  if (ln && n.iters_t != 1)
+    return fail(HYC_ENOTSUP, "hyc_layernorm_fwd_compress: rows of at most 1024 chunks per segment (H*bits/64 <= 1024)");
+  if (ln && bias && !aligned16(bias)) return fail(HYC_EINVAL, "hyc_layernorm_fwd_compress: bias must be 16-byte aligned");
   if (d->mode == HYC_MODE_CHANNEL && (!scales || (d->k > 0 && !vals))) return fail(HYC_EFAULT, "hyc_rmsnorm_fwd_compress: null vals/scales");
   if (!aligned16(x) || !aligned16(y) || !aligned16(w) || !aligned8(stored))
     return fail(HYC_EINVAL, "hyc_rmsnorm_fwd_compress: x, y, w must be 16-byte and stored 8-byte aligned");
@@ -778,7 +815,7 @@ int hyc_rmsnorm_fwd_compress(const void* x, const void* w, int32_t w_dtype, floa
   hipStream_t st = begin_launch(stream);
   const uint16_t* xp = static_cast<const uint16_t*>(x);
   // fast path: every lane owns one chunk per segment, group width known at compile time
-  if (d->mode == HYC_MODE_CHANNEL && n.iters == 1 && (lpg == 8 || lpg == 16) && d->bits != 1) {
+  if (!ln && d->mode == HYC_MODE_CHANNEL && n.iters == 1 && (lpg == 8 || lpg == 16) && d->bits != 1) {
     uint16_t* yp = static_cast<uint16_t*>(y);
     uint8_t* stp = static_cast<uint8_t*>(stored);
     uint16_t* vp = static_cast<uint16_t*>(vals);
@@ -803,17 +840,49 @@ int hyc_rmsnorm_fwd_compress(const void* x, const void* w, int32_t w_dtype, floa
 #undef HYC_FWD_FAST
     return check_launch("hyc_rmsnorm_fwd_compress");
   }
-#define HYC_FWD(MODE_, MT_)                                                                                        \
-  hipLaunchKernelGGL((k_rmsnorm_fwd<B, IT, MT_, MODE_>), dim3(grid), dim3(n.T), 0, st, xp, w, wf32, eps, M, H, g.cps, \
-                     ca, lpg, ta, perchan, static_cast<uint16_t*>(y), rstd, static_cast<uint8_t*>(stored),         \
+#define HYC_FWD_K(KERNEL_)                                                                                         \
+  hipLaunchKernelGGL(KERNEL_, dim3(grid), dim3(n.T), 0, st, xp, w, bias, wf32, eps, M, H, g.cps,                   \
+                     ca, lpg, ta, perchan, static_cast<uint16_t*>(y), mean, rstd, static_cast<uint8_t*>(stored),   \
                      static_cast<uint16_t*>(vals), static_cast<uint16_t*>(scales), row_counts)
+#define HYC_FWD(MODE_, MT_) HYC_FWD_K((k_rmsnorm_fwd<B, IT, MT_, MODE_>))
+#define HYC_FWD_LN(B_, MODE_)                                                                                      \
+  do {                                                                                                             \
+    if (n.T <= 256) HYC_FWD_K((k_rmsnorm_fwd<B_, 1, 256, MODE_, true>));                                           \
+    else HYC_FWD_K((k_rmsnorm_fwd<B_, 1, 1024, MODE_, true>));                                                     \
+  } while (0)
+  if (ln) {
+#define HYC_FWD_LN_BITS(MODE_)                                  \
+  switch (d->bits) {                                            \
+    case 1: HYC_FWD_LN(1, MODE_); break;                        \
+    case 2: HYC_FWD_LN(2, MODE_); break;                        \
+    case 4: HYC_FWD_LN(4, MODE_); break;                        \
+    default: HYC_FWD_LN(8, MODE_); break;                       \
+  }
+    if (d->mode == HYC_MODE_CHANNEL) { HYC_FWD_LN_BITS(0) } else { HYC_FWD_LN_BITS(1) }
+#undef HYC_FWD_LN_BITS
+    return check_launch("hyc_layernorm_fwd_compress");
+  }
   if (d->mode == HYC_MODE_CHANNEL) {
     HYC_BITS_ITERS(d->bits, n.iters_t, if (n.T <= 256) HYC_FWD(0, 256); else HYC_FWD(0, 1024));
   } else {
     HYC_BITS_ITERS(d->bits, n.iters_t, if (n.T <= 256) HYC_FWD(1, 256); else HYC_FWD(1, 1024));
   }
 #undef HYC_FWD
+#undef HYC_FWD_LN
+#undef HYC_FWD_K
   return check_launch("hyc_rmsnorm_fwd_compress");
+}
+
+int hyc_rmsnorm_fwd_compress(const void* x, const void* w, int32_t w_dtype, float eps, int64_t M, int64_t H,
+                             const hyc_desc* d, void* y, float* rstd, void* stored, void* vals, void* scales,
+                             int32_t* row_counts, void* stream) {
+  return norm_fwd_impl(x, w, nullptr, w_dtype, eps, M, H, d, y, nullptr, rstd, stored, vals, scales, row_counts, stream, false);
+}
+
+int hyc_layernorm_fwd_compress(const void* x, const void* w, const void* bias, int32_t w_dtype, float eps, int64_t M,
+                               int64_t H, const hyc_desc* d, void* y, float* mean, float* rstd, void* stored, void* vals,
+                               void* scales, int32_t* row_counts, void* stream) {
+  return norm_fwd_impl(x, w, bias, w_dtype, eps, M, H, d, y, mean, rstd, stored, vals, scales, row_counts, stream, true);
 }
 
 static int norm_bwd_impl(const void* dy, const void* stored, const void* vals, const void* scales, const void* w,

@@ -342,6 +342,67 @@ def rmsnorm_fwd_compress_threshold(x2d, w, eps, S, threshold, scale, bits, L=Non
     return y, rstd, ThresholdCompressed(stored, row_ptr, cols, vals, float(threshold), scale, L, R, bits, M, H, S)
 
 
+def layernorm_fwd_supported(H, bits):
+    """rows the one-pass LayerNorm forward covers"""
+    return bits in (1, 2, 4, 8) and H % (64 // bits) == 0 and H * bits // 64 <= 1024
+
+
+def _need_bias(bias, w, H):
+    if bias is None:
+        return None
+    if not bias.is_cuda or not bias.is_contiguous() or bias.numel() != H or bias.dtype != w.dtype:
+        raise ValueError("bias must be a contiguous CUDA tensor of %d elements in the weight's dtype" % H)
+    return bias
+
+
+def layernorm_fwd_compress_channel(x2d, w, bias, eps, plan, bits, group):
+    """-> (y bf16 [M,H], mean fp32 [M], rstd fp32 [M], ChannelCompressed of x), one pass over x"""
+    _need(x2d, BF16, "x")
+    M, H = x2d.shape
+    _need_weight(w, H)
+    _need_bias(bias, w, H)
+    lib = _abi.load()
+    check(lib.hyc_check_shape(H, bits, group, _abi.MODE_CHANNEL))
+    y = torch.empty_like(x2d)
+    mean = torch.empty(M, dtype=torch.float32, device=x2d.device)
+    rstd = torch.empty(M, dtype=torch.float32, device=x2d.device)
+    c = alloc_channel(M, H, plan, bits, group, x2d.device)
+    d = c.desc()
+    check(lib.hyc_layernorm_fwd_compress(_p(x2d), _p(w), _p(bias), _wdtype(w), float(eps), M, H, ctypes.byref(d), _p(y),
+                                         _p(mean), _p(rstd), _p(c.stored), _p(c.vals), _p(c.scales), None, _stream()))
+    return y, mean, rstd, c
+
+
+def layernorm_fwd_compress_threshold(x2d, w, bias, eps, S, threshold, scale, bits, L=None, R=None):
+    """-> (y, mean, rstd, ThresholdCompressed of x)"""
+    _need(x2d, BF16, "x")
+    _need(scale, BF16, "scale")
+    M, H = x2d.shape
+    _need_weight(w, H)
+    _need_bias(bias, w, H)
+    lib = _abi.load()
+    dev = x2d.device
+    if L is not None:
+        L = fit_rows(_need(L, BF16, "L"), S)
+        _need(R, BF16, "R")
+    y = torch.empty_like(x2d)
+    mean = torch.empty(M, dtype=torch.float32, device=dev)
+    rstd = torch.empty(M, dtype=torch.float32, device=dev)
+    stored = torch.empty((M, H * bits // 8), dtype=torch.int8 if bits == 8 else torch.uint8, device=dev)
+    counts = torch.empty(M, dtype=torch.int32, device=dev)
+    d = threshold_desc(threshold, scale, bits, S, H, L, R)
+    check(lib.hyc_layernorm_fwd_compress(_p(x2d), _p(w), _p(bias), _wdtype(w), float(eps), M, H, ctypes.byref(d), _p(y),
+                                         _p(mean), _p(rstd), _p(stored), None, None, _p(counts), _stream()))
+    row_ptr = torch.zeros(M + 1, dtype=torch.int32, device=dev)
+    torch.cumsum(counts, 0, out=row_ptr[1:])
+    nnz = int(row_ptr[-1].item())
+    cols = torch.empty(nnz, dtype=torch.int32, device=dev)
+    vals = torch.empty(nnz, dtype=BF16, device=dev)
+    check(lib.hyc_ref_outlier_fill(_p(x2d), M, H, ctypes.byref(d), _p(row_ptr), _p(cols) if nnz else None,
+                                   _p(vals) if nnz else None, _stream()))
+    return y, mean, rstd, ThresholdCompressed(stored, row_ptr, cols, vals, float(threshold), scale, L, R, bits, M, H, S)
+
+
 def _source(c, M, H):
     """(stored, vals, scales, desc) of a ChannelCompressed, or of a dense bf16 x_hat, that holds an [M, H] activation"""
     if isinstance(c, (ChannelCompressed, ThresholdCompressed)) and (c.M, c.H) != (M, H):

@@ -1,9 +1,10 @@
 """LayerNorm whose input is saved compressed.  Reference: operators/efficient_layernorm.py (forward kernel :15-61,
 backward :66-148, Function :203-330, module :333-405).
 
-The forward is PyTorch's own fused layer norm (y, mean, rstd in one pass) followed by the compress kernel; the
-backward is the fused decompress + dx + dw kernel of the RMSNorm path with the row mean folded in
-(xn = (x_hat - mean) * rstd), and db = sum of dy."""
+The forward is one kernel (statistics, y and the compressed x from a single read of x, the RMSNorm forward kernel
+with the row mean added); the backward is the fused decompress + dx + dw kernel of the RMSNorm path with the row mean
+folded in (xn = (x_hat - mean) * rstd), and db = sum of dy.  Rows too long for the one-pass forward (more than 1024
+chunks per segment) take the framework's layer norm followed by the compress kernel."""
 import torch
 
 from .. import kernels as K
@@ -19,6 +20,13 @@ def _forward_stats(x2, weight, bias, eps):
     else:
         y, mean, rstd = torch.native_layer_norm(x2, (x2.shape[-1],), weight, bias, eps)
     return y, mean.reshape(-1).float().contiguous(), rstd.reshape(-1).float().contiguous()
+
+
+def _affine(weight, bias):
+    """(w, b) as the kernels read them: contiguous, the bias in the weight's dtype"""
+    w = weight.detach().contiguous()
+    b = None if bias is None else bias.detach().to(w.dtype).contiguous()
+    return w, b
 
 
 def _backward(ctx, dy):
@@ -39,14 +47,21 @@ class EfficientMemoryLayerNormFunc(torch.autograd.Function):
         x2, _ = as_rows(x)
         if x2.shape[-1] * x.element_size() > 65536:
             raise RuntimeError("This layer norm doesn't support feature dim >= 64KB.")
-        y, mean, rstd = _forward_stats(x2, weight, bias, eps)
         if iteration < 2:
             outlier, L, R, scale = get_statistics(x, iteration, outlier_ratio, sub_outlier_ratio, sub_outlier_bit,
                                                   sub_outlier_quantize_method, rank)
         else:
             outlier, L, scale, R = static_value[0], static_value[1], static_value[2], static_value[3]
-        c, _ = compress_to_csr(x, outlier, scale, sub_outlier_bit, sub_outlier_ratio, L if rank > 0 else None,
-                               R if rank > 0 else None)
+        if (sub_outlier_ratio > 0. and sub_outlier_bit != 16 and x.dim() == 3
+                and K.layernorm_fwd_supported(x2.shape[-1], sub_outlier_bit)):
+            w, b = _affine(weight, bias)
+            y, mean, rstd, c = K.layernorm_fwd_compress_threshold(
+                x2, w, b, eps, x.shape[-2], float(outlier), scale.contiguous(), sub_outlier_bit,
+                L.contiguous() if rank > 0 else None, R.contiguous() if rank > 0 else None)
+        else:
+            y, mean, rstd = _forward_stats(x2, weight, bias, eps)
+            c, _ = compress_to_csr(x, outlier, scale, sub_outlier_bit, sub_outlier_ratio, L if rank > 0 else None,
+                                   R if rank > 0 else None)
         ctx.saved, ctx.mean, ctx.rstd, ctx.weight, ctx.bias = c, mean, rstd, weight, bias
         ctx.mark_non_differentiable(outlier, L, R, scale)
         return y.reshape(x.shape), outlier, L, R, scale
@@ -61,8 +76,12 @@ class _ChannelLayerNormFunc(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, weight, bias, eps, plan, bits, group):
         x2, _ = as_rows(x)
-        y, mean, rstd = _forward_stats(x2, weight, bias, eps)
-        ctx.saved = K.compress_channel(x2, plan, bits, group)
+        if K.layernorm_fwd_supported(x2.shape[-1], bits):
+            w, b = _affine(weight, bias)
+            y, mean, rstd, ctx.saved = K.layernorm_fwd_compress_channel(x2, w, b, eps, plan, bits, group)
+        else:
+            y, mean, rstd = _forward_stats(x2, weight, bias, eps)
+            ctx.saved = K.compress_channel(x2, plan, bits, group)
         ctx.mean, ctx.rstd, ctx.weight, ctx.bias = mean, rstd, weight, bias
         return y.reshape(x.shape)
 

@@ -167,9 +167,17 @@ int hyc_rmsnorm_bwd(const void* dy, const void* stored, const void* vals, const 
                     int32_t w_dtype, const float* rstd, int64_t M, int64_t H, const hyc_desc* d, int32_t c2_quirk,
                     void* dx, float* dw_partials, void* dw, void* stream);
 
+/* LayerNorm forward with the compression of x fused in (efficient_layernorm.py:15-61 kernel, :203-260 Function):
+ * mean = sum(x)/H, rstd = 1/sqrt(sum((x-mean)^2)/H + eps) (both fp32 [M]), y = bf16(((x-mean)*rstd)*w + b); bias may be
+ * NULL, else it has w's dtype.  Other arguments as hyc_rmsnorm_fwd_compress.  Rows of at most 1024 chunks per segment
+ * (H*bits/64 <= 1024), HYC_ENOTSUP beyond. */
+int hyc_layernorm_fwd_compress(const void* x, const void* w, const void* bias, int32_t w_dtype, float eps, int64_t M,
+                               int64_t H, const hyc_desc* d, void* y, float* mean, float* rstd, void* stored, void* vals,
+                               void* scales, int32_t* row_counts, void* stream);
+
 /* LayerNorm backward (efficient_layernorm.py:66-148, 262-330): xn = (xhat - mean)*rstd, dx as above with both
- * means (c1, c2), dw = sum_m dy*xn.  db = sum_m dy and the forward (mean, rstd, y) are plain reductions / one
- * library call and are left to the caller; x is compressed with hyc_compress.  Buffers as for hyc_rmsnorm_bwd. */
+ * means (c1, c2), dw = sum_m dy*xn.  db = sum_m dy is a plain reduction left to the caller.  Buffers as for
+ * hyc_rmsnorm_bwd. */
 int hyc_layernorm_bwd(const void* dy, const void* stored, const void* vals, const void* scales, const void* w,
                       int32_t w_dtype, const float* mean, const float* rstd, int64_t M, int64_t H, const hyc_desc* d,
                       void* dx, float* dw_partials, void* dw, void* stream);

@@ -139,6 +139,11 @@ def test_argument_errors_without_a_gpu(abi):
     assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 8192, null, 8192, 4, 4096, D, D, D, null, *nine, null) == abi.EFAULT
     assert lib.hyc_gated_act_fwd(abi.ACT_GELU_TANH, null, 8192, null, 8192, 0, 4096, D, D, D, null, *nine, null) == 0
     assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 65536, null, 65536, 4, 65536, D, D, D, null, *nine, null) == abi.ENOTSUP  # row too long
+    assert lib.hyc_layernorm_fwd_compress(null, null, null, 0, 1e-5, 4, 4096, None, null, null, null, null, null, null, null, null) == abi.EFAULT
+    assert lib.hyc_layernorm_fwd_compress(null, null, null, 7, 1e-5, 4, 4096, D, null, null, null, null, null, null, null, null) == abi.EINVAL
+    assert lib.hyc_layernorm_fwd_compress(null, null, null, 0, 1e-5, 4, 4096, D, null, null, null, null, null, null, null, null) == abi.EFAULT
+    assert lib.hyc_layernorm_fwd_compress(null, null, null, 0, 1e-5, 0, 4096, D, null, null, null, null, null, null, null, null) == 0
+    assert lib.hyc_layernorm_fwd_compress(null, null, null, 0, 1e-5, 4, 32768, D, null, null, null, null, null, null, null, null) in (abi.EFAULT, abi.ENOTSUP)
     assert lib.hyc_layernorm_bwd(null, null, null, null, null, 0, null, null, 4, 4096, D, null, null, null, null) == abi.EFAULT
     assert lib.hyc_layernorm_bwd(null, null, null, null, null, 0, null, null, 4, 4096, ctypes.byref(t), null, null, null, null) in (abi.EFAULT, abi.ENOTSUP)
     assert lib.hyc_rmsnorm_bwd_partial_rows(0, 4096, D) == 0

@@ -248,3 +248,54 @@ def test_gated_forward_equals_the_separate_calls(K, act, M, H, bits, group, k):
         assert bits_equal(got.scales, ref.scales) and bits_equal(got.vals, ref.vals)
     assert not K.gated_act_fwd_supported(4096, 2, 64) and K.gated_act_fwd_supported(11008, 4, 128)
     assert not K.gated_act_fwd_supported(14336, 4, 128)          # 896 chunks per segment: left to the separate calls
+
+
+@pytest.mark.parametrize("bits,group,M,H,k,wdt,with_bias", [
+    (4, 64, 80, 768, 8, torch.float32, True), (4, 128, 33, 1024, 10, torch.bfloat16, True),
+    (2, 64, 2100, 4096, 41, torch.float32, False), (8, 32, 9, 512, 5, torch.bfloat16, True),
+    (1, 64, 17, 1024, 0, torch.float32, True), (4, 128, 20, 11008, 110, torch.float32, True)])
+def test_layernorm_forward_channel(K, bits, group, M, H, k, wdt, with_bias):
+    """one pass = the reference's two-pass statistics and y (efficient_layernorm.py:15-61) plus hyc_compress of x"""
+    gen = torch.Generator().manual_seed(bits + M + H)
+    x = 0.7 + torch.randn(M, H, generator=gen)
+    x[:, torch.randperm(H, generator=gen)[:max(k, 1)]] *= 12
+    x = x.bfloat16()
+    w = (1 + 0.1 * torch.randn(H, generator=gen)).to(wdt)
+    b = (0.1 * torch.randn(H, generator=gen)).to(wdt) if with_bias else None
+    xd = x.cuda()
+    plan = K.select_channels(K.channel_absmax(xd), k)
+    y, mean, rstd, c = K.layernorm_fwd_compress_channel(xd, w.cuda(), None if b is None else b.cuda(), 1e-5, plan, bits, group)
+    y_o, mean_o, rstd_o = O.layernorm_fwd(x, w, b, 1e-5)
+    assert torch.allclose(mean.cpu(), mean_o, rtol=1e-5, atol=1e-6) and torch.allclose(rstd.cpu(), rstd_o, rtol=1e-5, atol=0)
+    # one bf16 ulp, or the absolute error that 1e-5 relative in mean / rstd leaves where (x - mean) * rstd * w + b cancels
+    diff = (y.cpu().float() - y_o.float()).abs()
+    assert bool(((bf16_ulp_diff(y.cpu(), y_o) <= 1) | (diff <= 2e-3)).all())
+    ref = K.compress_channel(xd, plan, bits, group)
+    assert torch.equal(c.stored.view(torch.uint8), ref.stored.view(torch.uint8))
+    assert bits_equal(c.scales, ref.scales) and bits_equal(c.vals, ref.vals)
+    with pytest.raises(ValueError):
+        K.layernorm_fwd_compress_channel(xd, w.cuda(), torch.zeros(H - 8, dtype=wdt, device="cuda"), 1e-5, plan, bits, group)
+
+
+@pytest.mark.parametrize("bits,method,rank", [(8, "per-channel", 2), (4, "per-token", 0), (2, "per-tensor", 0)])
+def test_layernorm_forward_threshold(K, bits, method, rank):
+    B, S, H = 2, 24, 768
+    gen = torch.Generator().manual_seed(40 + bits)
+    x = 0.3 + torch.randn(B, S, H, generator=gen)
+    x[..., :3] *= 15
+    x = x.bfloat16()
+    w = 1 + 0.1 * torch.randn(H, generator=gen)
+    b = 0.1 * torch.randn(H, generator=gen)
+    torch.manual_seed(1)
+    thr, L, R, scale = O.get_statistics(x, 0, 0.005, 1.0, bits, method, rank)
+    coo, stored, _ = O.ref_compress(x, thr, scale, bits, 1.0, L, R)
+    xh = O.ref_decompress(coo, stored, bits, scale, L=L, R=R).reshape(-1, H)
+    y, mean, rstd, c = K.layernorm_fwd_compress_threshold(x.reshape(-1, H).cuda(), w.cuda(), b.cuda(), 1e-5, S, float(thr),
+                                                          scale.cuda(), bits, L.cuda() if rank else None,
+                                                          R.cuda() if rank else None)
+    y_o, mean_o, rstd_o = O.layernorm_fwd(x.reshape(-1, H), w, b, 1e-5)
+    assert torch.allclose(mean.cpu(), mean_o, rtol=1e-5, atol=1e-6) and torch.allclose(rstd.cpu(), rstd_o, rtol=1e-5, atol=0)
+    diff = (y.cpu().float() - y_o.float()).abs()
+    assert bool(((bf16_ulp_diff(y.cpu(), y_o) <= 1) | (diff <= 2e-3)).all())
+    assert torch.equal(c.stored.cpu().reshape(stored.shape), stored)
+    assert bits_equal(K.decompress_threshold(c).cpu(), xh)

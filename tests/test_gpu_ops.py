@@ -326,9 +326,8 @@ def test_layernorm_module(ops, K, mode, H):
         y.backward(dy.cuda())
         w, b = mod.weight.detach().cpu(), mod.bias.detach().cpu()
         y_o, mean_o, rstd_o = O.layernorm_fwd(x, w, b, 1e-5)
-        # y is the framework's own fused layer norm (it folds mean and rstd into per-row coefficients): a rounding
-        # or two away from the reference's expression order where the terms cancel
-        assert torch.allclose(y.detach().cpu().float(), y_o.float(), rtol=2 ** -6, atol=4e-3)
+        # the kernel follows the reference's expression order; what is left is the summation order of mean and rstd
+        assert torch.allclose(y.detach().cpu().float(), y_o.float(), rtol=2 ** -7, atol=2e-3)
         xh = (K.decompress_threshold(saved) if mode == "ref" else K.decompress_channel(saved)).cpu().reshape(B, S, H)
         dx_o, dw_o, db_o = O.layernorm_bwd(dy, xh, w, mean_o, rstd_o)
         assert torch.allclose(xd.grad.cpu().float(), dx_o.float(), rtol=1e-2, atol=1e-3)
