@@ -62,6 +62,9 @@ SIGNATURES = {
                                   c_ptr, c_ptr, c_ptr, ctypes.POINTER(HycDesc), c_i64, c_i64, c_ptr, c_ptr, c_ptr]),
     "hyc_gated_act_fwd": (c_i32, [c_i32, c_ptr, c_i64, c_ptr, c_i64, c_i64, c_i64, ctypes.POINTER(HycDesc), ctypes.POINTER(HycDesc),
                                   ctypes.POINTER(HycDesc), c_ptr] + [c_ptr] * 9 + [c_ptr]),
+    "hyc_act_fwd_compress": (c_i32, [c_i32, c_ptr, c_i64, c_i64, c_i64, ctypes.POINTER(HycDesc), c_ptr, c_ptr, c_ptr, c_ptr, c_ptr]),
+    "hyc_hadamard_fwd_compress": (c_i32, [c_ptr, c_i64, c_ptr, c_i64, c_i64, c_i64, ctypes.POINTER(HycDesc), ctypes.POINTER(HycDesc),
+                                          c_ptr] + [c_ptr] * 6 + [c_ptr]),
     "hyc_softmax_fwd": (c_i32, [c_ptr, c_i64, c_i64, c_f32, c_ptr, c_ptr, c_ptr]),
     "hyc_softmax_causal_fwd": (c_i32, [c_ptr, c_i64, c_i64, c_i64, c_f32, c_ptr, c_ptr, c_ptr]),
     "hyc_softmax_fill": (c_i32, [c_ptr, c_i64, c_i64, c_f32, c_ptr, c_ptr, c_ptr, c_ptr]),

@@ -364,9 +364,19 @@ k_gated_act_bwd_fast(const uint16_t* __restrict__ g, const uint8_t* __restrict__
 // ---- forward of h = act(gate) * up with the three saves fused in ----------------------------------------------
 // The activation value as the framework computes it for a bf16 tensor: fp32 arithmetic with the accurate library
 // exp / erf, one rounding to bf16 (operators/efficient_silu.py:16 F.silu, operators/efficient_gelu.py:16 F.gelu).
+// SiLU takes a short cut that cannot change the bf16 result: x * rcp(1 + exp(-x)) with the hardware exp and a refined
+// reciprocal is within a few fp32 ulp of the library expression; only when that value lies within 32 ulp of a bf16
+// rounding boundary (1 element in 1000), or where the short cut loses accuracy (|x| >= 80, tiny results), is the
+// library expression evaluated.  Both forms then round to the same bf16 value for every input (tested on all 65 536).
 template <int ACT>
 __device__ __forceinline__ float act_value(float x) {
-  if (ACT == HYC_ACT_SILU) return x / (1.0f + expf(-x));
+  if (ACT == HYC_ACT_SILU) {
+    float f = x * rcp_pos(1.0f + exp_fast(-x));
+    const uint32_t low = __float_as_uint(f) & 0xFFFFu;            // the bits a bf16 rounding drops
+    const bool decided = (low - 0x7FE0u > 0x40u) && __builtin_fabsf(x) < 80.0f && __builtin_fabsf(f) > 1e-30f;
+    if (__builtin_expect(!decided, 0)) f = x / (1.0f + expf(-x));
+    return f;
+  }
   return (x * 0.5f) * (1.0f + erff(x * 0.70710678118654752440f));
 }
 
@@ -474,6 +484,100 @@ k_gated_act_fwd_fast(const uint16_t* __restrict__ gate, int64_t ldg, const uint1
 #pragma unroll
     for (int i = 0; i < NSEG; ++i) { graw[i] = g_n[i]; uraw[i] = u_n[i]; }
     grow += gstep; urow += ustep; hp += hstep; soff += sstep; scoff += scstep;
+  }
+}
+
+// The same idea for the operators taken one at a time (what a module swap installs): NIN = 1: y = act(x) and the
+// compressed x (EfficientMemorySiLU / GELU forward, efficient_silu.py:13-40, efficient_gelu.py:13-40);
+// NIN = 2: y = x1 * x2 and both operands compressed (EfficientMemoryHadamard forward, efficient_hadamard.py:11-53).
+// Every operand is read once.
+template <int BITS, int LPGT, int ACT, int NIN, int MAXT>
+__global__ void __launch_bounds__(MAXT)
+k_ew_fwd_fast(const uint16_t* __restrict__ x1, int64_t ld1, const uint16_t* __restrict__ x2, int64_t ld2, int64_t M, int64_t H,
+              int CPS, GatedFwdSite s1, GatedFwdSite s2, uint16_t* __restrict__ y) {
+  constexpr int NSEG = Q<BITS>::NSEG;
+  const int c = threadIdx.x;
+  if (c >= CPS) return;                                 // tail of the last wave; scale groups never straddle it
+  const int64_t SEG = (int64_t)CPS * 8;
+  const bool leader = (c & (LPGT - 1)) == 0;
+  const int shift = s1.ca.chunk_to_group_shift;
+  const int seg_groups = CPS >> shift;
+  const int gpr = s1.ca.groups_per_row;
+  uint32_t km[NIN][NSEG][4];
+  {
+    uint32_t plan[NSEG];
+    ChunkOutliers<NSEG> co;
+#pragma unroll
+    for (int n = 0; n < NIN; ++n) {
+      const ChanArgs& ca = n == 0 ? s1.ca : s2.ca;
+#pragma unroll
+      for (int i = 0; i < NSEG; ++i) plan[i] = ca.plan[i * CPS + c];
+      co.init(plan);
+#pragma unroll
+      for (int i = 0; i < NSEG; ++i) co.keep_masks(i, km[n][i]);
+    }
+  }
+  const int64_t stride = gridDim.x;
+  int64_t row = blockIdx.x;
+  const uint16_t* r1 = x1 + row * ld1;
+  const uint16_t* r2 = NIN == 2 ? x2 + row * ld2 : nullptr;
+  uint16_t* yp = y + row * H + 8 * c;
+  const int64_t step1 = stride * ld1, step2 = stride * ld2, ystep = stride * H, sstep = stride * SEG, scstep = stride * gpr;
+  int64_t soff = row * SEG + 8 * c, scoff = row * gpr + (c >> shift);
+  uint4 raw[NIN][NSEG];
+  if (row < M) {
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) {
+      raw[0][i] = *reinterpret_cast<const uint4*>(r1 + i * SEG + 8 * c);
+      if (NIN == 2) raw[NIN - 1][i] = *reinterpret_cast<const uint4*>(r2 + i * SEG + 8 * c);
+    }
+  }
+  for (; row < M; row += stride) {
+    uint4 nxt[NIN][NSEG];
+    if (row + stride < M) {
+#pragma unroll
+      for (int i = 0; i < NSEG; ++i) {
+        nxt[0][i] = *reinterpret_cast<const uint4*>(r1 + step1 + i * SEG + 8 * c);
+        if (NIN == 2) nxt[NIN - 1][i] = *reinterpret_cast<const uint4*>(r2 + step2 + i * SEG + 8 * c);
+      }
+    }
+    uint32_t lo[NIN], hi[NIN];
+#pragma unroll
+    for (int n = 0; n < NIN; ++n) { lo[n] = 0; hi[n] = 0; }
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) {
+      float a[8], v[8];
+      unpack8(raw[0][i], a);
+      if (NIN == 2) {
+        unpack8(raw[NIN - 1][i], v);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = a[j] * v[j];
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = act_value<ACT>(a[j]);
+      }
+      store_stream(yp + i * SEG, pack8(v));
+#pragma unroll
+      for (int n = 0; n < NIN; ++n) {
+        const uint4 r = raw[n][i];
+        unpack8(make_uint4(r.x & km[n][i][0], r.y & km[n][i][1], r.z & km[n][i][2], r.w & km[n][i][3]), v);
+        uint32_t cl, ch;
+        const float s = quant_seg<BITS, LPGT>(v, LPGT, cl, ch);
+        if (leader) (n == 0 ? s1.scales : s2.scales)[scoff + i * seg_groups] = f_to_bf(s);
+        if (BITS == 8) { lo[n] = cl; hi[n] = ch; } else { lo[n] |= cl << (i * BITS); hi[n] |= ch << (i * BITS); }
+      }
+    }
+    *reinterpret_cast<uint2*>(s1.stored + soff) = make_uint2(lo[0], hi[0]);
+    if (NIN == 2) *reinterpret_cast<uint2*>(s2.stored + soff) = make_uint2(lo[NIN - 1], hi[NIN - 1]);
+    for (int t = c; t < s1.ca.k; t += CPS) s1.vals[row * s1.ca.k + t] = r1[s1.ca.idx[t]];
+    if (NIN == 2)
+      for (int t = c; t < s2.ca.k; t += CPS) s2.vals[row * s2.ca.k + t] = r2[s2.ca.idx[t]];
+#pragma unroll
+    for (int n = 0; n < NIN; ++n)
+#pragma unroll
+      for (int i = 0; i < NSEG; ++i) raw[n][i] = nxt[n][i];
+    r1 += step1; if (NIN == 2) r2 += step2;
+    yp += ystep; soff += sstep; scoff += scstep;
   }
 }
 
@@ -738,6 +842,74 @@ int hyc_gated_act_fwd(int32_t act, const void* gate, int64_t ld_gate, const void
 #undef HYC_GFWD_T
 #undef HYC_GFWD
   return check_launch("hyc_gated_act_fwd");
+}
+
+// shared host part of hyc_act_fwd_compress (x2 = NULL) and hyc_hadamard_fwd_compress
+static int ew_fwd_impl(const char* who, int32_t act, const void* x1, int64_t ld1, const void* x2, int64_t ld2, int64_t M,
+                       int64_t H, const hyc_desc* d1, const hyc_desc* d2, void* y, void* stored1, void* vals1, void* scales1,
+                       void* stored2, void* vals2, void* scales2, void* stream) {
+  const bool two = d2 != nullptr;
+  if (!d1) return fail(HYC_EFAULT, "%s: null descriptor", who);
+  if (M < 0) return fail(HYC_EINVAL, "%s: M=%lld", who, (long long)M);
+  if (d1->mode != HYC_MODE_CHANNEL || (two && d2->mode != HYC_MODE_CHANNEL))
+    return fail(HYC_ENOTSUP, "%s: channel scheme only", who);
+  if (two && (d1->bits != d2->bits || d1->group != d2->group))
+    return fail(HYC_ENOTSUP, "%s: one code width and one group size for both operands", who);
+  if (ld1 < H || ld1 % 8 != 0 || (two && (ld2 < H || ld2 % 8 != 0)))
+    return fail(HYC_EINVAL, "%s: row pitch (at least H=%lld, a multiple of 8)", who, (long long)H);
+  RowGeom geo;
+  int rc = row_geom(H, d1->bits, &geo);
+  if (rc) return rc;
+  ChanArgs c1 = {}, c2 = {};
+  int lpg = 16;
+  if ((rc = make_chan_args(d1, geo, &c1, &lpg)) || (two && (rc = make_chan_args(d2, geo, &c2, &lpg)))) return rc;
+  // per-thread state grows with segments x operands: two operands of 2-bit codes do not fit the register file
+  if (geo.iters != 1 || d1->bits == 1 || (two && d1->bits == 2) || (lpg != 8 && lpg != 16))
+    return fail(HYC_ENOTSUP, "%s: needs 2-, 4- or 8-bit codes (4 or 8 for two operands), groups of 64 or 128 channels "
+                             "and rows of at most 1024 chunks per segment (use the separate calls otherwise)", who);
+  if (M == 0) return HYC_OK;
+  if (!x1 || !y || !stored1 || !scales1 || (d1->k > 0 && !vals1) ||
+      (two && (!x2 || !stored2 || !scales2 || (d2->k > 0 && !vals2))))
+    return fail(HYC_EFAULT, "%s: null buffer", who);
+  if (!aligned16(x1) || !aligned16(y) || !aligned8(stored1) || (two && (!aligned16(x2) || !aligned8(stored2))))
+    return fail(HYC_EINVAL, "%s: inputs and y must be 16-byte aligned, stored 8-byte", who);
+  const GatedFwdSite s1 = {c1, static_cast<uint8_t*>(stored1), static_cast<uint16_t*>(vals1), static_cast<uint16_t*>(scales1)};
+  const GatedFwdSite s2 = {c2, static_cast<uint8_t*>(stored2), static_cast<uint16_t*>(vals2), static_cast<uint16_t*>(scales2)};
+  const int64_t cap = 256 * (geo.threads >= 512 ? 3 : 8);
+  const int grid = (int)(M < cap ? M : cap);
+  hipStream_t st = begin_launch(stream);
+#define HYC_EW(B_, L_, A_, N_, MT_)                                                                                \
+  hipLaunchKernelGGL((k_ew_fwd_fast<B_, L_, A_, N_, MT_>), dim3(grid), dim3(geo.threads), 0, st,                   \
+                     static_cast<const uint16_t*>(x1), ld1, static_cast<const uint16_t*>(x2), ld2, M, H, geo.cps,  \
+                     s1, s2, static_cast<uint16_t*>(y))
+#define HYC_EW_T(B_, L_, A_, N_) do { if (geo.threads <= 256) HYC_EW(B_, L_, A_, N_, 256); else HYC_EW(B_, L_, A_, N_, 1024); } while (0)
+#define HYC_EW_L(B_, A_, N_) do { if (lpg == 8) HYC_EW_T(B_, 8, A_, N_); else HYC_EW_T(B_, 16, A_, N_); } while (0)
+  if (two) {
+    if (d1->bits == 4) HYC_EW_L(4, ACT_MUL, 2); else HYC_EW_L(8, ACT_MUL, 2);
+  } else if (act == HYC_ACT_SILU) {
+    if (d1->bits == 2) HYC_EW_L(2, HYC_ACT_SILU, 1); else if (d1->bits == 4) HYC_EW_L(4, HYC_ACT_SILU, 1); else HYC_EW_L(8, HYC_ACT_SILU, 1);
+  } else {
+    if (d1->bits == 2) HYC_EW_L(2, HYC_ACT_GELU_TANH, 1); else if (d1->bits == 4) HYC_EW_L(4, HYC_ACT_GELU_TANH, 1); else HYC_EW_L(8, HYC_ACT_GELU_TANH, 1);
+  }
+#undef HYC_EW_L
+#undef HYC_EW_T
+#undef HYC_EW
+  return check_launch(who);
+}
+
+int hyc_act_fwd_compress(int32_t act, const void* x, int64_t ldx, int64_t M, int64_t H, const hyc_desc* d, void* y,
+                         void* stored, void* vals, void* scales, void* stream) {
+  if (act != HYC_ACT_SILU && act != HYC_ACT_GELU_TANH) return fail(HYC_EINVAL, "hyc_act_fwd_compress: act=%d", act);
+  return ew_fwd_impl("hyc_act_fwd_compress", act, x, ldx, nullptr, 0, M, H, d, nullptr, y, stored, vals, scales, nullptr,
+                     nullptr, nullptr, stream);
+}
+
+int hyc_hadamard_fwd_compress(const void* x1, int64_t ld1, const void* x2, int64_t ld2, int64_t M, int64_t H,
+                              const hyc_desc* d1, const hyc_desc* d2, void* y, void* stored1, void* vals1, void* scales1,
+                              void* stored2, void* vals2, void* scales2, void* stream) {
+  if (!d2) return fail(HYC_EFAULT, "hyc_hadamard_fwd_compress: null descriptor");
+  return ew_fwd_impl("hyc_hadamard_fwd_compress", 0, x1, ld1, x2, ld2, M, H, d1, d2, y, stored1, vals1, scales1, stored2,
+                     vals2, scales2, stream);
 }
 
 }  // extern "C"

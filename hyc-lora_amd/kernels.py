@@ -506,6 +506,49 @@ def gated_act_bwd(act, g2d, src_act, src_up, src_gate):
     return d_gate, d_up
 
 
+def _row_kernel_fits(H, bits, group, widths):
+    return bits in widths and group in (64, 128) and H % (64 // bits) == 0 and H * bits // 64 <= 1024
+
+
+def act_fwd_compress_supported(H, bits, group):
+    """shapes the one-pass activation forward covers"""
+    return _row_kernel_fits(H, bits, group, (2, 4, 8))
+
+
+def hadamard_fwd_compress_supported(H, bits1, group1, bits2, group2):
+    return bits1 == bits2 and group1 == group2 and _row_kernel_fits(H, bits1, group1, (4, 8))
+
+
+def act_fwd_compress(act, x2d, plan, bits, group):
+    """y = act(x) (F.silu / F.gelu values) and the compressed x from one read of x -> (y, ChannelCompressed)"""
+    _need_rows(x2d, "x")
+    M, H = x2d.shape
+    c = alloc_channel(M, H, plan, bits, group, x2d.device)
+    d = c.desc()
+    y = torch.empty((M, H), dtype=BF16, device=x2d.device)
+    code = {"silu": _abi.ACT_SILU, "gelu": _abi.ACT_GELU_TANH}[act]
+    check(_abi.load().hyc_act_fwd_compress(code, _p(x2d), x2d.stride(0) if M > 1 else H, M, H, ctypes.byref(d), _p(y),
+                                           _p(c.stored), _p(c.vals), _p(c.scales), _stream()))
+    return y, c
+
+
+def hadamard_fwd_compress(a2d, b2d, plan_a, plan_b, bits, group):
+    """y = a * b and both operands compressed, each read once -> (y, c_a, c_b)"""
+    _need_rows(a2d, "x1")
+    _need_rows(b2d, "x2")
+    if a2d.shape != b2d.shape:
+        raise ValueError("x1 %s and x2 %s differ in shape" % (tuple(a2d.shape), tuple(b2d.shape)))
+    M, H = a2d.shape
+    ca = alloc_channel(M, H, plan_a, bits, group, a2d.device)
+    cb = alloc_channel(M, H, plan_b, bits, group, a2d.device)
+    da, db = ca.desc(), cb.desc()
+    y = torch.empty((M, H), dtype=BF16, device=a2d.device)
+    check(_abi.load().hyc_hadamard_fwd_compress(_p(a2d), a2d.stride(0) if M > 1 else H, _p(b2d), b2d.stride(0) if M > 1 else H,
+                                                M, H, ctypes.byref(da), ctypes.byref(db), _p(y), _p(ca.stored), _p(ca.vals),
+                                                _p(ca.scales), _p(cb.stored), _p(cb.vals), _p(cb.scales), _stream()))
+    return y, ca, cb
+
+
 def gated_act_fwd_supported(H, bits, group):
     """shapes the one-pass forward covers (the rest takes the activation, three compress calls and a product)"""
     return bits in (4, 8) and group in (64, 128) and H * bits // 64 <= 768 and H % (64 // bits) == 0

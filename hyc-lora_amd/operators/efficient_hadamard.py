@@ -41,6 +41,10 @@ class _ChannelHadamardFunc(torch.autograd.Function):
     def forward(ctx, x1, x2, plan1, plan2, bits1, bits2, group):
         a, _ = as_rows(x1)
         b, _ = as_rows(x2)
+        if a.shape == b.shape and K.hadamard_fwd_compress_supported(a.shape[-1], bits1, group, bits2, group):
+            y, c1, c2 = K.hadamard_fwd_compress(a, b, plan1, plan2, bits1, group)      # each operand read once
+            ctx.saved = (c1, c2)
+            return y.view(x1.shape)
         ctx.saved = (K.compress_channel(a, plan1, bits1, group), K.compress_channel(b, plan2, bits2, group))
         return x1 * x2
 

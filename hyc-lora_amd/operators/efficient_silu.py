@@ -54,8 +54,11 @@ class _ChannelActFunc(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, act, plan, bits, group):
         x2, _ = as_rows(x)
-        ctx.saved = K.compress_channel(x2, plan, bits, group)
         ctx.act = act
+        if K.act_fwd_compress_supported(x2.shape[-1], bits, group):
+            y, ctx.saved = K.act_fwd_compress(act, x2, plan, bits, group)      # one read of x
+            return y.view(x.shape)
+        ctx.saved = K.compress_channel(x2, plan, bits, group)
         return F.silu(x) if act == "silu" else F.gelu(x)
 
     @staticmethod

@@ -212,6 +212,20 @@ int hyc_gated_act_fwd(int32_t act, const void* gate, int64_t ld_gate, const void
                       void* scales_a, void* stored_u, void* vals_u, void* scales_u, void* stored_g, void* vals_g,
                       void* scales_g, void* stream);
 
+/* The operators taken one at a time, forward with the save fused in (every operand read once; channel scheme; the same
+ * bytes as the elementwise op followed by hyc_compress_rows):
+ *   hyc_act_fwd_compress       y = act(x) and x compressed (EfficientMemorySiLU / GELU forward, efficient_silu.py:13-40,
+ *                              efficient_gelu.py:13-40; act codes as for hyc_gated_act_fwd); 2-, 4- or 8-bit codes
+ *   hyc_hadamard_fwd_compress  y = x1 * x2 and both operands compressed (EfficientMemoryHadamard forward,
+ *                              efficient_hadamard.py:11-53); one code width (4 or 8 bits) and group size for both
+ * Inputs are bf16 [M, H] with row pitches in elements; groups of 64 or 128 channels, H * bits / 64 <= 1024;
+ * HYC_ENOTSUP otherwise. */
+int hyc_act_fwd_compress(int32_t act, const void* x, int64_t ldx, int64_t M, int64_t H, const hyc_desc* d, void* y,
+                         void* stored, void* vals, void* scales, void* stream);
+int hyc_hadamard_fwd_compress(const void* x1, int64_t ld1, const void* x2, int64_t ld2, int64_t M, int64_t H,
+                              const hyc_desc* d1, const hyc_desc* d2, void* y, void* stored1, void* vals1, void* scales1,
+                              void* stored2, void* vals2, void* scales2, void* stream);
+
 /* ---- softmax -------------------------------------------------------------------------------- */
 /* x bf16 [rows, N] -> y = softmax(x, -1) bf16 and counts[r] = #{j : y[r,j] > bf16(threshold)} (counts may be
  * NULL).  With x == NULL, y is taken as given and only the counts are produced.  For N <= 4096 y may be x itself

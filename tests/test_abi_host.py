@@ -139,6 +139,18 @@ def test_argument_errors_without_a_gpu(abi):
     assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 8192, null, 8192, 4, 4096, D, D, D, null, *nine, null) == abi.EFAULT
     assert lib.hyc_gated_act_fwd(abi.ACT_GELU_TANH, null, 8192, null, 8192, 0, 4096, D, D, D, null, *nine, null) == 0
     assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 65536, null, 65536, 4, 65536, D, D, D, null, *nine, null) == abi.ENOTSUP  # row too long
+    six = [null] * 6
+    assert lib.hyc_act_fwd_compress(9, null, 4096, 4, 4096, D, null, null, null, null, null) == abi.EINVAL
+    assert lib.hyc_act_fwd_compress(abi.ACT_SILU, null, 4096, 4, 4096, None, null, null, null, null, null) == abi.EFAULT
+    assert lib.hyc_act_fwd_compress(abi.ACT_SILU, null, 4096, 4, 4096, ctypes.byref(t), null, null, null, null, null) == abi.ENOTSUP
+    assert lib.hyc_act_fwd_compress(abi.ACT_SILU, null, 4000, 4, 4096, D, null, null, null, null, null) == abi.EINVAL
+    assert lib.hyc_act_fwd_compress(abi.ACT_GELU_TANH, null, 4096, 4, 4096, D, null, null, null, null, null) == abi.EFAULT
+    assert lib.hyc_act_fwd_compress(abi.ACT_GELU_TANH, null, 4096, 0, 4096, D, null, null, null, null, null) == 0
+    assert lib.hyc_hadamard_fwd_compress(null, 4096, null, 4096, 4, 4096, D, None, null, *six, null) == abi.EFAULT
+    assert lib.hyc_hadamard_fwd_compress(null, 4096, null, 4096, 4, 4096, D, ctypes.byref(d2), null, *six, null) == abi.ENOTSUP
+    assert lib.hyc_hadamard_fwd_compress(null, 4096, null, 4096, 4, 4096, d2b, d2b, null, *six, null) == abi.ENOTSUP   # two 2-bit operands
+    assert lib.hyc_hadamard_fwd_compress(null, 4096, null, 4100, 4, 4096, D, D, null, *six, null) == abi.EINVAL
+    assert lib.hyc_hadamard_fwd_compress(null, 4096, null, 4096, 4, 4096, D, D, null, *six, null) == abi.EFAULT
     assert lib.hyc_layernorm_fwd_compress(null, null, null, 0, 1e-5, 4, 4096, None, null, null, null, null, null, null, null, null) == abi.EFAULT
     assert lib.hyc_layernorm_fwd_compress(null, null, null, 7, 1e-5, 4, 4096, D, null, null, null, null, null, null, null, null) == abi.EINVAL
     assert lib.hyc_layernorm_fwd_compress(null, null, null, 0, 1e-5, 4, 4096, D, null, null, null, null, null, null, null, null) == abi.EFAULT

@@ -299,3 +299,40 @@ def test_layernorm_forward_threshold(K, bits, method, rank):
     assert bool(((bf16_ulp_diff(y.cpu(), y_o) <= 1) | (diff <= 2e-3)).all())
     assert torch.equal(c.stored.cpu().reshape(stored.shape), stored)
     assert bits_equal(K.decompress_threshold(c).cpu(), xh)
+
+
+@pytest.mark.parametrize("act,M,H,bits,group,k", [("silu", 333, 11008, 4, 128, 110), ("gelu", 64, 4096, 4, 128, 41),
+                                                  ("silu", 2100, 4096, 2, 64, 41), ("gelu", 40, 512, 8, 64, 5),
+                                                  ("silu", 17, 2048, 2, 128, 300)])
+def test_activation_forward_with_the_save_fused_in(K, act, M, H, bits, group, k):
+    """y = F.silu / F.gelu bit for bit and the compressed x equal to hyc_compress of x; x is a column slice"""
+    gen = torch.Generator().manual_seed(M + H + bits)
+    wide = torch.randn(M, H + 64, generator=gen)
+    wide[:, torch.randperm(H, generator=gen)[:k]] *= 15
+    x = wide.bfloat16().cuda()[:, :H]
+    plan = K.select_channels(K.channel_absmax(x), k)
+    y, c = K.act_fwd_compress(act, x, plan, bits, group)
+    want = torch.nn.functional.silu(x) if act == "silu" else torch.nn.functional.gelu(x)
+    assert bits_equal(y, want)
+    ref = K.compress_channel(x, plan, bits, group)
+    assert torch.equal(c.stored.view(torch.uint8), ref.stored.view(torch.uint8))
+    assert bits_equal(c.scales, ref.scales) and bits_equal(c.vals, ref.vals)
+    assert not K.act_fwd_compress_supported(4096, 1, 128) and not K.act_fwd_compress_supported(4096, 4, 32)
+
+
+@pytest.mark.parametrize("M,H,bits,group,k", [(333, 11008, 4, 128, 110), (2100, 4096, 4, 64, 41), (40, 512, 8, 64, 5),
+                                              (9, 2048, 8, 128, 300)])
+def test_product_forward_with_the_saves_fused_in(K, M, H, bits, group, k):
+    gen = torch.Generator().manual_seed(M + H + bits + 1)
+    both = torch.randn(M, 2 * H, generator=gen)
+    both[:, torch.randperm(2 * H, generator=gen)[:2 * k]] *= 15
+    both = both.bfloat16().cuda()
+    a, b = both[:, :H], both[:, H:]
+    pa, pb = (K.select_channels(K.channel_absmax(t), k) for t in (a, b))
+    y, ca, cb = K.hadamard_fwd_compress(a, b, pa, pb, bits, group)
+    assert bits_equal(y, a * b)
+    for got, t, p in ((ca, a, pa), (cb, b, pb)):
+        ref = K.compress_channel(t, p, bits, group)
+        assert torch.equal(got.stored.view(torch.uint8), ref.stored.view(torch.uint8))
+        assert bits_equal(got.scales, ref.scales) and bits_equal(got.vals, ref.vals)
+    assert not K.hadamard_fwd_compress_supported(4096, 2, 64, 2, 64) and not K.hadamard_fwd_compress_supported(4096, 4, 64, 8, 64)
