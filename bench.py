@@ -164,6 +164,10 @@ def kernel_tour(pkg, torch, reps=5):
             K.gated_act_bwd("silu", g, cs[2], cs[1], cs[0])
             if K.gated_act_fwd_supported(H, bits, G):
                 K.gated_act_fwd("silu", x, up, cs[2].plan, cs[1].plan, cs[0].plan, bits, G)
+            K.act_fwd_compress("silu", x, plan, bits, G)
+            K.act_fwd_compress("gelu", x, plan, bits, G)
+            if K.hadamard_fwd_compress_supported(H, bits, G, bits, G):
+                K.hadamard_fwd_compress(a, up, cs[2].plan, cs[1].plan, bits, G)
             K.gradw_gemm(dy16, cs[0])
             K.gradw_gemm(dyN, cs[0], staged=False)        # x_hat decoded inside the GEMM
             K.gradw_gemm(dyN, cs[0], staged=True)         # x_hat restored once, then the dense form of the kernel
