@@ -188,9 +188,16 @@ class _LoRAProjectionsFunc(torch.autograd.Function):
             dh = torch.addmm(zero, g, B[i], beta=0.0, alpha=s)    # [M, r]
             dhs.append(dh)
             dB.append(torch.addmm(zero, g.t(), ctx.h_all[:, i * r:(i + 1) * r], beta=0.0, alpha=s))
-            dA.append(K.gradw_gemm(dh, ctx.saved_x, out_dtype=A[i].dtype))
+        dh_all = dhs[0] if n == 1 else torch.cat(dhs, dim=1)         # [M, n*r]
+        # dA_i = dh_i^T @ x_hat: the projections of a group read the same saved activation, so their dh go through
+        # the weight-gradient kernel side by side (32 output rows per call, the widest its LoRA-shaped form takes)
+        # and x_hat is decoded once per call instead of once per projection
+        per_call = max(1, 32 // r) * r
+        for c0 in range(0, n * r, per_call):
+            block = K.gradw_gemm(dh_all[:, c0:c0 + per_call], ctx.saved_x, out_dtype=A[0].dtype)
+            dA.extend(block[j:j + r] for j in range(0, block.shape[0], r))
         # dX: all rank-r terms as one thin GEMM, then each base GEMM accumulates onto it in its epilogue
-        dx = (dhs[0] @ A[0]) if n == 1 else (torch.cat(dhs, dim=1) @ torch.cat(list(A), dim=0))
+        dx = dh_all @ (A[0] if n == 1 else torch.cat(list(A), dim=0))
         w_all = K.nf4_dequantize(mod.base_all)
         row = 0
         for i, out in enumerate(mod.out_features):

@@ -589,7 +589,7 @@ def gradw_gemm(dy2d, src, out_dtype=BF16, alpha=1.0, out=None, beta=0.0, staged=
     A compressed src is decoded inside the GEMM.  Every 256 output features decode the same activation tile again, so
     for wide outputs (N_out >= 2048; not a shape LoRA training has) it is cheaper to restore x_hat once into a
     transient matrix and run the same kernel on the dense operand (`staged`; None = by that rule)."""
-    _need(dy2d, BF16, "grad_output")
+    _need_rows(dy2d, "grad_output")                # rows may be a column slice of a wider matrix (pitch = stride(0))
     M, N_out = dy2d.shape
     if staged is None:
         staged = N_out >= STAGED_GRADW_MIN_FEATURES
@@ -606,7 +606,7 @@ def gradw_gemm(dy2d, src, out_dtype=BF16, alpha=1.0, out=None, beta=0.0, staged=
     ws_bytes = lib.hyc_gradw_workspace_bytes(M, N_out, H)
     ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=dy2d.device) if ws_bytes else None
     code = _abi.DTYPE_F32 if out.dtype == torch.float32 else _abi.DTYPE_BF16
-    check(lib.hyc_gradw_gemm(_p(dy2d), dy2d.stride(0), _p(stored), _p(vals), _p(scales), M, N_out, H, ctypes.byref(d),
+    check(lib.hyc_gradw_gemm(_p(dy2d), dy2d.stride(0) if M > 1 else N_out, _p(stored), _p(vals), _p(scales), M, N_out, H, ctypes.byref(d),
                              float(alpha), float(beta), _p(out), code, _p(ws), _stream()))
     return out
 
