@@ -336,3 +336,43 @@ def test_product_forward_with_the_saves_fused_in(K, M, H, bits, group, k):
         assert torch.equal(got.stored.view(torch.uint8), ref.stored.view(torch.uint8))
         assert bits_equal(got.scales, ref.scales) and bits_equal(got.vals, ref.vals)
     assert not K.hadamard_fwd_compress_supported(4096, 2, 64, 2, 64) and not K.hadamard_fwd_compress_supported(4096, 4, 64, 8, 64)
+
+
+def test_rows_beyond_two_gibi_elements(K):
+    """525 288 rows x 4096 channels = 2^31 + 4 M elements (4.3 GB): element offsets no longer fit 32 bits.  Rows are
+    independent, so the last rows (all of them past the 2^31-element mark) are checked against the oracle run on
+    those rows alone: codec, fused RMSNorm forward and backward, SiLU backward."""
+    M, H, k, bits, group = (1 << 31) // 4096 + 1000, 4096, 41, 4, 128
+    gen = torch.Generator(device="cuda").manual_seed(7)
+    x = torch.randn(M, H, generator=gen, device="cuda", dtype=torch.bfloat16)
+    x[:, 5::100] *= 20
+    tail = slice(M - 48, M)
+    xt = x[tail].cpu()
+    w = (1 + 0.1 * torch.randn(H, generator=torch.Generator().manual_seed(1)))
+    plan = K.select_channels(K.channel_absmax(x[:4096].contiguous()), k)
+    idx = plan.idx.cpu().long()
+    y, rstd, c = K.rmsnorm_fwd_compress_channel(x, w.cuda(), 1e-6, plan, bits, group)
+    vals, stored, scales = O.hyc_compress(xt, idx, bits, group)
+    assert torch.equal(c.stored[tail].cpu(), stored) and bits_equal(c.scales[tail].cpu(), scales)
+    assert bits_equal(c.vals[tail].cpu(), vals)
+    y_o, rstd_o = O.rmsnorm_fwd(xt, w, 1e-6)
+    assert bf16_ulp_diff(y[tail].cpu(), y_o).max() <= 1
+    del y
+    c2 = K.compress_channel(x, plan, bits, group)
+    assert torch.equal(c2.stored[tail], c.stored[tail]) and bits_equal(c2.vals[tail], c.vals[tail])
+    del c2
+    xh = K.decompress_channel(c)
+    xh_o = O.hyc_decompress(vals, stored, idx, scales, bits, group)
+    assert bits_equal(xh[tail].cpu(), xh_o)
+    del xh, x
+    dy = torch.zeros(M, H, device="cuda", dtype=torch.bfloat16)
+    dyt = (0.02 * torch.randn(48, H, generator=torch.Generator().manual_seed(2))).bfloat16()
+    dy[tail] = dyt.cuda()
+    dx, dw = K.rmsnorm_bwd(dy, c, w.cuda(), rstd)
+    dx_o, dw_o = O.rmsnorm_bwd(dyt, xh_o, w, rstd_o)            # every other row has dy = 0 and adds nothing to dw
+    assert torch.allclose(dx[tail].cpu().float(), dx_o.float(), rtol=1e-2, atol=1e-3)
+    assert torch.allclose(dw.cpu(), dw_o, rtol=1e-2, atol=1e-3)
+    assert float(dx[:M - 48].abs().max()) == 0.0
+    del dx
+    ds = K.act_bwd("silu", dy, c)
+    assert bits_equal(ds[tail].cpu(), O.silu_bwd(xh_o, dyt))

@@ -792,3 +792,34 @@ def test_flash_attention_module(ops, K, mode, lens, causal):
         mod(xg, cu, max(lens), window_size=(128, 0))
     with pytest.raises(ValueError):
         mod(xg, torch.tensor([0, total + 1], dtype=torch.int32, device="cuda"), total)
+
+
+def test_softmax_rows_beyond_two_gibi_elements(K):
+    """525 288 rows of 4096 probabilities: the last rows sit past the 2^31-element mark; forward, kept set and
+    backward of those rows against the oracle on the rows alone"""
+    rows, N = (1 << 31) // 4096 + 1000, 4096
+    gen = torch.Generator(device="cuda").manual_seed(11)
+    x = torch.randn(rows, N, generator=gen, device="cuda", dtype=torch.bfloat16) * 3
+    tail = slice(rows - 32, rows)
+    xt = x[tail].cpu()
+    thr = 0.004
+    y, sp = K.softmax_fwd(x, thr)
+    del x
+    y_o = torch.softmax(xt, dim=-1)
+    assert bf16_ulp_diff(y[tail].cpu(), y_o).max() <= 1
+    yt = y[tail].cpu()
+    del y
+    ptr = sp.row_ptr[rows - 32:].cpu().long()
+    assert int(ptr[-1]) == sp.cols.numel() and int(ptr[-1]) > (1 << 31) // 4096          # many rows, many entries
+    kept = torch.zeros(32, N, dtype=torch.bfloat16)
+    cols, vals = sp.cols[int(ptr[0]):].cpu().long(), sp.vals[int(ptr[0]):].cpu()
+    for r in range(32):
+        a, b = int(ptr[r] - ptr[0]), int(ptr[r + 1] - ptr[0])
+        kept[r, cols[a:b]] = vals[a:b]
+    assert bits_equal(kept, O.prune_softmax(yt, torch.tensor(thr)))
+    g = torch.zeros(rows, N, device="cuda", dtype=torch.bfloat16)
+    gt = (0.1 * torch.randn(32, N, generator=torch.Generator().manual_seed(3))).bfloat16()
+    g[tail] = gt.cuda()
+    dx = K.softmax_bwd(g, sp)
+    want = O.softmax_bwd(kept.float(), gt.float())
+    assert torch.allclose(dx[tail].cpu().float(), want.float(), rtol=1e-2, atol=1e-4)
