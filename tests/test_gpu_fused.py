@@ -376,3 +376,27 @@ def test_rows_beyond_two_gibi_elements(K):
     del dx
     ds = K.act_bwd("silu", dy, c)
     assert bits_equal(ds[tail].cpu(), O.silu_bwd(xh_o, dyt))
+
+
+def test_empty_batches_pass_through_every_launcher(K):
+    """M = 0: every launcher returns tensors of the right shape without a launch"""
+    H, k = 512, 5
+    e = torch.zeros(0, H, dtype=torch.bfloat16, device="cuda")
+    plan = K.select_channels(torch.zeros(H, device="cuda"), k)
+    w = torch.ones(H, device="cuda")
+    y, rstd, c = K.rmsnorm_fwd_compress_channel(e, w, 1e-6, plan, 4, 128)
+    assert y.shape == (0, H) and rstd.shape == (0,) and c.vals.shape == (0, k)
+    dx, dw = K.rmsnorm_bwd(e, c, w, rstd)
+    assert dx.shape == (0, H) and dw.shape == (H,) and float(dw.abs().max()) == 0.0
+    y, mean, rstd, c = K.layernorm_fwd_compress_channel(e, w, None, 1e-5, plan, 4, 128)
+    assert y.shape == (0, H) and mean.shape == (0,)
+    assert K.act_bwd("silu", e, c).shape == (0, H)
+    assert all(t.shape == (0, H) for t in K.hadamard_bwd(e, c, c))
+    assert all(t.shape == (0, H) for t in K.gated_act_bwd("gelu", e, c, c, c))
+    assert K.gated_act_fwd("silu", e, e, plan, plan, plan, 4, 128)[0].shape == (0, H)
+    assert K.act_fwd_compress("gelu", e, plan, 4, 128)[0].shape == (0, H)
+    assert K.hadamard_fwd_compress(e, e, plan, plan, 4, 128)[0].shape == (0, H)
+    gw = K.gradw_gemm(torch.zeros(0, 16, dtype=torch.bfloat16, device="cuda"), c, out_dtype=torch.float32)
+    assert gw.shape == (16, H) and float(gw.abs().max()) == 0.0
+    p, sp = K.softmax_fwd(e, 0.01)
+    assert p.shape == (0, H) and sp.cols.numel() == 0 and K.softmax_bwd(e, sp).shape == (0, H)
