@@ -173,6 +173,23 @@ def kernel_tour(pkg, torch, reps=5):
             K.gradw_gemm(dyN, cs[0], staged=True)         # x_hat restored once, then the dense form of the kernel
         torch.cuda.synchronize()
         del x, up, a, g, cs
+    # the reference snapshot's own scheme (element threshold, static scale) at config 2's shape: 1 % outlier
+    # elements, INT4, per-token and per-channel scales; consumers take the restored activation
+    M, H, S = 4096, 4096, 1024
+    x = mk(M, H, 20)
+    g = (0.02 * torch.randn(M, H, generator=gen, device="cuda")).bfloat16()
+    w = 1 + 0.1 * torch.randn(H, generator=gen, device="cuda")
+    thr = float(x.float().abs().flatten()[::7].kthvalue(int(M * H / 7 * 0.99)).values)
+    xf = x.float()
+    for scale in (((xf.amax(-1, keepdim=True) - xf.amin(-1, keepdim=True)) / 15)[:S].bfloat16().contiguous(),
+                  ((xf.amax(0, keepdim=True) - xf.amin(0, keepdim=True)) / 15).bfloat16().contiguous()):
+        for _ in range(reps):
+            c = K.compress_threshold(x, S, thr, scale, 4)
+            xh = K.decompress_threshold(c)
+            y, rstd, c2 = K.rmsnorm_fwd_compress_threshold(x, w, 1e-6, S, thr, scale, 4)
+            K.rmsnorm_bwd(g, xh, w, rstd)
+        torch.cuda.synchronize()
+    del x, xf, g, c, c2, xh, y
     # softmax at config 5's shape: probabilities [1, 32, 2048, 2048], 5 % kept
     x = (2.0 * torch.randn(1, 32, 2048, 2048, generator=gen, device="cuda")).bfloat16()
     g = (0.01 * torch.randn(1, 32, 2048, 2048, generator=gen, device="cuda")).bfloat16()

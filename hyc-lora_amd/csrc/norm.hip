@@ -164,7 +164,9 @@ k_rmsnorm_fwd_fast(const uint16_t* __restrict__ x, const void* __restrict__ w, f
 // b*slots + s, + gridDim.x*slots, ...: the rows in flight across the chip are adjacent in memory (rows that are far
 // apart would crowd onto a few memory channels).  Each slot keeps its own dw accumulators; they are added through
 // LDS at the end, in slot order, so a workgroup writes one fp32 partial row.
-template <int BITS, bool WF32, bool QUIRK, int MAXT>
+// DENSE: `stored` is the restored activation itself (bf16 [M, H]; what a threshold-scheme caller hands over after
+// hyc_decompress), read with the chunk mapping of 4-bit codes; nothing is decoded.
+template <int BITS, bool WF32, bool QUIRK, int MAXT, bool DENSE = false>
 __global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(4, 8)))
 k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ stored, const uint16_t* __restrict__ vals,
                    const uint16_t* __restrict__ scales, const void* __restrict__ w, const float* __restrict__ rstd,
@@ -204,7 +206,7 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[i][j] = 0.f;
     if (active) {
-      plan[i] = ca.plan[(seg0 + i) * CPS + c];
+      if (!DENSE) plan[i] = ca.plan[(seg0 + i) * CPS + c];
       if (slot == 0) {
         float wv[8];
         load_w8t<WF32>(w, (int64_t)(seg0 + i) * SEG + 8 * c, wv);
@@ -228,22 +230,30 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
   const char* cq = reinterpret_cast<const char*>(scales) + row * ca.groups_per_row * 2;
 
   uint2 pk = make_uint2(0, 0);
+  uint4 xraw[NSEG];                                                   // DENSE: the activation chunks of this row
   uint4 graw[NSEG];
   uint32_t sc[NSEG];   // one register each: a packed pair would be assembled right after the load and stall on it
   uint32_t o0[NSEG], o1[NSEG];
   float rs = 0.f, mu = 0.f;                                           // mu: LayerNorm's row mean (0 for RMSNorm)
 #pragma unroll
-  for (int i = 0; i < NSEG; ++i) { graw[i] = make_uint4(0, 0, 0, 0); sc[i] = 0; o0[i] = 0; o1[i] = 0; }
+  for (int i = 0; i < NSEG; ++i) {
+    graw[i] = make_uint4(0, 0, 0, 0); xraw[i] = make_uint4(0, 0, 0, 0); sc[i] = 0; o0[i] = 0; o1[i] = 0;
+  }
+  const char* xq = reinterpret_cast<const char*>(stored) + row * H * 2;      // DENSE only
   if (row < M && active) {
-    pk = *reinterpret_cast<const uint2*>(sq + so);
     rs = rstd[row];
     if (mean) mu = mean[row];
 #pragma unroll
-    for (int i = 0; i < NSEG; ++i) {
-      graw[i] = *reinterpret_cast<const uint4*>(gq + i * seg_b + xo);
-      sc[i] = *reinterpret_cast<const uint16_t*>(cq + i * grp_b + go);
+    for (int i = 0; i < NSEG; ++i) graw[i] = *reinterpret_cast<const uint4*>(gq + i * seg_b + xo);
+    if (DENSE) {
+#pragma unroll
+      for (int i = 0; i < NSEG; ++i) xraw[i] = *reinterpret_cast<const uint4*>(xq + i * seg_b + xo);
+    } else {
+      pk = *reinterpret_cast<const uint2*>(sq + so);
+#pragma unroll
+      for (int i = 0; i < NSEG; ++i) sc[i] = *reinterpret_cast<const uint16_t*>(cq + i * grp_b + go);
+      co.request(reinterpret_cast<const uint16_t*>(vq), o0, o1);
     }
-    co.request(reinterpret_cast<const uint16_t*>(vq), o0, o1);
   }
   int parity = 0;
   for (int64_t step = 0; step < steps; ++step, row += stride, parity ^= 1) {
@@ -266,11 +276,15 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
     for (int i = 0; i < NSEG; ++i) {
       float g[8];
       unpack8(graw[i], g);
-      const float sf = bf_to_f((uint16_t)sc[i]);
-      uint4 r = co.splice(i, dequant8<BITS>(pk.x, pk.y, seg0 + i, sf), o0[i], o1[i], sf);
-      if (co.more_pairs)
-        r = splice_more(r, co.more_pairs, ca.plan[(seg0 + i) * CPS + c], reinterpret_cast<const uint16_t*>(vq), valid, sf);
-      unpack8(r, xn[i]);
+      if (DENSE) {
+        unpack8(xraw[i], xn[i]);
+      } else {
+        const float sf = bf_to_f((uint16_t)sc[i]);
+        uint4 r = co.splice(i, dequant8<BITS>(pk.x, pk.y, seg0 + i, sf), o0[i], o1[i], sf);
+        if (co.more_pairs)
+          r = splice_more(r, co.more_pairs, ca.plan[(seg0 + i) * CPS + c], reinterpret_cast<const uint16_t*>(vq), valid, sf);
+        unpack8(r, xn[i]);
+      }
       uint32_t wo = wbase + (uint32_t)(i * 2 * CPS);
       asm volatile("" : "+v"(wo));                                    // re-read per row: do not keep the weights live
       const float4 wa = wl4[wo], wb = wl4[wo + CPS];
@@ -289,10 +303,15 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
     // The compressed row is decoded: its registers take the next row's codes, scales and outliers now (a row's
     // worth of registers less than requesting them at the top; the barrier and the second pass cover the latency).
     if (more) {
-      pk = *reinterpret_cast<const uint2*>(sq + sstep + so);
+      if (DENSE) {
 #pragma unroll
-      for (int i = 0; i < NSEG; ++i) sc[i] = *reinterpret_cast<const uint16_t*>(cq + gstep + i * grp_b + go);
-      co.request(reinterpret_cast<const uint16_t*>(vq + vstep), o0, o1);
+        for (int i = 0; i < NSEG; ++i) xraw[i] = *reinterpret_cast<const uint4*>(xq + xstep + i * seg_b + xo);
+      } else {
+        pk = *reinterpret_cast<const uint2*>(sq + sstep + so);
+#pragma unroll
+        for (int i = 0; i < NSEG; ++i) sc[i] = *reinterpret_cast<const uint16_t*>(cq + gstep + i * grp_b + go);
+        co.request(reinterpret_cast<const uint16_t*>(vq + vstep), o0, o1);
+      }
     }
     // two sums per slot, one barrier
     p1 = wave_sum(p1);
@@ -316,7 +335,7 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
     rs = rs_n; mu = mu_n;
 #pragma unroll
     for (int i = 0; i < NSEG; ++i) graw[i] = g_n[i];
-    gq += xstep; dq += xstep; sq += sstep; vq += vstep; cq += gstep;
+    gq += xstep; dq += xstep; sq += sstep; vq += vstep; cq += gstep; xq += xstep;
   }
   float* pr = dw_partials + (int64_t)blockIdx.x * H + (int64_t)seg0 * SEG + 8 * c;
 #pragma unroll
@@ -783,7 +802,7 @@ int64_t hyc_rmsnorm_bwd_partial_rows(int64_t M, int64_t H, const hyc_desc* d) {
   NormGeom n;
   if (row_geom(H, d->bits, &g) || norm_geom(g.cps, &n)) return 0;
   const BwdShape b = bwd_shape(M, d->bits, g.cps, n);
-  return (d->mode == HYC_MODE_CHANNEL && b.fast_ok) ? b.fast_P : b.P;
+  return ((d->mode == HYC_MODE_CHANNEL || (d->mode == HYC_MODE_DENSE && d->bits == 4)) && b.fast_ok) ? b.fast_P : b.P;
 }
 
 static int norm_fwd_impl(const void* x, const void* w, const void* bias, int32_t w_dtype, float eps, int64_t M, int64_t H,
@@ -904,7 +923,9 @@ static int norm_bwd_impl(const void* dy, const void* stored, const void* vals, c
   hipStream_t st = begin_launch(stream);
   const bool wf32 = w_dtype == HYC_DTYPE_F32;
   const BwdShape b = bwd_shape(M, d->bits, g.cps, n);
-  const bool fast = d->mode == HYC_MODE_CHANNEL && b.fast_ok;
+  // the dense source takes the fast kernel through the chunk mapping of 4-bit codes (two half rows per thread)
+  const bool dense_fast = d->mode == HYC_MODE_DENSE && d->bits == 4 && b.fast_ok;
+  const bool fast = (d->mode == HYC_MODE_CHANNEL && b.fast_ok) || dense_fast;
   const int64_t used_P = fast ? b.fast_P : b.P;
   if (M > 0) {
     if (!dy || !stored || !w || !rstd || !dx || !dw_partials) return fail(HYC_EFAULT, "hyc_rmsnorm_bwd: null buffer");
@@ -937,7 +958,25 @@ static int norm_bwd_impl(const void* dy, const void* stored, const void* vals, c
       default: HYC_BWD_FAST(B_, true, true, 1024); break;                                     \
     }                                                                                         \
   } while (0)
-      if (d->bits == 2) HYC_BWD_FAST_WQ(2);
+      if (dense_fast) {
+#define HYC_BWD_DENSE(W_, Q_, MT_)                                                                                 \
+  hipLaunchKernelGGL((k_rmsnorm_bwd_fast<4, W_, Q_, MT_, true>), dim3((unsigned)b.fast_P), dim3(fthreads), flds, st, gp, \
+                     static_cast<const uint8_t*>(stored), static_cast<const uint16_t*>(vals),                     \
+                     static_cast<const uint16_t*>(scales), w, rstd, mean, M, H, b.fast_T, g.cps, b.fast_slots, ca, \
+                     static_cast<uint16_t*>(dx), dw_partials)
+        switch ((wf32 ? 4 : 0) + (c2_quirk ? 2 : 0) + (fthreads <= 256 ? 0 : 1)) {
+          case 0: HYC_BWD_DENSE(false, false, 256); break;
+          case 1: HYC_BWD_DENSE(false, false, 1024); break;
+          case 2: HYC_BWD_DENSE(false, true, 256); break;
+          case 3: HYC_BWD_DENSE(false, true, 1024); break;
+          case 4: HYC_BWD_DENSE(true, false, 256); break;
+          case 5: HYC_BWD_DENSE(true, false, 1024); break;
+          case 6: HYC_BWD_DENSE(true, true, 256); break;
+          default: HYC_BWD_DENSE(true, true, 1024); break;
+        }
+#undef HYC_BWD_DENSE
+      }
+      else if (d->bits == 2) HYC_BWD_FAST_WQ(2);
       else if (d->bits == 4) HYC_BWD_FAST_WQ(4);
       else HYC_BWD_FAST_WQ(8);
 #undef HYC_BWD_FAST_WQ
