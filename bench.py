@@ -188,6 +188,8 @@ def kernel_tour(pkg, torch, reps=5):
             xh = K.decompress_threshold(c)
             y, rstd, c2 = K.rmsnorm_fwd_compress_threshold(x, w, 1e-6, S, thr, scale, 4)
             K.rmsnorm_bwd(g, xh, w, rstd)
+            K.act_bwd("silu", g, xh)
+            K.hadamard_bwd(g, xh, xh)
         torch.cuda.synchronize()
     del x, xf, g, c, c2, xh, y
     # softmax at config 5's shape: probabilities [1, 32, 2048, 2048], 5 % kept
