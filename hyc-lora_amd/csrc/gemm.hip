@@ -203,19 +203,46 @@ struct DirectArgs {
   float alpha, beta; void* out; int out_f32; float* partial;
 };
 
-struct DirectRegs {          // what one lane loads for one step
-  uint32_t blo[8], bhi[8], sc[8];
+template <int SPT>
+struct DirectRegs {          // what one lane loads for one step: a packed word and SPT group scales per token
+  uint32_t blo[8], bhi[8], sc[SPT][8];
 };
 
-// MAINT: true = a tile of 16 chunks of one segment (128 quantised channels), false = a tile of 16 outlier channels
+// MAINT: true = a tile of LC chunks of SPT segments, decoded from the same packed words (which are then read once
+//        per SPT segments); false = a tile of 16 outlier channels (bf16 values, nothing to decode)
 // NT = 16-row tiles of dY features (N_out <= 16*NT)
-template <int BITS, int NT, bool MAINT>
+// R:  0 = every lane applies its own group scale: x_hat = bf16((code - OFF) * s), LC = 16 chunks per tile.
+//     1, 2 = 1- and 2-bit codes with the scale folded into dY.  code - OFF is one of {-2, -1, 0, 1}, so
+//     x_hat = (code - OFF) * s is exact: nothing is rounded, and dW[n, h] = sum_t (dY[t, n] * s[t]) * (code[t, h] - OFF)
+//     is the same sum whenever all 16 columns of an MFMA lie in ONE scale group.  R lanes share a chunk and take
+//     every R-th byte of its packed word, so a tile is LC = 16/R chunks: group >= 128 channels: R = 1, 64 channels:
+//     R = 2.  (4-bit codes do round x_hat to bf16, which a folded scale cannot reproduce: they keep R = 0.)
+//     The A operand becomes dY * s, exactly, as two bf16 terms hi + lo (the product of two 8-bit significands has 16
+//     bits); the B operand is the integer code - OFF, which needs no arithmetic at all: bf16 has 8 significant bits,
+//     so the bit pattern of 2^BITS with the code in the top mantissa bits IS the number 2^BITS + code.  One byte
+//     permute picks the lane's byte of two tokens' words, one shift and one and-or put the code field of a segment
+//     under that pattern: 1 + 1/(2 SPT) operations per element plus 40 per segment and step for hi and lo (the fma
+//     form takes 3.9 per element).  The surplus 2^BITS + OFF per element is removed at the end through two more MFMAs
+//     per step whose B operand is all ones (sum_t A[n, t] in every column): dW -= (2^BITS + OFF) * that sum.
+//     Products are exact and fp32-accumulated either way; the partial sums are at most 6 times larger than the
+//     result's terms, so nothing is lost to cancellation.
+template <int BITS, int NT, bool MAINT, int SPT, int R>
 __device__ __forceinline__ void gradw_direct_tile(const DirectArgs& A, float* red, int hy, int64_t n0) {
-  constexpr uint32_t MASK = (BITS == 8) ? 0xFFu : Q<BITS>::CODE_MASK;
-  constexpr uint32_t REP = MASK * 0x01010101u;
+  static_assert(R == 0 || (BITS <= 2 && MAINT && (R == 1 || R == 2)), "the folded form serves 1- and 2-bit codes");
+  constexpr bool FOLD = R > 0;
+  constexpr int RR = FOLD ? R : 1;
+  constexpr int LC = 16 / RR;                                                    // chunks per tile
+  constexpr int NJ = 8 / RR;                                                     // MFMAs (16 channels each) per segment
+  constexpr uint32_t CMASK = (BITS == 8) ? 0xFFu : Q<BITS>::CODE_MASK;
+  constexpr uint32_t REP = CMASK * 0x01010101u;
   constexpr float OFFV = (BITS == 8) ? 128.f : (float)Q<BITS>::OFF;
-  constexpr int NB = MAINT ? 8 : 1;                                              // 16-column MFMA tiles per wave
+  constexpr int NB = MAINT ? NJ * SPT : 1;                                       // 16-column MFMA tiles per wave
   constexpr int RP = 17;                                                         // padded pitch of the reduction buffer
+  // folded form: bf16 pattern of 2^BITS, the code field's place under it, what to take off again
+  constexpr int FSH = 7 - (BITS & 7);                                            // code -> top mantissa bits
+  constexpr uint32_t FMAGIC = ((uint32_t)(127 + BITS) << 7) * 0x00010001u;
+  constexpr uint32_t FMASK = ((CMASK << FSH) & 0x7Fu) * 0x00010001u;
+  constexpr float FCORR = (float)(1 << (BITS & 7)) + OFFV;
   const ChanArgs& ca = A.ca;
   const int CPS = A.CPS, c_tiles = A.c_tiles;
   const int64_t ldy = A.ldy, N_out = A.N_out, H = A.H;
@@ -223,8 +250,10 @@ __device__ __forceinline__ void gradw_direct_tile(const DirectArgs& A, float* re
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);                     // uniform: token bases stay scalar
   const int l16 = lane & 15, kq = lane >> 4;                                     // column / token quarter
-  const int seg = MAINT ? hy / c_tiles : 0;
-  const int c = MAINT ? (hy - seg * c_tiles) * 16 + l16 : 0;                     // chunk inside the segment
+  const int sgrp = MAINT ? hy / c_tiles : 0;                                     // group of SPT segments
+  const int seg = sgrp * SPT;                                                    // its first segment
+  const int hsel = l16 / LC;                                                     // which of the R byte subsets (0 when R <= 1)
+  const int c = MAINT ? (hy - sgrp * c_tiles) * LC + (l16 % LC) : 0;             // chunk inside the segment
   const int q = MAINT ? 0 : hy * 16 + l16;                                       // outlier number
   const int shs = (BITS == 8) ? 0 : seg * BITS;
   const int64_t m_begin = (int64_t)blockIdx.z * A.tokens_per_split;
@@ -239,7 +268,9 @@ __device__ __forceinline__ void gradw_direct_tile(const DirectArgs& A, float* re
   const char* asrc = reinterpret_cast<const char*>(A.dy);
   const int cc = c < CPS ? c : CPS - 1, qc = q < ca.k ? q : ca.k - 1;           // clamped: see fetch()
   const uint32_t lane_b = MAINT ? 8u * (uint32_t)cc : 2u * (uint32_t)qc;
-  const uint32_t lane_s = 2u * (uint32_t)((seg * CPS + cc) >> ca.chunk_to_group_shift);
+  uint32_t lane_s[SPT];
+#pragma unroll
+  for (int g = 0; g < SPT; ++g) lane_s[g] = 2u * (uint32_t)(((seg + g) * CPS + cc) >> ca.chunk_to_group_shift);
   uint32_t lane_a[NT], aoff[NT];                                                 // feature 16a + l16, clamped
 #pragma unroll
   for (int a = 0; a < NT; ++a) {
@@ -247,34 +278,64 @@ __device__ __forceinline__ void gradw_direct_tile(const DirectArgs& A, float* re
     aoff[a] = (uint32_t)(8 * kq * dy_b) + lane_a[a];
   }
   const uint32_t boff = (uint32_t)(8 * kq * tok_b) + lane_b;
-  const uint32_t soff = (uint32_t)(8 * kq * sc_b) + lane_s;
+  uint32_t soff[SPT];
+#pragma unroll
+  for (int g = 0; g < SPT; ++g) soff[g] = (uint32_t)(8 * kq * sc_b) + lane_s[g];
+
+  // Where this thread will write at the end; its plan word (outlier mask of the chunk) or outlier channel index is
+  // requested now, so that the load is over long before the write-out needs it.
+  constexpr int COLS = MAINT ? SPT * LC * 8 : 16;                                // channels of the tile
+  static_assert(COLS <= 256, "one thread per channel of the tile");
+  const int mode = A.partial != nullptr ? 0 : (A.out_f32 ? 1 : 2);
+  const bool wo_vec = MAINT && mode == 0;                                        // 4 channels per thread (the workspace is 16-byte aligned)
+  const int wo_col = wo_vec ? (tid % (COLS / 4)) * 4 : tid % COLS;
+  const int wo_tb = MAINT ? (wo_col & 7) : 0, wo_tcl = MAINT ? ((wo_col >> 3) % LC) : 0, wo_tg = MAINT ? wo_col / (8 * LC) : 0;
+  bool wo_in;
+  uint32_t wo_pword = 0;
+  int64_t wo_h;
+  if (MAINT) {
+    const int tc = (hy - sgrp * c_tiles) * LC + wo_tcl;                          // chunk of this thread's channel(s)
+    wo_in = tc < CPS;
+    if (wo_in) wo_pword = ca.plan[(seg + wo_tg) * CPS + tc];
+    wo_h = (int64_t)(seg + wo_tg) * CPS * 8 + 8 * tc + wo_tb;                    // a segment spans CPS*8 channels
+  } else {
+    wo_in = hy * 16 + wo_col < ca.k;
+    wo_h = wo_in ? ca.idx[hy * 16 + wo_col] : 0;
+  }
 
   floatx4_t acc[NT][NB];
+  floatx4_t accs[FOLD ? SPT : 1][NT];                                            // folded form: sum_t A[n, t] per segment
 #pragma unroll
-  for (int a = 0; a < NT; ++a)
+  for (int a = 0; a < NT; ++a) {
 #pragma unroll
     for (int b = 0; b < NB; ++b) acc[a][b] = (floatx4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int g = 0; g < (FOLD ? SPT : 1); ++g) accs[g][a] = (floatx4_t){0.f, 0.f, 0.f, 0.f};
+  }
 
   // Every load is unconditional: lanes past the last chunk / outlier / feature read their neighbour's data (the
   // results are dropped at the write-out), tokens past the end read the last token with a zeroed dY operand.
-  auto fetch = [&](int64_t m0, DirectRegs& R, uint32_t (&ar)[NT][8]) __attribute__((always_inline)) {
+  auto fetch = [&](int64_t m0, DirectRegs<SPT>& Rg, uint32_t (&ar)[NT][8]) __attribute__((always_inline)) {
     const int left = (int)(m_end - m0 < DK ? m_end - m0 : DK);                  // valid tokens of the step
     const char* ab = asrc + m0 * dy_b;
     const char* bb = bsrc + m0 * tok_b;
     const char* sb = ssrc + m0 * sc_b;
     if (left == DK) {                                                            // all steps but the last: scalar base + lane offset
-      uint32_t bo = boff, so = soff, ao[NT];
-      asm volatile("" : "+v"(bo), "+v"(so));                                     // keep them 32-bit values of this block
+      uint32_t bo = boff, so[SPT], ao[NT];
+      asm volatile("" : "+v"(bo));                                               // keep them 32-bit values of this block
+#pragma unroll
+      for (int g = 0; g < SPT; ++g) { so[g] = soff[g]; asm volatile("" : "+v"(so[g])); }
 #pragma unroll
       for (int a = 0; a < NT; ++a) { ao[a] = aoff[a]; asm volatile("" : "+v"(ao[a])); }
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         if (MAINT) {
           const uint2 w = *reinterpret_cast<const uint2*>(bb + bo);
-          R.blo[e] = w.x; R.bhi[e] = w.y;
-          R.sc[e] = *reinterpret_cast<const uint16_t*>(sb + so);
+          Rg.blo[e] = w.x; Rg.bhi[e] = w.y;
+#pragma unroll
+          for (int g = 0; g < SPT; ++g) Rg.sc[g][e] = *reinterpret_cast<const uint16_t*>(sb + so[g]);
         } else {
-          R.blo[e] = *reinterpret_cast<const uint16_t*>(bb + bo);
+          Rg.blo[e] = *reinterpret_cast<const uint16_t*>(bb + bo);
         }
 #pragma unroll
         for (int a = 0; a < NT; ++a) ar[a][e] = *reinterpret_cast<const uint16_t*>(ab + ao[a]);
@@ -287,10 +348,11 @@ __device__ __forceinline__ void gradw_direct_tile(const DirectArgs& A, float* re
         const int tc = t < left ? t : left - 1;
         if (MAINT) {
           const uint2 w = *reinterpret_cast<const uint2*>(bb + tc * tok_b + lane_b);
-          R.blo[e] = w.x; R.bhi[e] = w.y;
-          R.sc[e] = *reinterpret_cast<const uint16_t*>(sb + tc * sc_b + lane_s);
+          Rg.blo[e] = w.x; Rg.bhi[e] = w.y;
+#pragma unroll
+          for (int g = 0; g < SPT; ++g) Rg.sc[g][e] = *reinterpret_cast<const uint16_t*>(sb + tc * sc_b + lane_s[g]);
         } else {
-          R.blo[e] = *reinterpret_cast<const uint16_t*>(bb + tc * tok_b + lane_b);
+          Rg.blo[e] = *reinterpret_cast<const uint16_t*>(bb + tc * tok_b + lane_b);
         }
 #pragma unroll
         for (int a = 0; a < NT; ++a) {
@@ -300,48 +362,135 @@ __device__ __forceinline__ void gradw_direct_tile(const DirectArgs& A, float* re
       }
     }
   };
-  auto step = [&](DirectRegs& R, uint32_t (&ar)[NT][8]) __attribute__((always_inline)) {
-    bf16x8_t bfrag[NB];
-    if (MAINT) {
-      float s[8], ns[8];
+  auto step = [&](DirectRegs<SPT>& Rg, uint32_t (&ar)[NT][8]) __attribute__((always_inline)) {
+    if (FOLD) {
+      uint32_t magic = FMAGIC;
+      asm volatile("" : "+v"(magic));                  // in a vector register, so that (x & mask) | magic is one v_and_or_b32
+      const bf16x8_t ones = __builtin_bit_cast(bf16x8_t, (u32x4_t){0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u});
+      // A operands of segment g: dY * s is a product of two 8-bit significands, so it is exactly hi + lo with
+      // hi = bf16(dY * s) and lo = dY * s - hi, both bf16; their row sums through the all-ones B operand
+      auto make_a = [&](int g, bf16x8_t (&ahi)[NT], bf16x8_t (&alo)[NT]) __attribute__((always_inline)) {
+        float sg[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        s[e] = bf_to_f((uint16_t)R.sc[e]); ns[e] = -OFFV * s[e];
-        // this segment's code of every byte, as a byte
-        R.blo[e] = (BITS == 8) ? R.blo[e] ^ 0x80808080u : (R.blo[e] >> shs) & REP;
-        R.bhi[e] = (BITS == 8) ? R.bhi[e] ^ 0x80808080u : (R.bhi[e] >> shs) & REP;
-      }
+        for (int e = 0; e < 8; ++e) sg[e] = bf_to_f((uint16_t)Rg.sc[g][e]);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        uint32_t wj[4];
+        for (int a = 0; a < NT; ++a) {
+          uint32_t wh[4], wl[4];
 #pragma unroll
-        for (int e = 0; e < 8; e += 2) {
-          float f[2];
-#pragma unroll
-          for (int d = 0; d < 2; ++d) {
-            const uint32_t w = (j < 4) ? R.blo[e + d] : R.bhi[e + d];
-            f[d] = __builtin_fmaf((float)((w >> (8 * (j & 3))) & 0xFFu), s[e + d], ns[e + d]);
+          for (int e = 0; e < 8; e += 2) {
+            const float p0 = __uint_as_float(ar[a][e] << 16) * sg[e], p1 = __uint_as_float(ar[a][e + 1] << 16) * sg[e + 1];
+            wh[e >> 1] = pack_bf16(p0, p1);
+            wl[e >> 1] = pack_bf16(p0 - bf_lo(wh[e >> 1]), p1 - bf_hi(wh[e >> 1]));
           }
-          wj[e >> 1] = pack_bf16(f[0], f[1]);
+          ahi[a] = __builtin_bit_cast(bf16x8_t, (u32x4_t){wh[0], wh[1], wh[2], wh[3]});
+          alo[a] = __builtin_bit_cast(bf16x8_t, (u32x4_t){wl[0], wl[1], wl[2], wl[3]});
+          accs[g][a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ahi[a], ones, accs[g][a], 0, 0, 0);
+          accs[g][a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(alo[a], ones, accs[g][a], 0, 0, 0);
         }
-        bfrag[j] = __builtin_bit_cast(bf16x8_t, (u32x4_t){wj[0], wj[1], wj[2], wj[3]});
+      };
+      // B operands: for byte slot jj of the lane, the raw bytes of two tokens side by side ...
+      auto make_d = [&](int jj, uint32_t (&d)[4]) __attribute__((always_inline)) {
+        const uint32_t sel = 0x0C040C00u + (uint32_t)(RR * (jj % (4 / RR)) + hsel) * 0x00010001u;
+#pragma unroll
+        for (int ep = 0; ep < 4; ++ep) {
+          const uint32_t w0 = (jj < NJ / 2) ? Rg.blo[2 * ep] : Rg.bhi[2 * ep];
+          const uint32_t w1 = (jj < NJ / 2) ? Rg.blo[2 * ep + 1] : Rg.bhi[2 * ep + 1];
+          d[ep] = __builtin_amdgcn_perm(w1, w0, sel);                            // [byte of token 2ep, 0, byte of token 2ep+1, 0]
+          if (SPT != Q<BITS>::NSEG) d[ep] >>= shs;                               // first segment of the tile to bit 0
+        }
+      };
+      // ... then the code field of segment g under the bf16 pattern, and the MFMAs of (g, jj)
+      auto mfmas = [&](int g, int jj, const uint32_t (&d)[4], const bf16x8_t (&ahi)[NT], const bf16x8_t (&alo)[NT])
+                       __attribute__((always_inline)) {
+        const int sh = FSH - g * BITS;                                           // compile-time after unrolling
+        const int shl = sh > 0 ? sh : 0, shr = sh < 0 ? -sh : 0;
+        uint32_t w[4];
+#pragma unroll
+        for (int ep = 0; ep < 4; ++ep) w[ep] = (((d[ep] << shl) >> shr) & FMASK) | magic;
+        const bf16x8_t bf = __builtin_bit_cast(bf16x8_t, (u32x4_t){w[0], w[1], w[2], w[3]});
+#pragma unroll
+        for (int a = 0; a < NT; ++a) {
+          acc[a][g * NJ + jj] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ahi[a], bf, acc[a][g * NJ + jj], 0, 0, 0);
+          acc[a][g * NJ + jj] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(alo[a], bf, acc[a][g * NJ + jj], 0, 0, 0);
+        }
+      };
+      // whichever of the two intermediate sets is smaller stays live across the other loop
+      if (SPT * NT * 8 <= NJ * 4) {
+        bf16x8_t ahi[SPT][NT], alo[SPT][NT];
+#pragma unroll
+        for (int g = 0; g < SPT; ++g) make_a(g, ahi[g], alo[g]);
+#pragma unroll
+        for (int jj = 0; jj < NJ; ++jj) {
+          uint32_t d[4];
+          make_d(jj, d);
+#pragma unroll
+          for (int g = 0; g < SPT; ++g) mfmas(g, jj, d, ahi[g], alo[g]);
+        }
+      } else {
+        uint32_t d[NJ][4];
+#pragma unroll
+        for (int jj = 0; jj < NJ; ++jj) make_d(jj, d[jj]);
+#pragma unroll
+        for (int g = 0; g < SPT; ++g) {
+          bf16x8_t ahi[NT], alo[NT];
+          make_a(g, ahi, alo);
+#pragma unroll
+          for (int jj = 0; jj < NJ; ++jj) mfmas(g, jj, d[jj], ahi, alo);
+        }
+      }
+      return;
+    }
+    bf16x8_t af[NT];
+#pragma unroll
+    for (int a = 0; a < NT; ++a)
+      af[a] = __builtin_bit_cast(bf16x8_t, (u32x4_t){ar[a][0] | (ar[a][1] << 16), ar[a][2] | (ar[a][3] << 16),
+                                                     ar[a][4] | (ar[a][5] << 16), ar[a][6] | (ar[a][7] << 16)});
+    if (MAINT) {
+#pragma unroll
+      for (int g = 0; g < SPT; ++g) {                  // one segment at a time: decode its 8 fragments, then their MFMAs
+        bf16x8_t bfrag[8];
+        float s[8], ns[8];
+        uint32_t clo[8], chi[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          s[e] = bf_to_f((uint16_t)Rg.sc[g][e]); ns[e] = -OFFV * s[e];
+          // segment seg + g's code of every byte, as a byte
+          clo[e] = (BITS == 8) ? Rg.blo[e] ^ 0x80808080u : (Rg.blo[e] >> (shs + g * BITS)) & REP;
+          chi[e] = (BITS == 8) ? Rg.bhi[e] ^ 0x80808080u : (Rg.bhi[e] >> (shs + g * BITS)) & REP;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          uint32_t wj[4];
+#pragma unroll
+          for (int e = 0; e < 8; e += 2) {
+            float f[2];
+#pragma unroll
+            for (int d = 0; d < 2; ++d) {
+              const uint32_t w = (j < 4) ? clo[e + d] : chi[e + d];
+              f[d] = __builtin_fmaf((float)((w >> (8 * (j & 3))) & 0xFFu), s[e + d], ns[e + d]);
+            }
+            wj[e >> 1] = pack_bf16(f[0], f[1]);
+          }
+          bfrag[j] = __builtin_bit_cast(bf16x8_t, (u32x4_t){wj[0], wj[1], wj[2], wj[3]});
+        }
+#pragma unroll
+        for (int a = 0; a < NT; ++a)
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            acc[a][8 * g + j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[a], bfrag[j], acc[a][8 * g + j], 0, 0, 0);
+        if (g + 1 < SPT) __builtin_amdgcn_sched_barrier(0);   // keep the segments apart: decoding both first spills
       }
     } else {
-      bfrag[0] = __builtin_bit_cast(bf16x8_t, (u32x4_t){R.blo[0] | (R.blo[1] << 16), R.blo[2] | (R.blo[3] << 16),
-                                                       R.blo[4] | (R.blo[5] << 16), R.blo[6] | (R.blo[7] << 16)});
-    }
+      const bf16x8_t bfrag = __builtin_bit_cast(bf16x8_t, (u32x4_t){Rg.blo[0] | (Rg.blo[1] << 16), Rg.blo[2] | (Rg.blo[3] << 16),
+                                                                   Rg.blo[4] | (Rg.blo[5] << 16), Rg.blo[6] | (Rg.blo[7] << 16)});
 #pragma unroll
-    for (int a = 0; a < NT; ++a) {
-      const bf16x8_t af = __builtin_bit_cast(bf16x8_t, (u32x4_t){ar[a][0] | (ar[a][1] << 16), ar[a][2] | (ar[a][3] << 16),
-                                                                ar[a][4] | (ar[a][5] << 16), ar[a][6] | (ar[a][7] << 16)});
-#pragma unroll
-      for (int b = 0; b < NB; ++b) acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, bfrag[b], acc[a][b], 0, 0, 0);
+      for (int a = 0; a < NT; ++a) acc[a][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[a], bfrag, acc[a][0], 0, 0, 0);
     }
   };
 
   // wave w takes steps w, w+4, ... of the workgroup's token range; two steps of loads are in flight
   constexpr int64_t WS = 4 * DK;
-  DirectRegs R0, R1;
+  DirectRegs<SPT> R0, R1;
   uint32_t a0[NT][8], a1[NT][8];
   int64_t m0 = m_begin + (int64_t)wave * DK;
   if (m0 < m_end) fetch(m0, R0, a0);
@@ -354,84 +503,142 @@ __device__ __forceinline__ void gradw_direct_tile(const DirectArgs& A, float* re
       if (m0 + 3 * WS < m_end) fetch(m0 + 3 * WS, R1, a1);
     }
   }
+  if (FOLD) {                                                                    // take the 2^BITS + OFF per element off again
+#pragma unroll
+    for (int a = 0; a < NT; ++a)
+#pragma unroll
+      for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) acc[a][b][v] = __builtin_fmaf(-FCORR, accs[b / NJ][a][v], acc[a][b][v]);
+  }
 
-  // ---- the four waves add up in LDS, in wave order; layout [row n][tile b][lane] with a padded pitch ----
+  // ---- the four waves add up in LDS: (wave 0 + wave 2) in one half of `red`, (wave 1 + wave 3) in the other, the
+  // two halves are added by the write-out; layout of a half [row n][tile b][lane] with a padded pitch ----
   // lane holds column (lane mod 16) and rows 4*(lane/16) + v of each 16x16 tile
-  for (int w = 0; w < 4; ++w) {
-    if (wave == w) {
+  constexpr int HALF = 16 * NT * NB * RP;
+  float* mine = red + (wave & 1) * HALF;
+  if (wave < 2) {
 #pragma unroll
-      for (int a = 0; a < NT; ++a)
+    for (int a = 0; a < NT; ++a)
 #pragma unroll
-        for (int b = 0; b < NB; ++b)
+      for (int b = 0; b < NB; ++b)
 #pragma unroll
-          for (int v = 0; v < 4; ++v) {
-            const int n = 16 * a + 4 * kq + v;
-            float* r = &red[(n * NB + b) * RP + l16];
-            *r = (w == 0) ? acc[a][b][v] : *r + acc[a][b][v];
-          }
-    }
-    __syncthreads();
+        for (int v = 0; v < 4; ++v) mine[((16 * a + 4 * kq + v) * NB + b) * RP + l16] = acc[a][b][v];
   }
+  __syncthreads();
+  if (wave >= 2) {
+    // all reads first, then the adds and writes: written as read-add-write per element the compiler keeps them in
+    // program order (it cannot see that the addresses differ) and every element waits out the LDS latency
+#pragma unroll
+    for (int a = 0; a < NT; ++a)
+#pragma unroll
+      for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) acc[a][b][v] += mine[((16 * a + 4 * kq + v) * NB + b) * RP + l16];
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int a = 0; a < NT; ++a)
+#pragma unroll
+      for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) mine[((16 * a + 4 * kq + v) * NB + b) * RP + l16] = acc[a][b][v];
+  }
+  __syncthreads();
   // ---- write-out by all threads, neighbouring threads = neighbouring channels ----
-  constexpr int COLS = 16 * NB;                                                  // channels of the tile
-  const int mode = A.partial != nullptr ? 0 : (A.out_f32 ? 1 : 2);
   const float alpha = A.alpha, beta = A.beta;
-  const int col = tid % COLS, nfirst = tid / COLS;                               // thread's channel, first row
-  constexpr int NSTEP = 256 / COLS;
-  const int tb = MAINT ? (col & 7) : 0, tl = MAINT ? (col >> 3) : col;           // tile (= byte of the word), lane
-  bool keep;
-  int64_t h;
-  if (MAINT) {
-    const int tc = (hy - seg * c_tiles) * 16 + tl;                               // chunk of this thread's channel
-    keep = tc < CPS;
-    const uint32_t pword = keep ? ca.plan[seg * CPS + tc] : 0u;
-    keep = keep && ((pword >> tb) & 1u) == 0;                                    // outlier channels belong to the outlier launch
-    h = (int64_t)seg * CPS * 8 + 8 * tc + tb;                                    // a segment spans CPS*8 channels
-  } else {
-    keep = hy * 16 + col < ca.k;
-    h = keep ? ca.idx[hy * 16 + col] : 0;
+  if (!wo_in) return;
+  // channel = (segment tg of the tile, chunk tcl of the tile, byte tb of the packed word): MFMA tile 8/R*tg + tb/R,
+  // lane (tb mod R) * LC + tcl
+  if (wo_vec) {                                        // partial sums of a main tile: 16-byte stores, 4 channels per thread
+    constexpr int NSTEP4 = 256 / (COLS / 4);
+    int ro[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) ro[i] = (wo_tg * NJ + (wo_tb + i) / RR) * RP + ((wo_tb + i) % RR) * LC + wo_tcl;
+    const uint32_t m4 = (wo_pword >> wo_tb) & 0xFu;    // outlier channels belong to the outlier tiles
+    for (int nl = tid / (COLS / 4); nl < 16 * NT && n0 + nl < N_out; nl += NSTEP4) {
+      float v[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = red[nl * NB * RP + ro[i]] + red[HALF + nl * NB * RP + ro[i]];
+      float* o = A.partial + ((int64_t)blockIdx.z * N_out + n0 + nl) * H + wo_h;
+      if (m4 == 0) {
+        *reinterpret_cast<float4*>(o) = make_float4(v[0], v[1], v[2], v[3]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) if (!((m4 >> i) & 1u)) o[i] = v[i];
+      }
+    }
+    return;
   }
-  if (!keep) return;
-  for (int nl = nfirst; nl < 16 * NT && n0 + nl < N_out; nl += NSTEP) {
-    const float val = red[(nl * NB + tb) * RP + tl];
+  if (MAINT && ((wo_pword >> wo_tb) & 1u)) return;
+  const int rb = MAINT ? wo_tg * NJ + wo_tb / RR : 0, rl = MAINT ? (wo_tb % RR) * LC + wo_tcl : tid % COLS;
+  for (int nl = tid / COLS; nl < 16 * NT && n0 + nl < N_out; nl += 256 / COLS) {
+    const float val = red[(nl * NB + rb) * RP + rl] + red[HALF + (nl * NB + rb) * RP + rl];
     const int64_t n = n0 + nl;
     if (mode == 0) {
-      A.partial[((int64_t)blockIdx.z * N_out + n) * H + h] = val;
+      A.partial[((int64_t)blockIdx.z * N_out + n) * H + wo_h] = val;
     } else if (mode == 1) {
-      float* o = static_cast<float*>(A.out) + n * H + h;
+      float* o = static_cast<float*>(A.out) + n * H + wo_h;
       *o = (beta != 0.f) ? alpha * val + beta * *o : alpha * val;
     } else {
-      uint16_t* o = static_cast<uint16_t*>(A.out) + n * H + h;
+      uint16_t* o = static_cast<uint16_t*>(A.out) + n * H + wo_h;
       *o = f_to_bf((beta != 0.f) ? alpha * val + beta * bf_to_f(*o) : alpha * val);
     }
   }
 }
 
-// one launch: blockIdx.y < NSEG * c_tiles are the tiles of quantised channels, the rest the outlier tiles
+// one launch: blockIdx.y < (NSEG / SPT) * c_tiles are the tiles of quantised channels, the rest the outlier tiles
 // (two waves per SIMD at least: with 256 registers or fewer the accumulators stay in ordinary vector registers)
-template <int BITS, int NT>
+template <int BITS, int NT, int SPT, int R>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) k_gradw_direct(DirectArgs A) {
-  __shared__ float red[16 * NT * 8 * 17];
-  const int main_tiles = Q<BITS>::NSEG * A.c_tiles;
+  static_assert(Q<BITS>::NSEG % SPT == 0, "segments per tile must divide the segments of a packed word");
+  constexpr int NB = (R > 0 ? 8 / R : 8) * SPT;
+  __shared__ float red[2 * 16 * NT * NB * 17];
+  const int main_tiles = (Q<BITS>::NSEG / SPT) * A.c_tiles;
   const int64_t n0 = (int64_t)blockIdx.x * (16 * NT);                            // first feature of the workgroup
-  if ((int)blockIdx.y < main_tiles) gradw_direct_tile<BITS, NT, true>(A, red, (int)blockIdx.y, n0);
-  else gradw_direct_tile<BITS, NT, false>(A, red, (int)blockIdx.y - main_tiles, n0);
+  if ((int)blockIdx.y < main_tiles) gradw_direct_tile<BITS, NT, true, SPT, R>(A, red, (int)blockIdx.y, n0);
+  else gradw_direct_tile<BITS, NT, false, 1, 0>(A, red, (int)blockIdx.y - main_tiles, n0);
 }
 
-// the streaming kernel serves N_out <= DIRECT_MAX_N; its token splits are a function of the shape only
+// How a shape is laid on the kernel: R (see above) from the group width, SPT from the registers the accumulators of
+// NT x SPT x 8/R tiles leave, LC chunks per tile.
+struct DirectPlan { int r, spt, lc; };
+static DirectPlan direct_plan(int bits, int lpg, int64_t N_out) {
+  DirectPlan p;
+  const int nseg = 8 / bits, nt = N_out <= 16 ? 1 : 2;
+  p.r = (bits > 2 || lpg < 8) ? 0 : (lpg >= 16 ? 1 : (nt == 1 ? 2 : 0));
+  p.spt = p.r == 0 ? 1 : (nt == 1 ? 2 : 1);
+  if (p.spt > nseg) p.spt = nseg;
+  p.lc = p.r == 2 ? 8 : 16;
+  return p;
+}
+
+// The streaming kernel serves N_out <= DIRECT_MAX_N.  Token splits: as many as keep the whole grid resident at once
+// (two workgroups per CU, DIRECT_BLOCKS in all).  The kernel is bound by its decode work, so a grid a little over that
+// leaves most of the chip idle during a second round (65 536 x 4096 INT4: 560 workgroups 88 us, 494 workgroups 61 us).
 constexpr int64_t DIRECT_MAX_N = 32;
-#ifndef DIRECT_BLOCKS
-#define DIRECT_BLOCKS 512                                 // workgroups to aim for (tiles x token splits)
-#endif
-static int direct_splits(int64_t M, int64_t N_out, int64_t H) {
-  (void)N_out;
-  const int64_t tiles = (H + 127) / 128;
-  int64_t s = (DIRECT_BLOCKS + tiles - 1) / tiles;
+constexpr int64_t DIRECT_BLOCKS = 512;
+static int direct_splits(int64_t M, int64_t y_tiles) {
+  int64_t s = DIRECT_BLOCKS / (y_tiles > 0 ? y_tiles : 1);
   const int64_t max_by_tokens = (M + 8 * DK - 1) / (8 * DK);      // at least two steps per wave
   if (s > max_by_tokens) s = max_by_tokens;
   if (s < 1) s = 1;
   if (s > 64) s = 64;
   return (int)s;
+}
+static int64_t direct_y_tiles(int64_t H, int bits, int lpg, int k, int64_t N_out) {
+  const DirectPlan p = direct_plan(bits, lpg, N_out);
+  const int64_t cps = (H * bits + 63) / 64;
+  return (8 / bits / p.spt) * ((cps + p.lc - 1) / p.lc) + (k + 15) / 16;
+}
+// the most splits any code width and group width can ask for (the workspace query does not know them)
+static int direct_splits_max(int64_t M, int64_t N_out, int64_t H) {
+  int best = 1;
+  for (int bits = 1; bits <= 8; bits *= 2)
+    for (int lpg = 4; lpg <= 16; lpg *= 2) {
+      const int sp = direct_splits(M, direct_y_tiles(H, bits, lpg, 0, N_out));
+      if (sp > best) best = sp;
+    }
+  return best;
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -820,7 +1027,7 @@ int64_t hyc_gradw_workspace_bytes(int64_t M, int64_t N_out, int64_t H) {
   const int64_t tiles = ((N_out + BN - 1) / BN) * (H / GH);
   int splits = choose_splits(M, tiles);                   // dense source
   if (N_out <= DIRECT_MAX_N) {                            // channel-compressed source, few output rows
-    const int ds = direct_splits(M, N_out, H);
+    const int ds = direct_splits_max(M, N_out, H);
     if (ds > splits) splits = ds;
   }
   return splits > 1 ? (int64_t)splits * N_out * H * 4 : 0;
@@ -856,29 +1063,37 @@ int hyc_gradw_gemm(const void* dy, int64_t ldy, const void* stored, const void* 
   if (chan && N_out <= DIRECT_MAX_N) {
     if (M > 0 && (!dy || !stored || !scales || (d->k > 0 && !vals))) return fail(HYC_EFAULT, "hyc_gradw_gemm: null buffer");
     if (M > 0 && !aligned8(stored)) return fail(HYC_EINVAL, "hyc_gradw_gemm: stored must be 8-byte aligned");
-    const int splits = M > 0 ? direct_splits(M, N_out, H) : 1;
+    const DirectPlan pl = direct_plan(d->bits, lpg, N_out);
+    const int c_tiles = (g.cps + pl.lc - 1) / pl.lc, o_tiles = (d->k + 15) / 16;
+    const int y_tiles = (g.nseg / pl.spt) * c_tiles + o_tiles;
+    const int splits = M > 0 ? direct_splits(M, y_tiles) : 1;
     if (splits > 1 && !workspace) return fail(HYC_EFAULT, "hyc_gradw_gemm: workspace of hyc_gradw_workspace_bytes() bytes required");
+    if (splits > 1 && !aligned16(workspace)) return fail(HYC_EINVAL, "hyc_gradw_gemm: workspace must be 16-byte aligned");
     int64_t tps = (M + splits - 1) / splits;
     tps = ((tps + DK - 1) / DK) * DK;
     if (tps < DK) tps = DK;
     float* partial = splits > 1 ? static_cast<float*>(workspace) : nullptr;
-    const int c_tiles = (g.cps + 15) / 16, o_tiles = (d->k + 15) / 16;
     const int nt = N_out <= 16 ? 1 : 2;
-    const dim3 grid(1, (unsigned)(g.nseg * c_tiles + o_tiles), (unsigned)splits);
+    const dim3 grid(1, (unsigned)y_tiles, (unsigned)splits);
     const int of32 = out_dtype == HYC_DTYPE_F32;
     DirectArgs da = {static_cast<const uint16_t*>(dy), ldy, M, N_out, H, static_cast<const uint8_t*>(stored),
                      static_cast<const uint16_t*>(vals), static_cast<const uint16_t*>(scales), ca, g.cps, c_tiles, tps,
                      alpha, beta, out, of32, partial};
-#define HYC_DIRECT_N(B_, N_) hipLaunchKernelGGL((k_gradw_direct<B_, N_>), grid, dim3(256), 0, st, da)
+#define HYC_DIRECT_K(B_, N_, S_, R_) hipLaunchKernelGGL((k_gradw_direct<B_, N_, S_, R_>), grid, dim3(256), 0, st, da)
 #define HYC_DIRECT(B_)                                                                                 \
-  do { if (nt == 1) HYC_DIRECT_N(B_, 1); else HYC_DIRECT_N(B_, 2); } while (0)
+  do {                                                                                                 \
+    constexpr int NS = 8 / B_;                         /* the SPT of direct_plan() */                  \
+    if (pl.r == 0) { if (nt == 1) HYC_DIRECT_K(B_, 1, 1, 0); else HYC_DIRECT_K(B_, 2, 1, 0); }         \
+    else if (pl.r == 1) { if (nt == 1) HYC_DIRECT_K(B_, 1, (NS < 2 ? NS : 2), 1); else HYC_DIRECT_K(B_, 2, 1, 1); } \
+    else HYC_DIRECT_K(B_, 1, (NS < 2 ? NS : 2), 2);     /* direct_plan() keeps R = 2 to N_out <= 16 */ \
+  } while (0)
     switch (d->bits) {
       case 1: HYC_DIRECT(1); break;
       case 2: HYC_DIRECT(2); break;
-      case 4: HYC_DIRECT(4); break;
-      default: HYC_DIRECT(8); break;
+      case 4: if (nt == 1) HYC_DIRECT_K(4, 1, 1, 0); else HYC_DIRECT_K(4, 2, 1, 0); break;
+      default: if (nt == 1) HYC_DIRECT_K(8, 1, 1, 0); else HYC_DIRECT_K(8, 2, 1, 0); break;
     }
-#undef HYC_DIRECT_N
+#undef HYC_DIRECT_K
 #undef HYC_DIRECT
     if ((rc = check_launch("hyc_gradw_gemm"))) return rc;
     if (splits > 1) {

@@ -249,7 +249,7 @@ int hyc_softmax_dense(int64_t rows, int64_t N, const int32_t* row_ptr, const int
 /* ---- weight gradient ------------------------------------------------------------------------- */
 /* out[n, h] = alpha * sum_m dy[m, n] * x_hat[m, h] + beta * out[n, h]; dy bf16 [M, N_out] with row stride ldy,
  * x_hat dequantised on the fly (channel mode) or read as bf16 (HYC_MODE_DENSE); out [N_out, H] bf16 or fp32.
- * workspace: hyc_gradw_workspace_bytes() bytes of device memory (may be 0 -> NULL). */
+ * workspace: hyc_gradw_workspace_bytes() bytes of device memory, 16-byte aligned (may be 0 -> NULL). */
 int64_t hyc_gradw_workspace_bytes(int64_t M, int64_t N_out, int64_t H);
 int hyc_gradw_gemm(const void* dy, int64_t ldy, const void* stored, const void* vals, const void* scales, int64_t M,
                    int64_t N_out, int64_t H, const hyc_desc* d, float alpha, float beta, void* out, int32_t out_dtype,

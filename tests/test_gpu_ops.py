@@ -51,7 +51,11 @@ def test_gradw_channel(K, bits, group, M, H, N, k):
     assert torch.allclose(got16.float(), want, rtol=1e-2, atol=1e-3 * float(want.abs().max()) + 1e-3)
     if H % 128 == 0:
         dense = K.gradw_gemm(dy.cuda(), xh, out_dtype=torch.float32).cpu()
-        assert torch.allclose(dense, got32, rtol=1e-5, atol=1e-5 * float(want.abs().max()))
+        # The few-row kernel folds the group scale into dY (A = bf16(dY * s), B = the integer codes) when all 16
+        # columns of an MFMA share a scale group: one more bf16 rounding per product than decoding x_hat first.
+        folded = N <= 32 and bits < 8 and (group >= 128 or (group == 64 and N <= 16))
+        tol = 1e-3 if folded else 1e-5
+        assert torch.allclose(dense, got32, rtol=tol, atol=tol * float(want.abs().max()))
         # the staged route (restore once, then the same kernel on the dense operand) is what wide outputs default to
         assert torch.equal(K.gradw_gemm(dy.cuda(), c, out_dtype=torch.float32, staged=True).cpu(), dense)
         assert torch.equal(K.gradw_gemm(dy.cuda(), c, out_dtype=torch.float32).cpu(), dense if N >= 2048 else got32)
