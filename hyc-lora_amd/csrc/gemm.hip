@@ -614,7 +614,7 @@ static DirectPlan direct_plan(int bits, int lpg, int64_t N_out) {
 
 // The streaming kernel serves N_out <= DIRECT_MAX_N.  Token splits: as many as keep the whole grid resident at once
 // (two workgroups per CU, DIRECT_BLOCKS in all).  The kernel is bound by its decode work, so a grid a little over that
-// leaves most of the chip idle during a second round (65 536 x 4096 INT4: 560 workgroups 88 us, 494 workgroups 61 us).
+// leaves most of the chip idle during a second round (65 536 x 4096 INT4: 560 workgroups 88 us, 490 workgroups 65 us).
 constexpr int64_t DIRECT_MAX_N = 32;
 constexpr int64_t DIRECT_BLOCKS = 512;
 static int direct_splits(int64_t M, int64_t y_tiles) {
