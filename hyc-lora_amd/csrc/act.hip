@@ -27,7 +27,7 @@ __device__ __forceinline__ float rcp_pos(float d) {
 __device__ __forceinline__ float sigmoid_f(float x) { return rcp_pos(1.0f + exp_fast(-x)); }
 // tanh: odd polynomial below 0.05 (where 1 - e^{-2|y|} cancels), (1 - e)/(1 + e) above
 __device__ __forceinline__ float tanh_f(float y) {
-  const float a = __builtin_fabsf(y);
+  const float a = __builtin_fminf(__builtin_fabsf(y), 32.0f);   // tanh(32) is 1 in fp32; keeps e^{-2|y|} away from inf * 0
   const float e = exp_fast(-2.0f * a);
   const float big = (1.0f - e) * rcp_pos(1.0f + e);
   const float y2 = a * a;
@@ -38,7 +38,16 @@ __device__ __forceinline__ float tanh_f(float y) {
 }
 
 // two elements at a time: every intermediate is rounded to bf16 where torch rounds it, pairs share the conversion
+// the derivative alone (a bf16 value): what the gradient is multiplied with
+__device__ __forceinline__ void silu_deriv2(float x0, float x1, float& d0, float& d1);
+__device__ __forceinline__ void gelu_tanh_deriv2(float x0, float x1, float& d0, float& d1);
 __device__ __forceinline__ void silu_grad2(float x0, float x1, float g0, float g1, float& o0, float& o1) {
+  float d0, d1;
+  silu_deriv2(x0, x1, d0, d1);
+  o0 = d0 * g0;           // the caller's pack8 performs the last rounding
+  o1 = d1 * g1;
+}
+__device__ __forceinline__ void silu_deriv2(float x0, float x1, float& d0, float& d1) {
   float s0 = sigmoid_f(x0), s1 = sigmoid_f(x1);
   bfr2(s0, s1);
   float a0 = x0 + 1.0f, a1 = x1 + 1.0f;
@@ -47,13 +56,17 @@ __device__ __forceinline__ void silu_grad2(float x0, float x1, float g0, float g
   bfr2(b0, b1);
   float c0 = a0 - b0, c1 = a1 - b1;
   bfr2(c0, c1);
-  float d0 = s0 * c0, d1 = s1 * c1;
+  d0 = s0 * c0; d1 = s1 * c1;
   bfr2(d0, d1);
-  o0 = d0 * g0;           // the caller's pack8 performs the last rounding
-  o1 = d1 * g1;
 }
 
 __device__ __forceinline__ void gelu_tanh_grad2(float x0, float x1, float g0, float g1, float& o0, float& o1) {
+  float d0, d1;
+  gelu_tanh_deriv2(x0, x1, d0, d1);
+  o0 = d0 * g0;
+  o1 = d1 * g1;
+}
+__device__ __forceinline__ void gelu_tanh_deriv2(float x0, float x1, float& d0, float& d1) {
   const float gamma = 0.7978845608028654f;   // sqrt(2/pi)
   const float kappa = 0.044715f;
   const float kappa3 = (float)(3 * 0.044715);
@@ -87,9 +100,7 @@ __device__ __forceinline__ void gelu_tanh_grad2(float x0, float x1, float g0, fl
   bfr2(G0, G1);
   float H0 = A0 + G0, H1 = A1 + G1;
   bfr2(H0, H1);
-  float I0 = 0.5f * H0, I1 = 0.5f * H1;                  // exact
-  o0 = I0 * g0;
-  o1 = I1 * g1;
+  d0 = 0.5f * H0; d1 = 0.5f * H1;                        // exact
 }
 
 template <int ACT>
@@ -102,13 +113,58 @@ __device__ __forceinline__ void act_grad8(const float (&x)[8], const float (&g)[
   }
 }
 
+// The derivative is a function of one bf16 value, and the reference rounds every step of it to bf16, so a table
+// of it is exact by construction.  LUT_EXP binades from 2^LUT_LOG_LO up, both signs; smaller magnitudes (zero
+// included) share the first entry (the derivative is the constant 0.5 there), larger ones are computed.
+constexpr int LUT_LOG_LO = -12, LUT_EXP = 20;
+constexpr uint32_t LUT_LO = (uint32_t)(127 + LUT_LOG_LO) << 7;
+constexpr uint32_t LUT_N = LUT_EXP * 128;              // entries per sign
+constexpr uint32_t LUT_NEG = 4096;                     // first entry of the negative half
+static_assert(LUT_N <= LUT_NEG, "the sign bit is or-ed into the index");
+
+template <int ACT>
+__device__ __forceinline__ void lut_fill(uint16_t* lut) {
+  for (uint32_t i = 2 * threadIdx.x; i < 2 * LUT_N; i += 2 * blockDim.x) {
+    const uint32_t neg = i >= LUT_N ? 1u : 0u, u = i - neg * LUT_N;
+    const float x0 = __uint_as_float(((neg << 15) | (LUT_LO + u)) << 16), x1 = __uint_as_float(((neg << 15) | (LUT_LO + u + 1)) << 16);
+    float d0, d1;
+    if (ACT == HYC_ACT_SILU) silu_deriv2(x0, x1, d0, d1); else gelu_tanh_deriv2(x0, x1, d0, d1);
+    lut[neg * LUT_NEG + u] = (uint16_t)(__float_as_uint(d0) >> 16);
+    lut[neg * LUT_NEG + u + 1] = (uint16_t)(__float_as_uint(d1) >> 16);
+  }
+}
+// dx of one chunk through the table; false (nothing written) if a lane of the wave holds a value beyond the table
+__device__ __forceinline__ bool lut_grad8(const uint16_t* lut, const uint4& xr, const float (&g)[8], float (&o)[8]) {
+  const uint32_t w[4] = {xr.x, xr.y, xr.z, xr.w};
+  uint32_t idx[8], worst = 0;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const uint32_t e0 = w[j] & 0x7FFFu, e1 = (w[j] >> 16) & 0x7FFFu;
+    const uint32_t u0 = e0 > LUT_LO ? e0 - LUT_LO : 0u, u1 = e1 > LUT_LO ? e1 - LUT_LO : 0u;
+    worst = worst > u0 ? worst : u0;
+    worst = worst > u1 ? worst : u1;
+    idx[2 * j] = ((w[j] >> 3) & LUT_NEG) | u0;
+    idx[2 * j + 1] = ((w[j] >> 19) & LUT_NEG) | u1;
+  }
+  if (__builtin_amdgcn_ballot_w64(worst >= LUT_N) != 0) return false;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) o[j] = __uint_as_float((uint32_t)lut[idx[j]] << 16) * g[j];
+  return true;
+}
+
 // fast path: channel source, every lane owns one chunk per segment, next row requested ahead
 template <int BITS, int ACT, int MAXT>
 __global__ void __launch_bounds__(MAXT)
 k_act_bwd_fast(const uint16_t* __restrict__ g, const uint8_t* __restrict__ stored, const uint16_t* __restrict__ vals,
                const uint16_t* __restrict__ scales, int64_t M, int64_t H, int CPS, ChanArgs ca,
-               uint16_t* __restrict__ dx) {
+               uint16_t* __restrict__ dx, int use_lut) {
   constexpr int NSEG = Q<BITS>::NSEG;
+  constexpr bool HAS_LUT = ACT == HYC_ACT_SILU || ACT == HYC_ACT_GELU_TANH;
+  __shared__ uint16_t lut[HAS_LUT ? LUT_NEG + LUT_N : 1];
+  if (HAS_LUT && use_lut) {
+    lut_fill<ACT>(lut);
+    __syncthreads();
+  }
   const int c = threadIdx.x;
   if (c >= CPS) return;                                 // tail of the last wave
   const int64_t SEG = (int64_t)CPS * 8;
@@ -155,9 +211,11 @@ k_act_bwd_fast(const uint16_t* __restrict__ g, const uint8_t* __restrict__ store
       const float sf = bf_to_f((uint16_t)sc[i]);
       uint4 r = co.splice(i, dequant8<BITS>(pk.x, pk.y, i, sf), o0[i], o1[i], sf);
       if (co.more_pairs) r = splice_more(r, co.more_pairs, ca.plan[i * CPS + c], vp, true, sf);
-      unpack8(r, xv);
       unpack8(graw[i], gv);
-      act_grad8<ACT>(xv, gv, o);
+      if (!(HAS_LUT && use_lut && lut_grad8(lut, r, gv, o))) {
+        unpack8(r, xv);
+        act_grad8<ACT>(xv, gv, o);
+      }
       store_stream(dxp + i * SEG, pack8(o));
     }
     pk = pk_n;
@@ -641,13 +699,16 @@ static int launch_act(const void* g, const void* stored, const void* vals, const
       hipLaunchKernelGGL((k_act_bwd_fast<B_, ACT, 256>), dim3(grid), dim3(geo.threads), 0, st,                 \
                          static_cast<const uint16_t*>(g), static_cast<const uint8_t*>(stored),                 \
                          static_cast<const uint16_t*>(vals), static_cast<const uint16_t*>(scales), M, H, geo.cps, ca, \
-                         static_cast<uint16_t*>(dx));                                                          \
+                         static_cast<uint16_t*>(dx), use_lut);                                                 \
     else                                                                                                       \
       hipLaunchKernelGGL((k_act_bwd_fast<B_, ACT, 1024>), dim3(grid), dim3(geo.threads), 0, st,                \
                          static_cast<const uint16_t*>(g), static_cast<const uint8_t*>(stored),                 \
                          static_cast<const uint16_t*>(vals), static_cast<const uint16_t*>(scales), M, H, geo.cps, ca, \
-                         static_cast<uint16_t*>(dx));                                                          \
+                         static_cast<uint16_t*>(dx), use_lut);                                                 \
   } while (0)
+    // the derivative table costs a workgroup 2 LUT_N evaluations and saves four fifths of one per element
+    const int64_t rows_per_wg = (M + grid - 1) / grid;
+    const int use_lut = rows_per_wg * geo.threads * 16 * 4 >= (int64_t)2 * LUT_N * 5;
     if (d->bits == 2) HYC_ACT_FAST(2);
     else if (d->bits == 4) HYC_ACT_FAST(4);
     else HYC_ACT_FAST(8);

@@ -828,3 +828,30 @@ def test_softmax_rows_beyond_two_gibi_elements(K):
     dx = K.softmax_bwd(g, sp)
     want = O.softmax_bwd(kept.float(), gt.float())
     assert torch.allclose(dx[tail].cpu().float(), want.float(), rtol=1e-2, atol=1e-4)
+
+
+@pytest.mark.parametrize("act", ["silu", "gelu"])
+def test_act_bwd_every_bf16_value(K, act):
+    """the backward kernels look the derivative up in a table once a workgroup has enough rows to pay for building it
+    (values beyond the table are computed): every bf16 pattern as the restored activation, against the oracle.  All
+    channels are outlier channels here, so x_hat is x itself."""
+    H = 4096
+    pat = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16).view(-1, H)      # 16 rows
+    x = pat.repeat(512, 1).cuda()                                                                      # 8192 rows
+    gen = torch.Generator().manual_seed(5)
+    g16 = (0.5 + torch.rand(16, H, generator=gen)).bfloat16()
+    g = g16.repeat(512, 1).cuda()
+    plan = K.select_channels(torch.ones(H, device="cuda"), H)
+    c = K.compress_channel(x, plan, 4, 128)
+    xh = K.decompress_channel(c)[:16].cpu()                 # x itself, except that -0 comes back as (-0) + (+0) = +0
+    assert int((xh.view(torch.int16) != pat.view(torch.int16)).sum()) == 1
+    dx = K.act_bwd(act, g, c).cpu()
+    want = (O.silu_bwd if act == "silu" else O.gelu_bwd)(xh, g16)
+    same = (torch.isnan(want) & torch.isnan(dx[:16])) | (dx[:16].view(torch.int16) == want.view(torch.int16))
+    # sigmoid(-88) is a subnormal fp32 number on the CPU and zero from the GPU's reciprocal: three inputs, |dx| < 1e-36
+    same |= (want.float().abs() < 1e-30) & (dx[:16].float().abs() < 1e-30)
+    assert bool(same.all()), [hex(int(b) & 0xFFFF) for b in pat.view(torch.int16)[~same][:8]]
+    rep = dx.view(512, 16, H).view(torch.int16)
+    assert torch.equal(rep, rep[:1].expand_as(rep))
+    few = K.act_bwd(act, g[:16].contiguous(), K.compress_channel(x[:16].contiguous(), plan, 4, 128)).cpu()   # one row per workgroup: no table
+    assert torch.equal(few.view(torch.int16), dx[:16].view(torch.int16))
