@@ -122,6 +122,12 @@ constexpr uint32_t LUT_N = LUT_EXP * 128;              // entries per sign
 constexpr uint32_t LUT_NEG = 4096;                     // first entry of the negative half
 static_assert(LUT_N <= LUT_NEG, "the sign bit is or-ed into the index");
 
+// the table costs a workgroup 2 LUT_N evaluations and saves about four fifths of one per element (16 per thread and row)
+static inline int lut_pays(int64_t M, int grid, int threads) {
+  const int64_t rows_per_wg = (M + grid - 1) / grid;
+  return rows_per_wg * threads * 16 * 4 >= (int64_t)2 * LUT_N * 5;
+}
+
 template <int ACT>
 __device__ __forceinline__ void lut_fill(uint16_t* lut) {
   for (uint32_t i = 2 * threadIdx.x; i < 2 * LUT_N; i += 2 * blockDim.x) {
@@ -370,8 +376,14 @@ k_gated_act_bwd_fast(const uint16_t* __restrict__ g, const uint8_t* __restrict__
                      const uint16_t* __restrict__ s_a, ChanArgs c_a, const uint8_t* __restrict__ st_u,
                      const uint16_t* __restrict__ v_u, const uint16_t* __restrict__ s_u, ChanArgs c_u,
                      const uint8_t* __restrict__ st_g, const uint16_t* __restrict__ v_g, const uint16_t* __restrict__ s_g,
-                     ChanArgs c_g, int64_t M, int64_t H, int CPS, uint16_t* __restrict__ d_gate, uint16_t* __restrict__ d_up) {
+                     ChanArgs c_g, int64_t M, int64_t H, int CPS, uint16_t* __restrict__ d_gate, uint16_t* __restrict__ d_up,
+                     int use_lut) {
   constexpr int NSEG = Q<BITS>::NSEG;
+  __shared__ uint16_t lut[LUT_NEG + LUT_N];             // the activation's derivative, see lut_fill
+  if (use_lut) {
+    lut_fill<ACT>(lut);
+    __syncthreads();
+  }
   const int c = threadIdx.x;
   if (c >= CPS) return;                                 // tail of the last wave
   const int64_t SEG = (int64_t)CPS * 8;
@@ -410,7 +422,7 @@ k_gated_act_bwd_fast(const uint16_t* __restrict__ g, const uint8_t* __restrict__
       for (int j = 0; j < 8; ++j) { r[j] = xa[j] * gv[j]; t[j] = gv[j] * xu[j]; }
       store_stream(dup + i * SEG, pack8(r));
       unpack8(pack8(t), t);                             // the gradient of act(gate), rounded to bf16 as a tensor would be
-      act_grad8<ACT>(xg, t, r);
+      if (!(use_lut && lut_grad8(lut, pack8(xg), t, r))) act_grad8<ACT>(xg, t, r);
       store_stream(dgp + i * SEG, pack8(r));
     }
 #pragma unroll
@@ -438,6 +450,35 @@ __device__ __forceinline__ float act_value(float x) {
   return (x * 0.5f) * (1.0f + erff(x * 0.70710678118654752440f));
 }
 
+// The forward value is a function of one bf16 input as well: the same table layout, filled with bf16(act(x)).
+// Nothing is shared below the table here (act(x) ~ x/2 near zero): such inputs, zero included, are computed.
+template <int ACT>
+__device__ __forceinline__ void lut_fill_value(uint16_t* lut) {
+  for (uint32_t i = threadIdx.x; i < 2 * LUT_N; i += blockDim.x) {
+    const uint32_t neg = i >= LUT_N ? 1u : 0u, u = i - neg * LUT_N;
+    lut[neg * LUT_NEG + u] = f_to_bf(act_value<ACT>(__uint_as_float(((neg << 15) | (LUT_LO + u)) << 16)));
+  }
+}
+// bf16(act(x)) of one chunk through the table; false (nothing written) if a lane of the wave holds a value outside it
+__device__ __forceinline__ bool lut_value8(const uint16_t* lut, const uint4& xr, uint4& out) {
+  const uint32_t w[4] = {xr.x, xr.y, xr.z, xr.w};
+  uint32_t idx[8], worst = 0;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const uint32_t u0 = (w[j] & 0x7FFFu) - LUT_LO, u1 = ((w[j] >> 16) & 0x7FFFu) - LUT_LO;     // wraps below the table
+    worst = worst > u0 ? worst : u0;
+    worst = worst > u1 ? worst : u1;
+    idx[2 * j] = ((w[j] >> 3) & LUT_NEG) | u0;
+    idx[2 * j + 1] = ((w[j] >> 19) & LUT_NEG) | u1;
+  }
+  if (__builtin_amdgcn_ballot_w64(worst >= LUT_N) != 0) return false;
+  out.x = (uint32_t)lut[idx[0]] | ((uint32_t)lut[idx[1]] << 16);
+  out.y = (uint32_t)lut[idx[2]] | ((uint32_t)lut[idx[3]] << 16);
+  out.z = (uint32_t)lut[idx[4]] | ((uint32_t)lut[idx[5]] << 16);
+  out.w = (uint32_t)lut[idx[6]] | ((uint32_t)lut[idx[7]] << 16);
+  return true;
+}
+
 struct GatedFwdSite {       // one compressed output
   ChanArgs ca;
   uint8_t* stored;
@@ -451,8 +492,14 @@ struct GatedFwdSite {       // one compressed output
 template <int BITS, int LPGT, int ACT, int MAXT>
 __global__ void __launch_bounds__(MAXT)
 k_gated_act_fwd_fast(const uint16_t* __restrict__ gate, int64_t ldg, const uint16_t* __restrict__ up, int64_t ldu, int64_t M,
-                     int64_t H, int CPS, GatedFwdSite sa, GatedFwdSite su, GatedFwdSite sg, uint16_t* __restrict__ h) {
+                     int64_t H, int CPS, GatedFwdSite sa, GatedFwdSite su, GatedFwdSite sg, uint16_t* __restrict__ h,
+                     int use_lut) {
   constexpr int NSEG = Q<BITS>::NSEG;
+  __shared__ uint16_t lut[LUT_NEG + LUT_N];
+  if (use_lut) {
+    lut_fill_value<ACT>(lut);
+    __syncthreads();
+  }
   const int c = threadIdx.x;
   if (c >= CPS) return;                                 // tail of the last wave; scale groups never straddle it
   const int64_t SEG = (int64_t)CPS * 8;
@@ -508,11 +555,14 @@ k_gated_act_fwd_fast(const uint16_t* __restrict__ gate, int64_t ldg, const uint1
 #pragma unroll
     for (int i = 0; i < NSEG; ++i) {
       float gv[8], uv[8], av[8], v[8];
-      unpack8(graw[i], gv);
       unpack8(uraw[i], uv);
+      uint4 araw;                                       // act(gate) as the bf16 tensor the framework would hold
+      if (!(use_lut && lut_value8(lut, graw[i], araw))) {
+        unpack8(graw[i], gv);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) av[j] = act_value<ACT>(gv[j]);
-      const uint4 araw = pack8(av);                     // act(gate) as the bf16 tensor the framework would hold
+        for (int j = 0; j < 8; ++j) av[j] = act_value<ACT>(gv[j]);
+        araw = pack8(av);
+      }
       unpack8(araw, av);
 #pragma unroll
       for (int j = 0; j < 8; ++j) v[j] = av[j] * uv[j];
@@ -552,8 +602,14 @@ k_gated_act_fwd_fast(const uint16_t* __restrict__ gate, int64_t ldg, const uint1
 template <int BITS, int LPGT, int ACT, int NIN, int MAXT>
 __global__ void __launch_bounds__(MAXT)
 k_ew_fwd_fast(const uint16_t* __restrict__ x1, int64_t ld1, const uint16_t* __restrict__ x2, int64_t ld2, int64_t M, int64_t H,
-              int CPS, GatedFwdSite s1, GatedFwdSite s2, uint16_t* __restrict__ y) {
+              int CPS, GatedFwdSite s1, GatedFwdSite s2, uint16_t* __restrict__ y, int use_lut) {
   constexpr int NSEG = Q<BITS>::NSEG;
+  constexpr bool HAS_LUT = NIN == 1;
+  __shared__ uint16_t lut[HAS_LUT ? LUT_NEG + LUT_N : 1];
+  if (HAS_LUT && use_lut) {
+    lut_fill_value<ACT == ACT_MUL ? HYC_ACT_SILU : ACT>(lut);
+    __syncthreads();
+  }
   const int c = threadIdx.x;
   if (c >= CPS) return;                                 // tail of the last wave; scale groups never straddle it
   const int64_t SEG = (int64_t)CPS * 8;
@@ -605,16 +661,20 @@ k_ew_fwd_fast(const uint16_t* __restrict__ x1, int64_t ld1, const uint16_t* __re
 #pragma unroll
     for (int i = 0; i < NSEG; ++i) {
       float a[8], v[8];
-      unpack8(raw[0][i], a);
+      uint4 yraw;
       if (NIN == 2) {
+        unpack8(raw[0][i], a);
         unpack8(raw[NIN - 1][i], v);
 #pragma unroll
         for (int j = 0; j < 8; ++j) v[j] = a[j] * v[j];
-      } else {
+        yraw = pack8(v);
+      } else if (!(use_lut && lut_value8(lut, raw[0][i], yraw))) {
+        unpack8(raw[0][i], a);
 #pragma unroll
         for (int j = 0; j < 8; ++j) v[j] = act_value<ACT>(a[j]);
+        yraw = pack8(v);
       }
-      store_stream(yp + i * SEG, pack8(v));
+      store_stream(yp + i * SEG, yraw);
 #pragma unroll
       for (int n = 0; n < NIN; ++n) {
         const uint4 r = raw[n][i];
@@ -706,9 +766,7 @@ static int launch_act(const void* g, const void* stored, const void* vals, const
                          static_cast<const uint16_t*>(vals), static_cast<const uint16_t*>(scales), M, H, geo.cps, ca, \
                          static_cast<uint16_t*>(dx), use_lut);                                                 \
   } while (0)
-    // the derivative table costs a workgroup 2 LUT_N evaluations and saves four fifths of one per element
-    const int64_t rows_per_wg = (M + grid - 1) / grid;
-    const int use_lut = rows_per_wg * geo.threads * 16 * 4 >= (int64_t)2 * LUT_N * 5;
+    const int use_lut = lut_pays(M, grid, geo.threads);
     if (d->bits == 2) HYC_ACT_FAST(2);
     else if (d->bits == 4) HYC_ACT_FAST(4);
     else HYC_ACT_FAST(8);
@@ -822,6 +880,7 @@ int hyc_gated_act_bwd(int32_t act, const void* g, const void* stored_a, const vo
   const int64_t cap = 256 * (geo.threads >= 512 ? 3 : 8);
   const int grid = (int)(M < cap ? M : cap);
   hipStream_t st = begin_launch(stream);
+  const int use_lut = lut_pays(M, grid, geo.threads);
 #define HYC_GATED(B_, A_, MT_)                                                                                     \
   hipLaunchKernelGGL((k_gated_act_bwd_fast<B_, A_, MT_>), dim3(grid), dim3(geo.threads), 0, st,                    \
                      static_cast<const uint16_t*>(g), static_cast<const uint8_t*>(stored_a),                       \
@@ -829,7 +888,7 @@ int hyc_gated_act_bwd(int32_t act, const void* g, const void* stored_a, const vo
                      static_cast<const uint8_t*>(stored_u), static_cast<const uint16_t*>(vals_u),                  \
                      static_cast<const uint16_t*>(scales_u), c_u, static_cast<const uint8_t*>(stored_g),           \
                      static_cast<const uint16_t*>(vals_g), static_cast<const uint16_t*>(scales_g), c_g, M, H,      \
-                     geo.cps, static_cast<uint16_t*>(d_gate), static_cast<uint16_t*>(d_up))
+                     geo.cps, static_cast<uint16_t*>(d_gate), static_cast<uint16_t*>(d_up), use_lut)
 #define HYC_GATED_T(B_, A_)                                                       \
   do {                                                                            \
     if (geo.threads <= 256) HYC_GATED(B_, A_, 256);                               \
@@ -886,10 +945,11 @@ int hyc_gated_act_fwd(int32_t act, const void* gate, int64_t ld_gate, const void
   const int64_t cap = 256 * (geo.threads >= 512 ? 3 : 8);
   const int grid = (int)(M < cap ? M : cap);
   hipStream_t st = begin_launch(stream);
+  const int use_lut = lut_pays(M, grid, geo.threads);
 #define HYC_GFWD(B_, L_, A_, MT_)                                                                                  \
   hipLaunchKernelGGL((k_gated_act_fwd_fast<B_, L_, A_, MT_>), dim3(grid), dim3(geo.threads), 0, st,                \
                      static_cast<const uint16_t*>(gate), ld_gate, static_cast<const uint16_t*>(up), ld_up, M, H,   \
-                     geo.cps, sa, su, sg, static_cast<uint16_t*>(h))
+                     geo.cps, sa, su, sg, static_cast<uint16_t*>(h), use_lut)
 #define HYC_GFWD_T(B_, L_, A_) /* H = 11008: 704 threads, up to 168 registers each */ \
   do { if (geo.threads <= 256) HYC_GFWD(B_, L_, A_, 256); else HYC_GFWD(B_, L_, A_, 768); } while (0)
 #define HYC_GFWD_L(B_, A_) do { if (lpg == 8) HYC_GFWD_T(B_, 8, A_); else HYC_GFWD_T(B_, 16, A_); } while (0)
@@ -939,10 +999,11 @@ static int ew_fwd_impl(const char* who, int32_t act, const void* x1, int64_t ld1
   const int64_t cap = 256 * (geo.threads >= 512 ? 3 : 8);
   const int grid = (int)(M < cap ? M : cap);
   hipStream_t st = begin_launch(stream);
+  const int use_lut = !two && lut_pays(M, grid, geo.threads);
 #define HYC_EW(B_, L_, A_, N_, MT_)                                                                                \
   hipLaunchKernelGGL((k_ew_fwd_fast<B_, L_, A_, N_, MT_>), dim3(grid), dim3(geo.threads), 0, st,                   \
                      static_cast<const uint16_t*>(x1), ld1, static_cast<const uint16_t*>(x2), ld2, M, H, geo.cps,  \
-                     s1, s2, static_cast<uint16_t*>(y))
+                     s1, s2, static_cast<uint16_t*>(y), use_lut)
 #define HYC_EW_T(B_, L_, A_, N_) do { if (geo.threads <= 256) HYC_EW(B_, L_, A_, N_, 256); else HYC_EW(B_, L_, A_, N_, 1024); } while (0)
 #define HYC_EW_L(B_, A_, N_) do { if (lpg == 8) HYC_EW_T(B_, 8, A_, N_); else HYC_EW_T(B_, 16, A_, N_); } while (0)
   if (two) {

@@ -400,3 +400,39 @@ def test_empty_batches_pass_through_every_launcher(K):
     assert gw.shape == (16, H) and float(gw.abs().max()) == 0.0
     p, sp = K.softmax_fwd(e, 0.01)
     assert p.shape == (0, H) and sp.cols.numel() == 0 and K.softmax_bwd(e, sp).shape == (0, H)
+
+
+@pytest.mark.parametrize("act", ["silu", "gelu"])
+def test_forward_activation_tables_match_the_framework_for_every_bf16_value(K, act):
+    """with enough rows per workgroup the forward kernels look act(x) up in a table built from the same arithmetic
+    (inputs outside it are computed): all 65 536 bf16 patterns again, through the one-pass gated forward, the
+    activation forward with its save, and the gated backward's derivative table against the separate backward calls"""
+    H = 4096
+    pat = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16).view(-1, H)      # 16 rows
+    gate = pat.repeat(512, 1).cuda()                                                                   # 8192 rows
+    up = torch.ones_like(gate)
+    plan = K.select_channels(torch.zeros(H, device="cuda"), 0)
+    want = torch.nn.functional.silu(gate) if act == "silu" else torch.nn.functional.gelu(gate)
+
+    def same(a, b):
+        return bool(((torch.isnan(a) & torch.isnan(b)) | (a.view(torch.int16) == b.view(torch.int16))).all())
+
+    h, c_a, c_u, c_g = K.gated_act_fwd(act, gate, up, plan, plan, plan, 4, 128)
+    assert same(h, want)
+    y, c_x = K.act_fwd_compress(act, gate, plan, 4, 128)
+    assert same(y, want)
+    assert torch.equal(c_x.stored, c_g.stored) and torch.equal(c_x.scales.view(torch.int16), c_g.scales.view(torch.int16))
+    # finite inputs for the backward comparison (codes of a row holding inf / nan are not meaningful)
+    fin = gate[:, :2048].contiguous().clamp(-300, 300)
+    finp = K.select_channels(K.channel_absmax(fin), 20)
+    g = torch.full_like(fin, 0.75)
+    ones = torch.ones_like(fin)
+    a = torch.nn.functional.silu(fin) if act == "silu" else torch.nn.functional.gelu(fin)
+    ca, cu, cg = (K.compress_channel(t, finp, 4, 128) for t in (a, ones, fin))
+    d_gate, d_up = K.gated_act_bwd(act, g, ca, cu, cg)
+    d_a, d_u = K.hadamard_bwd(g, ca, cu)
+    assert same(d_up, d_u) and same(d_gate, K.act_bwd(act, d_a, cg))
+    few = slice(0, 16)                                         # one row per workgroup: no table
+    cf = [K.compress_channel(t[few].contiguous(), finp, 4, 128) for t in (a, ones, fin)]
+    dg_few, _ = K.gated_act_bwd(act, g[few].contiguous(), *cf)
+    assert same(dg_few, d_gate[few])
