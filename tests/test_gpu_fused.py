@@ -423,7 +423,7 @@ def test_forward_activation_tables_match_the_framework_for_every_bf16_value(K, a
     assert same(y, want)
     assert torch.equal(c_x.stored, c_g.stored) and torch.equal(c_x.scales.view(torch.int16), c_g.scales.view(torch.int16))
     # finite inputs for the backward comparison (codes of a row holding inf / nan are not meaningful)
-    fin = gate[:, :2048].contiguous().clamp(-300, 300)
+    fin = torch.nan_to_num(gate).clamp(-300, 300)             # 4 rows x 256 threads per workgroup: the tables are in use
     finp = K.select_channels(K.channel_absmax(fin), 20)
     g = torch.full_like(fin, 0.75)
     ones = torch.ones_like(fin)
