@@ -708,8 +708,14 @@ template <int BITS, int SRC, int ACT>
 __global__ void __launch_bounds__(1024)
 k_act_bwd(const uint16_t* __restrict__ g, const uint8_t* __restrict__ stored, const uint16_t* __restrict__ vals,
           const uint16_t* __restrict__ scales, int64_t M, int64_t H, int CPS, int iters, ChanArgs ca,
-          uint16_t* __restrict__ dx) {
+          uint16_t* __restrict__ dx, int use_lut) {
   constexpr int NSEG = Q<BITS>::NSEG;
+  constexpr bool HAS_LUT = ACT == HYC_ACT_SILU || ACT == HYC_ACT_GELU_TANH;
+  __shared__ uint16_t lut[HAS_LUT ? LUT_NEG + LUT_N : 1];   // the derivative table of the fast kernel
+  if (HAS_LUT && use_lut) {
+    lut_fill<ACT>(lut);
+    __syncthreads();
+  }
   const int64_t SEG = (int64_t)CPS * 8;
   for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
     for (int it = 0; it < iters; ++it) {
@@ -724,10 +730,16 @@ k_act_bwd(const uint16_t* __restrict__ g, const uint8_t* __restrict__ stored, co
         for (int i = 0; i < NSEG; ++i) {
           const int64_t col = i * SEG + 8 * c;
           float xv[8], gv[8], o[8];
-          if (SRC == 0) decode_chan<BITS>(pk.x, pk.y, i, c, CPS, ca, vals + row * ca.k, scales + row * ca.groups_per_row, xv);
-          else unpack8(*reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(stored) + row * H + col), xv);
+          uint4 xr;
+          if (SRC == 0) {
+            decode_chan<BITS>(pk.x, pk.y, i, c, CPS, ca, vals + row * ca.k, scales + row * ca.groups_per_row, xv);
+            if (HAS_LUT) xr = pack8(xv);
+          } else {
+            xr = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(stored) + row * H + col);
+            unpack8(xr, xv);
+          }
           unpack8(graw[i], gv);
-          act_grad8<ACT>(xv, gv, o);
+          if (!(HAS_LUT && use_lut && lut_grad8(lut, xr, gv, o))) act_grad8<ACT>(xv, gv, o);
           *reinterpret_cast<uint4*>(dx + row * H + col) = pack8(o);
         }
       }
@@ -756,6 +768,7 @@ static int launch_act(const void* g, const void* stored, const void* vals, const
   const int64_t cap = 256 * (geo.threads >= 512 ? 3 : 8);
   const int grid = (int)(M < cap ? M : cap);
   hipStream_t st = begin_launch(stream);
+  const int use_lut = lut_pays(M, grid, geo.threads * geo.iters, LUT_PAYS_BWD);
   if (d->mode == HYC_MODE_CHANNEL && geo.iters == 1 && d->bits != 1) {
 #define HYC_ACT_FAST(B_)                                                                                       \
   do {                                                                                                         \
@@ -770,7 +783,6 @@ static int launch_act(const void* g, const void* stored, const void* vals, const
                          static_cast<const uint16_t*>(vals), static_cast<const uint16_t*>(scales), M, H, geo.cps, ca, \
                          static_cast<uint16_t*>(dx), use_lut);                                                 \
   } while (0)
-    const int use_lut = lut_pays(M, grid, geo.threads, LUT_PAYS_BWD);
     if (d->bits == 2) HYC_ACT_FAST(2);
     else if (d->bits == 4) HYC_ACT_FAST(4);
     else HYC_ACT_FAST(8);
@@ -781,7 +793,7 @@ static int launch_act(const void* g, const void* stored, const void* vals, const
   hipLaunchKernelGGL((k_act_bwd<B_, S_, ACT>), dim3(grid), dim3(geo.threads), 0, st,                      \
                      static_cast<const uint16_t*>(g), static_cast<const uint8_t*>(stored),                \
                      static_cast<const uint16_t*>(vals), static_cast<const uint16_t*>(scales), M, H, geo.cps, \
-                     geo.iters, ca, static_cast<uint16_t*>(dx))
+                     geo.iters, ca, static_cast<uint16_t*>(dx), use_lut)
   if (d->mode == HYC_MODE_CHANNEL) {
     switch (d->bits) {
       case 1: HYC_ACT_LAUNCH(1, 0); break;

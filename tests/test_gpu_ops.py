@@ -855,3 +855,11 @@ def test_act_bwd_every_bf16_value(K, act):
     assert torch.equal(rep, rep[:1].expand_as(rep))
     few = K.act_bwd(act, g[:16].contiguous(), K.compress_channel(x[:16].contiguous(), plan, 4, 128)).cpu()   # one row per workgroup: no table
     assert torch.equal(few.view(torch.int16), dx[:16].view(torch.int16))
+    # a restored (dense) activation takes the general kernel, which has the same table
+    dense = K.act_bwd(act, g, x).cpu()
+    want_d = (O.silu_bwd if act == "silu" else O.gelu_bwd)(pat, g16)
+    same = (torch.isnan(want_d) & torch.isnan(dense[:16])) | (dense[:16].view(torch.int16) == want_d.view(torch.int16))
+    same |= (want_d.float().abs() < 1e-30) & (dense[:16].float().abs() < 1e-30)
+    assert bool(same.all()), [hex(int(b) & 0xFFFF) for b in pat.view(torch.int16)[~same][:8]]
+    repd = dense.view(512, 16, H).view(torch.int16)
+    assert torch.equal(repd, repd[:1].expand_as(repd))
