@@ -229,7 +229,9 @@ def test_gated_forward_activation_matches_the_framework_for_every_bf16_value(K, 
 
 @pytest.mark.parametrize("act,M,H,bits,group,k", [("silu", 333, 11008, 4, 128, 110), ("gelu", 64, 4096, 4, 128, 41),
                                                   ("silu", 2100, 4096, 4, 64, 41), ("silu", 40, 512, 8, 64, 5),
-                                                  ("gelu", 130, 2048, 8, 128, 300)])
+                                                  ("gelu", 130, 2048, 8, 128, 300),
+                                                  # three rows of 704 threads per workgroup: the activation table is in use
+                                                  ("silu", 2100, 11008, 4, 128, 110), ("gelu", 1600, 11008, 4, 128, 110)])
 def test_gated_forward_equals_the_separate_calls(K, act, M, H, bits, group, k):
     """one pass = F.silu / F.gelu, three hyc_compress calls and a product, bit for bit; gate and up are column slices of
     one wider matrix, as a fused gate/up projection hands them over"""
