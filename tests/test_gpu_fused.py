@@ -172,7 +172,8 @@ def test_hadamard_bwd(K, M, H, b1, g1, b2, g2):
 
 
 @pytest.mark.parametrize("act", ["silu", "gelu"])
-@pytest.mark.parametrize("M,H,bits,group", [(40, 4096, 4, 128), (2100, 11008, 2, 64), (33, 2048, 8, 64)])
+@pytest.mark.parametrize("M,H,bits,group", [(40, 4096, 4, 128), (2100, 11008, 2, 64), (33, 2048, 8, 64),
+                                            (2100, 11008, 4, 128)])      # three 704-thread rows per workgroup: derivative table
 def test_gated_act_bwd_equals_the_two_steps(K, act, M, H, bits, group):
     """one pass over (act(gate), up, gate) = hadamard backward followed by the activation backward, bit for bit"""
     k = K.num_outlier_channels(H, 0.01)
