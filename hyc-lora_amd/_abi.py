@@ -12,6 +12,8 @@ LIB_PATH = os.path.join(_HERE, "lib", "libhyc_gfx950.so")
 MODE_CHANNEL, MODE_THRESHOLD, MODE_DENSE = 0, 1, 2
 DTYPE_BF16, DTYPE_F32 = 0, 1
 ACT_SILU, ACT_GELU_TANH = 0, 1
+SCALE_RANGE, SCALE_ABSMAX = 0, 1
+ABI_VERSION = 2
 EINVAL, EFAULT, ENOTSUP, ELAUNCH = -22, -14, -95, -5
 
 c_i32, c_i64, c_f32, c_ptr = ctypes.c_int32, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
@@ -26,7 +28,7 @@ class HycDesc(ctypes.Structure):
         ("scale", c_ptr),
         ("scale_stride_token", c_i64), ("scale_stride_channel", c_i64), ("S", c_i64),
         ("L", c_ptr), ("R", c_ptr),
-        ("rank", c_i32), ("reserved", c_i32),
+        ("rank", c_i32), ("scale_rule", c_i32),
         ("csr_row_ptr", c_ptr), ("csr_cols", c_ptr), ("csr_vals", c_ptr),
         ("chan_idx", c_ptr),
     ]
@@ -103,8 +105,9 @@ def load():
         fn = getattr(lib, name)           # AttributeError if a declared symbol is not exported
         fn.restype = res
         fn.argtypes = args
-    if lib.hyc_abi_version() != 1:
-        raise RuntimeError("libhyc ABI version %d, expected 1" % lib.hyc_abi_version())
+    if lib.hyc_abi_version() != ABI_VERSION:
+        raise RuntimeError("libhyc ABI version %d, expected %d: rebuild it with `python hyc-lora_amd/build.py`"
+                           % (lib.hyc_abi_version(), ABI_VERSION))
     _lib = lib
     return lib
 

@@ -21,6 +21,9 @@ int make_chan_args(const hyc_desc* d, const RowGeom& g, ChanArgs* a, int* lpg) {
   a->k = d->k;
   a->groups_per_row = (int)(g.H / d->group);
   a->chunk_to_group_shift = ilog2(*lpg);
+  if (d->scale_rule != HYC_SCALE_RANGE && d->scale_rule != HYC_SCALE_ABSMAX)
+    return fail(HYC_EINVAL, "scale_rule=%d: HYC_SCALE_RANGE (0) or HYC_SCALE_ABSMAX (1)", d->scale_rule);
+  a->absmax = d->scale_rule == HYC_SCALE_ABSMAX;
   return HYC_OK;
 }
 

@@ -573,15 +573,15 @@ k_gated_act_fwd_fast(const uint16_t* __restrict__ gate, int64_t ldg, const uint1
       store_stream(hp + i * SEG, pack8(v));
       uint32_t cl, ch;
       unpack8(make_uint4(araw.x & km_a[i][0], araw.y & km_a[i][1], araw.z & km_a[i][2], araw.w & km_a[i][3]), v);
-      float s = quant_seg<BITS, LPGT>(v, LPGT, cl, ch);
+      float s = quant_seg<BITS, LPGT>(v, LPGT, cl, ch, sa.ca.absmax != 0);
       if (leader) sa.scales[scoff + i * seg_groups] = f_to_bf(s);
       if (BITS == 8) { lo_a = cl; hi_a = ch; } else { lo_a |= cl << (i * BITS); hi_a |= ch << (i * BITS); }
       unpack8(make_uint4(uraw[i].x & km_u[i][0], uraw[i].y & km_u[i][1], uraw[i].z & km_u[i][2], uraw[i].w & km_u[i][3]), v);
-      s = quant_seg<BITS, LPGT>(v, LPGT, cl, ch);
+      s = quant_seg<BITS, LPGT>(v, LPGT, cl, ch, su.ca.absmax != 0);
       if (leader) su.scales[scoff + i * seg_groups] = f_to_bf(s);
       if (BITS == 8) { lo_u = cl; hi_u = ch; } else { lo_u |= cl << (i * BITS); hi_u |= ch << (i * BITS); }
       unpack8(make_uint4(graw[i].x & km_g[i][0], graw[i].y & km_g[i][1], graw[i].z & km_g[i][2], graw[i].w & km_g[i][3]), v);
-      s = quant_seg<BITS, LPGT>(v, LPGT, cl, ch);
+      s = quant_seg<BITS, LPGT>(v, LPGT, cl, ch, sg.ca.absmax != 0);
       if (leader) sg.scales[scoff + i * seg_groups] = f_to_bf(s);
       if (BITS == 8) { lo_g = cl; hi_g = ch; } else { lo_g |= cl << (i * BITS); hi_g |= ch << (i * BITS); }
     }
@@ -684,7 +684,7 @@ k_ew_fwd_fast(const uint16_t* __restrict__ x1, int64_t ld1, const uint16_t* __re
         const uint4 r = raw[n][i];
         unpack8(make_uint4(r.x & km[n][i][0], r.y & km[n][i][1], r.z & km[n][i][2], r.w & km[n][i][3]), v);
         uint32_t cl, ch;
-        const float s = quant_seg<BITS, LPGT>(v, LPGT, cl, ch);
+        const float s = quant_seg<BITS, LPGT>(v, LPGT, cl, ch, (n == 0 ? s1.ca.absmax : s2.ca.absmax) != 0);
         if (leader) (n == 0 ? s1.scales : s2.scales)[scoff + i * seg_groups] = f_to_bf(s);
         if (BITS == 8) { lo[n] = cl; hi[n] = ch; } else { lo[n] |= cl << (i * BITS); hi[n] |= ch << (i * BITS); }
       }

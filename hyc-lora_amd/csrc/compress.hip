@@ -64,7 +64,7 @@ k_decompress_chan(const uint8_t* __restrict__ stored, const uint16_t* __restrict
 // Fast paths: every lane owns exactly one chunk per segment (CPS == blockDim.x), the group width is a template
 // parameter, plan words are loaded once, pointers advance by a constant and the next row is requested before the
 // current one is processed.
-template <int BITS, int LPGT, int MAXT>
+template <int BITS, int LPGT, int MAXT, int RULE>
 __global__ void __launch_bounds__(MAXT)
 k_compress_chan_fast(const uint16_t* __restrict__ x, int64_t M, int64_t H /* row pitch of x */, int CPS, ChanArgs a,
                      uint8_t* __restrict__ stored, uint16_t* __restrict__ vals, uint16_t* __restrict__ scales) {
@@ -115,7 +115,7 @@ k_compress_chan_fast(const uint16_t* __restrict__ x, int64_t M, int64_t H /* row
       float v[8];
       unpack8(make_uint4(raw[i].x & km[i][0], raw[i].y & km[i][1], raw[i].z & km[i][2], raw[i].w & km[i][3]), v);
       uint32_t cl, ch;
-      const float s = quant_seg<BITS, LPGT>(v, LPGT, cl, ch);
+      const float s = quant_seg<BITS, LPGT, RULE>(v, LPGT, cl, ch, false);
       if (leader) scp[i * seg_groups] = f_to_bf(s);
       if (BITS == 8) { lo = cl; hi = ch; }
       else { lo |= cl << (i * BITS); hi |= ch << (i * BITS); }
@@ -415,18 +415,23 @@ int hyc_compress_rows(const void* x, int64_t ldx, int64_t M, int64_t H, const hy
     if (!aligned16(x) || !aligned8(stored)) return fail(HYC_EINVAL, "hyc_compress: x must be 16-byte and stored 8-byte aligned");
     const int grid = row_grid(M, g.threads);
     if (g.iters == 1 && (lpg == 8 || lpg == 16) && d->bits != 1) {
-#define HYC_CF(B_, L_)                                                                                             \
+#define HYC_CF_R(B_, L_, R_)                                                                                       \
   do {                                                                                                             \
     if (g.threads <= 256)                                                                                          \
-      hipLaunchKernelGGL((k_compress_chan_fast<B_, L_, 256>),                                                      \
-                         dim3(long_input_grid<k_compress_chan_fast<B_, L_, 256>>(M, g.threads, grid)), dim3(g.threads), 0, st, \
+      hipLaunchKernelGGL((k_compress_chan_fast<B_, L_, 256, R_>),                                                  \
+                         dim3(long_input_grid<k_compress_chan_fast<B_, L_, 256, R_>>(M, g.threads, grid)), dim3(g.threads), 0, st, \
                          static_cast<const uint16_t*>(x), M, ldx, g.cps, a, static_cast<uint8_t*>(stored),               \
                          static_cast<uint16_t*>(vals), static_cast<uint16_t*>(scales));                            \
     else                                                                                                           \
-      hipLaunchKernelGGL((k_compress_chan_fast<B_, L_, 1024>),                                                     \
-                         dim3(long_input_grid<k_compress_chan_fast<B_, L_, 1024>>(M, g.threads, grid)), dim3(g.threads), 0, st, \
+      hipLaunchKernelGGL((k_compress_chan_fast<B_, L_, 1024, R_>),                                                 \
+                         dim3(long_input_grid<k_compress_chan_fast<B_, L_, 1024, R_>>(M, g.threads, grid)), dim3(g.threads), 0, st, \
                          static_cast<const uint16_t*>(x), M, ldx, g.cps, a, static_cast<uint8_t*>(stored),               \
                          static_cast<uint16_t*>(vals), static_cast<uint16_t*>(scales));                            \
+  } while (0)
+#define HYC_CF(B_, L_)                                           \
+  do {                                                           \
+    if (a.absmax) HYC_CF_R(B_, L_, SCALE_ABSMAX);                \
+    else HYC_CF_R(B_, L_, SCALE_RANGE);                          \
   } while (0)
       switch (d->bits * 100 + lpg) {
         case 208: HYC_CF(2, 8); break;
@@ -436,6 +441,7 @@ int hyc_compress_rows(const void* x, int64_t ldx, int64_t M, int64_t H, const hy
         case 808: HYC_CF(8, 8); break;
         default: HYC_CF(8, 16); break;
       }
+#undef HYC_CF_R
 #undef HYC_CF
       return check_launch("hyc_compress");
     }

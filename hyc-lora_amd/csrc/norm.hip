@@ -58,7 +58,7 @@ __device__ __forceinline__ float block_sum1(float a, float (*red)[16], int parit
   return t;
 }
 
-template <int BITS, int LPGT, bool WF32, int MAXT>
+template <int BITS, int LPGT, bool WF32, int MAXT, int RULE>
 __global__ void __launch_bounds__(MAXT)
 k_rmsnorm_fwd_fast(const uint16_t* __restrict__ x, const void* __restrict__ w, float eps, int64_t M, int64_t H,
                    int CPS, ChanArgs ca, uint16_t* __restrict__ y, float* __restrict__ rstd_out, uint8_t* __restrict__ stored,
@@ -132,7 +132,7 @@ k_rmsnorm_fwd_fast(const uint16_t* __restrict__ x, const void* __restrict__ w, f
       for (int j = 0; j < 8; ++j) ss = __builtin_fmaf(v[j], v[j], ss);
       unpack8(make_uint4(raw[i].x & km[i][0], raw[i].y & km[i][1], raw[i].z & km[i][2], raw[i].w & km[i][3]), v);
       uint32_t cl, ch;
-      const float s = quant_seg<BITS, LPGT>(v, LPGT, cl, ch);
+      const float s = quant_seg<BITS, LPGT, RULE>(v, LPGT, cl, ch, false);
       if (leader) scp[i * seg_groups] = f_to_bf(s);
       if (BITS == 8) { lo = cl; hi = ch; }
       else { lo |= cl << (i * BITS); hi |= ch << (i * BITS); }
@@ -430,7 +430,7 @@ k_rmsnorm_fwd(const uint16_t* __restrict__ x, const void* __restrict__ w, const 
 #pragma unroll
           for (int j = 0; j < 8; ++j) ss = LN ? ss + v[j] : __builtin_fmaf(v[j], v[j], ss);
           uint32_t cl, ch;
-          const float s = encode_seg<BITS>(raw[it][i], v, plan[it][i], lpg, vals + row * ca.k, cl, ch);
+          const float s = encode_seg<BITS>(raw[it][i], v, plan[it][i], lpg, vals + row * ca.k, cl, ch, ca.absmax != 0);
           if (act[it] && (c & (lpg - 1)) == 0)
             scales[row * ca.groups_per_row + ((i * CPS + c) >> ca.chunk_to_group_shift)] = f_to_bf(s);
           if (BITS == 8) { lo = cl; hi = ch; }
@@ -840,8 +840,14 @@ static int norm_fwd_impl(const void* x, const void* w, const void* bias, int32_t
     uint16_t* vp = static_cast<uint16_t*>(vals);
     uint16_t* scp = static_cast<uint16_t*>(scales);
 #define HYC_FWD_FAST(B_, L_, W_, MT_)                                                                              \
-  hipLaunchKernelGGL((k_rmsnorm_fwd_fast<B_, L_, W_, MT_>), dim3(grid), dim3(n.T), 0, st, xp, w, eps, M, H, g.cps, ca, yp, \
-                     rstd, stp, vp, scp)
+  do {                                                                                                             \
+    if (ca.absmax)                                                                                                 \
+      hipLaunchKernelGGL((k_rmsnorm_fwd_fast<B_, L_, W_, MT_, SCALE_ABSMAX>), dim3(grid), dim3(n.T), 0, st, xp, w, eps, M, H, \
+                         g.cps, ca, yp, rstd, stp, vp, scp);                                                       \
+    else                                                                                                           \
+      hipLaunchKernelGGL((k_rmsnorm_fwd_fast<B_, L_, W_, MT_, SCALE_RANGE>), dim3(grid), dim3(n.T), 0, st, xp, w, eps, M, H, \
+                         g.cps, ca, yp, rstd, stp, vp, scp);                                                       \
+  } while (0)
 #define HYC_FWD_FAST_W(B_, L_)                                                        \
   do {                                                                                \
     if (n.T <= 256) { if (wf32) HYC_FWD_FAST(B_, L_, true, 256); else HYC_FWD_FAST(B_, L_, false, 256); }  \

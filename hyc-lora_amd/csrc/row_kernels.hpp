@@ -18,13 +18,15 @@ __device__ __forceinline__ uint16_t raw16(const uint4& r, int j) {
 // plan word `p` (see hyc_desc.chan_plan) marks the outlier channels of the chunk; their values go to vals_row and
 // they are quantised as exact zeros.  Cross-lane: every lane of the wave must take part.
 // Returns the group scale; the caller stores it from the first lane of each group.
-template <int BITS, int LPGT>
-__device__ __forceinline__ float quant_seg(float (&v)[8], int lpg, uint32_t& cl, uint32_t& ch);
+// RULE: the group scale rule, SCALE_RANGE / SCALE_ABSMAX, or SCALE_RUNTIME = decided by the flag `absmax` (uniform).
+constexpr int SCALE_RANGE = 0, SCALE_ABSMAX = 1, SCALE_RUNTIME = -1;
+template <int BITS, int LPGT, int RULE = SCALE_RUNTIME>
+__device__ __forceinline__ float quant_seg(float (&v)[8], int lpg, uint32_t& cl, uint32_t& ch, bool absmax);
 
 // LPGT: lanes per scale group when known at compile time, 0 = use the runtime value `lpg`.
 template <int BITS, int LPGT = 0>
 __device__ __forceinline__ float encode_seg(const uint4& rawseg, float (&v)[8], uint32_t p, int lpg, uint16_t* vals_row,
-                                            uint32_t& cl, uint32_t& ch) {
+                                            uint32_t& cl, uint32_t& ch, bool absmax) {
   if (__builtin_expect((p & 0xFFu) != 0, 0)) {         // rare: ~k/(H/8) of the chunks
     const uint32_t m8 = p & 0xFFu;
     const int first = (int)(p >> 16);
@@ -36,27 +38,45 @@ __device__ __forceinline__ float encode_seg(const uint4& rawseg, float (&v)[8], 
       }
     }
   }
-  return quant_seg<BITS, LPGT>(v, lpg, cl, ch);
+  return quant_seg<BITS, LPGT>(v, lpg, cl, ch, absmax);
 }
 
-// group min/max -> scale -> 8 code bytes, no outlier handling (the caller has zeroed the outlier channels)
-template <int BITS, int LPGT>
-__device__ __forceinline__ float quant_seg(float (&v)[8], int lpg, uint32_t& cl, uint32_t& ch) {
-  float mx = __builtin_elementwise_maximum(__builtin_elementwise_maximum(v[0], v[1]), v[2]);
-  float mn = __builtin_elementwise_minimum(__builtin_elementwise_minimum(v[0], v[1]), v[2]);
-  mx = __builtin_elementwise_maximum(__builtin_elementwise_maximum(mx, v[3]), v[4]);
-  mn = __builtin_elementwise_minimum(__builtin_elementwise_minimum(mn, v[3]), v[4]);
-  mx = __builtin_elementwise_maximum(__builtin_elementwise_maximum(mx, v[5]), v[6]);
-  mn = __builtin_elementwise_minimum(__builtin_elementwise_minimum(mn, v[5]), v[6]);
-  mx = __builtin_elementwise_maximum(mx, v[7]);
-  mn = __builtin_elementwise_minimum(mn, v[7]);
-  if (LPGT > 0) {
-    group_maxmin<LPGT>(mx, mn);
+// group statistics -> scale -> 8 code bytes, no outlier handling (the caller has zeroed the outlier channels).
+//   range rule    s = bf16(bf16(max - min) / (2^b - 1))      the reference's formula, compress_function.py:328-334
+//   abs-max rule  s = bf16(bf16(2 max|x|) / (2^b - 1))       the same formula over the interval made symmetric about 0,
+//                 [-max|x|, max|x|]: no element is off by more than half a step, one butterfly instead of two
+//                 (1-bit codes, {-1, 0}: s = max|x|)
+// Both quotients are formed as a product with the rounded reciprocal: the dividend is a bf16 value (an integer below
+// 256 times a power of two) and the divisor an integer below 256, so the exact quotient never lies within 2^-17
+// (relative) of a bf16 rounding boundary, far more than the 2^-23 the product can be off by.
+template <int BITS, int LPGT, int RULE>
+__device__ __forceinline__ float quant_seg(float (&v)[8], int lpg, uint32_t& cl, uint32_t& ch, bool absmax) {
+  float s;
+  if (RULE == SCALE_ABSMAX || (RULE == SCALE_RUNTIME && absmax)) {
+    float am = __builtin_elementwise_maximum(__builtin_elementwise_maximum(__builtin_fabsf(v[0]), __builtin_fabsf(v[1])), __builtin_fabsf(v[2]));
+    am = __builtin_elementwise_maximum(__builtin_elementwise_maximum(am, __builtin_fabsf(v[3])), __builtin_fabsf(v[4]));
+    am = __builtin_elementwise_maximum(__builtin_elementwise_maximum(am, __builtin_fabsf(v[5])), __builtin_fabsf(v[6]));
+    am = __builtin_elementwise_maximum(am, __builtin_fabsf(v[7]));
+    if (LPGT > 0) am = group_reduce<LPGT>(am, OpMax());
+    else am = group_reduce_rt(am, lpg, OpMax());
+    s = BITS == 1 ? am : bfr((am + am) * Q<BITS>::INV_LEVELS);
   } else {
-    mx = group_reduce_rt(mx, lpg, OpMax());
-    mn = group_reduce_rt(mn, lpg, OpMin());
+    float mx = __builtin_elementwise_maximum(__builtin_elementwise_maximum(v[0], v[1]), v[2]);
+    float mn = __builtin_elementwise_minimum(__builtin_elementwise_minimum(v[0], v[1]), v[2]);
+    mx = __builtin_elementwise_maximum(__builtin_elementwise_maximum(mx, v[3]), v[4]);
+    mn = __builtin_elementwise_minimum(__builtin_elementwise_minimum(mn, v[3]), v[4]);
+    mx = __builtin_elementwise_maximum(__builtin_elementwise_maximum(mx, v[5]), v[6]);
+    mn = __builtin_elementwise_minimum(__builtin_elementwise_minimum(mn, v[5]), v[6]);
+    mx = __builtin_elementwise_maximum(mx, v[7]);
+    mn = __builtin_elementwise_minimum(mn, v[7]);
+    if (LPGT > 0) {
+      group_maxmin<LPGT>(mx, mn);
+    } else {
+      mx = group_reduce_rt(mx, lpg, OpMax());
+      mn = group_reduce_rt(mn, lpg, OpMin());
+    }
+    s = bfr(bfr(mx - mn) * Q<BITS>::INV_LEVELS);
   }
-  const float s = bfr(bfr(mx - mn) * Q<BITS>::INV_LEVELS);   // == bf16(bf16(max-min)/levels): same integer-ratio argument
   codes8<BITS>(v, s, cl, ch);
   return s;
 }
@@ -76,7 +96,7 @@ __device__ __forceinline__ void encode_chan(const uint4* raw, bool active, int c
     const int cg = i * CPS + c;                        // chunk index within the full row
     const uint32_t p = active ? a.plan[cg] : 0u;
     uint32_t cl, ch;
-    const float s = encode_seg<BITS>(raw[i], v, p, lpg, vals_row, cl, ch);
+    const float s = encode_seg<BITS>(raw[i], v, p, lpg, vals_row, cl, ch, a.absmax != 0);
     if (active && (c & (lpg - 1)) == 0) scales_row[cg >> a.chunk_to_group_shift] = f_to_bf(s);
     if (BITS == 8) { lo = cl; hi = ch; }
     else { lo |= cl << (i * BITS); hi |= ch << (i * BITS); }

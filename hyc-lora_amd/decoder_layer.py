@@ -46,6 +46,7 @@ class LayerConfig:
     linear_group: int = 64
     act_bits: int = 4                # norm inputs, q / k / v, gate / act(gate) / up
     act_group: int = 128
+    scale_rule: str = "absmax"       # how a (token, group) scale is formed, see kernels.ChannelPlan
     compress: bool = True            # False: the same functions keep their activations in bf16 (formula check)
     attention: str = "eager"         # "eager": scores, softmax, p @ v with the kept probabilities (the path the
                                      # reference wires into its models); "flash": the library's fused attention with
@@ -83,7 +84,8 @@ class LoRAProjections(torch.nn.Module):
             self.base.append(K.NF4Weight(self.base_all.packed[lo // 2:hi // 2], self.base_all.absmax[lo // 64:hi // 64],
                                          (out, in_features)))
             row += out
-        self.site = CompressionSite(cfg.outlier_ratio, 1.0, cfg.linear_bits, "per-token", 0, "hyc", cfg.linear_group)
+        self.site = CompressionSite(cfg.outlier_ratio, 1.0, cfg.linear_bits, "per-token", 0, "hyc", cfg.linear_group,
+                                    cfg.scale_rule)
         self.iteration = 0
         self.record = None
         self._fused_choice = {}
@@ -228,7 +230,8 @@ class CompressedAttention(torch.nn.Module):
         if cfg.attention not in ("eager", "flash"):
             raise ValueError("attention must be 'eager' or 'flash', got %r" % (cfg.attention,))
         self.cfg = cfg
-        mk = lambda: CompressionSite(cfg.outlier_ratio, 1.0, cfg.act_bits, "per-token", 0, "hyc", cfg.act_group)
+        mk = lambda: CompressionSite(cfg.outlier_ratio, 1.0, cfg.act_bits, "per-token", 0, "hyc", cfg.act_group,
+                                     cfg.scale_rule)
         self.site_q, self.site_k, self.site_v, self.site_o = mk(), mk(), mk(), mk()
         self.iteration = 0
         self.static_value = None          # probability threshold, as in EfficientMemorySoftmax
@@ -425,7 +428,8 @@ class DecoderLayer(torch.nn.Module):
             norm = lambda: EfficientMemoryRMSNorm(H, eps=cfg.rms_eps, elementwise_affine=True, bias=False,
                                                   outlier_ratio=cfg.outlier_ratio, sub_outlier_ratio=1.0,
                                                   sub_outlier_bit=cfg.act_bits, sub_outlier_quantize_method="per-token",
-                                                  rank=0, mode="hyc", group_size=cfg.act_group).to(device).to(BF16)
+                                                  rank=0, mode="hyc", group_size=cfg.act_group,
+                                                  scale_rule=cfg.scale_rule).to(device).to(BF16)
         else:
             norm = lambda: _PlainRMSNorm(H, cfg.rms_eps, device)
         self.input_layernorm = norm()
@@ -436,7 +440,7 @@ class DecoderLayer(torch.nn.Module):
         self.down_proj = LoRAProjections(I, [H], cfg, device)
         self.attention = CompressedAttention(cfg)
         self.act = EfficientMemoryGatedAct("silu", cfg.outlier_ratio, 1.0, cfg.act_bits, "per-token", 0,
-                                           group_size=cfg.act_group) if cfg.compress else None
+                                           group_size=cfg.act_group, scale_rule=cfg.scale_rule) if cfg.compress else None
         self._rope = None
 
     def forward(self, x):

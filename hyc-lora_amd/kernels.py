@@ -62,13 +62,21 @@ def num_outlier_channels(H, ratio):
 # ----------------------------------------------------------------------------------------------------
 # channel mode
 # ----------------------------------------------------------------------------------------------------
+SCALE_RULES = {"range": _abi.SCALE_RANGE, "absmax": _abi.SCALE_ABSMAX}
+DEFAULT_SCALE_RULE = "absmax"
+
+
 @dataclass
 class ChannelPlan:
-    """the static outlier-channel set of one activation site"""
+    """the static part of one activation site: its outlier-channel set and the rule its group scales follow
+    ("absmax": 2 max|x| / (2^bits - 1), the reference's formula over the interval made symmetric about zero, so that no
+    element ends up more than half a step away; "range": the reference's (max - min) / (2^bits - 1) as it stands,
+    which has no zero point and clips groups that are not centred on 0)"""
     H: int
     k: int
     idx: torch.Tensor    # int32 [k], ascending
     plan: torch.Tensor   # int32 [H/8] (bit pattern of the uint32 lookup words)
+    scale_rule: str = DEFAULT_SCALE_RULE
 
 
 def kth_value(x, k):
@@ -100,7 +108,9 @@ def channel_absmax(x2d, amax=None):
     return amax
 
 
-def select_channels(amax, k):
+def select_channels(amax, k, scale_rule=DEFAULT_SCALE_RULE):
+    if scale_rule not in SCALE_RULES:
+        raise ValueError("scale_rule must be 'absmax' or 'range', got %r" % (scale_rule,))
     _need(amax, torch.float32, "amax")
     H = amax.numel()
     if H % 8 or not 0 <= k <= H:
@@ -108,14 +118,31 @@ def select_channels(amax, k):
     idx = torch.empty(max(k, 1), dtype=torch.int32, device=amax.device)[:k]
     plan = torch.empty(H // 8, dtype=torch.int32, device=amax.device)
     check(_abi.load().hyc_select_channels(_p(amax), H, k, _p(idx), _p(plan), _stream()))
-    return ChannelPlan(H, k, idx, plan)
+    return ChannelPlan(H, k, idx, plan, scale_rule)
 
 
-def channel_desc(plan: ChannelPlan, bits, group):
+def _check_plan(plan, device=None):
+    """the kernels index plan.plan [H/8] and plan.idx [k] without further checks, so they must be int32 device
+    tensors of exactly those sizes, on the device of the activation they are used with"""
+    for name, t, n in (("plan.plan", plan.plan, plan.H // 8), ("plan.idx", plan.idx, plan.k)):
+        if not isinstance(t, torch.Tensor) or not t.is_cuda:
+            raise ValueError("%s must be a CUDA (ROCm) tensor; after loading a checkpoint on the host, move the "
+                             "calibration state to the GPU (load_calibration_state does)" % name)
+        if t.dtype != torch.int32 or not t.is_contiguous() or t.numel() != n:
+            raise ValueError("%s must be a contiguous int32 tensor of %d elements" % (name, n))
+        if device is not None and t.device != device:
+            raise ValueError("%s lives on %s, the activation on %s" % (name, t.device, device))
+    if plan.scale_rule not in SCALE_RULES:
+        raise ValueError("scale_rule must be 'absmax' or 'range', got %r" % (plan.scale_rule,))
+
+
+def channel_desc(plan: ChannelPlan, bits, group, device=None):
+    _check_plan(plan, device)
     d = HycDesc()
     d.mode, d.bits, d.group, d.k = _abi.MODE_CHANNEL, bits, group, plan.k
     d.chan_plan = plan.plan.data_ptr()
     d.chan_idx = plan.idx.data_ptr() if plan.k else None
+    d.scale_rule = SCALE_RULES[plan.scale_rule]
     return d
 
 
@@ -138,7 +165,7 @@ class ChannelCompressed:
     H: int
 
     def desc(self):
-        return channel_desc(self.plan, self.bits, self.group)
+        return channel_desc(self.plan, self.bits, self.group, self.stored.device)
 
     def nbytes(self):
         return self.stored.numel() * self.stored.element_size() + 2 * self.vals.numel() + 2 * self.scales.numel()
@@ -147,6 +174,7 @@ class ChannelCompressed:
 def alloc_channel(M, H, plan, bits, group, device):
     if plan.H != H:
         raise ValueError("the outlier-channel plan was made for %d channels, the activation has %d" % (plan.H, H))
+    _check_plan(plan, torch.device(device) if not isinstance(device, torch.device) else device)
     stored = torch.empty((M, H * bits // 8), dtype=torch.int8 if bits == 8 else torch.uint8, device=device)
     vals = torch.empty((M, plan.k), dtype=BF16, device=device)
     scales = torch.empty((M, H // group), dtype=BF16, device=device)

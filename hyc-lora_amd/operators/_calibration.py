@@ -44,9 +44,11 @@ class CompressionSite:
     """per-activation state: the reference's (iteration, static_value) pair plus the channel-mode plan"""
 
     def __init__(self, outlier_ratio, sub_outlier_ratio, sub_outlier_bit, sub_outlier_quantize_method, rank,
-                 mode="ref", group_size=128):
+                 mode="ref", group_size=128, scale_rule=K.DEFAULT_SCALE_RULE):
         if mode not in MODES:
             raise ValueError("mode must be 'ref' or 'hyc', got %r" % (mode,))
+        if scale_rule not in K.SCALE_RULES:
+            raise ValueError("scale_rule must be 'absmax' or 'range', got %r" % (scale_rule,))
         self.outlier_ratio = outlier_ratio
         self.sub_outlier_ratio = sub_outlier_ratio
         self.sub_outlier_bit = sub_outlier_bit
@@ -54,6 +56,7 @@ class CompressionSite:
         self.rank = rank
         self.mode = mode
         self.group_size = group_size
+        self.scale_rule = scale_rule   # hyc mode: how the (token, group) scales are formed, see kernels.ChannelPlan
         self.amax = None     # hyc mode: running channel abs-max (fp32 [H])
         self.plan = None     # hyc mode: ChannelPlan
 
@@ -63,7 +66,7 @@ class CompressionSite:
         if iteration < 2 or self.plan is None:
             self.amax = K.channel_absmax(x2d, self.amax)
             k = K.num_outlier_channels(x2d.shape[-1], self.outlier_ratio)
-            self.plan = K.select_channels(self.amax, k)
+            self.plan = K.select_channels(self.amax, k, self.scale_rule)
         return self.plan
 
 
@@ -81,7 +84,8 @@ def as_rows(x):
 def _site_state(site):
     if site.plan is None:
         return None
-    return {"amax": site.amax, "H": site.plan.H, "k": site.plan.k, "idx": site.plan.idx, "plan": site.plan.plan}
+    return {"amax": site.amax, "H": site.plan.H, "k": site.plan.k, "idx": site.plan.idx, "plan": site.plan.plan,
+            "scale_rule": site.plan.scale_rule}
 
 
 def calibration_state(model):
@@ -102,9 +106,11 @@ def calibration_state(model):
     return out
 
 
-def load_calibration_state(model, state, strict=True):
-    """inverse of calibration_state; tensors are moved to the device of the module's parameters when it has any.
-    Returns the names in `state` that matched no module."""
+def load_calibration_state(model, state, strict=True, device=None):
+    """inverse of calibration_state.  Every tensor of the state is moved to `device`; by default that is the device
+    of the module's parameters or, for the modules that have none (activations, products, GEMMs), the current GPU:
+    the kernels read the outlier-channel plans and static scales through raw device pointers, so a state that was
+    loaded with map_location="cpu" must not stay on the host.  Returns the names in `state` that matched no module."""
     modules = dict(model.named_modules())
     unknown = []
     for name, entry in state.items():
@@ -112,12 +118,19 @@ def load_calibration_state(model, state, strict=True):
         if mod is None or not hasattr(mod, "iteration"):
             unknown.append(name)
             continue
-        param = next(mod.parameters(), None)
+        target = device
+        if target is None:
+            param = next(mod.parameters(), None)
+            if param is not None and param.is_cuda:
+                target = param.device
+            elif torch.cuda.is_available():
+                target = torch.device("cuda", torch.cuda.current_device())
+        if target is None:
+            raise ValueError("load_calibration_state: module %s has no GPU parameters and no GPU is available; "
+                             "pass device=" % name)
 
         def place(t):
-            if isinstance(t, torch.Tensor) and param is not None:
-                return t.to(param.device)
-            return t
+            return t.to(target) if isinstance(t, torch.Tensor) else t
 
         for key, val in entry.items():
             if key == "iteration":
@@ -130,7 +143,10 @@ def load_calibration_state(model, state, strict=True):
                     site.amax, site.plan = None, None
                 else:
                     site.amax = place(val["amax"])
-                    site.plan = K.ChannelPlan(val["H"], val["k"], place(val["idx"]), place(val["plan"]))
+                    # states written before the scale rule existed used the range rule
+                    site.plan = K.ChannelPlan(val["H"], val["k"], place(val["idx"]).to(torch.int32).contiguous(),
+                                              place(val["plan"]).to(torch.int32).contiguous(),
+                                              val.get("scale_rule", "range"))
     if strict and unknown:
         raise KeyError("no memory-efficient module named %s" % ", ".join(unknown))
     return unknown

@@ -156,7 +156,7 @@ class EfficientFlashAttnVarlenQKVPacked(torch.nn.Module):
 
     def __init__(self, outlier_ratio: float = 0.01, sub_outlier_ratio: float = 0.2, sub_outlier_bit: int = 8,
                  sub_outlier_quantize_method: str = 'per-tensor', rank: int = 16, *, mode: str = "ref",
-                 group_size: int = 128):
+                 group_size: int = 128, scale_rule: str = "absmax"):
         super(EfficientFlashAttnVarlenQKVPacked, self).__init__()
         self.outlier_ratio = outlier_ratio
         self.sub_outlier_ratio = sub_outlier_ratio
@@ -166,7 +166,7 @@ class EfficientFlashAttnVarlenQKVPacked(torch.nn.Module):
         self.mode = mode
         self.group_size = group_size
         mk = lambda: CompressionSite(outlier_ratio, sub_outlier_ratio, sub_outlier_bit, sub_outlier_quantize_method, rank,
-                                     mode, group_size)
+                                     mode, group_size, scale_rule)
         self.site_q, self.site_k, self.site_v, self.site_o = mk(), mk(), mk(), mk()
         self.iteration = 0
         self.q_static_value = [None, None, None, None]

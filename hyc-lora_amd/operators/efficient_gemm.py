@@ -89,7 +89,7 @@ class EfficientMemoryGEMM(torch.nn.Module):
                  sub_outlier_quantize_method_1: str = 'per-tensor', outlier_ratio_2: float = 0.01,
                  sub_outlier_ratio_2: float = 0.2, sub_outlier_bit_2: int = 8,
                  sub_outlier_quantize_method_2: str = 'per-tensor', rank: int = 16, *, mode: str = "ref",
-                 group_size: int = 128):
+                 group_size: int = 128, scale_rule: str = "absmax"):
         super().__init__()
         self.outlier_ratio_1, self.sub_outlier_ratio_1 = outlier_ratio_1, sub_outlier_ratio_1
         self.sub_outlier_bit_1, self.sub_outlier_quantize_method_1 = sub_outlier_bit_1, sub_outlier_quantize_method_1
@@ -99,9 +99,9 @@ class EfficientMemoryGEMM(torch.nn.Module):
         self.mode = mode
         self.group_size = group_size
         self.site_1 = CompressionSite(outlier_ratio_1, sub_outlier_ratio_1, sub_outlier_bit_1,
-                                      sub_outlier_quantize_method_1, rank, mode, group_size)
+                                      sub_outlier_quantize_method_1, rank, mode, group_size, scale_rule)
         self.site_2 = CompressionSite(outlier_ratio_2, sub_outlier_ratio_2, sub_outlier_bit_2,
-                                      sub_outlier_quantize_method_2, rank, mode, group_size)
+                                      sub_outlier_quantize_method_2, rank, mode, group_size, scale_rule)
         self.iteration = 0
         self.static_value_1 = [None, None, None, None]
         self.static_value_2 = [None, None, None, None]
@@ -175,7 +175,7 @@ class _ChannelGEMMWithSoftmaxFunc(torch.autograd.Function):
 class EfficientMemoryGEMMWithSoftmax(torch.nn.Module):
     def __init__(self, outlier_ratio_1: float = 0.01, outlier_ratio_2: float = 0.01, sub_outlier_ratio_2: float = 0.2,
                  sub_outlier_bit_2: int = 8, sub_outlier_quantize_method_2: str = 'per-tensor', rank: int = 16, *,
-                 mode: str = "ref", group_size: int = 128):
+                 mode: str = "ref", group_size: int = 128, scale_rule: str = "absmax"):
         super().__init__()
         self.outlier_ratio_1 = outlier_ratio_1
         self.outlier_ratio_2, self.sub_outlier_ratio_2 = outlier_ratio_2, sub_outlier_ratio_2
@@ -184,7 +184,7 @@ class EfficientMemoryGEMMWithSoftmax(torch.nn.Module):
         self.mode = mode
         self.group_size = group_size
         self.site_2 = CompressionSite(outlier_ratio_2, sub_outlier_ratio_2, sub_outlier_bit_2,
-                                      sub_outlier_quantize_method_2, rank, mode, group_size)
+                                      sub_outlier_quantize_method_2, rank, mode, group_size, scale_rule)
         self.iteration = 0
         self.static_value_1 = None
         self.static_value_2 = [None, None, None, None]

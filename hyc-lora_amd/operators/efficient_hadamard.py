@@ -60,7 +60,7 @@ class EfficientMemoryHadamard(torch.nn.Module):
                  sub_outlier_quantize_method_1: str = 'per-tensor', outlier_ratio_2: float = 0.01,
                  sub_outlier_ratio_2: float = 0.2, sub_outlier_bit_2: int = 8,
                  sub_outlier_quantize_method_2: str = 'per-tensor', rank: int = 16, *, mode: str = "ref",
-                 group_size: int = 128):
+                 group_size: int = 128, scale_rule: str = "absmax"):
         super().__init__()
         self.outlier_ratio_1, self.sub_outlier_ratio_1 = outlier_ratio_1, sub_outlier_ratio_1
         self.sub_outlier_bit_1, self.sub_outlier_quantize_method_1 = sub_outlier_bit_1, sub_outlier_quantize_method_1
@@ -70,9 +70,9 @@ class EfficientMemoryHadamard(torch.nn.Module):
         self.mode = mode
         self.group_size = group_size
         self.site_1 = CompressionSite(outlier_ratio_1, sub_outlier_ratio_1, sub_outlier_bit_1,
-                                      sub_outlier_quantize_method_1, rank, mode, group_size)
+                                      sub_outlier_quantize_method_1, rank, mode, group_size, scale_rule)
         self.site_2 = CompressionSite(outlier_ratio_2, sub_outlier_ratio_2, sub_outlier_bit_2,
-                                      sub_outlier_quantize_method_2, rank, mode, group_size)
+                                      sub_outlier_quantize_method_2, rank, mode, group_size, scale_rule)
         self.iteration = 0
         self.static_value_1 = [None, None, None, None]
         self.static_value_2 = [None, None, None, None]
@@ -145,13 +145,13 @@ class EfficientMemoryGatedAct(torch.nn.Module):
 
     def __init__(self, act: str = "silu", outlier_ratio: float = 0.01, sub_outlier_ratio: float = 1.0,
                  sub_outlier_bit: int = 4, sub_outlier_quantize_method: str = 'per-token', rank: int = 0, *,
-                 group_size: int = 128):
+                 group_size: int = 128, scale_rule: str = "absmax"):
         super().__init__()
         if act not in ("silu", "gelu"):
             raise ValueError("act must be 'silu' or 'gelu'")
         self.act, self.sub_outlier_bit, self.group_size = act, sub_outlier_bit, group_size
         mk = lambda: CompressionSite(outlier_ratio, sub_outlier_ratio, sub_outlier_bit, sub_outlier_quantize_method,
-                                     rank, "hyc", group_size)
+                                     rank, "hyc", group_size, scale_rule)
         self.site_act, self.site_up, self.site_gate = mk(), mk(), mk()
         self.iteration = 0
 

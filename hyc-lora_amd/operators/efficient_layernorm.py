@@ -94,7 +94,7 @@ class _ChannelLayerNormFunc(torch.autograd.Function):
 class EfficientMemoryLayerNorm(torch.nn.LayerNorm):
     def __init__(self, normalized_shape, eps=1e-05, elementwise_affine=True, bias=True, outlier_ratio: float = 0.01,
                  sub_outlier_ratio: float = 0.2, sub_outlier_bit: int = 8, sub_outlier_quantize_method: str = 'per-tensor',
-                 rank: int = 16, *, mode: str = "ref", group_size: int = 128):
+                 rank: int = 16, *, mode: str = "ref", group_size: int = 128, scale_rule: str = "absmax"):
         super(EfficientMemoryLayerNorm, self).__init__(normalized_shape, eps, elementwise_affine, bias)
         self.outlier_ratio = outlier_ratio
         self.sub_outlier_ratio = sub_outlier_ratio
@@ -104,7 +104,7 @@ class EfficientMemoryLayerNorm(torch.nn.LayerNorm):
         self.mode = mode
         self.group_size = group_size
         self.site = CompressionSite(outlier_ratio, sub_outlier_ratio, sub_outlier_bit, sub_outlier_quantize_method, rank,
-                                    mode, group_size)
+                                    mode, group_size, scale_rule)
         self.iteration = 0
         self.static_value = [None, None, None, None]
 

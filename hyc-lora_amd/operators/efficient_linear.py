@@ -75,7 +75,7 @@ class _ChannelLinearFunc(torch.autograd.Function):
 class EfficientMemoryLinear(torch.nn.Linear):
     def __init__(self, in_features: int, out_features: int, bias: bool = False, outlier_ratio: float = 0.01,
                  sub_outlier_ratio: float = 0.2, sub_outlier_bit: int = 8, sub_outlier_quantize_method: str = 'per-tensor',
-                 rank: int = 16, *, mode: str = "ref", group_size: int = 128):
+                 rank: int = 16, *, mode: str = "ref", group_size: int = 128, scale_rule: str = "absmax"):
         super(EfficientMemoryLinear, self).__init__(in_features, out_features, bias)
         self.outlier_ratio = outlier_ratio
         self.sub_outlier_ratio = sub_outlier_ratio
@@ -85,7 +85,7 @@ class EfficientMemoryLinear(torch.nn.Linear):
         self.mode = mode
         self.group_size = group_size
         self.site = CompressionSite(outlier_ratio, sub_outlier_ratio, sub_outlier_bit, sub_outlier_quantize_method, rank,
-                                    mode, group_size)
+                                    mode, group_size, scale_rule)
         self.iteration = 0
         self.static_value = [None, None, None, None]
 

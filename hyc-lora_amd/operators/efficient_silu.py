@@ -73,10 +73,10 @@ class _ActModule(torch.nn.Module):
 
     def __init__(self, outlier_ratio: float = 0.01, sub_outlier_ratio: float = 0.2, sub_outlier_bit: int = 8,
                  sub_outlier_quantize_method: str = 'per-tensor', rank: int = 16, *, mode: str = "ref",
-                 group_size: int = 128):
+                 group_size: int = 128, scale_rule: str = "absmax"):
         super().__init__()
         self.site = CompressionSite(outlier_ratio, sub_outlier_ratio, sub_outlier_bit, sub_outlier_quantize_method,
-                                    rank, mode, group_size)
+                                    rank, mode, group_size, scale_rule)
         self.outlier_ratio = outlier_ratio
         self.sub_outlier_ratio = sub_outlier_ratio
         self.sub_outlier_bit = sub_outlier_bit

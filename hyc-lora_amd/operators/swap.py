@@ -25,10 +25,11 @@ def _knobs(section):
                 sub_outlier_quantize_method=section["sub_outlier_quant_method"])
 
 
-def replace_module_for_quantization(module, compress_config, model_args=None, *, mode="ref", group_size=128):
+def replace_module_for_quantization(module, compress_config, model_args=None, *, mode="ref", group_size=128,
+                                    scale_rule="absmax"):
     """In place, like the reference's.  `model_args` is read for `model_name_or_path` only (a name containing "gemma"
     selects the Gemma RMSNorm)."""
-    extra = dict(mode=mode, group_size=group_size)
+    extra = dict(mode=mode, group_size=group_size, scale_rule=scale_rule)
     gemma = model_args is not None and "gemma" in str(getattr(model_args, "model_name_or_path", ""))
 
     for name, child in module.named_children():
@@ -87,4 +88,5 @@ def replace_module_for_quantization(module, compress_config, model_args=None, *,
                 sub_outlier_bit_2=h["sub_outlier_bit"], sub_outlier_quantize_method_2=h["sub_outlier_quant_method"],
                 rank=h["rank"], **extra))
         else:
-            replace_module_for_quantization(child, compress_config, model_args, mode=mode, group_size=group_size)
+            replace_module_for_quantization(child, compress_config, model_args, mode=mode, group_size=group_size,
+                                            scale_rule=scale_rule)

@@ -48,8 +48,8 @@
  *            byte j of a row = sum_i code[j + i*H/n] << (i*bits), n = 8/bits, code = q + 2^(bits-1),
  *            q = clamp(rint(bf16(x / scale)), -2^(bits-1), 2^(bits-1)-1)   (compress_function.py:170-197)
  *   HYC_MODE_CHANNEL   k outlier channels kept verbatim: vals bf16 [M, k] (column i = channel idx[i],
- *            idx ascending); scales bf16 [M, H/group], scale = bf16(bf16(max-min) / (2^bits-1)) over
- *            the group's channels after the outlier channels were zeroed.
+ *            idx ascending); scales bf16 [M, H/group], one per token and group of channels, formed by
+ *            the descriptor's scale_rule (HYC_SCALE_*) after the outlier channels were zeroed.
  *   HYC_MODE_THRESHOLD outliers are the elements with |x - base| > threshold (CSR: row_ptr int32 [M+1],
  *            cols int32 [nnz] ascending within a row, vals bf16 [nnz]); static scale read through two
  *            strides (per-tensor 0/0, per-channel 0/1, per-token 1/0) at row (m mod S);
@@ -64,7 +64,7 @@
 extern "C" {
 #endif
 
-#define HYC_ABI_VERSION 1
+#define HYC_ABI_VERSION 2
 
 /* error codes (negative errno values) */
 #define HYC_OK 0
@@ -76,6 +76,14 @@ extern "C" {
 #define HYC_MODE_CHANNEL 0
 #define HYC_MODE_THRESHOLD 1
 #define HYC_MODE_DENSE 2 /* consumers only: `stored` is the already decompressed bf16 [M,H] */
+
+/* group scale of the channel scheme, over the group's channels after the outlier channels were zeroed:
+ *   HYC_SCALE_RANGE   bf16(bf16(max - min) / (2^bits - 1)), the reference's formula (compress_function.py:328-334).
+ *                     There is no zero point, so a group that is not centred on 0 clips at the code bounds.
+ *   HYC_SCALE_ABSMAX  bf16(bf16(2 max|x|) / (2^bits - 1)): the same formula over the interval made symmetric about 0,
+ *                     [-max|x|, max|x|]; no element is reconstructed more than half a step away.  (1-bit codes: max|x|.) */
+#define HYC_SCALE_RANGE 0
+#define HYC_SCALE_ABSMAX 1
 
 #define HYC_DTYPE_BF16 0
 #define HYC_DTYPE_F32 1
@@ -100,7 +108,8 @@ typedef struct hyc_desc {
   const void* L;              /* device bf16 [S, rank] or NULL when rank == 0 */
   const void* R;              /* device bf16 [rank, H] */
   int32_t rank;
-  int32_t reserved;
+  /* ---- HYC_MODE_CHANNEL: how the encoders form the scale of a (token, group); decoders only read scales ---- */
+  int32_t scale_rule; /* HYC_SCALE_* */
   /* outliers as CSR; consumed by decompress / backward entry points, produced by hyc_ref_outlier_fill */
   const int32_t* csr_row_ptr; /* device [M+1] */
   const int32_t* csr_cols;    /* device [nnz] */

@@ -293,14 +293,32 @@ def hyc_select_channels(scores, k):
     return torch.sort(order).values.to(torch.int32)
 
 
+def hyc_group_scales(rest, bits, group, rule="absmax"):
+    """bf16 [M, H/G] scales of the channel scheme from `rest` = x with the outlier channels zeroed.  No reference code
+    exists for either rule; both are evaluated with the reference's arithmetic (bf16 tensor ops, each rounding to
+    nearest even) and pinned in tests/test_oracle_pins.py by an integer-arithmetic model and by invariants.
+
+    "range"   (max - min) / (2^b - 1): the reference's scale formula (compress_function.py:328-334) per token and
+              group.  The codes have no zero point, so a group that is not centred on 0 clips at the code bounds.
+    "absmax"  (2 max|x|) / (2^b - 1): the same formula over the interval made symmetric about zero,
+              [-max|x|, max|x|]; every element lands within half a step of a code (1-bit codes, {-1, 0}: max|x|)."""
+    M, H = rest.shape
+    g = rest.reshape(M, H // group, group)
+    if rule == "range":
+        return (g.amax(dim=-1) - g.amin(dim=-1)) / (2 ** bits - 1)
+    if rule == "absmax":
+        am = g.abs().amax(dim=-1)
+        return am if bits == 1 else (am + am) / (2 ** bits - 1)
+    raise ValueError("rule must be 'range' or 'absmax'")
+
+
 @torch.no_grad()
-def hyc_compress(x, idx, bits, group):
+def hyc_compress(x, idx, bits, group, rule="absmax"):
     """x [M,H] bf16, idx [k] ascending -> (vals [M,k] bf16, stored, scales [M,H/G] bf16).
 
     Composition of the reference steps (:149-151 zero-out, :170 quantise, :175-197 pack) with
-    the channel mask in place of the threshold mask, and the reference scale formula
-    (max - min) / (2^b - 1) (:328-334) evaluated per token and group of G channels.
-    0/0 (an all-zero group) is given q = 0, i.e. code = offset."""
+    the channel mask in place of the threshold mask and a scale per token and group of G channels
+    (hyc_group_scales).  0/0 (an all-zero group) is given q = 0, i.e. code = offset."""
     M, H = x.shape
     idx = idx.long()
     hot = torch.zeros(H, dtype=torch.bool)
@@ -308,9 +326,8 @@ def hyc_compress(x, idx, bits, group):
     big = x * hot
     vals = big[:, idx].contiguous()
     rest = x - big
-    g = rest.reshape(M, H // group, group)
-    scales = (g.amax(dim=-1) - g.amin(dim=-1)) / (2 ** bits - 1)
-    q = quantize_q(g, scales[..., None], bits, define_nan=True).reshape(M, H)
+    scales = hyc_group_scales(rest, bits, group, rule)
+    q = quantize_q(rest.reshape(M, H // group, group), scales[..., None], bits, define_nan=True).reshape(M, H)
     return vals, encode_q(q, bits), scales
 
 

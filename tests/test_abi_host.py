@@ -33,7 +33,7 @@ def test_every_declared_symbol_is_exported_and_bound(abi):
         assert hasattr(lib, n), n
         assert n in abi.SIGNATURES, "no ctypes prototype for " + n
     assert sorted(abi.SIGNATURES) == names
-    assert lib.hyc_abi_version() == 1
+    assert lib.hyc_abi_version() == 2
 
 
 def test_desc_layout_matches_header(abi):
@@ -316,7 +316,8 @@ def test_calibration_state_round_trip(hyc, tmp_path):
     src = build()
     src[0].iteration = 5
     src[0].site.amax = torch.arange(16, dtype=torch.float32)
-    src[0].site.plan = K.ChannelPlan(16, 1, torch.tensor([15], dtype=torch.int32), torch.tensor([0, 7], dtype=torch.int32))
+    src[0].site.plan = K.ChannelPlan(16, 1, torch.tensor([15], dtype=torch.int32), torch.tensor([0, 7], dtype=torch.int32),
+                                     "range")
     src[1].iteration, src[1].static_value = 2, torch.tensor(0.25)
     src[2].iteration = 2
     src[2].static_value_1 = [torch.tensor(1.5), torch.zeros(4, 16).bfloat16(), torch.ones(1, 8).bfloat16(), torch.zeros(16, 8).bfloat16()]
@@ -327,7 +328,17 @@ def test_calibration_state_round_trip(hyc, tmp_path):
     torch.save(state, path)
     state = torch.load(path, weights_only=True)
     dst = build()
-    assert ops.load_calibration_state(dst, state) == []
+    if not torch.cuda.is_available():
+        # the default target of a parameterless module is the current GPU: without one the call says so
+        with pytest.raises(ValueError, match="device"):
+            ops.load_calibration_state(build(), state)
+    assert ops.load_calibration_state(dst, state, device="cpu") == []
+    assert dst[0].site.plan.scale_rule == "range" and dst[0].site.plan.idx.device.type == "cpu"
+    # a plan that stayed on the host is refused before any pointer reaches a kernel
+    with pytest.raises(ValueError, match="CUDA"):
+        K.channel_desc(dst[0].site.plan, 4, 16)
+    with pytest.raises(ValueError, match="CUDA"):
+        K.alloc_channel(2, 16, dst[0].site.plan, 4, 16, "cpu")
     assert dst[0].iteration == 5 and torch.equal(dst[0].site.amax, src[0].site.amax)
     assert dst[0].site.plan.k == 1 and torch.equal(dst[0].site.plan.idx, src[0].site.plan.idx)
     assert torch.equal(dst[0].site.plan.plan, src[0].site.plan.plan)

@@ -70,18 +70,22 @@ CH_CASES = [
 ]
 
 
+@pytest.mark.parametrize("rule", ["absmax", "range"])
 @pytest.mark.parametrize("bits,group,M,H,k", CH_CASES)
-def test_channel_roundtrip(K, bits, group, M, H, k):
+def test_channel_roundtrip(K, bits, group, M, H, k, rule):
     x, _ = make_x(bits * 1000 + H + M, M, H, max(k, 1), 30.0)
+    if M > 8:
+        x[5] = x[5].abs()         # one-sided rows: where the two scale rules differ most
+        x[6] = -x[6].abs()
     if M > 3:
         x[1, :group] = 0          # a constant (zero-scale) group
         x[2, group:2 * group] = 1.5
     idx = O.hyc_select_channels(O.hyc_channel_scores(x), k)
     xd = x.cuda()
-    plan = K.select_channels(K.channel_absmax(xd), k)
+    plan = K.select_channels(K.channel_absmax(xd), k, rule)
     assert torch.equal(plan.idx.cpu(), idx)
     c = K.compress_channel(xd, plan, bits, group)
-    vals, stored, scales = O.hyc_compress(x, idx, bits, group)
+    vals, stored, scales = O.hyc_compress(x, idx, bits, group, rule)
     assert bits_equal(c.scales.cpu(), scales)
     assert bits_equal(c.vals.cpu(), vals)
     assert c.stored.dtype == stored.dtype and torch.equal(c.stored.cpu(), stored)
@@ -89,6 +93,46 @@ def test_channel_roundtrip(K, bits, group, M, H, k):
     want = O.hyc_decompress(vals, stored, idx, scales, bits, group)
     assert bits_equal(xh, want)
     assert bits_equal(xh[:, idx.long()], x[:, idx.long()])
+
+
+@pytest.mark.parametrize("rule", ["absmax", "range"])
+@pytest.mark.parametrize("bits", [1, 2, 4, 8])
+@pytest.mark.parametrize("group,fused", [(128, False), (32, False), (128, True)])
+def test_group_scale_of_every_bf16_value(K, bits, group, fused, rule):
+    """The kernels form the scale as bf16(d * fl(1 / levels)) where the bf16 tensor expression divides.  Every finite
+    non-negative bf16 value d is made the range (and twice the abs-max) of one group: both signs of the extreme, both
+    rules, all code widths, the standalone encoder (group 32: generic kernel, group 128: fast kernel) and the encoder
+    inside the RMSNorm forward; scales and codes must equal the oracle's, which divides."""
+    H = 1024
+    pats = torch.arange(0, 0x7F80, dtype=torch.int32)                      # +0 ... largest finite, subnormals included
+    per_row = H // group
+    M = (pats.numel() + per_row - 1) // per_row
+    d = torch.zeros(M * per_row, dtype=torch.int32)
+    d[:pats.numel()] = pats
+    ext = d.to(torch.int16).view(torch.bfloat16).reshape(M, per_row)
+    gen = torch.Generator().manual_seed(bits * 10 + group)
+    # the rest of a group: values between 0 and the extreme, so that the extreme is both the range and the abs-max
+    x = (torch.rand(M, per_row, group, generator=gen) * ext.float()[..., None]).bfloat16()
+    x = torch.minimum(x, ext[..., None])
+    x[..., 0] = 0
+    x[..., 3] = ext
+    x[1::2] = -x[1::2]                                                      # odd rows: the extreme is the minimum
+    if rule == "absmax":
+        x = (x.float() * 0.5).bfloat16()                                    # 2 * max|x| runs over every bf16 value (exact halving
+                                                                            # except in the lowest binade, which is covered as is)
+    x = x.reshape(M, H).contiguous()
+    idx = torch.tensor([], dtype=torch.int32)
+    plan = K.select_channels(torch.zeros(H, device="cuda"), 0, rule)
+    vals, stored, scales = O.hyc_compress(x, idx, bits, group, rule)
+    if fused:
+        if bits == 1:
+            pytest.skip("1-bit codes take the generic forward kernel, covered by group 32")
+        w = torch.ones(H, device="cuda")
+        _, _, c = K.rmsnorm_fwd_compress_channel(x.cuda(), w, 1e-6, plan, bits, group)
+    else:
+        c = K.compress_channel(x.cuda(), plan, bits, group)
+    assert bits_equal(c.scales.cpu(), scales)
+    assert torch.equal(c.stored.cpu(), stored)
 
 
 @pytest.mark.parametrize("bits,group", [(4, 64), (2, 64), (8, 128)])
@@ -273,24 +317,26 @@ FULL_SIZE = [  # (name, M, H, bits, group, hot channels, gain)
 ]
 
 
+@pytest.mark.parametrize("rule", ["absmax", "range"])
 @pytest.mark.parametrize("name,M,H,bits,group,n_hot,gain", FULL_SIZE)
-def test_full_size_configurations(K, name, M, H, bits, group, n_hot, gain):
+def test_full_size_configurations(K, name, M, H, bits, group, n_hot, gain, rule):
     """At the configurations' own sizes: the channel choice equals the oracle's; rows are independent, so the packed
     bytes, scales, outlier values and the reconstruction of a seeded sample of 96 rows must equal, bit for bit, the
     oracle run on those rows alone; and over ALL rows the properties the scheme guarantees hold: outlier channels
     come back exactly, every other element is within half a quantisation step (one bf16 ulp of slack) of the
-    original unless its code sits on the clamp, and the scale of each group is bf16(bf16(max - min) / levels)."""
+    original unless its code sits on the clamp, and the scale of each group is bf16(bf16(max - min) / levels) under the
+    range rule, bf16(bf16(2 max|x|) / levels) under the abs-max rule."""
     x, hot = make_x(len(name), M, H, n_hot, gain)
     k = K.num_outlier_channels(H, 0.01)
     xd = x.cuda()
-    plan = K.select_channels(K.channel_absmax(xd), k)
+    plan = K.select_channels(K.channel_absmax(xd), k, rule)
     idx = O.hyc_select_channels(O.hyc_channel_scores(x), k)
     assert torch.equal(plan.idx.cpu(), idx)
     assert set(hot.tolist()) <= set(idx.tolist()) or n_hot > k
     c = K.compress_channel(xd, plan, bits, group)
     xh = K.decompress_channel(c)
     rows = torch.randperm(M, generator=torch.Generator().manual_seed(M + H))[:96].sort().values
-    vals, stored, scales = O.hyc_compress(x[rows], idx, bits, group)
+    vals, stored, scales = O.hyc_compress(x[rows], idx, bits, group, rule)
     assert torch.equal(c.stored.cpu()[rows].view(torch.uint8), stored.view(torch.uint8))
     assert bits_equal(c.scales.cpu()[rows], scales) and bits_equal(c.vals.cpu()[rows], vals)
     assert bits_equal(xh.cpu()[rows], O.hyc_decompress(vals, stored, idx, scales, bits, group))
@@ -300,7 +346,7 @@ def test_full_size_configurations(K, name, M, H, bits, group, n_hot, gain):
     keep[plan.idx.long()] = False
     assert torch.equal(xd[:, ~keep], xh[:, ~keep])
     inl = torch.where(keep, xf, torch.zeros((), device="cuda")).view(M, H // group, group)
-    span = (inl.amax(-1) - inl.amin(-1)).bfloat16().float()
+    span = ((inl.amax(-1) - inl.amin(-1)) if rule == "range" else 2 * inl.abs().amax(-1)).bfloat16().float()
     levels = float(2 ** bits - 1)
     assert bits_equal((span / levels).bfloat16().cpu(), c.scales.cpu())
     s = c.scales.float().repeat_interleave(group, dim=1)

@@ -44,21 +44,22 @@ NORM_CASES = [(4, 128, 96, 4096, 41, torch.float32), (4, 128, 96, 4096, 41, torc
               (2, 64, 2300, 4096, 41, torch.bfloat16)]
 
 
+@pytest.mark.parametrize("rule", ["absmax", "range"])
 @pytest.mark.parametrize("bits,group,M,H,k,wdt", NORM_CASES)
-def test_rmsnorm_channel(K, bits, group, M, H, k, wdt):
+def test_rmsnorm_channel(K, bits, group, M, H, k, wdt, rule):
     x, gen = make_x(H + bits, M, H, k // 2, 30.0)
     w = (1 + 0.1 * torch.randn(H, generator=gen)).to(wdt)
     dy = (0.02 * torch.randn(M, H, generator=gen)).bfloat16()
     eps = 1e-6
     xd = x.cuda()
-    plan = K.select_channels(K.channel_absmax(xd), k)
+    plan = K.select_channels(K.channel_absmax(xd), k, rule)
     idx = plan.idx.cpu()
     assert torch.equal(idx, O.hyc_select_channels(O.hyc_channel_scores(x), k))
     y, rstd, c = K.rmsnorm_fwd_compress_channel(xd, w.cuda(), eps, plan, bits, group)
     y_o, rstd_o = O.rmsnorm_fwd(x, w, eps)
     assert torch.allclose(rstd.cpu(), rstd_o, rtol=2e-6, atol=0)
     assert bf16_ulp_diff(y.cpu(), y_o).max() <= 1
-    vals, stored, scales = O.hyc_compress(x, idx, bits, group)
+    vals, stored, scales = O.hyc_compress(x, idx, bits, group, rule)
     assert torch.equal(c.stored.cpu(), stored) and bits_equal(c.scales.cpu(), scales) and bits_equal(c.vals.cpu(), vals)
     # backward
     xh = O.hyc_decompress(vals, stored, idx, scales, bits, group)
@@ -242,7 +243,9 @@ def test_gated_forward_equals_the_separate_calls(K, act, M, H, bits, group, k):
     both = both.bfloat16().cuda()
     gate, up = both[:, :H], both[:, H:]
     a = torch.nn.functional.silu(gate) if act == "silu" else torch.nn.functional.gelu(gate)
-    plans = [K.select_channels(K.channel_absmax(t), k) for t in (a, up, gate)]
+    # each site carries its own scale rule
+    rules = ("absmax", "range", "absmax") if M % 2 else ("range", "absmax", "range")
+    plans = [K.select_channels(K.channel_absmax(t), k, r) for t, r in zip((a, up, gate), rules)]
     want = [K.compress_channel(t, p, bits, group) for t, p in zip((a, up, gate), plans)]
     h, c_a, c_u, c_g = K.gated_act_fwd(act, gate, up, plans[0], plans[1], plans[2], bits, group)
     assert bits_equal(h, a * up)
@@ -307,13 +310,14 @@ def test_layernorm_forward_threshold(K, bits, method, rank):
 @pytest.mark.parametrize("act,M,H,bits,group,k", [("silu", 333, 11008, 4, 128, 110), ("gelu", 64, 4096, 4, 128, 41),
                                                   ("silu", 2100, 4096, 2, 64, 41), ("gelu", 40, 512, 8, 64, 5),
                                                   ("silu", 17, 2048, 2, 128, 300)])
-def test_activation_forward_with_the_save_fused_in(K, act, M, H, bits, group, k):
+@pytest.mark.parametrize("rule", ["absmax", "range"])
+def test_activation_forward_with_the_save_fused_in(K, act, M, H, bits, group, k, rule):
     """y = F.silu / F.gelu bit for bit and the compressed x equal to hyc_compress of x; x is a column slice"""
     gen = torch.Generator().manual_seed(M + H + bits)
     wide = torch.randn(M, H + 64, generator=gen)
     wide[:, torch.randperm(H, generator=gen)[:k]] *= 15
     x = wide.bfloat16().cuda()[:, :H]
-    plan = K.select_channels(K.channel_absmax(x), k)
+    plan = K.select_channels(K.channel_absmax(x), k, rule)
     y, c = K.act_fwd_compress(act, x, plan, bits, group)
     want = torch.nn.functional.silu(x) if act == "silu" else torch.nn.functional.gelu(x)
     assert bits_equal(y, want)
@@ -331,7 +335,7 @@ def test_product_forward_with_the_saves_fused_in(K, M, H, bits, group, k):
     both[:, torch.randperm(2 * H, generator=gen)[:2 * k]] *= 15
     both = both.bfloat16().cuda()
     a, b = both[:, :H], both[:, H:]
-    pa, pb = (K.select_channels(K.channel_absmax(t), k) for t in (a, b))
+    pa, pb = (K.select_channels(K.channel_absmax(t), k, r) for t, r in ((a, "absmax"), (b, "range")))
     y, ca, cb = K.hadamard_fwd_compress(a, b, pa, pb, bits, group)
     assert bits_equal(y, a * b)
     for got, t, p in ((ca, a, pa), (cb, b, pb)):

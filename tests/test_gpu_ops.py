@@ -497,7 +497,12 @@ def test_calibration_state_resume(ops, mode):
     for x in xs[:2]:
         a(x.clone().requires_grad_(True))
     b = torch.nn.Sequential(ops.EfficientMemorySiLU(mode=mode, group_size=64, **kw))
-    ops.load_calibration_state(b, ops.calibration_state(a))
+    # as after torch.load(..., map_location="cpu"): the module has no parameters, the state must still end up on the GPU
+    state = {name: {k: ([t.cpu() if isinstance(t, torch.Tensor) else t for t in v] if isinstance(v, list) else
+                        {kk: (t.cpu() if isinstance(t, torch.Tensor) else t) for kk, t in v.items()} if isinstance(v, dict)
+                        else (v.cpu() if isinstance(v, torch.Tensor) else v))
+                    for k, v in entry.items()} for name, entry in ops.calibration_state(a).items()}
+    ops.load_calibration_state(b, state)
     g = torch.ones_like(xs[2])
     grads = []
     for m in (a, b):

@@ -163,6 +163,158 @@ def test_hyc_invariants(bits, group):
     assert torch.all(err[ok] <= sc[ok] * (0.5 + off * 2 ** -7) + 1e-30)
 
 
+# ---- the (token, group) scale rules of the channel scheme: no reference code exists for them, so they are pinned by
+# ---- (i) an independent integer-arithmetic model, (ii) invariants a wrong rule breaks, (iii) the special case that
+# ---- reduces to the golden-pinned threshold scheme
+def _bf16_bits(t):
+    return t.contiguous().view(torch.int16).numpy().astype(np.uint16).astype(np.uint32)
+
+
+def _scale_model(values, bits, rule):
+    """one group, pure Python over its elements: IEEE fp32 steps (numpy scalars) each followed by an integer
+    round-to-nearest-even to bf16 - what a bf16 tensor expression does op by op"""
+    fl = [np.float32(v) for v in values]
+    if rule == "range":
+        mx, mn = fl[0], fl[0]
+        for v in fl[1:]:
+            mx = v if v > mx else mx
+            mn = v if v < mn else mn
+        d = _bf16_to_f32(_f32_to_bf16_rne(np.array([mx - mn], dtype=np.float32)))[0]
+        q = np.array([d / np.float32(2 ** bits - 1)], dtype=np.float32)
+    else:
+        am = np.float32(0)
+        for v in fl:
+            a = -v if v < 0 else v
+            am = a if a > am else am
+        if bits == 1:
+            q = np.array([am], dtype=np.float32)
+        else:
+            two = _bf16_to_f32(_f32_to_bf16_rne(np.array([am + am], dtype=np.float32)))[0]
+            q = np.array([two / np.float32(2 ** bits - 1)], dtype=np.float32)
+    return int(_f32_to_bf16_rne(q)[0])
+
+
+@pytest.mark.parametrize("rule", ["range", "absmax"])
+@pytest.mark.parametrize("bits,group", [(1, 32), (2, 64), (4, 32), (8, 64)])
+def test_group_scale_rule_integer_model(rule, bits, group):
+    gen = torch.Generator().manual_seed(bits * 7 + group)
+    M, H = 6, 4 * group
+    x = torch.randn(M, H, generator=gen)
+    x[0] = x[0].abs() * 3 + 0.5                      # a non-negative row
+    x[1] = -x[1].abs()                               # a non-positive row
+    x[2] = x[2] * 1e-3 + 7.25                        # far from zero, narrow
+    x[3, :group] = 0                                 # an all-zero group
+    x[4] *= 2.0 ** -120                              # tiny magnitudes
+    x = x.bfloat16()
+    got = _bf16_bits(O.hyc_group_scales(x, bits, group, rule))
+    xf = x.float().numpy()
+    for m in range(M):
+        for g in range(H // group):
+            want = _scale_model(xf[m, g * group:(g + 1) * group], bits, rule)
+            assert int(got[m, g]) == want, (m, g, hex(int(got[m, g])), hex(want))
+
+
+@pytest.mark.parametrize("bits,group", [(2, 64), (4, 128), (8, 32)])
+def test_range_rule_spans_all_codes(bits, group):
+    """range rule: a group's maximum and minimum lie 2^b - 1 steps apart, up to the two bf16 roundings of the scale
+    (each at most 2^-8 relative), and without bias over many groups (the quotient by 255 is not checked for bias: a
+    bf16 dividend over 255 rounds down more often than up; the integer model above pins it exactly).  A divisor of 2^b, an abs-max rule or a doubled
+    scale all break this."""
+    gen = torch.Generator().manual_seed(40 + bits)
+    M, H = 64, 4 * group
+    x = (torch.randn(M, H, generator=gen) * torch.rand(M, 1, generator=gen) * 4 + torch.randn(M, 1, generator=gen)).bfloat16()
+    sc = O.hyc_group_scales(x, bits, group, "range").double()
+    g = x.double().reshape(M, H // group, group)
+    steps = (g.amax(-1) - g.amin(-1)) / sc / (2 ** bits - 1)
+    assert torch.all((steps - 1).abs() <= 2 ** -7 * 1.01), (float(steps.min()), float(steps.max()))
+    if bits <= 4:                                      # in codes: 2^b - 1 apart, one more or less through rint
+        assert abs(float(steps.mean()) - 1) < 1.5e-3, float(steps.mean())
+        span = torch.round(g.amax(-1) / sc) - torch.round(g.amin(-1) / sc)
+        assert abs(float(span.mean()) - (2 ** bits - 1)) < 0.25
+
+
+@pytest.mark.parametrize("bits,group", [(2, 64), (4, 128), (8, 32)])
+def test_absmax_rule_extreme_code_and_half_step_bound(bits, group):
+    """abs-max rule: the interval [-max|x|, max|x|] is 2^b - 1 steps long (up to the bf16 roundings of the scale); the
+    element of largest magnitude gets the extreme code of its side; every element, whatever the sign pattern of the
+    group, comes back within half a step.  A divisor of 2^b or 2^(b-1), the range rule or a halved scale break one of
+    these."""
+    gen = torch.Generator().manual_seed(50 + bits)
+    M, H = 32, 4 * group
+    x = torch.randn(M, H, generator=gen) * 3
+    x[::2] = x[::2].abs()                             # half the rows non-negative (activation outputs)
+    x[1::4] = -x[1::4].abs()
+    x = x.bfloat16()
+    idx = torch.tensor([], dtype=torch.int32)
+    vals, stored, scales = O.hyc_compress(x, idx, bits, group, rule="absmax")
+    codes = O.unpack_codes(stored, bits).long() if bits < 8 else stored.long() + 128
+    off, levels = 2 ** (bits - 1), 2 ** bits - 1
+    g = x.double().reshape(M, H // group, group)
+    cg = codes.reshape(M, H // group, group)
+    steps = 2 * g.abs().amax(-1) / scales.double() / levels
+    assert torch.all((steps - 1).abs() <= 2 ** -7 * 1.01), (float(steps.min()), float(steps.max()))
+    where = g.abs().argmax(-1, keepdim=True)
+    big = torch.gather(g, -1, where).squeeze(-1)
+    code_big = torch.gather(cg, -1, where).squeeze(-1)
+    # +levels/2 rounds to the even 2^(b-1) and clamps to the top code; -levels/2 is the bottom code or, when the scale
+    # was rounded up, the one above it
+    assert torch.all(code_big[big > 0] >= levels - (1 if bits == 8 else 0))
+    assert torch.all(code_big[big < 0] <= 1)
+    xh = O.hyc_decompress(vals, stored, idx, scales, bits, group).double().reshape(M, H // group, group)
+    sc = scales.double()[..., None]
+    # half a step, plus the bf16 roundings of the quotient and of code * scale (each at most |q| 2^-8 steps)
+    assert torch.all((xh - g).abs() <= sc * (0.5 + off * 2 ** -7) + 1e-30)
+
+
+@pytest.mark.parametrize("bits", [2, 4, 8])
+def test_range_rule_with_one_group_is_the_reference_per_token_scheme(bits):
+    """group = H and no outlier channels: the channel scheme under the range rule must reproduce, byte for byte, the
+    reference's per-token scheme (get_statistics' per-token scale + compress, both pinned by golden vectors)."""
+    gen = torch.Generator().manual_seed(60 + bits)
+    S, H = 16, 256
+    x = torch.randn(1, S, H, generator=gen)
+    x = x + torch.randn(1, S, 1, generator=gen)        # rows with different offsets
+    if float(x.max()) < float(-x.min()):
+        x = -x                                         # the signed quantile of ratio 0 is the maximum: keep |min| below it
+    x = x.bfloat16()
+    thr, L, R, scale = O.get_statistics(x, 0, 0.0, 1.0, bits, "per-token", 0)
+    coo, stored_ref, _ = O.ref_compress(x, thr, scale, bits, 1.0, L, R)
+    assert coo.coalesce().values().numel() == 0        # no element outliers: the comparison is about the codes only
+    vals, stored, scales = O.hyc_compress(x[0], torch.tensor([], dtype=torch.int32), bits, H, rule="range")
+    assert bits_equal(scales.reshape(-1), scale.reshape(-1))
+    assert torch.equal(stored, stored_ref[0])
+
+
+def _roundtrip_rel_rms(x, bits, group, rule, k):
+    idx = O.hyc_select_channels(O.hyc_channel_scores(x), k)
+    vals, stored, scales = O.hyc_compress(x, idx, bits, group, rule)
+    xh = O.hyc_decompress(vals, stored, idx, scales, bits, group)
+    return float((xh.float() - x.float()).pow(2).mean().sqrt() / x.float().pow(2).mean().sqrt())
+
+
+def test_absmax_rule_roundtrip_error_is_bounded_on_uncentred_data():
+    """what the activation sites hold: zero-mean inputs, SiLU outputs, magnitudes.  The abs-max rule stays within
+    half a percent relative RMS at 8 bits and 8 % at 4 bits on all of them (the kept outlier channels included in the
+    norm); the range rule (no zero point) clips the one-sided ones and is off by 10 % even at 8 bits, which is why it is
+    not the default.  On zero-mean data the two rules give the same scale up to the asymmetry of the sample."""
+    gen = torch.Generator().manual_seed(70)
+    M, H, G, k = 64, 1024, 128, 10
+    z = torch.randn(M, H, generator=gen)
+    z[:, torch.randperm(H, generator=gen)[:k]] *= 20
+    cases = {"gaussian": z, "silu": torch.nn.functional.silu(z), "magnitude": z.abs()}
+    for name, t in cases.items():
+        t = t.bfloat16()
+        e8 = _roundtrip_rel_rms(t, 8, G, "absmax", k)
+        e4 = _roundtrip_rel_rms(t, 4, G, "absmax", k)
+        assert e8 < 0.006, (name, e8)
+        assert e4 < 0.08, (name, e4)
+    assert _roundtrip_rel_rms(cases["silu"].bfloat16(), 8, G, "range", k) > 0.05
+    assert _roundtrip_rel_rms(cases["magnitude"].bfloat16(), 8, G, "range", k) > 0.08
+    e2a = _roundtrip_rel_rms(cases["gaussian"].bfloat16(), 2, 64, "absmax", k)
+    e2r = _roundtrip_rel_rms(cases["gaussian"].bfloat16(), 2, 64, "range", k)
+    assert e2a < 0.26 and abs(e2a - e2r) < 0.05, (e2a, e2r)
+
+
 def test_ref_static_scale_idempotent():
     """with a static scale, compressing a decompressed tensor reproduces the same codes."""
     gen = torch.Generator().manual_seed(11)
@@ -182,12 +334,19 @@ def test_hyc_constant_group_is_defined():
     x = torch.zeros(2, 256).bfloat16()
     x[0, :128] = 3.0
     idx = torch.tensor([], dtype=torch.int32)
-    vals, stored, scales = O.hyc_compress(x, idx, 4, 128)
-    assert torch.all(scales == 0)
+    vals, stored, scales = O.hyc_compress(x, idx, 4, 128, rule="range")
+    assert torch.all(scales == 0)                   # max == min: the range rule has nothing to divide
     codes = O.unpack_codes(stored, 4)
     assert torch.all(codes[0, :128] == 15)          # 3/0 = +inf clamps to the top code
     assert torch.all(codes[0, 128:] == 8) and torch.all(codes[1] == 8)   # 0/0 is defined as q = 0
     assert torch.all(O.hyc_decompress(vals, stored, idx, scales, 4, 128) == 0)
+    # the abs-max rule keeps a constant group: 3 / (6/15) = 7.5 -> 8 -> clamped to 7, i.e. 7 * 0.4 = 2.8
+    vals, stored, scales = O.hyc_compress(x, idx, 4, 128, rule="absmax")
+    assert float(scales[0, 0]) == float(torch.tensor(6.0 / 15).bfloat16()) and torch.all(scales.flatten()[1:] == 0)
+    codes = O.unpack_codes(stored, 4)
+    assert torch.all(codes[0, :128] == 15) and torch.all(codes[0, 128:] == 8) and torch.all(codes[1] == 8)
+    xh = O.hyc_decompress(vals, stored, idx, scales, 4, 128)
+    assert torch.all((xh[0, :128].float() - 3.0).abs() <= 0.5 * 0.4 + 0.02) and torch.all(xh[1] == 0)
 
 
 # ------------------------------------------------------------------ RMSNorm
