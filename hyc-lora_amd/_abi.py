@@ -14,6 +14,7 @@ DTYPE_BF16, DTYPE_F32 = 0, 1
 ACT_SILU, ACT_GELU_TANH = 0, 1
 SCALE_RANGE, SCALE_ABSMAX = 0, 1
 ABI_VERSION = 2
+RMSNORM_BWD_STATIC_MAX_FLOATS = 4 * 1024 * 1024
 EINVAL, EFAULT, ENOTSUP, ELAUNCH = -22, -14, -95, -5
 
 c_i32, c_i64, c_f32, c_ptr = ctypes.c_int32, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
@@ -55,6 +56,8 @@ SIGNATURES = {
                                            c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr]),
     "hyc_rmsnorm_bwd": (c_i32, [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_i32, c_ptr, c_i64, c_i64,
                                 ctypes.POINTER(HycDesc), c_i32, c_ptr, c_ptr, c_ptr, c_ptr]),
+    "hyc_rmsnorm_bwd_static": (c_i32, [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_i32, c_ptr, c_i64, c_i64,
+                                       ctypes.POINTER(HycDesc), c_i32, c_ptr, c_ptr, c_ptr]),
     "hyc_layernorm_bwd": (c_i32, [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_i32, c_ptr, c_ptr, c_i64, c_i64,
                                   ctypes.POINTER(HycDesc), c_ptr, c_ptr, c_ptr, c_ptr]),
     "hyc_act_bwd": (c_i32, [c_i32, c_ptr, c_ptr, c_ptr, c_ptr, c_i64, c_i64, ctypes.POINTER(HycDesc), c_ptr, c_ptr]),

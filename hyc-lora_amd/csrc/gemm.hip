@@ -193,7 +193,6 @@ k_gradw(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_out, 
 // ------------------------------------------------------------------------------------------------
 constexpr int DK = 32;     // tokens per step = one MFMA k-step
 
-typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 typedef float floatx4_t __attribute__((ext_vector_type(4)));
 
 struct DirectArgs {
@@ -653,25 +652,6 @@ constexpr int WN = 128;     // dY features per workgroup: WN (four waves) or 2*W
 constexpr int WH = 256;     // channels per workgroup
 constexpr int WPAD = 32;    // row padding of the wide kernel's LDS tiles, in elements
 
-// Buffer loads: a resource is (base, bytes); an offset at or beyond `bytes` reads as zero instead of faulting.
-typedef __amdgpu_buffer_rsrc_t BufferRsrc;
-typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
-typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ BufferRsrc make_rsrc(const void* base, uint32_t bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
-}
-__device__ __forceinline__ uint4 load_b128(BufferRsrc r, uint32_t off) {
-  const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, 0);
-  return make_uint4(v.x, v.y, v.z, v.w);
-}
-__device__ __forceinline__ uint2 load_b64(BufferRsrc r, uint32_t off) {
-  const u32x2_t v = __builtin_amdgcn_raw_buffer_load_b64(r, (int)off, 0, 0);
-  return make_uint2(v.x, v.y);
-}
-__device__ __forceinline__ uint32_t load_b16(BufferRsrc r, uint32_t off) {
-  return (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(r, (int)off, 0, 0);
-}
-
 template <int NSEG, int A_PER, int B_PER>
 struct WideRegs {            // one stage of global data per thread
   uint4 a[A_PER];            // dY chunks
@@ -740,7 +720,6 @@ k_gradw_wide(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_
   // is a per-thread constant.
   const uint32_t gpr = (uint32_t)ca.groups_per_row, kk2 = 2u * (uint32_t)ca.k;
   const uint32_t b_pitch = (SRC == 0) ? (uint32_t)SEG : 2u * (uint32_t)H;          // bytes per token of the x operand
-  constexpr uint32_t NOWHERE = 0x80000000u;              // beyond any resource of at most 2 GiB
   uint32_t va[A_PER], vb[B_PER], vs[B_PER][NST], vo0[B_PER][NST], vo1[B_PER][NST];
 #pragma unroll
   for (int u = 0; u < A_PER; ++u) {

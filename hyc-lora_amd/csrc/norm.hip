@@ -1,6 +1,8 @@
 // RMSNorm forward fused with the compression of its input, and RMSNorm backward fused with the
 // decompression.  A row lives in registers (x is read from HBM once); the next row's loads are issued before the
 // current row is processed so that memory requests stay in flight during the arithmetic.
+#include <atomic>
+
 #include "abi_util.hpp"
 #include "row_kernels.hpp"
 
@@ -160,6 +162,38 @@ k_rmsnorm_fwd_fast(const uint16_t* __restrict__ x, const void* __restrict__ w, f
   }
 }
 
+// ---- rows staged through LDS -------------------------------------------------------------------------------------
+// gfx950 can load 16 bytes per lane from memory straight into LDS (global_load_lds_dwordx4: lane i of a wave lands at
+// the wave's LDS base + 16 i).  A wave uses that as a prefetch queue of its own: the incoming-gradient chunks of the
+// rows it will process next wait in LDS, not in registers, so several rows can be in flight per wave at no cost in
+// occupancy.  Every wave only ever reads what it requested itself, so no barrier guards the queue.
+//
+// Completion: vector memory operations of a wave complete in issue order.  The small per-row loads that go to
+// registers (codes, scales, outlier values, rstd) are issued AFTER the queue entry of the same row, and a queue entry
+// is read only after one of those registers has been used, so the compiler's own wait for that register covers the
+// entry.  The LDS reads are written in assembly: a read the compiler can see would make it wait for EVERY outstanding
+// load into the queue array (it cannot tell the stages apart), which would undo the prefetch.
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+typedef const __attribute__((address_space(1))) void* gbl_void_ptr;
+constexpr int RING_D = 3;                                             // rows per wave in the queue: being read, next, after next
+
+__device__ __forceinline__ uint32_t lds_offset(const void* p) {
+  return (uint32_t)(size_t)(__attribute__((address_space(3))) const char*)p;
+}
+// NSEG chunks of 16 bytes per lane, 1 KB apart, at LDS byte address `addr` (this lane's); `after` is any register
+// whose load was issued after the queue entry: naming it here keeps this read behind the wait for it
+template <int NSEG>
+__device__ __forceinline__ void queue_read(uint32_t addr, uint32_t after, uint4 (&g)[NSEG]) {
+  u32x4_t a, b = {0, 0, 0, 0};
+  if (NSEG == 2)
+    asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %2 offset:1024\n\ts_waitcnt lgkmcnt(0)"
+                 : "=&v"(a), "=&v"(b) : "v"(addr), "v"(after) : "memory");
+  else
+    asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=&v"(a) : "v"(addr), "v"(after) : "memory");
+  g[0] = make_uint4(a.x, a.y, a.z, a.w);
+  if (NSEG == 2) g[NSEG - 1] = make_uint4(b.x, b.y, b.z, b.w);
+}
+
 // Backward fast path.  A workgroup is `slots` row slots of CPS threads; slot s of workgroup b handles rows
 // b*slots + s, + gridDim.x*slots, ...: the rows in flight across the chip are adjacent in memory (rows that are far
 // apart would crowd onto a few memory channels).  Each slot keeps its own dw accumulators; they are added through
@@ -170,194 +204,234 @@ template <int BITS, bool WF32, bool QUIRK, int MAXT, bool DENSE = false>
 __global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(4, 8)))
 k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ stored, const uint16_t* __restrict__ vals,
                    const uint16_t* __restrict__ scales, const void* __restrict__ w, const float* __restrict__ rstd,
-                   const float* __restrict__ mean, int64_t M, int64_t H, int T, int CPS, int slots, ChanArgs ca,
+                   const float* __restrict__ mean, int64_t M, int64_t H, int T, int CPS, int slots, int steps, ChanArgs ca,
                    uint16_t* __restrict__ dx, float* __restrict__ dw_partials) {
   // A thread decodes at most two segments of its packed word: with four segments (2-bit codes) two threads share
   // a word, which keeps the per-thread state (and so the occupancy) the same for every bit width.
   constexpr int NSEG = Q<BITS>::NSEG > 2 ? 2 : Q<BITS>::NSEG;         // segments per thread
   constexpr int PARTS = Q<BITS>::NSEG / NSEG;                         // threads per packed word
-  __shared__ float red[2][16][2][16];                                 // [parity][slot][value][wave]
+  constexpr int STAGE_B = MAXT * NSEG * 16;                           // bytes of one queue stage of the workgroup
+  __shared__ float red[2][4][2][16];                                  // [parity][slot][value][wave]
+  __shared__ __align__(16) uint4 queue[RING_D * MAXT * NSEG];         // [stage][wave][segment][lane]: dy chunks on their way in
   // dynamic LDS: the weight row as fp32 [segment][half chunk][CPS] float4 (read again for every row: sixteen
-  // registers fewer than keeping the thread's weights live), then [slots-1][T][8] floats for the final dw sum
+  // registers fewer than keeping the thread's weights live)
   extern __shared__ __align__(16) float lds_dyn[];
   float4* wl4 = reinterpret_cast<float4*>(lds_dyn);
-  float* xslot = lds_dyn + H;
   // T = PARTS*CPS rounded up to whole waves, so the slot is the same for a whole wave: row bases stay scalar
-  const int slot = __builtin_amdgcn_readfirstlane((int)threadIdx.x / T);
+  // (at most four slots and two threads per packed word: comparisons instead of integer divisions)
+  const int tid_u = __builtin_amdgcn_readfirstlane((int)threadIdx.x & ~63);
+  const int slot = (tid_u >= T) + (tid_u >= 2 * T) + (tid_u >= 3 * T);
   const int u = (int)threadIdx.x - slot * T;
   const bool active = u < PARTS * CPS;
-  const int part = PARTS > 1 ? u / CPS : 0, c = u - part * CPS;
+  const int part = (PARTS > 1 && u >= CPS) ? 1 : 0, c = u - part * CPS;
+  static_assert(PARTS <= 2, "two threads per packed word at most");
   const int seg0 = part * NSEG;                                       // first segment of this thread
   const int SEG = CPS * 8;                                            // channels per segment = bytes per stored row
   const float invH = 1.0f / (float)H;
   const int wave = u >> 6, nw = T >> 6;
   const int seg_groups = CPS >> ca.chunk_to_group_shift;
-  // byte offsets of the thread inside a row of each tensor; 32 bits, added to a scalar row base by the load itself
-  const uint32_t xo = (uint32_t)(seg0 * SEG + 8 * c) * 2u;
-  const uint32_t so = 8u * (uint32_t)c;
-  const uint32_t go = (uint32_t)(seg0 * seg_groups + (c >> ca.chunk_to_group_shift)) * 2u;
-  const int64_t seg_b = (int64_t)SEG * 2, grp_b = (int64_t)seg_groups * 2;
+  // Byte offsets of the thread inside a row of each tensor.  Every memory instruction of the row loop is a buffer
+  // operation on a resource that spans one row (zero bytes for a row past the end), and lanes past the end of the
+  // row (the tail of a slot's last wave) carry the offset NOWHERE: nothing is predicated or branched on.
+  const uint32_t xo = active ? (uint32_t)(seg0 * SEG + 8 * c) * 2u : NOWHERE;
+  const uint32_t so = active ? 8u * (uint32_t)c : NOWHERE;
+  const uint32_t go = active ? (uint32_t)(seg0 * seg_groups + (c >> ca.chunk_to_group_shift)) * 2u : NOWHERE;
+  const uint32_t seg_b = (uint32_t)SEG * 2u, grp_b = (uint32_t)seg_groups * 2u;
+  const uint32_t row_b = (uint32_t)H * 2u, sc_b = (uint32_t)ca.groups_per_row * 2u, val_b = (uint32_t)ca.k * 2u;
+  // the wave's place in a queue stage, and this lane's
+  const int wv = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+  char* const qwave = reinterpret_cast<char*>(queue) + wv * (NSEG * 1024);
+  const uint32_t qlane = lds_offset(queue) + (uint32_t)(wv * (NSEG * 1024)) + 16u * (threadIdx.x & 63);
 
+  const uint32_t wbase = active ? (uint32_t)(seg0 * 2 * CPS + c) : 0u;
+  const int64_t stride = (int64_t)gridDim.x * slots;
+  int64_t row = (int64_t)blockIdx.x * slots + slot;
+  // (steps = ceil(M / stride), the same for every slot so that barriers stay matched; divided on the host)
+  // row r of a tensor whose rows are `bytes` long, as a resource; empty when the row does not exist
+  auto row_of = [&](const void* base, int64_t r, uint32_t bytes) __attribute__((always_inline)) {
+    return make_rsrc(static_cast<const char*>(base) + r * (int64_t)bytes, r < M ? bytes : 0u);
+  };
+  // the dy chunks of row r into queue stage `stage_b` (a byte offset)
+  auto request_dy = [&](int64_t r, int stage_b) __attribute__((always_inline)) {
+    const BufferRsrc rs_g = row_of(dy, r, row_b);
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) load_b128_to_lds(rs_g, xo + (uint32_t)i * seg_b, qwave + stage_b + i * 1024);
+  };
+
+  uint2 pk = make_uint2(0, 0);
+  uint4 xraw[NSEG];                                                   // DENSE: the activation chunks of this row
+  uint32_t sc[NSEG];   // one register each: a packed pair would be assembled right after the load and stall on it
+  uint32_t o0[NSEG], o1[NSEG];
+  uint32_t vo0[NSEG], vo1[NSEG];                                      // offsets of the chunk's first two outlier values
+  float rs = 0.f, mu = 0.f;                                           // mu: LayerNorm's row mean (0 for RMSNorm)
+  const uint16_t* vrow = vals;                                        // outlier values of the current row
+  // the small operands of row r, to registers: codes, scales, rstd ...
+  auto request_codes = [&](int64_t r) __attribute__((always_inline)) {
+    // (vector loads although rstd is the same for the whole slot: a scalar load in flight would turn every wait for
+    // an LDS read into a wait for it, too)
+    rs = __uint_as_float(load_b32(row_of(rstd, r, 4u), 0u));
+    if (mean) mu = __uint_as_float(load_b32(row_of(mean, r, 4u), 0u));
+    if (DENSE) {
+      const BufferRsrc rs_x = row_of(stored, r, row_b);
+#pragma unroll
+      for (int i = 0; i < NSEG; ++i) xraw[i] = load_b128(rs_x, xo + (uint32_t)i * seg_b);
+    } else {
+      pk = load_b64(row_of(stored, r, (uint32_t)SEG), so);
+      const BufferRsrc rs_c = row_of(scales, r, sc_b);
+#pragma unroll
+      for (int i = 0; i < NSEG; ++i) sc[i] = load_b16(rs_c, go + (uint32_t)i * grp_b);
+    }
+  };
+  // ... and the chunk's first two outlier values (needs the selectors)
+  auto request_outliers = [&](int64_t r) __attribute__((always_inline)) {
+    if (!DENSE) {
+      const BufferRsrc rs_v = row_of(vals, r, val_b);
+#pragma unroll
+      for (int i = 0; i < NSEG; ++i) { o0[i] = load_b16(rs_v, vo0[i]); o1[i] = load_b16(rs_v, vo1[i]); }
+      vrow = vals + (r < M ? r : M - 1) * ca.k;
+    }
+  };
+
+  // What the row loop needs first is asked for first: the thread's plan words and (first slot) its weights; then the
+  // first two rows of dy and the first row's codes, which travel while the plan is turned into selectors and the
+  // weight row goes to LDS; the first row's outlier values last (their place follows from the selectors).  Row 0's
+  // registers are requested after row 0's queue entry, see above (row 1's entry is older too, so the first row waits
+  // for both; they were requested together).
   uint32_t plan[NSEG];
-  float acc[NSEG][8];
+  float acc[NSEG][8], wv8[NSEG][8];
 #pragma unroll
   for (int i = 0; i < NSEG; ++i) {
     plan[i] = 0;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc[i][j] = 0.f;
+    for (int j = 0; j < 8; ++j) { acc[i][j] = 0.f; wv8[i][j] = 0.f; }
     if (active) {
       if (!DENSE) plan[i] = ca.plan[(seg0 + i) * CPS + c];
-      if (slot == 0) {
-        float wv[8];
-        load_w8t<WF32>(w, (int64_t)(seg0 + i) * SEG + 8 * c, wv);
-        wl4[((seg0 + i) * 2 + 0) * CPS + c] = make_float4(wv[0], wv[1], wv[2], wv[3]);
-        wl4[((seg0 + i) * 2 + 1) * CPS + c] = make_float4(wv[4], wv[5], wv[6], wv[7]);
-      }
+      if (slot == 0) load_w8t<WF32>(w, (int64_t)(seg0 + i) * SEG + 8 * c, wv8[i]);
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  request_dy(row, 0);
+  request_dy(row + stride, STAGE_B);
+  __builtin_amdgcn_sched_barrier(0);
+  request_codes(row);
+  __builtin_amdgcn_sched_barrier(0);
+  if (active && slot == 0) {
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) {
+      wl4[((seg0 + i) * 2 + 0) * CPS + c] = make_float4(wv8[i][0], wv8[i][1], wv8[i][2], wv8[i][3]);
+      wl4[((seg0 + i) * 2 + 1) * CPS + c] = make_float4(wv8[i][4], wv8[i][5], wv8[i][6], wv8[i][7]);
     }
   }
   ChunkOutliers<NSEG> co;
   co.init(plan);
-  __syncthreads();                                                    // the weight row is in LDS
-  const uint32_t wbase = active ? (uint32_t)(seg0 * 2 * CPS + c) : 0u;
-  const int64_t stride = (int64_t)gridDim.x * slots;
-  int64_t row = (int64_t)blockIdx.x * slots + slot;
-  const int64_t steps = (M + stride - 1) / stride;                    // the same for every slot: barriers stay matched
-  const int64_t xstep = stride * H * 2, sstep = stride * SEG, vstep = stride * ca.k * 2, gstep = stride * ca.groups_per_row * 2;
-  const char* gq = reinterpret_cast<const char*>(dy) + row * H * 2;
-  char* dq = reinterpret_cast<char*>(dx) + row * H * 2;
-  const char* sq = reinterpret_cast<const char*>(stored) + row * SEG;
-  const char* vq = reinterpret_cast<const char*>(vals) + row * ca.k * 2;
-  const char* cq = reinterpret_cast<const char*>(scales) + row * ca.groups_per_row * 2;
-
-  uint2 pk = make_uint2(0, 0);
-  uint4 xraw[NSEG];                                                   // DENSE: the activation chunks of this row
-  uint4 graw[NSEG];
-  uint32_t sc[NSEG];   // one register each: a packed pair would be assembled right after the load and stall on it
-  uint32_t o0[NSEG], o1[NSEG];
-  float rs = 0.f, mu = 0.f;                                           // mu: LayerNorm's row mean (0 for RMSNorm)
 #pragma unroll
   for (int i = 0; i < NSEG; ++i) {
-    graw[i] = make_uint4(0, 0, 0, 0); xraw[i] = make_uint4(0, 0, 0, 0); sc[i] = 0; o0[i] = 0; o1[i] = 0;
+    vo0[i] = co.has0[i] ? co.vb[i] : NOWHERE;
+    vo1[i] = co.has1[i] ? co.vb[i] + 2u : NOWHERE;
   }
-  const char* xq = reinterpret_cast<const char*>(stored) + row * H * 2;      // DENSE only
-  if (row < M && active) {
-    rs = rstd[row];
-    if (mean) mu = mean[row];
-#pragma unroll
-    for (int i = 0; i < NSEG; ++i) graw[i] = *reinterpret_cast<const uint4*>(gq + i * seg_b + xo);
-    if (DENSE) {
-#pragma unroll
-      for (int i = 0; i < NSEG; ++i) xraw[i] = *reinterpret_cast<const uint4*>(xq + i * seg_b + xo);
-    } else {
-      pk = *reinterpret_cast<const uint2*>(sq + so);
-#pragma unroll
-      for (int i = 0; i < NSEG; ++i) sc[i] = *reinterpret_cast<const uint16_t*>(cq + i * grp_b + go);
-      co.request(reinterpret_cast<const uint16_t*>(vq), o0, o1);
-    }
-  }
+  request_outliers(row);
+  __builtin_amdgcn_sched_barrier(0);
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");     // the weight row is in LDS (no wait for the queue)
+  int st_b = 0;                                                       // queue stage of the current row, as a byte offset
   int parity = 0;
-  for (int64_t step = 0; step < steps; ++step, row += stride, parity ^= 1) {
-    const bool valid = row < M && active;
-    const bool more = row + stride < M && active;
-    uint4 g_n[NSEG];                                                  // the bulk of the next row: requested a row ahead
-    float rs_n = 0.f, mu_n = 0.f;
-#pragma unroll
-    for (int i = 0; i < NSEG; ++i) g_n[i] = make_uint4(0, 0, 0, 0);
-    if (more) {
-      rs_n = rstd[row + stride];
-      if (mean) mu_n = mean[row + stride];
-#pragma unroll
-      for (int i = 0; i < NSEG; ++i) g_n[i] = *reinterpret_cast<const uint4*>(gq + xstep + i * seg_b + xo);
-    }
+  for (int step = 0; step < steps; ++step, row += stride, parity ^= 1) {
+    const bool live = row < M;                                        // the same for the whole slot
     float xn[NSEG][8], wdy[NSEG][8];
     float p1 = 0.f, p2 = 0.f;
-    const float nm = -mu * rs;                                        // xn = (x_hat - mean) * rstd as one fma
+    const float rs_c = rs;
+    if (live) {
+      const float nm = -mu * rs;                                      // xn = (x_hat - mean) * rstd as one fma
+      uint4 graw[NSEG];
+      queue_read<NSEG>(qlane + (uint32_t)st_b, DENSE ? xraw[0].x : sc[0], graw);
 #pragma unroll
-    for (int i = 0; i < NSEG; ++i) {
-      float g[8];
-      unpack8(graw[i], g);
-      if (DENSE) {
-        unpack8(xraw[i], xn[i]);
-      } else {
-        const float sf = bf_to_f((uint16_t)sc[i]);
-        uint4 r = co.splice(i, dequant8<BITS>(pk.x, pk.y, seg0 + i, sf), o0[i], o1[i], sf);
-        if (co.more_pairs)
-          r = splice_more(r, co.more_pairs, ca.plan[(seg0 + i) * CPS + c], reinterpret_cast<const uint16_t*>(vq), valid, sf);
-        unpack8(r, xn[i]);
-      }
-      uint32_t wo = wbase + (uint32_t)(i * 2 * CPS);
-      asm volatile("" : "+v"(wo));                                    // re-read per row: do not keep the weights live
-      const float4 wa = wl4[wo], wb = wl4[wo + CPS];
-      const float wv[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
+      for (int i = 0; i < NSEG; ++i) {
+        float g[8];
+        unpack8(graw[i], g);
+        if (DENSE) {
+          unpack8(xraw[i], xn[i]);
+        } else {
+          const float sf = bf_to_f((uint16_t)sc[i]);
+          uint4 r = co.splice(i, dequant8<BITS>(pk.x, pk.y, seg0 + i, sf), o0[i], o1[i], sf);
+          if (co.more_pairs) r = splice_more(r, co.more_pairs, ca.plan[(seg0 + i) * CPS + c], vrow, active, sf);
+          unpack8(r, xn[i]);
+        }
+        uint32_t wo = wbase + (uint32_t)(i * 2 * CPS);
+        asm volatile("" : "+v"(wo));                                  // re-read per row: do not keep the weights live
+        const float4 wa = wl4[wo], wb = wl4[wo + CPS];
+        const float wv8[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const float n = __builtin_fmaf(xn[i][j], rs, nm);
-        const float t = wv[j] * g[j];
-        xn[i][j] = n;
-        wdy[i][j] = t;
-        p1 = __builtin_fmaf(n, t, p1);
-        if (QUIRK) p2 += t;
-        acc[i][j] = __builtin_fmaf(g[j], n, acc[i][j]);
+        for (int j = 0; j < 8; ++j) {
+          const float n = __builtin_fmaf(xn[i][j], rs, nm);
+          const float t = wv8[j] * g[j];
+          xn[i][j] = n;
+          wdy[i][j] = t;
+          p1 = __builtin_fmaf(n, t, p1);
+          if (QUIRK) p2 += t;
+          acc[i][j] = __builtin_fmaf(g[j], n, acc[i][j]);
+        }
       }
+      // lanes past the end of the row hold whatever their queue entries and registers happened to contain
+      p1 = active ? p1 : 0.f;
+      if (QUIRK) p2 = active ? p2 : 0.f;
     }
-    // The compressed row is decoded: its registers take the next row's codes, scales and outliers now (a row's
-    // worth of registers less than requesting them at the top; the barrier and the second pass cover the latency).
-    if (more) {
-      if (DENSE) {
-#pragma unroll
-        for (int i = 0; i < NSEG; ++i) xraw[i] = *reinterpret_cast<const uint4*>(xq + xstep + i * seg_b + xo);
-      } else {
-        pk = *reinterpret_cast<const uint2*>(sq + sstep + so);
-#pragma unroll
-        for (int i = 0; i < NSEG; ++i) sc[i] = *reinterpret_cast<const uint16_t*>(cq + gstep + i * grp_b + go);
-        co.request(reinterpret_cast<const uint16_t*>(vq + vstep), o0, o1);
-      }
-    }
+    // The row is decoded: its registers take the next row's codes, scales and outliers now, and the row after that
+    // goes into the queue stage that was read two rows ago.  Order matters, see above.
+    __builtin_amdgcn_sched_barrier(0);
+    request_codes(row + stride);
+    request_outliers(row + stride);
+    __builtin_amdgcn_sched_barrier(0);
+    request_dy(row + 2 * stride, st_b >= STAGE_B ? st_b - STAGE_B : st_b + 2 * STAGE_B);
+    __builtin_amdgcn_sched_barrier(0);
     // two sums per slot, one barrier
     p1 = wave_sum(p1);
     if (QUIRK) p2 = wave_sum(p2);
     if ((u & 63) == 0) { red[parity][slot][0][wave] = p1; if (QUIRK) red[parity][slot][1][wave] = p2; }
-    __syncthreads();
+    // a bare barrier: __syncthreads() would also wait for every load on its way into the queue
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     float t1 = red[parity][slot][0][0], t2 = QUIRK ? red[parity][slot][1][0] : 0.f;
     for (int i = 1; i < nw; ++i) { t1 += red[parity][slot][0][i]; if (QUIRK) t2 += red[parity][slot][1][i]; }
     // dx = (wdy - (xn*c1 + c2)) * rstd, arranged as two fused multiply-adds
-    const float k1 = -(t1 * invH) * rs;
-    const float k2 = QUIRK ? -(t2 * invH) * rs : 0.f;
-    if (valid) {
+    const float k1 = -(t1 * invH) * rs_c;
+    const float k2 = QUIRK ? -(t2 * invH) * rs_c : 0.f;
+    const BufferRsrc rs_o = row_of(dx, row, row_b);
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) {
+      float o[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) o[j] = __builtin_fmaf(xn[i][j], k1, __builtin_fmaf(wdy[i][j], rs_c, k2));
+      store_b128_stream(rs_o, xo + (uint32_t)i * seg_b, pack8(o));
+    }
+    st_b = st_b >= 2 * STAGE_B ? 0 : st_b + STAGE_B;
+  }
+  // The slots' dw sums are added in slot order through the queue's memory, which nobody reads any more.
+  float* pr = dw_partials + (int64_t)blockIdx.x * H + (int64_t)seg0 * SEG + 8 * c;
+  if (slots > 1) {
+    float4* xs = reinterpret_cast<float4*>(queue);                     // [slots-1][T][NSEG][2] float4
+    __syncthreads();
+    if (slot > 0) {
 #pragma unroll
       for (int i = 0; i < NSEG; ++i) {
-        float o[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) o[j] = __builtin_fmaf(xn[i][j], k1, __builtin_fmaf(wdy[i][j], rs, k2));
-        store_stream(reinterpret_cast<uint16_t*>(dq + i * seg_b + xo), pack8(o));
-      }
-    }
-    rs = rs_n; mu = mu_n;
-#pragma unroll
-    for (int i = 0; i < NSEG; ++i) graw[i] = g_n[i];
-    gq += xstep; dq += xstep; sq += sstep; vq += vstep; cq += gstep; xq += xstep;
-  }
-  float* pr = dw_partials + (int64_t)blockIdx.x * H + (int64_t)seg0 * SEG + 8 * c;
-#pragma unroll
-  for (int i = 0; i < NSEG; ++i) {
-    if (slots > 1) {
-      __syncthreads();
-      if (slot > 0) {
-        float4* o = reinterpret_cast<float4*>(xslot + ((int64_t)(slot - 1) * T + u) * 8);
+        float4* o = xs + (((int64_t)(slot - 1) * T + u) * NSEG + i) * 2;
         o[0] = make_float4(acc[i][0], acc[i][1], acc[i][2], acc[i][3]);
         o[1] = make_float4(acc[i][4], acc[i][5], acc[i][6], acc[i][7]);
       }
-      __syncthreads();
-      if (slot == 0) {
-        for (int s2 = 1; s2 < slots; ++s2) {
-          const float4* o = reinterpret_cast<const float4*>(xslot + ((int64_t)(s2 - 1) * T + u) * 8);
+    }
+    __syncthreads();
+    if (slot == 0) {
+      for (int s2 = 1; s2 < slots; ++s2) {
+#pragma unroll
+        for (int i = 0; i < NSEG; ++i) {
+          const float4* o = xs + (((int64_t)(s2 - 1) * T + u) * NSEG + i) * 2;
           const float4 a = o[0], b = o[1];
           acc[i][0] += a.x; acc[i][1] += a.y; acc[i][2] += a.z; acc[i][3] += a.w;
           acc[i][4] += b.x; acc[i][5] += b.y; acc[i][6] += b.z; acc[i][7] += b.w;
         }
       }
     }
-    if (slot == 0 && active) {
+  }
+  if (slot == 0 && active) {
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) {
       float4* o = reinterpret_cast<float4*>(pr + (int64_t)i * SEG);
       o[0] = make_float4(acc[i][0], acc[i][1], acc[i][2], acc[i][3]);
       o[1] = make_float4(acc[i][4], acc[i][5], acc[i][6], acc[i][7]);
@@ -740,6 +814,16 @@ static inline BwdShape bwd_shape(int64_t M, int bits, int cps, const NormGeom& n
   const int parts = bits == 2 ? 2 : 1;
   b.fast_T = ((parts * cps + 63) / 64) * 64;
   b.fast_ok = n.iters == 1 && bits != 1 && b.fast_T <= 1024;
+  if (b.fast_ok) {
+    // LDS of the fast kernel: the dy queue and the row sums (static, sized by the kernel's thread bound) and the
+    // weight row (dynamic); 160 KB per workgroup on gfx950
+    int fs0 = 1024 / b.fast_T;
+    if (fs0 > BWD_FAST_SLOTS_MAX) fs0 = BWD_FAST_SLOTS_MAX;
+    const int64_t maxt = fs0 * b.fast_T <= 256 ? 256 : 1024, nseg = bits == 8 ? 1 : 2;
+    const int64_t H = (int64_t)cps * 64 / bits;
+    const int64_t lds = RING_D * maxt * nseg * 16 + 1024 + H * 4;
+    b.fast_ok = lds <= 160 * 1024;
+  }
   b.slots = n.T <= 256 ? BWD_SLOTS_SMALL : 1;
   b.threads = b.slots * n.T;
   // about a thousand row slots in flight; each walks at least four rows so the partial rows stay few
@@ -943,12 +1027,13 @@ static int norm_bwd_impl(const void* dy, const void* stored, const void* vals, c
     const size_t lds = b.slots > 1 ? (size_t)(b.slots - 1) * n.T * 8 * sizeof(float) : 0;
     if (fast) {
       const int fthreads = b.fast_slots * b.fast_T;
-      const size_t flds = (size_t)H * sizeof(float) +
-                          (b.fast_slots > 1 ? (size_t)(b.fast_slots - 1) * b.fast_T * 8 * sizeof(float) : 0);
+      const size_t flds = (size_t)H * sizeof(float);
+      const int64_t fstride = b.fast_P * b.fast_slots;
+      const int fsteps = (int)((M + fstride - 1) / fstride);
 #define HYC_BWD_FAST(B_, W_, Q_, MT_)                                                                              \
   hipLaunchKernelGGL((k_rmsnorm_bwd_fast<B_, W_, Q_, MT_>), dim3((unsigned)b.fast_P), dim3(fthreads), flds, st, gp,  \
                      static_cast<const uint8_t*>(stored), static_cast<const uint16_t*>(vals),                     \
-                     static_cast<const uint16_t*>(scales), w, rstd, mean, M, H, b.fast_T, g.cps, b.fast_slots, ca, \
+                     static_cast<const uint16_t*>(scales), w, rstd, mean, M, H, b.fast_T, g.cps, b.fast_slots, fsteps, ca, \
                      static_cast<uint16_t*>(dx), dw_partials)
 #define HYC_BWD_FAST_WQ(B_)                                                                   \
   do {                                                                                        \
@@ -968,7 +1053,7 @@ static int norm_bwd_impl(const void* dy, const void* stored, const void* vals, c
 #define HYC_BWD_DENSE(W_, Q_, MT_)                                                                                 \
   hipLaunchKernelGGL((k_rmsnorm_bwd_fast<4, W_, Q_, MT_, true>), dim3((unsigned)b.fast_P), dim3(fthreads), flds, st, gp, \
                      static_cast<const uint8_t*>(stored), static_cast<const uint16_t*>(vals),                     \
-                     static_cast<const uint16_t*>(scales), w, rstd, mean, M, H, b.fast_T, g.cps, b.fast_slots, ca, \
+                     static_cast<const uint16_t*>(scales), w, rstd, mean, M, H, b.fast_T, g.cps, b.fast_slots, fsteps, ca, \
                      static_cast<uint16_t*>(dx), dw_partials)
         switch ((wf32 ? 4 : 0) + (c2_quirk ? 2 : 0) + (fthreads <= 256 ? 0 : 1)) {
           case 0: HYC_BWD_DENSE(false, false, 256); break;
@@ -1020,6 +1105,49 @@ int hyc_rmsnorm_bwd(const void* dy, const void* stored, const void* vals, const 
                     int32_t w_dtype, const float* rstd, int64_t M, int64_t H, const hyc_desc* d, int32_t c2_quirk,
                     void* dx, float* dw_partials, void* dw, void* stream) {
   return norm_bwd_impl(dy, stored, vals, scales, w, w_dtype, rstd, nullptr, M, H, d, c2_quirk, dx, dw_partials, dw, stream);
+}
+
+// ---- the backward for callers that cannot allocate -------------------------------------------------------------
+// The fp32 partial rows of dw live in a file-scope device array instead of a caller buffer.  In host code the
+// array's name is only a handle: the address the kernels need is asked from the runtime once per device (each
+// device holds its own copy of the array) and kept.
+static __device__ __align__(256) float scratch[HYC_RMSNORM_BWD_STATIC_MAX_FLOATS];
+
+static int static_scratch(float** out) {
+  static std::atomic<float*> per_device[64];
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(HYC_ELAUNCH, "hyc_rmsnorm_bwd_static: hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= 64) return fail(HYC_ENOTSUP, "hyc_rmsnorm_bwd_static: device ordinal %d (0..63 are covered)", dev);
+  float* p = per_device[dev].load(std::memory_order_acquire);
+  if (!p) {
+    void* sym = nullptr;
+    e = hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !sym) {
+      (void)hipGetLastError();
+      return fail(HYC_ELAUNCH, "hyc_rmsnorm_bwd_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    }
+    p = static_cast<float*>(sym);
+    per_device[dev].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return HYC_OK;
+}
+
+int hyc_rmsnorm_bwd_static(const void* dy, const void* stored, const void* vals, const void* scales, const void* w,
+                           int32_t w_dtype, const float* rstd, int64_t M, int64_t H, const hyc_desc* d, int32_t c2_quirk,
+                           void* dx, void* dw, void* stream) {
+  if (!d) return fail(HYC_EFAULT, "hyc_rmsnorm_bwd_static: null descriptor");
+  if (M > 0 && !dw) return fail(HYC_EFAULT, "hyc_rmsnorm_bwd_static: dw is required (the partial rows are not the caller's)");
+  const int64_t rows = hyc_rmsnorm_bwd_partial_rows(M, H, d);
+  if (rows * H > (int64_t)HYC_RMSNORM_BWD_STATIC_MAX_FLOATS)
+    return fail(HYC_EINVAL, "hyc_rmsnorm_bwd_static: %lld partial rows of %lld floats exceed the static workspace of %lld floats; "
+                "use hyc_rmsnorm_bwd with a caller workspace", (long long)rows, (long long)H,
+                (long long)HYC_RMSNORM_BWD_STATIC_MAX_FLOATS);
+  float* partials = nullptr;
+  const int rc = static_scratch(&partials);
+  if (rc) return rc;
+  return norm_bwd_impl(dy, stored, vals, scales, w, w_dtype, rstd, nullptr, M, H, d, c2_quirk, dx, partials, dw, stream);
 }
 
 int hyc_layernorm_bwd(const void* dy, const void* stored, const void* vals, const void* scales, const void* w,

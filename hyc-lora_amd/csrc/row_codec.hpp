@@ -53,6 +53,41 @@ __device__ __forceinline__ void store_stream(uint16_t* p, const uint4& v) {
   __builtin_nontemporal_store(t, reinterpret_cast<u32x4_t*>(p));
 }
 
+// ---- buffer addressing ----------------------------------------------------------------------------
+// A resource is (base, bytes); a lane whose offset is at or beyond `bytes` reads zeros / has its store dropped
+// instead of faulting.  Kernels use that to keep their memory instructions unconditional: rows past the end get a
+// resource of zero bytes, lanes without data the offset NOWHERE.  (Straight-line code lets the compiler count the
+// operations in flight exactly, so it waits for the one it needs and no more.)
+typedef __amdgpu_buffer_rsrc_t BufferRsrc;
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+constexpr uint32_t NOWHERE = 0x80000000u;                // beyond any resource (sizes stay below 2 GiB)
+__device__ __forceinline__ BufferRsrc make_rsrc(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ uint4 load_b128(BufferRsrc r, uint32_t off) {
+  const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, 0);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ uint2 load_b64(BufferRsrc r, uint32_t off) {
+  const u32x2_t v = __builtin_amdgcn_raw_buffer_load_b64(r, (int)off, 0, 0);
+  return make_uint2(v.x, v.y);
+}
+__device__ __forceinline__ uint32_t load_b32(BufferRsrc r, uint32_t off) {
+  return (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(r, (int)off, 0, 0);
+}
+__device__ __forceinline__ uint32_t load_b16(BufferRsrc r, uint32_t off) {
+  return (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(r, (int)off, 0, 0);
+}
+// streaming 16-byte store (written once, not read again by this kernel)
+__device__ __forceinline__ void store_b128_stream(BufferRsrc r, uint32_t off, const uint4& v) {
+  const u32x4_t t = {v.x, v.y, v.z, v.w};
+  __builtin_amdgcn_raw_buffer_store_b128(t, r, (int)off, 0, 2);
+}
+// 16 bytes per lane from memory straight into LDS: lane i of the wave lands at `lds_wave_base` + 16 i
+__device__ __forceinline__ void load_b128_to_lds(BufferRsrc r, uint32_t off, void* lds_wave_base) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void*)lds_wave_base, 16, (int)off, 0, 0, 0);
+}
+
 // ---- cross-lane -------------------------------------------------------------------------------
 // value of another lane of the same 16-lane row.  OLD_ZERO: lanes without a source read 0 (lets the compiler fold
 // the move into v_add_f32_dpp).

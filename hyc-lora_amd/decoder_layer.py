@@ -288,7 +288,7 @@ class _AttentionFunc(torch.autograd.Function):
                 p, _ = K.softmax_fwd(scores, causal_period=s, inplace=True)
                 thr = get_statistics_softmax(p.view(b, nh, s, s), it, cfg.softmax_ratio)
                 mod.static_value = running_mean(mod.static_value, thr, it)
-                kept.append(K.softmax_sparsify(p, float(thr)))
+                kept.append(K.softmax_sparsify(p, K.threshold_value(thr)))
             del scores
             torch.bmm(p, v3[c0:c1], out=out3[c0:c1])
             if mod.record is not None:

@@ -53,6 +53,22 @@ def _need_weight(w, H):
     return w
 
 
+def threshold_value(t):
+    """Python float of a threshold.  A device tensor costs one host round trip the first time; the float is then kept
+    on the tensor object, so the frozen threshold of a calibrated module (the same 0-d tensor call after call) is
+    read back once, not at every step.  (A caller that changes such a tensor in place must drop `_hyc_float`.)"""
+    if not isinstance(t, torch.Tensor):
+        return float(t)
+    v = getattr(t, "_hyc_float", None)
+    if v is None:
+        v = float(t)
+        try:
+            t._hyc_float = v
+        except AttributeError:
+            pass
+    return v
+
+
 def num_outlier_channels(H, ratio):
     """k = floor(ratio*H + 1/2)"""
     import math

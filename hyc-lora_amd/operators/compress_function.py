@@ -87,7 +87,7 @@ def compress_to_csr(x, outlier, scale, sub_outlier_bit, sub_outlier_ratio, L, R)
     x = x.contiguous()
     S, H = x.shape[-2], x.shape[-1]
     rank0 = L is None or not bool(L.shape[-1]) or (L.shape[-1] == 16 and getattr(L, "_hyc_zero", False))
-    c = K.compress_threshold(x.reshape(-1, H), S, float(outlier), scale.contiguous(), sub_outlier_bit,
+    c = K.compress_threshold(x.reshape(-1, H), S, K.threshold_value(outlier), scale.contiguous(), sub_outlier_bit,
                              None if rank0 else L.contiguous(), None if rank0 else R.contiguous())
     return c, tuple(x.shape)
 

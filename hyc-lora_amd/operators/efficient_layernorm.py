@@ -56,7 +56,7 @@ class EfficientMemoryLayerNormFunc(torch.autograd.Function):
                 and K.layernorm_fwd_supported(x2.shape[-1], sub_outlier_bit)):
             w, b = _affine(weight, bias)
             y, mean, rstd, c = K.layernorm_fwd_compress_threshold(
-                x2, w, b, eps, x.shape[-2], float(outlier), scale.contiguous(), sub_outlier_bit,
+                x2, w, b, eps, x.shape[-2], K.threshold_value(outlier), scale.contiguous(), sub_outlier_bit,
                 L.contiguous() if rank > 0 else None, R.contiguous() if rank > 0 else None)
         else:
             y, mean, rstd = _forward_stats(x2, weight, bias, eps)

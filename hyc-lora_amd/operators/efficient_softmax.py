@@ -22,12 +22,12 @@ class EfficientMemorySoftmaxFunc(torch.autograd.Function):
         scores = x.contiguous()
         if iteration >= _CALIBRATION_CALLS:
             threshold = static_value
-            probs, ctx.kept = K.softmax_fwd(scores, float(threshold))
+            probs, ctx.kept = K.softmax_fwd(scores, K.threshold_value(threshold))
         else:
             # the threshold of this call comes from its own probabilities, so they are needed before the pruning
             probs, _ = K.softmax_fwd(scores)
             threshold = get_statistics_softmax(probs, iteration, outlier_ratio)
-            ctx.kept = K.softmax_sparsify(probs, float(threshold))
+            ctx.kept = K.softmax_sparsify(probs, K.threshold_value(threshold))
         ctx.mark_non_differentiable(threshold)
         return probs, threshold
 

@@ -24,6 +24,8 @@
  *   hyc_rmsnorm_bwd
  *       EfficientMemoryRMSNormFunc.backward + _rms_norm_bwd_dx_fused + _rms_norm_bwd_dwdb,
  *       operators/efficient_rmsnorm.py:215-269, :63-143
+ *   hyc_rmsnorm_bwd_static
+ *       no counterpart in the reference: hyc_rmsnorm_bwd for callers that cannot allocate (see its declaration)
  *   hyc_act_bwd
  *       EfficientMemorySiLUFunc.backward operators/efficient_silu.py:44-53,
  *       EfficientMemoryGELUFunc.backward operators/efficient_gelu.py:44-64,
@@ -175,6 +177,19 @@ int hyc_rmsnorm_fwd_compress(const void* x, const void* w, int32_t w_dtype, floa
 int hyc_rmsnorm_bwd(const void* dy, const void* stored, const void* vals, const void* scales, const void* w,
                     int32_t w_dtype, const float* rstd, int64_t M, int64_t H, const hyc_desc* d, int32_t c2_quirk,
                     void* dx, float* dw_partials, void* dw, void* stream);
+
+/* hyc_rmsnorm_bwd for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid allocation): the same kernels and results, but the fp32 partial rows of dw live in a device
+ * array inside the library, so there is no dw_partials argument and the call allocates nothing.  It has no counterpart
+ * in the reference.  Limits: hyc_rmsnorm_bwd_partial_rows(M, H, d) * H <= HYC_RMSNORM_BWD_STATIC_MAX_FLOATS (16 MiB of
+ * fp32; with 2- or 4-bit codes every width up to 16384 channels fits at any M: at most 256 rows), HYC_EINVAL beyond; dw must not be
+ * NULL.  Each GPU the library runs on holds its own 16 MiB array until the process ends; every call on a GPU uses that
+ * GPU's array, so two calls that overlap on one GPU (different streams) race: serialise them or use hyc_rmsnorm_bwd.
+ * The first call on a device asks the runtime for the array's address (no allocation, but make it outside a capture). */
+#define HYC_RMSNORM_BWD_STATIC_MAX_FLOATS (4 * 1024 * 1024)
+int hyc_rmsnorm_bwd_static(const void* dy, const void* stored, const void* vals, const void* scales, const void* w,
+                           int32_t w_dtype, const float* rstd, int64_t M, int64_t H, const hyc_desc* d, int32_t c2_quirk,
+                           void* dx, void* dw, void* stream);
 
 /* LayerNorm forward with the compression of x fused in (efficient_layernorm.py:15-61 kernel, :203-260 Function):
  * mean = sum(x)/H, rstd = 1/sqrt(sum((x-mean)^2)/H + eps) (both fp32 [M]), y = bf16(((x-mean)*rstd)*w + b); bias may be

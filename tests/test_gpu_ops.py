@@ -310,6 +310,31 @@ def test_rmsnorm_module(ops, K, mode):
     assert mod.iteration == 3
 
 
+@pytest.mark.parametrize("mode", ["ref", "hyc"])
+def test_rmsnorm_modules_with_different_settings_do_not_share_state(ops, K, mode):
+    """two modules that differ in ref_c2_quirk, their forwards interleaved before either backward runs: each backward
+    uses its own module's setting (the settings travel with the call, not through a class attribute)"""
+    B, S, H = 1, 32, 512
+    gen = torch.Generator().manual_seed(17)
+    kw = dict(eps=1e-6, bias=False, outlier_ratio=0.01, sub_outlier_ratio=1.0, sub_outlier_bit=8,
+              sub_outlier_quantize_method='per-token', rank=0, mode=mode, group_size=128)
+    mods = [ops.EfficientMemoryRMSNorm(H, ref_c2_quirk=q, **kw).cuda() for q in (True, False)]
+    x = torch.randn(B, S, H, generator=gen).bfloat16()
+    dy = (0.5 + 0.1 * torch.randn(B, S, H, generator=gen)).bfloat16()          # a non-zero mean makes the c2 term visible
+    xs = [x.cuda().requires_grad_(True) for _ in mods]
+    ys = [m(xi) for m, xi in zip(mods, xs)]                                     # both forwards first
+    saved = [y.grad_fn.saved for y in ys]
+    for y in ys:
+        y.backward(dy.cuda())
+    w = mods[0].weight.detach().cpu()
+    _, rstd_o = O.rmsnorm_fwd(x, w, 1e-6)
+    for quirk, xi, c in zip((True, False), xs, saved):
+        xh = (K.decompress_threshold(c) if mode == "ref" else K.decompress_channel(c)).cpu().reshape(B, S, H)
+        dx_o, _ = O.rmsnorm_bwd(dy, xh, w, rstd_o, c2_quirk=quirk)
+        assert torch.allclose(xi.grad.cpu().float(), dx_o.float(), rtol=1e-2, atol=1e-3)
+    assert not torch.allclose(xs[0].grad.float(), xs[1].grad.float(), rtol=1e-2, atol=1e-3)
+
+
 @pytest.mark.parametrize("mode,H", [("ref", 768), ("hyc", 768), ("hyc", 4096)])
 def test_layernorm_module(ops, K, mode, H):
     """EfficientMemoryLayerNorm (efficient_layernorm.py:333-405): y, dx, dw, db against the oracle on the activation the
