@@ -335,11 +335,12 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
   int st_b = 0;                                                       // queue stage of the current row, as a byte offset
   int parity = 0;
   for (int step = 0; step < steps; ++step, row += stride, parity ^= 1) {
-    const bool live = row < M;                                        // the same for the whole slot
     float xn[NSEG][8], wdy[NSEG][8];
     float p1 = 0.f, p2 = 0.f;
     const float rs_c = rs;
-    if (live) {
+    {
+      // (a row past the end, and lanes past the end of a row, have read zeros for every operand - queue entries
+      // included - so they add exact zeros to the sums below: no branch, no selects)
       const float nm = -mu * rs;                                      // xn = (x_hat - mean) * rstd as one fma
       uint4 graw[NSEG];
       queue_read<NSEG>(qlane + (uint32_t)st_b, DENSE ? xraw[0].x : sc[0], graw);
@@ -350,19 +351,20 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
         if (DENSE) {
           unpack8(xraw[i], xn[i]);
         } else {
-          const float sf = bf_to_f((uint16_t)sc[i]);
-          uint4 r = co.splice(i, dequant8<BITS>(pk.x, pk.y, seg0 + i, sf), o0[i], o1[i], sf);
-          if (co.more_pairs) r = splice_more(r, co.more_pairs, ca.plan[(seg0 + i) * CPS + c], vrow, active, sf);
+          // dx and dw are compared to a tolerance: the lean decode (scales of 1e30 and beyond and the sign of a zero
+          // outlier are not its concern)
+          uint4 r = co.splice_value(i, dequant8_fast<BITS>(pk.x, pk.y, seg0 + i, bf_to_f((uint16_t)sc[i])), o0[i], o1[i]);
+          if (co.more_pairs) r = splice_more(r, co.more_pairs, ca.plan[(seg0 + i) * CPS + c], vrow, active, 1.f);
           unpack8(r, xn[i]);
         }
         uint32_t wo = wbase + (uint32_t)(i * 2 * CPS);
         asm volatile("" : "+v"(wo));                                  // re-read per row: do not keep the weights live
         const float4 wa = wl4[wo], wb = wl4[wo + CPS];
-        const float wv8[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
+        const float wv[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           const float n = __builtin_fmaf(xn[i][j], rs, nm);
-          const float t = wv8[j] * g[j];
+          const float t = wv[j] * g[j];
           xn[i][j] = n;
           wdy[i][j] = t;
           p1 = __builtin_fmaf(n, t, p1);
@@ -370,9 +372,6 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
           acc[i][j] = __builtin_fmaf(g[j], n, acc[i][j]);
         }
       }
-      // lanes past the end of the row hold whatever their queue entries and registers happened to contain
-      p1 = active ? p1 : 0.f;
-      if (QUIRK) p2 = active ? p2 : 0.f;
     }
     // The row is decoded: its registers take the next row's codes, scales and outliers now, and the row after that
     // goes into the queue stage that was read two rows ago.  Order matters, see above.
@@ -797,6 +796,9 @@ static inline int norm_geom(int cps, NormGeom* n) {
 #ifndef BWD_FAST_SLOTS_MAX
 #define BWD_FAST_SLOTS_MAX 4
 #endif
+#ifndef HYC_BWD_BIG
+#define HYC_BWD_BIG 1024
+#endif
 #ifndef BWD_SLOTS_SMALL
 #define BWD_SLOTS_SMALL 1
 #endif
@@ -819,10 +821,11 @@ static inline BwdShape bwd_shape(int64_t M, int bits, int cps, const NormGeom& n
     // weight row (dynamic); 160 KB per workgroup on gfx950
     int fs0 = 1024 / b.fast_T;
     if (fs0 > BWD_FAST_SLOTS_MAX) fs0 = BWD_FAST_SLOTS_MAX;
-    const int64_t maxt = fs0 * b.fast_T <= 256 ? 256 : 1024, nseg = bits == 8 ? 1 : 2;
+    const int64_t maxt = fs0 * b.fast_T <= 256 ? 256 : HYC_BWD_BIG, nseg = bits == 8 ? 1 : 2;
+    if (fs0 * b.fast_T > HYC_BWD_BIG) b.fast_ok = false;
     const int64_t H = (int64_t)cps * 64 / bits;
     const int64_t lds = RING_D * maxt * nseg * 16 + 1024 + H * 4;
-    b.fast_ok = lds <= 160 * 1024;
+    b.fast_ok = b.fast_ok && lds <= 160 * 1024;
   }
   b.slots = n.T <= 256 ? BWD_SLOTS_SMALL : 1;
   b.threads = b.slots * n.T;
@@ -1040,13 +1043,13 @@ static int norm_bwd_impl(const void* dy, const void* stored, const void* vals, c
     const int key_ = (wf32 ? 4 : 0) + (c2_quirk ? 2 : 0) + (fthreads <= 256 ? 0 : 1);        \
     switch (key_) {                                                                           \
       case 0: HYC_BWD_FAST(B_, false, false, 256); break;                                     \
-      case 1: HYC_BWD_FAST(B_, false, false, 1024); break;                                    \
+      case 1: HYC_BWD_FAST(B_, false, false, HYC_BWD_BIG); break;                                    \
       case 2: HYC_BWD_FAST(B_, false, true, 256); break;                                      \
-      case 3: HYC_BWD_FAST(B_, false, true, 1024); break;                                     \
+      case 3: HYC_BWD_FAST(B_, false, true, HYC_BWD_BIG); break;                                     \
       case 4: HYC_BWD_FAST(B_, true, false, 256); break;                                      \
-      case 5: HYC_BWD_FAST(B_, true, false, 1024); break;                                     \
+      case 5: HYC_BWD_FAST(B_, true, false, HYC_BWD_BIG); break;                                     \
       case 6: HYC_BWD_FAST(B_, true, true, 256); break;                                       \
-      default: HYC_BWD_FAST(B_, true, true, 1024); break;                                     \
+      default: HYC_BWD_FAST(B_, true, true, HYC_BWD_BIG); break;                                     \
     }                                                                                         \
   } while (0)
       if (dense_fast) {
@@ -1057,13 +1060,13 @@ static int norm_bwd_impl(const void* dy, const void* stored, const void* vals, c
                      static_cast<uint16_t*>(dx), dw_partials)
         switch ((wf32 ? 4 : 0) + (c2_quirk ? 2 : 0) + (fthreads <= 256 ? 0 : 1)) {
           case 0: HYC_BWD_DENSE(false, false, 256); break;
-          case 1: HYC_BWD_DENSE(false, false, 1024); break;
+          case 1: HYC_BWD_DENSE(false, false, HYC_BWD_BIG); break;
           case 2: HYC_BWD_DENSE(false, true, 256); break;
-          case 3: HYC_BWD_DENSE(false, true, 1024); break;
+          case 3: HYC_BWD_DENSE(false, true, HYC_BWD_BIG); break;
           case 4: HYC_BWD_DENSE(true, false, 256); break;
-          case 5: HYC_BWD_DENSE(true, false, 1024); break;
+          case 5: HYC_BWD_DENSE(true, false, HYC_BWD_BIG); break;
           case 6: HYC_BWD_DENSE(true, true, 256); break;
-          default: HYC_BWD_DENSE(true, true, 1024); break;
+          default: HYC_BWD_DENSE(true, true, HYC_BWD_BIG); break;
         }
 #undef HYC_BWD_DENSE
       }

@@ -292,6 +292,9 @@ __device__ __forceinline__ uint4 dequant8(uint32_t lo, uint32_t hi, int seg, flo
   uint32_t a, b;
   if (BITS == 8) { a = lo ^ REP; b = hi ^ REP; }             // int8 -> biased unsigned (q + 128)
   else { a = (lo >> (seg * BITS)) & REP; b = (hi >> (seg * BITS)) & REP; }
+  // opaque from here on: the four codes of a word are then converted by v_cvt_f32_ubyte0..3, one instruction each
+  // (left to itself the compiler extracts every field from the packed word first: two instructions per code)
+  asm volatile("" : "+v"(a), "+v"(b));
   float c[8] = {(float)(a & 0xFFu), (float)((a >> 8) & 0xFFu), (float)((a >> 16) & 0xFFu), (float)(a >> 24),
                 (float)(b & 0xFFu), (float)((b >> 8) & 0xFFu), (float)((b >> 16) & 0xFFu), (float)(b >> 24)};
   constexpr float OFFV = (BITS == 8) ? 128.f : (float)Q<BITS>::OFF;
@@ -316,6 +319,7 @@ __device__ __forceinline__ uint4 dequant8_fast(uint32_t lo, uint32_t hi, int seg
   uint32_t a, b;
   if (BITS == 8) { a = lo ^ REP; b = hi ^ REP; }
   else { a = (lo >> (seg * BITS)) & REP; b = (hi >> (seg * BITS)) & REP; }
+  asm volatile("" : "+v"(a), "+v"(b));                       // see dequant8
   float c[8] = {(float)(a & 0xFFu), (float)((a >> 8) & 0xFFu), (float)((a >> 16) & 0xFFu), (float)(a >> 24),
                 (float)(b & 0xFFu), (float)((b >> 8) & 0xFFu), (float)((b >> 16) & 0xFFu), (float)(b >> 24)};
   constexpr float OFFV = (BITS == 8) ? 128.f : (float)Q<BITS>::OFF;
