@@ -2,6 +2,7 @@
 // decompression.  A row lives in registers (x is read from HBM once); the next row's loads are issued before the
 // current row is processed so that memory requests stay in flight during the arithmetic.
 #include <atomic>
+#include <stdlib.h>
 
 #include "abi_util.hpp"
 #include "row_kernels.hpp"
@@ -60,19 +61,80 @@ __device__ __forceinline__ float block_sum1(float a, float (*red)[16], int parit
   return t;
 }
 
+// ---- rows staged through LDS -------------------------------------------------------------------------------------
+// gfx950 can load 16 bytes per lane from memory straight into LDS (global_load_lds_dwordx4: lane i of a wave lands at
+// the wave's LDS base + 16 i).  A wave uses that as a prefetch queue of its own: the incoming-gradient chunks of the
+// rows it will process next wait in LDS, not in registers, so several rows can be in flight per wave at no cost in
+// occupancy.  Every wave only ever reads what it requested itself, so no barrier guards the queue.
+//
+// Completion: vector memory operations of a wave complete in issue order.  The small per-row loads that go to
+// registers (codes, scales, outlier values, rstd) are issued AFTER the queue entry of the same row, and a queue entry
+// is read only after one of those registers has been used, so the compiler's own wait for that register covers the
+// entry.  The LDS reads are written in assembly: a read the compiler can see would make it wait for EVERY outstanding
+// load into the queue array (it cannot tell the stages apart), which would undo the prefetch.
+typedef float floatx4_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+typedef const __attribute__((address_space(1))) void* gbl_void_ptr;
+constexpr int RING_D = 3;                                             // rows per wave in the queue: being read, next, after next
+
+__device__ __forceinline__ uint32_t lds_offset(const void* p) {
+  return (uint32_t)(size_t)(__attribute__((address_space(3))) const char*)p;
+}
+// NSEG chunks of 16 bytes per lane, 1 KB apart, at LDS byte address `addr` (this lane's); `after` is any register
+// whose load was issued after the queue entry: naming it here keeps this read behind the wait for it
+template <int NSEG>
+__device__ __forceinline__ void queue_read(uint32_t addr, uint32_t after, uint4 (&g)[NSEG]) {
+  static_assert(NSEG == 1 || NSEG == 2 || NSEG == 4, "chunks per lane");
+  u32x4_t a, b = {0, 0, 0, 0}, c = {0, 0, 0, 0}, d = {0, 0, 0, 0};
+  if (NSEG == 4)
+    asm volatile("ds_read_b128 %0, %4\n\tds_read_b128 %1, %4 offset:1024\n\tds_read_b128 %2, %4 offset:2048\n\t"
+                 "ds_read_b128 %3, %4 offset:3072\n\ts_waitcnt lgkmcnt(0)"
+                 : "=&v"(a), "=&v"(b), "=&v"(c), "=&v"(d) : "v"(addr), "v"(after) : "memory");
+  else if (NSEG == 2)
+    asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %2 offset:1024\n\ts_waitcnt lgkmcnt(0)"
+                 : "=&v"(a), "=&v"(b) : "v"(addr), "v"(after) : "memory");
+  else
+    asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=&v"(a) : "v"(addr), "v"(after) : "memory");
+  const u32x4_t v[4] = {a, b, c, d};
+#pragma unroll
+  for (int i = 0; i < NSEG; ++i) g[i] = make_uint4(v[i].x, v[i].y, v[i].z, v[i].w);
+}
+
+// rows per wave in the forward kernel's queue: three, or two where three would not leave room (long rows of 2-bit codes)
+constexpr int fwd_queue_depth(int maxt, int nseg) { return RING_D * maxt * nseg * 16 <= 128 * 1024 ? RING_D : 2; }
+
 template <int BITS, int LPGT, bool WF32, int MAXT, int RULE>
 __global__ void __launch_bounds__(MAXT)
 k_rmsnorm_fwd_fast(const uint16_t* __restrict__ x, const void* __restrict__ w, float eps, int64_t M, int64_t H,
                    int CPS, ChanArgs ca, uint16_t* __restrict__ y, float* __restrict__ rstd_out, uint8_t* __restrict__ stored,
                    uint16_t* __restrict__ vals, uint16_t* __restrict__ scales) {
   constexpr int NSEG = Q<BITS>::NSEG;
+  constexpr int D = fwd_queue_depth(MAXT, NSEG);                      // rows in the queue
   __shared__ float red[2][16];
+  // dynamic LDS, D stages of blockDim.x * NSEG chunks: [stage][wave][segment][lane], x chunks on their way in
+  extern __shared__ __align__(16) uint4 queue[];
+  const int STAGE_B = (int)blockDim.x * NSEG * 16;                    // bytes of one queue stage of the workgroup
   const int c = threadIdx.x;
   const bool active = c < CPS;                                    // false only in the tail of the last wave
-  const int64_t SEG = (int64_t)CPS * 8;
+  const uint32_t SEG = (uint32_t)CPS * 8u;
   const float invH = 1.0f / (float)H;
-  const int wave = c >> 6, nw = blockDim.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(c >> 6), nw = blockDim.x >> 6;
   const bool leader = active && (c & (LPGT - 1)) == 0;
+  const int seg_groups = CPS >> ca.chunk_to_group_shift;          // scale groups per segment
+  // Every memory instruction of the row loop is a buffer operation on a resource that spans one row (zero bytes for a
+  // row past the end); lanes without data carry the offset NOWHERE.  Nothing is predicated or branched on.
+  const uint32_t row_b = (uint32_t)H * 2u, seg_b = SEG * 2u;
+  const uint32_t xo = active ? 16u * (uint32_t)c : NOWHERE;                                       // y: chunk c of segment 0
+  // (the same for x on its way into the queue, except that lanes past the end of the row re-read its first chunk: a
+  // load into LDS with some of its lanes out of range runs several times slower - measured - than one with all or none)
+  const uint32_t qo = active ? 16u * (uint32_t)c : 0u;
+  const uint32_t so = active ? 8u * (uint32_t)c : NOWHERE;                                        // packed word
+  const uint32_t go = leader ? 2u * (uint32_t)(c >> ca.chunk_to_group_shift) : NOWHERE;           // group scale (leaders)
+  const uint32_t ro = c == 0 ? 0u : NOWHERE;                                                      // rstd (one lane)
+  const bool gather = active && c < ca.k;                         // thread c copies outlier channel idx[c] to vals
+  const uint32_t gi = gather ? 2u * (uint32_t)ca.idx[c] : NOWHERE, vo = gather ? 2u * (uint32_t)c : NOWHERE;
+  char* const qwave = reinterpret_cast<char*>(queue) + wave * (NSEG * 1024);
+  const uint32_t qlane = lds_offset(queue) + (uint32_t)(wave * (NSEG * 1024)) + 16u * (uint32_t)(c & 63);
 
   uint32_t km[NSEG][4];                                            // AND masks that zero the outlier channels
   float wv[NSEG][8];
@@ -85,7 +147,7 @@ k_rmsnorm_fwd_fast(const uint16_t* __restrict__ x, const void* __restrict__ w, f
       for (int j = 0; j < 8; ++j) wv[i][j] = 0.f;
       if (active) {
         plan[i] = ca.plan[i * CPS + c];
-        load_w8t<WF32>(w, i * SEG + 8 * c, wv[i]);
+        load_w8t<WF32>(w, (int64_t)i * SEG + 8 * c, wv[i]);
       }
     }
     ChunkOutliers<NSEG> co;
@@ -93,37 +155,55 @@ k_rmsnorm_fwd_fast(const uint16_t* __restrict__ x, const void* __restrict__ w, f
 #pragma unroll
     for (int i = 0; i < NSEG; ++i) co.keep_masks(i, km[i]);
   }
-  const bool gather = active && c < ca.k;                                  // thread c copies outlier channel idx[c] to vals
-  const int idx0 = gather ? ca.idx[c] : 0;
   const int64_t stride = gridDim.x;
   int64_t row = blockIdx.x;
-  const uint16_t* xrow = x + row * H;
-  const uint16_t* xp = xrow + 8 * c;
-  uint16_t* yp = y + row * H + 8 * c;
-  uint8_t* sp = stored + row * SEG + 8 * c;
-  uint16_t* vp = vals + row * ca.k;
-  uint16_t* scp = scales + row * ca.groups_per_row + (c >> ca.chunk_to_group_shift);
-  const int64_t xstep = stride * H, sstep = stride * SEG, vstep = stride * ca.k, scstep = stride * ca.groups_per_row;
-  const int seg_groups = CPS >> ca.chunk_to_group_shift;          // scale groups per segment
-
-  uint4 raw[NSEG];
-  uint16_t o = 0;
+  auto row_of = [&](const void* base, int64_t r, uint32_t bytes) __attribute__((always_inline)) {
+    return make_rsrc(static_cast<const char*>(base) + r * (int64_t)bytes, r < M ? bytes : 0u);
+  };
+  // row r into queue stage `stage_b`
+  auto request = [&](int64_t r, int stage_b) __attribute__((always_inline)) {
+    const BufferRsrc rs_x = row_of(x, r, row_b);
 #pragma unroll
-  for (int i = 0; i < NSEG; ++i) raw[i] = make_uint4(0, 0, 0, 0);
-  if (row < M && active) {
+    for (int i = 0; i < NSEG; ++i) load_b128_to_lds(rs_x, qo + (uint32_t)i * seg_b, qwave + stage_b + i * 1024);
+  };
+  // The outlier channel this thread copies to vals[r, :] goes to a register.  It is requested after row r's queue
+  // entry and before the next entry, so having used it vouches for row r's entry and for nothing younger (see above).
+  auto request_outlier = [&](int64_t r) __attribute__((always_inline)) { return load_b16(row_of(x, r, row_b), gi); };
+  // The compiler sizes each wait by the fewest memory operations that can have been issued since the load it waits
+  // for, over every path to that point.  Entering the loop must therefore look like coming around it: the requests
+  // made ahead of the loop are followed by as many stores as a loop iteration issues after its requests (here to
+  // nowhere: dropped before they reach memory).  Without them the wait at the top of the loop would be sized for the
+  // first row and would drain the queue on every row.
+  request(row, 0);
+  __builtin_amdgcn_sched_barrier(0);
+  uint32_t og = request_outlier(row);
+  __builtin_amdgcn_sched_barrier(0);
+  if (D > 2) request(row + stride, STAGE_B);
+  {
+    const BufferRsrc nothing = make_rsrc(x, 0u);
+    store_b32(nothing, NOWHERE, 0u);                                 // stands for: rstd
+    store_b64(nothing, NOWHERE + 8u, 0u, 0u);                        // the packed word
 #pragma unroll
-    for (int i = 0; i < NSEG; ++i) raw[i] = *reinterpret_cast<const uint4*>(xp + i * SEG);
-    if (gather) o = xrow[idx0];
+    for (int i = 0; i < NSEG; ++i) store_b16(nothing, NOWHERE + 2u * (i + 1), (uint16_t)0);   // NSEG scales
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) store_b128_stream(nothing, NOWHERE + 16u * (i + 1), make_uint4(0, 0, 0, 0));   // NSEG chunks of y
+    // (distinct offsets: identical stores would be folded into one)
   }
-  int parity = 0;
+  __builtin_amdgcn_sched_barrier(0);
+  int st_b = 0, parity = 0;
   for (; row < M; row += stride, parity ^= 1) {
-    uint4 nxt[NSEG];
-    uint16_t o_n = 0;
-    if (row + stride < M && active) {
-#pragma unroll
-      for (int i = 0; i < NSEG; ++i) nxt[i] = *reinterpret_cast<const uint4*>(xp + xstep + i * SEG);
-      if (gather) o_n = xrow[xstep + idx0];
-    }
+    uint4 raw[NSEG];
+    queue_read<NSEG>(qlane + (uint32_t)st_b, og, raw);
+    const BufferRsrc rs_s = row_of(stored, row, SEG), rs_c = row_of(scales, row, 2u * (uint32_t)ca.groups_per_row);
+    const BufferRsrc rs_v = row_of(vals, row, 2u * (uint32_t)ca.k);
+    // the row's outlier value leaves at once and the next row's takes the register; then the row after next (two
+    // ahead; one with a short queue) goes into the stage that was read one row ago
+    store_b16(rs_v, vo, (uint16_t)og);
+    __builtin_amdgcn_sched_barrier(0);
+    og = request_outlier(row + stride);
+    __builtin_amdgcn_sched_barrier(0);
+    request(row + (D - 1) * stride, st_b >= STAGE_B ? st_b - STAGE_B : st_b + (D - 1) * STAGE_B);
+    __builtin_amdgcn_sched_barrier(0);
     float ss = 0.f;
     uint32_t lo = 0, hi = 0;
 #pragma unroll
@@ -135,63 +215,45 @@ k_rmsnorm_fwd_fast(const uint16_t* __restrict__ x, const void* __restrict__ w, f
       unpack8(make_uint4(raw[i].x & km[i][0], raw[i].y & km[i][1], raw[i].z & km[i][2], raw[i].w & km[i][3]), v);
       uint32_t cl, ch;
       const float s = quant_seg<BITS, LPGT, RULE>(v, LPGT, cl, ch, false);
-      if (leader) scp[i * seg_groups] = f_to_bf(s);
+      store_b16(rs_c, go + 2u * (uint32_t)(i * seg_groups), f_to_bf(s));
       if (BITS == 8) { lo = cl; hi = ch; }
       else { lo |= cl << (i * BITS); hi |= ch << (i * BITS); }
     }
-    if (active) *reinterpret_cast<uint2*>(sp) = make_uint2(lo, hi);
-    if (gather) {
-      vp[c] = o;
-      for (int t = c + CPS; t < ca.k; t += CPS) vp[t] = xrow[ca.idx[t]];   // only when k exceeds the workgroup size
+    store_b64(rs_s, so, lo, hi);
+    if (ca.k > CPS) {                                               // more outlier channels than threads (uniform, rare)
+      const uint16_t* xrow = x + row * H;
+      for (int t = c + CPS; t < ca.k; t += CPS) vals[row * ca.k + t] = xrow[ca.idx[t]];
     }
-    ss = block_sum1(active ? ss : 0.f, red, parity, wave, nw);      // inactive lanes hold no data
-    const float rstd = 1.0f / __builtin_sqrtf(ss * invH + eps);
-    if (c == 0) rstd_out[row] = rstd;
+    // sum over the waves of the workgroup: one bare barrier (__syncthreads() would also wait for the loads on their way
+    // into the queue), alternating buffers so that the next row's partial sums never overwrite values still being read
+    // (lanes past the end of the row hold a copy of its first chunk: they stay out of the sum, and what they encode is
+    // stored nowhere; scale groups never straddle the end of a row)
+    ss = wave_sum(active ? ss : 0.f);
+    if ((c & 63) == 0) red[parity][wave] = ss;
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    float tot = red[parity][0];
+    for (int i = 1; i < nw; ++i) tot += red[parity][i];
+    const float rstd = 1.0f / __builtin_sqrtf(tot * invH + eps);
+    store_b32(row_of(rstd_out, row, 4u), ro, __float_as_uint(rstd));
+    const BufferRsrc rs_y = row_of(y, row, row_b);
 #pragma unroll
     for (int i = 0; i < NSEG; ++i) {
       float v[8];
       unpack8(raw[i], v);
 #pragma unroll
       for (int j = 0; j < 8; ++j) v[j] = (v[j] * rstd) * wv[i][j];
-      if (active) store_stream(yp + i * SEG, pack8(v));
+      store_b128_stream(rs_y, xo + (uint32_t)i * seg_b, pack8(v));
     }
-#pragma unroll
-    for (int i = 0; i < NSEG; ++i) raw[i] = nxt[i];
-    o = o_n;
-    xrow += xstep; xp += xstep; yp += xstep; sp += sstep; vp += vstep; scp += scstep;
+    st_b = st_b >= (D - 1) * STAGE_B ? 0 : st_b + STAGE_B;
   }
 }
 
-// ---- rows staged through LDS -------------------------------------------------------------------------------------
-// gfx950 can load 16 bytes per lane from memory straight into LDS (global_load_lds_dwordx4: lane i of a wave lands at
-// the wave's LDS base + 16 i).  A wave uses that as a prefetch queue of its own: the incoming-gradient chunks of the
-// rows it will process next wait in LDS, not in registers, so several rows can be in flight per wave at no cost in
-// occupancy.  Every wave only ever reads what it requested itself, so no barrier guards the queue.
-//
-// Completion: vector memory operations of a wave complete in issue order.  The small per-row loads that go to
-// registers (codes, scales, outlier values, rstd) are issued AFTER the queue entry of the same row, and a queue entry
-// is read only after one of those registers has been used, so the compiler's own wait for that register covers the
-// entry.  The LDS reads are written in assembly: a read the compiler can see would make it wait for EVERY outstanding
-// load into the queue array (it cannot tell the stages apart), which would undo the prefetch.
-typedef __attribute__((address_space(3))) void* lds_void_ptr;
-typedef const __attribute__((address_space(1))) void* gbl_void_ptr;
-constexpr int RING_D = 3;                                             // rows per wave in the queue: being read, next, after next
-
-__device__ __forceinline__ uint32_t lds_offset(const void* p) {
-  return (uint32_t)(size_t)(__attribute__((address_space(3))) const char*)p;
-}
-// NSEG chunks of 16 bytes per lane, 1 KB apart, at LDS byte address `addr` (this lane's); `after` is any register
-// whose load was issued after the queue entry: naming it here keeps this read behind the wait for it
-template <int NSEG>
-__device__ __forceinline__ void queue_read(uint32_t addr, uint32_t after, uint4 (&g)[NSEG]) {
-  u32x4_t a, b = {0, 0, 0, 0};
-  if (NSEG == 2)
-    asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %2 offset:1024\n\ts_waitcnt lgkmcnt(0)"
-                 : "=&v"(a), "=&v"(b) : "v"(addr), "v"(after) : "memory");
-  else
-    asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=&v"(a) : "v"(addr), "v"(after) : "memory");
-  g[0] = make_uint4(a.x, a.y, a.z, a.w);
-  if (NSEG == 2) g[NSEG - 1] = make_uint4(b.x, b.y, b.z, b.w);
+// two float4 at LDS byte addresses `addr` and `addr + second`
+__device__ __forceinline__ void lds_read_8f(uint32_t addr, uint32_t second, float (&o)[8]) {
+  floatx4_t a, b;
+  asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %3\n\ts_waitcnt lgkmcnt(0)"
+               : "=&v"(a), "=&v"(b) : "v"(addr), "v"(addr + second) : "memory");
+  o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w; o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
 }
 
 // Backward fast path.  A workgroup is `slots` row slots of CPS threads; slot s of workgroup b handles rows
@@ -211,8 +273,9 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
   constexpr int NSEG = Q<BITS>::NSEG > 2 ? 2 : Q<BITS>::NSEG;         // segments per thread
   constexpr int PARTS = Q<BITS>::NSEG / NSEG;                         // threads per packed word
   constexpr int STAGE_B = MAXT * NSEG * 16;                           // bytes of one queue stage of the workgroup
+  constexpr int D = RING_D;                                           // rows in the queue
   __shared__ float red[2][4][2][16];                                  // [parity][slot][value][wave]
-  __shared__ __align__(16) uint4 queue[RING_D * MAXT * NSEG];         // [stage][wave][segment][lane]: dy chunks on their way in
+  __shared__ __align__(16) uint4 queue[D * MAXT * NSEG];              // [stage][wave][segment][lane]: dy chunks on their way in
   // dynamic LDS: the weight row as fp32 [segment][half chunk][CPS] float4 (read again for every row: sixteen
   // registers fewer than keeping the thread's weights live)
   extern __shared__ __align__(16) float lds_dyn[];
@@ -234,6 +297,9 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
   // operation on a resource that spans one row (zero bytes for a row past the end), and lanes past the end of the
   // row (the tail of a slot's last wave) carry the offset NOWHERE: nothing is predicated or branched on.
   const uint32_t xo = active ? (uint32_t)(seg0 * SEG + 8 * c) * 2u : NOWHERE;
+  // (into the queue, lanes past the end of the row re-read its first chunk: a load into LDS with some of its lanes out
+  // of range runs several times slower - measured - than one with all or none; what they read is zeroed below)
+  const uint32_t qo = active ? xo : 0u;
   const uint32_t so = active ? 8u * (uint32_t)c : NOWHERE;
   const uint32_t go = active ? (uint32_t)(seg0 * seg_groups + (c >> ca.chunk_to_group_shift)) * 2u : NOWHERE;
   const uint32_t seg_b = (uint32_t)SEG * 2u, grp_b = (uint32_t)seg_groups * 2u;
@@ -243,7 +309,7 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
   char* const qwave = reinterpret_cast<char*>(queue) + wv * (NSEG * 1024);
   const uint32_t qlane = lds_offset(queue) + (uint32_t)(wv * (NSEG * 1024)) + 16u * (threadIdx.x & 63);
 
-  const uint32_t wbase = active ? (uint32_t)(seg0 * 2 * CPS + c) : 0u;
+  const uint32_t wl_lane = lds_offset(wl4) + (active ? (uint32_t)(seg0 * 2 * CPS + c) : 0u) * 16u;   // this thread's weights in LDS
   const int64_t stride = (int64_t)gridDim.x * slots;
   int64_t row = (int64_t)blockIdx.x * slots + slot;
   // (steps = ceil(M / stride), the same for every slot so that barriers stay matched; divided on the host)
@@ -255,7 +321,7 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
   auto request_dy = [&](int64_t r, int stage_b) __attribute__((always_inline)) {
     const BufferRsrc rs_g = row_of(dy, r, row_b);
 #pragma unroll
-    for (int i = 0; i < NSEG; ++i) load_b128_to_lds(rs_g, xo + (uint32_t)i * seg_b, qwave + stage_b + i * 1024);
+    for (int i = 0; i < NSEG; ++i) load_b128_to_lds(rs_g, qo + (uint32_t)i * seg_b, qwave + stage_b + i * 1024);
   };
 
   uint2 pk = make_uint2(0, 0);
@@ -331,6 +397,16 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
   }
   request_outliers(row);
   __builtin_amdgcn_sched_barrier(0);
+  // The compiler sizes each wait by the fewest memory operations that can have been issued since the load it waits
+  // for, over every path to that point.  In the loop a row's registers are followed by a queue request and the
+  // previous row's stores; entering the loop must look the same, or the waits at the top of the loop would be sized
+  // for the first row and drain the queue on every row.  So: a request for a row past the end (zeros into the stage
+  // that the first iteration requests next) and as many stores to nowhere (dropped before they reach memory).
+  request_dy(M, (D - 1) * STAGE_B);
+#pragma unroll
+  for (int i = 0; i < NSEG; ++i)   // (distinct offsets: identical stores would be folded into one)
+    store_b128_stream(make_rsrc(dx, 0u), NOWHERE + 16u * i, make_uint4(0, 0, 0, 0));
+  __builtin_amdgcn_sched_barrier(0);
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");     // the weight row is in LDS (no wait for the queue)
   int st_b = 0;                                                       // queue stage of the current row, as a byte offset
   int parity = 0;
@@ -357,10 +433,10 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
           if (co.more_pairs) r = splice_more(r, co.more_pairs, ca.plan[(seg0 + i) * CPS + c], vrow, active, 1.f);
           unpack8(r, xn[i]);
         }
-        uint32_t wo = wbase + (uint32_t)(i * 2 * CPS);
-        asm volatile("" : "+v"(wo));                                  // re-read per row: do not keep the weights live
-        const float4 wa = wl4[wo], wb = wl4[wo + CPS];
-        const float wv[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
+        // the thread's weights, re-read per row (sixteen registers fewer than keeping them live); in assembly for the
+        // same reason as the queue reads: a read of dynamic LDS that the compiler can see waits for the queue to drain
+        float wv[8];
+        lds_read_8f(wl_lane + (uint32_t)(i * 2 * CPS) * 16u, (uint32_t)CPS * 16u, wv);
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           const float n = __builtin_fmaf(xn[i][j], rs, nm);
@@ -372,6 +448,10 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
           acc[i][j] = __builtin_fmaf(g[j], n, acc[i][j]);
         }
       }
+      // (lanes past the end of the row hold the row's first chunk of dy and weights: they stay out of the row sums;
+      // their dw sums are never stored)
+      p1 = active ? p1 : 0.f;
+      if (QUIRK) p2 = active ? p2 : 0.f;
     }
     // The row is decoded: its registers take the next row's codes, scales and outliers now, and the row after that
     // goes into the queue stage that was read two rows ago.  Order matters, see above.
@@ -379,7 +459,7 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
     request_codes(row + stride);
     request_outliers(row + stride);
     __builtin_amdgcn_sched_barrier(0);
-    request_dy(row + 2 * stride, st_b >= STAGE_B ? st_b - STAGE_B : st_b + 2 * STAGE_B);
+    request_dy(row + (D - 1) * stride, st_b >= STAGE_B ? st_b - STAGE_B : st_b + (D - 1) * STAGE_B);
     __builtin_amdgcn_sched_barrier(0);
     // two sums per slot, one barrier
     p1 = wave_sum(p1);
@@ -400,7 +480,7 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
       for (int j = 0; j < 8; ++j) o[j] = __builtin_fmaf(xn[i][j], k1, __builtin_fmaf(wdy[i][j], rs_c, k2));
       store_b128_stream(rs_o, xo + (uint32_t)i * seg_b, pack8(o));
     }
-    st_b = st_b >= 2 * STAGE_B ? 0 : st_b + STAGE_B;
+    st_b = st_b >= (D - 1) * STAGE_B ? 0 : st_b + STAGE_B;
   }
   // The slots' dw sums are added in slot order through the queue's memory, which nobody reads any more.
   float* pr = dw_partials + (int64_t)blockIdx.x * H + (int64_t)seg0 * SEG + 8 * c;
@@ -916,7 +996,9 @@ static int norm_fwd_impl(const void* x, const void* w, const void* bias, int32_t
   if (!aligned16(x) || !aligned16(y) || !aligned16(w) || !aligned8(stored))
     return fail(HYC_EINVAL, "hyc_rmsnorm_fwd_compress: x, y, w must be 16-byte and stored 8-byte aligned");
   const bool wf32 = w_dtype == HYC_DTYPE_F32;
-  const int64_t cap = 256 * (n.T >= 512 ? 2 : 8);
+  // workgroups: about four rows each (measured: 1024 workgroups at 4096 rows, 16 384 at 65 536), at least one round
+  // of the chip, and two per CU when a row takes more than eight waves
+  int64_t cap = n.T >= 512 ? 512 : (M / 4 < 1024 ? 1024 : (M / 4 > 16384 ? 16384 : M / 4));
   const int grid = (int)(M < cap ? M : cap);
   hipStream_t st = begin_launch(stream);
   const uint16_t* xp = static_cast<const uint16_t*>(x);
@@ -928,11 +1010,12 @@ static int norm_fwd_impl(const void* x, const void* w, const void* bias, int32_t
     uint16_t* scp = static_cast<uint16_t*>(scales);
 #define HYC_FWD_FAST(B_, L_, W_, MT_)                                                                              \
   do {                                                                                                             \
+    const size_t qb_ = (size_t)fwd_queue_depth(MT_, Q<B_>::NSEG) * n.T * Q<B_>::NSEG * 16;                         \
     if (ca.absmax)                                                                                                 \
-      hipLaunchKernelGGL((k_rmsnorm_fwd_fast<B_, L_, W_, MT_, SCALE_ABSMAX>), dim3(grid), dim3(n.T), 0, st, xp, w, eps, M, H, \
+      hipLaunchKernelGGL((k_rmsnorm_fwd_fast<B_, L_, W_, MT_, SCALE_ABSMAX>), dim3(grid), dim3(n.T), qb_, st, xp, w, eps, M, H, \
                          g.cps, ca, yp, rstd, stp, vp, scp);                                                       \
     else                                                                                                           \
-      hipLaunchKernelGGL((k_rmsnorm_fwd_fast<B_, L_, W_, MT_, SCALE_RANGE>), dim3(grid), dim3(n.T), 0, st, xp, w, eps, M, H, \
+      hipLaunchKernelGGL((k_rmsnorm_fwd_fast<B_, L_, W_, MT_, SCALE_RANGE>), dim3(grid), dim3(n.T), qb_, st, xp, w, eps, M, H, \
                          g.cps, ca, yp, rstd, stp, vp, scp);                                                       \
   } while (0)
 #define HYC_FWD_FAST_W(B_, L_)                                                        \

@@ -83,6 +83,16 @@ __device__ __forceinline__ void store_b128_stream(BufferRsrc r, uint32_t off, co
   const u32x4_t t = {v.x, v.y, v.z, v.w};
   __builtin_amdgcn_raw_buffer_store_b128(t, r, (int)off, 0, 2);
 }
+__device__ __forceinline__ void store_b64(BufferRsrc r, uint32_t off, uint32_t lo, uint32_t hi) {
+  const u32x2_t t = {lo, hi};
+  __builtin_amdgcn_raw_buffer_store_b64(t, r, (int)off, 0, 0);
+}
+__device__ __forceinline__ void store_b32(BufferRsrc r, uint32_t off, uint32_t v) {
+  __builtin_amdgcn_raw_buffer_store_b32(v, r, (int)off, 0, 0);
+}
+__device__ __forceinline__ void store_b16(BufferRsrc r, uint32_t off, uint16_t v) {
+  __builtin_amdgcn_raw_buffer_store_b16((short)v, r, (int)off, 0, 0);
+}
 // 16 bytes per lane from memory straight into LDS: lane i of the wave lands at `lds_wave_base` + 16 i
 __device__ __forceinline__ void load_b128_to_lds(BufferRsrc r, uint32_t off, void* lds_wave_base) {
   __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void*)lds_wave_base, 16, (int)off, 0, 0, 0);
