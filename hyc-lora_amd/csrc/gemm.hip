@@ -10,6 +10,7 @@
 // Because of the segment packing, one packed tile [tokens, 8c bytes] feeds NSEG separate ranges of output
 // columns; a workgroup owns all of them so the packed bytes are read once.
 #include <algorithm>
+#include <utility>
 
 #include "abi_util.hpp"
 #include "row_kernels.hpp"
@@ -641,14 +642,15 @@ static int direct_splits_max(int64_t M, int64_t N_out, int64_t H) {
 }
 
 // ------------------------------------------------------------------------------------------------
-// Large output (N_out > 32): workgroup tile 128 (n) x 256 (h), four waves of 64 x 128, two LDS stages.
-// While the MFMAs of stage s run, the global loads of stage s+1 are in flight; they are decoded into the other LDS
+// Large output (N_out > 32), first form: workgroup tile 128 (n) x 256 (h), four waves of 64 x 128, two LDS stages.
+// While the MFMAs of stage s run, the global loads of stage s+1 are in flight; they are written into the other LDS
 // buffer after the MFMAs have been issued, and one barrier per stage separates the two.  128 accumulator registers
-// per lane; at least two waves per SIMD so that they stay in ordinary vector registers and a second workgroup's
-// decode overlaps this one's MFMAs.
+// per lane and two waves per SIMD.  It is launched for a dense activation whose tile grid is too small for the
+// 256-feature form below (the template still carries the eight-wave and channel-scheme variants it was written with;
+// k_gradw_big has taken their place).
 // ------------------------------------------------------------------------------------------------
 constexpr int WK = 32;      // tokens per stage
-constexpr int WN = 128;     // dY features per workgroup: WN (four waves) or 2*WN (eight waves)
+constexpr int WN = 128;     // dY features per workgroup of this form (the second form takes 2 * WN)
 constexpr int WH = 256;     // channels per workgroup
 constexpr int WPAD = 32;    // row padding of the wide kernel's LDS tiles, in elements
 
@@ -958,6 +960,344 @@ k_gradw_wide(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Large output, second form: workgroup tile 256 (n) x 256 (h) on FOUR waves of 128 x 128, one per SIMD.  A wave's 256
+// fp32 accumulators live in the accumulation registers (the compiler puts them there by itself at one wave per SIMD),
+// which leaves the 256 ordinary registers to operand fragments and to the data of the next three stages.  Against the
+// 64 x 128 wave tile this halves the operand bytes read from LDS per MFMA (8 fragments per 16 MFMAs instead of 6 per
+// 8) - the traffic that bounds the eight-wave form.  With a single wave per SIMD nothing but the wave's own next
+// instructions can fill the 32 cycles of an MFMA (eight issue slots: the MFMA and seven others), so a stage of 32
+// tokens is laid out by hand as 32 slots, one MFMA each:
+//   slots  0- 7  read the fragments of the stage's second 16 tokens
+//   slots  0-15  decode stage s+1 (two elements per slot; its registers were requested two stages ago)
+//   slots  8-15  request stage s+3 into the register set that held stage s
+//   slots 16-23  write stage s+1 to the next LDS buffer, move the buffer resources on
+//   slot  24     the stage's one barrier; slots 24-31 read the fragments of the first 16 tokens of stage s+1
+// ------------------------------------------------------------------------------------------------
+template <int V> struct StageNo { static constexpr int value = V; };
+// f(StageNo<0>), f(StageNo<1>), ... : a loop whose bodies are separate instantiations (no unroll threshold applies)
+template <class F, int... T>
+__device__ __forceinline__ void for_each_slot(F&& f, std::integer_sequence<int, T...>) { (f(StageNo<T>{}), ...); }
+
+template <int BITS, int SRC>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+k_gradw_big(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_out, int64_t H,
+            const uint8_t* __restrict__ stored, const uint16_t* __restrict__ vals, const uint16_t* __restrict__ scales,
+            ChanArgs ca, int CPS, int64_t tokens_per_split, float alpha, float beta,
+            void* __restrict__ out, int out_f32, float* __restrict__ partial) {
+  constexpr int NSEG = (SRC == 0) ? Q<BITS>::NSEG : 1;
+  constexpr int TN = 256;                     // dY features per workgroup
+  constexpr int HS = WH / NSEG;               // columns of the tile that come from one segment
+  constexpr int CPR = HS / 8;                 // packed 8-byte chunks (channel scheme) / 16-byte chunks (dense) per token row and segment
+  constexpr int THREADS = 256;
+  constexpr int AP = TN + WPAD, BP = WH + WPAD;
+  constexpr int NBUF = 3;
+  __shared__ __align__(16) uint16_t lds[NBUF * WK * (AP + BP)];
+#define HYC_AS(b_) (lds + (b_) * (WK * AP))
+#define HYC_BS(b_) (lds + NBUF * (WK * AP) + (b_) * (WK * BP))
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int64_t n0 = (int64_t)blockIdx.x * TN;
+  const int64_t SEG = (SRC == 0) ? (int64_t)CPS * 8 : H;
+  const int64_t j0 = (int64_t)blockIdx.y * HS;          // first column of the tile inside each segment
+  const int64_t m_begin = (int64_t)blockIdx.z * tokens_per_split;
+  const int64_t m_end = m_begin + tokens_per_split < M ? m_begin + tokens_per_split : M;
+  const int wn = (wave >> 1) * 128, wh = (wave & 1) * 128;
+
+  floatx16_t acc[4][4];
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
+
+  constexpr int A_PER = WK * TN / 8 / THREADS;            // 16-byte chunks of the dY stage per thread (4)
+  constexpr int B_ITEMS = WK * CPR;
+  constexpr int B_PER = (B_ITEMS + THREADS - 1) / THREADS;
+  static_assert(B_ITEMS % THREADS == 0 || B_ITEMS < THREADS, "items per stage");
+  // Narrow codes give fewer packed words per stage than threads: PARTS threads then share a word, NST segments each.
+  constexpr int PARTS = (SRC == 0 && B_ITEMS < THREADS) ? THREADS / B_ITEMS : 1;
+  constexpr int NST = NSEG / PARTS;                       // segments a thread decodes
+  static_assert(NSEG % PARTS == 0 && (PARTS == 1 || PARTS * B_ITEMS == THREADS), "threads per packed word");
+  constexpr int NCH = B_PER * NST;                        // 16-byte chunks of the x stage per thread
+  static_assert(A_PER == 4 && NCH == 4, "the slot plan below is written for four chunks of either operand");
+  const int seg0 = (PARTS > 1 ? tid / B_ITEMS : 0) * NST; // first of them
+  const int item0 = PARTS > 1 ? tid % B_ITEMS : tid;      // the thread's first item
+  typedef WideRegs<NST, A_PER, B_PER> Regs;
+  ChunkOutliers<NST> co;
+  {
+    uint32_t pw[NST];
+#pragma unroll
+    for (int i = 0; i < NST; ++i)
+      pw[i] = (SRC == 0) ? ca.plan[(seg0 + i) * CPS + (int)(j0 / 8) + item0 % CPR] : 0u;
+    co.init(pw);
+  }
+
+  // Every operand of the token loop is read through a buffer resource that starts at the stage's first token and
+  // ends with the workgroup's token range: nothing is clamped, predicated or branched on, a stage past the end
+  // reads zeros, and the addresses are per-thread constants.
+  const uint32_t gpr = (uint32_t)ca.groups_per_row, kk2 = 2u * (uint32_t)ca.k;
+  const uint32_t a_pitch = 2u * (uint32_t)ldy;
+  const uint32_t b_pitch = (SRC == 0) ? (uint32_t)SEG : 2u * (uint32_t)H;          // bytes per token of the x operand
+  uint32_t va[A_PER], vb[B_PER], vs[B_PER][NST], vo0[B_PER][NST], vo1[B_PER][NST];
+  int a_at[A_PER], b_at[NCH];                                                       // element offsets inside an LDS buffer
+#pragma unroll
+  for (int u = 0; u < A_PER; ++u) {
+    const int idx = tid + u * THREADS;
+    const int row = idx / (TN / 8), cc = idx % (TN / 8);
+    va[u] = n0 + 8 * cc < N_out ? 2u * ((uint32_t)row * (uint32_t)ldy + (uint32_t)n0 + 8u * cc) : NOWHERE;
+    a_at[u] = row * AP + 8 * cc;
+  }
+#pragma unroll
+  for (int u = 0; u < B_PER; ++u) {
+    const int idx = item0 + u * THREADS;
+    const int row = idx / CPR, cc = idx % CPR;
+    if (SRC == 0) {
+      const int c = (int)(j0 / 8) + cc;
+      vb[u] = (uint32_t)row * b_pitch + 8u * c;
+#pragma unroll
+      for (int i = 0; i < NST; ++i) {
+        vs[u][i] = 2u * ((uint32_t)row * gpr + (uint32_t)(((seg0 + i) * CPS + c) >> ca.chunk_to_group_shift));
+        vo0[u][i] = co.has0[i] ? (uint32_t)row * kk2 + co.vb[i] : NOWHERE;
+        vo1[u][i] = co.has1[i] ? (uint32_t)row * kk2 + co.vb[i] + 2u : NOWHERE;
+        b_at[u * NST + i] = row * BP + (seg0 + i) * HS + 8 * cc;
+      }
+    } else {
+      vb[u] = (uint32_t)row * b_pitch + 2u * ((uint32_t)j0 + 8u * cc);
+      b_at[u] = row * BP + 8 * cc;
+    }
+  }
+  // the resources of the next stage to request
+  const char* pa = reinterpret_cast<const char*>(dy + m_begin * ldy);
+  const char* pb = reinterpret_cast<const char*>(stored) + m_begin * (int64_t)b_pitch;
+  const char* ps = reinterpret_cast<const char*>(scales + m_begin * (int64_t)gpr);
+  const char* po = reinterpret_cast<const char*>(vals + m_begin * (int64_t)ca.k);
+  int left = (int)(m_end - m_begin);                                                // tokens from that stage to the end
+  BufferRsrc rs_a = make_rsrc(pa, (uint32_t)left * a_pitch), rs_b = make_rsrc(pb, __builtin_amdgcn_readfirstlane((uint32_t)left * b_pitch));
+  BufferRsrc rs_s = make_rsrc(ps, (uint32_t)left * 2u * gpr), rs_o = make_rsrc(po, __builtin_amdgcn_readfirstlane((uint32_t)left * kk2));
+  // (the empty asm statements keep the scalar arithmetic in the slot it is written in, and in scalar registers)
+  auto renew = [&](BufferRsrc& rs, const char*& ptr, uint32_t step, uint32_t pitch) __attribute__((always_inline)) {
+    const uint64_t next = reinterpret_cast<uint64_t>(ptr) + step;
+    uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)next), hi = __builtin_amdgcn_readfirstlane((uint32_t)(next >> 32));
+    uint32_t bytes = __builtin_amdgcn_readfirstlane((uint32_t)left * pitch);
+    asm volatile("" : "+s"(lo), "+s"(hi), "+s"(bytes));
+    ptr = reinterpret_cast<const char*>(((uint64_t)hi << 32) | lo);
+    rs = make_rsrc(ptr, bytes);
+  };
+  auto advance = [&](int part) __attribute__((always_inline)) {                     // four parts, one resource each
+    if (part == 0) {
+      left = left > WK ? left - WK : 0;
+      renew(rs_a, pa, WK * a_pitch, a_pitch);
+    } else if (part == 1) {
+      renew(rs_b, pb, WK * b_pitch, b_pitch);
+    } else if (part == 2 && SRC == 0) {
+      renew(rs_s, ps, WK * 2u * gpr, 2u * gpr);
+    } else if (part == 3 && SRC == 0) {
+      renew(rs_o, po, WK * kk2, kk2);
+    }
+  };
+  // The requests of a stage, numbered: codes and scales (decoded first) before dY and the outlier values.
+  constexpr int NLOAD = A_PER + (SRC == 0 ? B_PER * (1 + 3 * NST) : B_PER);
+  auto request = [&](Regs& R, int j) __attribute__((always_inline)) {
+    if (SRC != 0) {
+      if (j < B_PER) R.b[j] = load_b128(rs_b, vb[j]);
+      else R.a[j - B_PER] = load_b128(rs_a, va[j - B_PER]);
+    } else if (j < B_PER) {
+      const uint2 pk = load_b64(rs_b, vb[j]);
+      R.b[j] = make_uint4(pk.x, pk.y, 0, 0);
+    } else if (j < B_PER + NCH) {
+      const int c = j - B_PER;
+      R.s[c / NST][c % NST] = load_b16(rs_s, vs[c / NST][c % NST]);
+    } else if (j < B_PER + NCH + A_PER) {
+      const int u = j - B_PER - NCH;
+      R.a[u] = load_b128(rs_a, va[u]);
+    } else {
+      const int q = j - B_PER - NCH - A_PER, c = q >> 1;
+      if (q & 1) R.o1[c / NST][c % NST] = load_b16(rs_o, vo1[c / NST][c % NST]);
+      else R.o0[c / NST][c % NST] = load_b16(rs_o, vo0[c / NST][c % NST]);
+    }
+  };
+  auto request_all = [&](Regs& R) __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < NLOAD; ++j) request(R, j);
+#pragma unroll
+    for (int part = 0; part < 4; ++part) advance(part);
+  };
+  // Chunks with more than two outlier channels (rare; the flag is the same for the whole wave): the remaining values
+  // are written over the decoded chunk in LDS, element by element, after the chunk itself.
+  auto patch_more = [&](uint16_t* Bb, int64_t mb) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < B_PER; ++u) {
+      const int idx = item0 + u * THREADS;
+      const int row = idx / CPR, cc = idx % CPR;
+      if (mb + row < m_end) {
+        const uint16_t* vrow = vals + (mb + row) * ca.k;
+#pragma unroll
+        for (int i = 0; i < NST; ++i) {
+          const uint32_t p = ca.plan[(seg0 + i) * CPS + (int)(j0 / 8) + cc];
+          uint32_t m = p & 0xFFu;
+          m &= m - 1; m &= m - 1;                                       // the first two are in place already
+          int at = (int)(p >> 16) + 2;
+          while (m != 0) {
+            Bb[b_at[u * NST + i] + (__ffs(m) - 1)] = vrow[at++];
+            m &= m - 1;
+          }
+        }
+      }
+    }
+  };
+  // decode one stage of registers (tokens mb ..) into an LDS buffer all at once (before the loop)
+  auto stash = [&](uint16_t* Ab, uint16_t* Bb, const Regs& R, int64_t mb) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < A_PER; ++u) *reinterpret_cast<uint4*>(&Ab[a_at[u]]) = R.a[u];
+#pragma unroll
+    for (int u = 0; u < B_PER; ++u) {
+      if (SRC == 0) {
+#pragma unroll
+        for (int i = 0; i < NST; ++i)
+          *reinterpret_cast<uint4*>(&Bb[b_at[u * NST + i]]) =
+              co.splice_value(i, dequant8_fast<BITS>(R.b[u].x, R.b[u].y, seg0 + i, bf_to_f((uint16_t)R.s[u][i])), R.o0[u][i], R.o1[u][i]);
+      } else {
+        *reinterpret_cast<uint4*>(&Bb[b_at[u]]) = R.b[u];
+      }
+    }
+    if (SRC == 0 && co.more_pairs) patch_more(Bb, mb);
+  };
+  bf16x8_t fa0[4], fb0[4], fa1[4], fb1[4];                    // operand fragments of the stage's first / second 16 tokens
+  // fragment q of 8 of a 16-token half: the x fragment of the first MFMAs, the four dY fragments, the other three of x
+  auto read_frag = [&](const uint16_t* Ab, const uint16_t* Bb, int kk, int q, bf16x8_t (&fa)[4], bf16x8_t (&fb)[4]) __attribute__((always_inline)) {
+    if (q == 0) fb[0] = frag32(Bb, BP, wh, kk);
+    else if (q <= 4) fa[q - 1] = frag32(Ab, AP, wn + 32 * (q - 1), kk);
+    else fb[q - 4] = frag32(Bb, BP, wh + 32 * (q - 4), kk);
+  };
+  // One stage: the MFMAs on LDS buffer B; the register set Rd (stage s+1, tokens m1 ..) goes to buffer B+1 on the
+  // way and the set Rf is requested anew (stage s+3).
+  auto stage = [&](auto bno, const Regs& Rd, Regs& Rf, int64_t m1) __attribute__((always_inline)) {
+    constexpr int B = decltype(bno)::value, NB = (B + 1) % NBUF;
+    constexpr uint32_t REP = (BITS == 8) ? 0x80808080u : Q<BITS>::CODE_MASK * 0x01010101u;
+    constexpr float OFFV = (BITS == 8) ? 128.f : (float)Q<BITS>::OFF;
+    uint32_t cw[NCH][2], res[NCH][4];
+    float sc[NCH], ns[NCH];
+    auto slot = [&](auto tno) __attribute__((always_inline)) {
+      constexpr int t = decltype(tno)::value;
+      __builtin_amdgcn_sched_barrier(0);
+      {
+        constexpr int a = t & 3, b = (t >> 2) & 3;
+        acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(t < 16 ? fa0[a] : fa1[a], t < 16 ? fb0[b] : fb1[b], acc[a][b], 0, 0, 0);
+      }
+      if constexpr (t < 8) read_frag(HYC_AS(B), HYC_BS(B), 16, t, fa1, fb1);
+      if constexpr (SRC == 0 && t < 16) {                               // two elements of chunk c of stage s+1
+        constexpr int c = t >> 2, w = t & 3, u = c / NST, i = c % NST;
+        if constexpr (w == 0) {
+          cw[c][0] = (BITS == 8) ? Rd.b[u].x ^ REP : (Rd.b[u].x >> ((seg0 + i) * BITS)) & REP;
+          cw[c][1] = (BITS == 8) ? Rd.b[u].y ^ REP : (Rd.b[u].y >> ((seg0 + i) * BITS)) & REP;
+          asm volatile("" : "+v"(cw[c][0]), "+v"(cw[c][1]));            // (keeps the byte-wise conversions below)
+          sc[c] = bf_to_f((uint16_t)Rd.s[u][i]);
+          ns[c] = -OFFV * sc[c];
+        }
+        const uint32_t src = cw[c][w >> 1];
+        const float f0 = __builtin_fmaf((float)((src >> (16 * (w & 1))) & 0xFFu), sc[c], ns[c]);
+        const float f1 = __builtin_fmaf((float)((src >> (16 * (w & 1) + 8)) & 0xFFu), sc[c], ns[c]);
+        res[c][w] = pack_bf16(f0, f1);
+      }
+      if constexpr (t >= 8 && t < 16) {
+        constexpr int j0_ = (t - 8) * NLOAD / 8, j1_ = (t - 7) * NLOAD / 8;
+        for_each_slot([&](auto jno) __attribute__((always_inline)) { request(Rf, j0_ + decltype(jno)::value); },
+                      std::make_integer_sequence<int, j1_ - j0_>{});
+      }
+      if constexpr (t >= 16 && t < 20) {
+        *reinterpret_cast<uint4*>(&HYC_AS(NB)[a_at[t - 16]]) = Rd.a[t - 16];
+        advance(t - 16);
+      }
+      if constexpr (t >= 20 && t < 24) {
+        constexpr int c = t - 20, u = c / NST, i = c % NST;
+        if constexpr (SRC == 0)
+          *reinterpret_cast<uint4*>(&HYC_BS(NB)[b_at[c]]) =
+              co.splice_value(i, make_uint4(res[c][0], res[c][1], res[c][2], res[c][3]), Rd.o0[u][i], Rd.o1[u][i]);
+        else
+          *reinterpret_cast<uint4*>(&HYC_BS(NB)[b_at[c]]) = Rd.b[c];
+        if constexpr (t == 23 && SRC == 0) {
+          if (co.more_pairs) patch_more(HYC_BS(NB), m1);
+        }
+      }
+      if constexpr (t == 24) __syncthreads();                           // buffer NB is complete, buffer B read for the last time
+      if constexpr (t >= 24) read_frag(HYC_AS(NB), HYC_BS(NB), 0, t - 24, fa0, fb0);
+    };
+    for_each_slot(slot, std::make_integer_sequence<int, 32>{});
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  if (m_begin < m_end) {
+    Regs R0, R1, R2;
+    const int64_t nstages = (m_end - m_begin + WK - 1) / WK;
+    request_all(R0);
+    request_all(R1);
+    request_all(R2);
+    stash(HYC_AS(0), HYC_BS(0), R0, m_begin);
+    __syncthreads();
+#pragma unroll
+    for (int q = 0; q < 8; ++q) read_frag(HYC_AS(0), HYC_BS(0), 0, q, fa0, fb0);
+    int64_t m1 = m_begin + WK;
+    for (int64_t s = 0; s < nstages; s += 3) {                         // a stage past the end holds zeros
+      stage(StageNo<0>{}, R1, R0, m1);
+      stage(StageNo<1>{}, R2, R1, m1 + WK);
+      stage(StageNo<2>{}, R0, R2, m1 + 2 * WK);
+      m1 += 3 * WK;
+    }
+  }
+#undef HYC_AS
+#undef HYC_BS
+
+  // ---- epilogue.  A lane holds column (lane mod 32), rows 8*(v/4) + 4*(lane/32) + (v mod 4) of each 32x32 tile.  The
+  // wave turns 32 rows x 128 columns at a time around in a private piece of LDS so that every lane stores eight
+  // neighbouring columns (16 bytes of bf16, 32 of fp32) and a row leaves as one contiguous run. ----
+  constexpr int EPP = 128 + 4;                               // floats per staged row
+  static_assert(4 * 32 * EPP * 4 <= (int)sizeof(lds), "epilogue staging");
+  __syncthreads();                                           // the last fragments have been read
+  float* ep = reinterpret_cast<float*>(lds) + wave * (32 * EPP);
+  const int er = lane >> 4, ec = 8 * (lane & 15);
+  const int hl = wh + ec;                                    // first of the lane's columns inside the tile
+  const int64_t h = (int64_t)(hl / HS) * SEG + j0 + (hl % HS);
+#pragma unroll
+  for (int a = 0; a < 4; ++a) {
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) ep[(8 * (v >> 2) + 4 * (lane >> 5) + (v & 3)) * EPP + 32 * b + (lane & 31)] = acc[a][b][v];
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");       // (one wave: LDS keeps its order, the compiler must too)
+#pragma unroll
+    for (int p = 0; p < 8; ++p) {
+      const int r = 4 * p + er;
+      const int64_t n = n0 + wn + 32 * a + r;
+      float4 lo = *reinterpret_cast<const float4*>(&ep[r * EPP + ec]);
+      float4 hi = *reinterpret_cast<const float4*>(&ep[r * EPP + ec + 4]);
+      if (n < N_out) {
+        if (partial != nullptr) {
+          float4* o = reinterpret_cast<float4*>(partial + ((int64_t)blockIdx.z * N_out + n) * H + h);
+          o[0] = lo; o[1] = hi;
+        } else if (out_f32) {
+          float4* o = reinterpret_cast<float4*>(static_cast<float*>(out) + n * H + h);
+          float4 p0 = make_float4(0.f, 0.f, 0.f, 0.f), p1 = p0;
+          if (beta != 0.f) { p0 = o[0]; p1 = o[1]; }
+          o[0] = make_float4(alpha * lo.x + beta * p0.x, alpha * lo.y + beta * p0.y, alpha * lo.z + beta * p0.z, alpha * lo.w + beta * p0.w);
+          o[1] = make_float4(alpha * hi.x + beta * p1.x, alpha * hi.y + beta * p1.y, alpha * hi.z + beta * p1.z, alpha * hi.w + beta * p1.w);
+        } else {
+          uint4* o = reinterpret_cast<uint4*>(static_cast<uint16_t*>(out) + n * H + h);
+          uint4 q = make_uint4(0, 0, 0, 0);
+          if (beta != 0.f) q = *o;
+          auto mix = [&](float x0, float x1, uint32_t old) __attribute__((always_inline)) {
+            return pack_bf16(alpha * x0 + beta * bf_to_f((uint16_t)(old & 0xFFFFu)), alpha * x1 + beta * bf_to_f((uint16_t)(old >> 16)));
+          };
+          *o = make_uint4(mix(lo.x, lo.y, q.x), mix(lo.z, lo.w, q.y), mix(hi.x, hi.y, q.z), mix(hi.z, hi.w, q.w));
+        }
+      }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  }
+}
+
 // out = alpha * sum_z partial[z] + beta * out, splits added in increasing z
 __global__ void __launch_bounds__(256)
 k_gradw_finish(const float* __restrict__ partial, int splits, int64_t total, float alpha, float beta,
@@ -994,6 +1334,23 @@ static int choose_splits(int64_t M, int64_t tiles) {
   return (int)s;
 }
 
+// ... for the 256 x 256 tiles of k_gradw_big, one workgroup per CU at a time.  A split costs a partial result written
+// and read again: 8 bytes per output element at about 4 TB/s against 2*M flop per element at about 1.1 PFLOP/s, i.e.
+// 1100 / M of the product's own time per split; the rounds of workgroups cost 1 / (filled share of the last round).
+static int choose_splits_big(int64_t M, int64_t tiles) {
+  const int64_t cus = 256;
+  const int64_t max_by_tokens = std::max<int64_t>(1, M / (8 * WK));   // at least 8 stages per split
+  int best = 1;
+  double best_cost = 0.0;
+  for (int64_t s = 1; s <= 16 && s <= max_by_tokens; ++s) {
+    const int64_t wgs = tiles * s;
+    const double rounds = (double)(((wgs + cus - 1) / cus) * cus) / (double)wgs;
+    const double cost = rounds + (s > 1 ? (double)s * 1100.0 / (double)M : 0.0);
+    if (s == 1 || cost < best_cost - 1e-9) { best_cost = cost; best = (int)s; }
+  }
+  return best;
+}
+
 }  // namespace hyc
 
 using namespace hyc;
@@ -1005,6 +1362,8 @@ int64_t hyc_gradw_workspace_bytes(int64_t M, int64_t N_out, int64_t H) {
   const int BN = N_out <= 32 ? 32 : 128;
   const int64_t tiles = ((N_out + BN - 1) / BN) * (H / GH);
   int splits = choose_splits(M, tiles);                   // dense source
+  if (N_out >= 2 * WN && H % GH == 0)                     // 256 x 256 tiles
+    splits = std::max(splits, choose_splits_big(M, ((N_out + 2 * WN - 1) / (2 * WN)) * ((H + WH - 1) / WH)));
   if (N_out <= DIRECT_MAX_N) {                            // channel-compressed source, few output rows
     const int ds = direct_splits_max(M, N_out, H);
     if (ds > splits) splits = ds;
@@ -1085,11 +1444,14 @@ int hyc_gradw_gemm(const void* dy, int64_t ldy, const void* stored, const void* 
   }
   const int BN = N_out <= 32 ? 32 : 128;
   const int64_t n_tiles = (N_out + BN - 1) / BN, h_tiles = H / GH;
-  const int splits = M > 0 ? choose_splits(M, n_tiles * h_tiles) : 1;     // (the wide kernel has half the tiles: same value)
   if (M > 0 && (!dy || !stored)) return fail(HYC_EFAULT, "hyc_gradw_gemm: null buffer");
-  // wide tiles (128 x 256) when the output is large and the tile grid fits the packing
-  // (the channel scheme uses the eight-wave form only: its four-wave form runs out of registers)
+  // wide tiles (256 columns) when the output is large and the tile grid fits the packing
+  // (the channel scheme has the 256-feature form only)
   const bool wide = chan ? (N_out >= 2 * WN && g.seg % (WH / g.nseg) == 0) : (N_out >= WN && H % WH == 0);
+  // 256 features per workgroup (four waves of 128 x 128) when the tile grid fills the chip, else 128 (dense only)
+  const int wnt = !wide ? 0 : chan || (N_out >= 2 * WN && ((N_out + 2 * WN - 1) / (2 * WN)) * (H / WH) >= 128) ? 2 * WN : WN;
+  const int splits = M <= 0 ? 1 : wnt == 2 * WN ? choose_splits_big(M, ((N_out + 2 * WN - 1) / (2 * WN)) * (H / WH))
+                                                : choose_splits(M, n_tiles * h_tiles);   // (128 x 256 tiles: same value)
   if (chan && M > 0 && (!scales || (d->k > 0 && !vals))) return fail(HYC_EFAULT, "hyc_gradw_gemm: null vals/scales");
   if (M > 0 && (!aligned16(dy) || !aligned8(stored) || (!chan && !aligned16(stored))))
     return fail(HYC_EINVAL, "hyc_gradw_gemm: dy must be 16-byte aligned, stored 8-byte (16 when dense)");
@@ -1104,26 +1466,28 @@ int hyc_gradw_gemm(const void* dy, int64_t ldy, const void* stored, const void* 
                                               chan ? std::max<int64_t>(2 * (H / d->group), 2 * (int64_t)d->k) : 0);
   const bool fits32 = (tps + WK) * pitch_max < ((int64_t)1 << 31);
   if (wide && fits32) {
-    // eight waves (256 features per workgroup) halve the decode work per MFMA; four waves fill the chip better
-    // when the output is small
-    const int wnt = chan || (N_out >= 2 * WN && ((N_out + 2 * WN - 1) / (2 * WN)) * (H / WH) >= 128) ? 2 * WN : WN;
     const dim3 wgrid((unsigned)((N_out + wnt - 1) / wnt), (unsigned)(H / WH), (unsigned)splits);
 #define HYC_WIDE_W(B_, S_, W_)                                                                                    \
   hipLaunchKernelGGL((k_gradw_wide<B_, S_, W_>), wgrid, dim3(2 * W_), 0, st, static_cast<const uint16_t*>(dy), ldy, M, \
                      N_out, H, static_cast<const uint8_t*>(stored), static_cast<const uint16_t*>(vals),          \
                      static_cast<const uint16_t*>(scales), ca, g.cps, tps, alpha, beta, out, of32, partial)
-    if (chan) {
-      switch (d->bits) {
-        case 1: HYC_WIDE_W(1, 0, 2 * WN); break;
-        case 2: HYC_WIDE_W(2, 0, 2 * WN); break;
-        case 4: HYC_WIDE_W(4, 0, 2 * WN); break;
-        default: HYC_WIDE_W(8, 0, 2 * WN); break;
-      }
-    } else if (wnt == WN) {
+#define HYC_BIG(B_, S_)                                                                                            \
+  hipLaunchKernelGGL((k_gradw_big<B_, S_>), wgrid, dim3(256), 0, st, static_cast<const uint16_t*>(dy), ldy, M,     \
+                     N_out, H, static_cast<const uint8_t*>(stored), static_cast<const uint16_t*>(vals),          \
+                     static_cast<const uint16_t*>(scales), ca, g.cps, tps, alpha, beta, out, of32, partial)
+    if (wnt == WN) {
       HYC_WIDE_W(4, 2, WN);
+    } else if (chan) {
+      switch (d->bits) {
+        case 1: HYC_BIG(1, 0); break;
+        case 2: HYC_BIG(2, 0); break;
+        case 4: HYC_BIG(4, 0); break;
+        default: HYC_BIG(8, 0); break;
+      }
     } else {
-      HYC_WIDE_W(4, 2, 2 * WN);
+      HYC_BIG(4, 2);
     }
+#undef HYC_BIG
 #undef HYC_WIDE_W
   } else {
 #define HYC_GEMM(B_, S_, N_)                                                                                     \

@@ -37,7 +37,9 @@ GEMM_CASES = [(4, 128, 200, 512, 16, 5), (2, 64, 300, 2048, 512, 20), (1, 64, 20
               # few output rows with the scale folded into dY: group 128 / 256 (16 chunks per tile), group 64 (8 chunks,
               # two lanes per chunk), one and two 16-row tiles of dY, ragged token counts, a partial last tile
               (2, 128, 333, 2048, 16, 20), (2, 128, 257, 2048, 32, 20), (2, 256, 190, 1024, 24, 10), (1, 128, 200, 2048, 16, 20),
-              (1, 64, 130, 1024, 8, 10), (2, 64, 77, 11008, 16, 110), (2, 64, 2100, 1024, 32, 10), (2, 64, 31, 512, 16, 0)]
+              (1, 64, 130, 1024, 8, 10), (2, 64, 77, 11008, 16, 110), (2, 64, 2100, 1024, 32, 10), (2, 64, 31, 512, 16, 0),
+              # 256-feature tiles: fewer tokens than the stages in flight, and a tile grid small enough for token splits
+              (2, 64, 40, 1024, 256, 10), (4, 128, 8200, 1024, 256, 10), (8, 128, 8192, 512, 264, 5)]
 
 
 @pytest.mark.parametrize("bits,group,M,H,N,k", GEMM_CASES)
