@@ -19,11 +19,25 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch at the bench workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
-# `bench.py --pmc-probe`, scaled by what the same counters read for a plain copy of known size
-# (profiles/rmsnorm_fwd_bwd_config2.md): FETCH_SIZE 16516.5 / 21039.0 KiB x 1.9986, WRITE_SIZE 41792.2 / 36888.7 KiB.
-TRAFFIC_FWD = int((16516.5 * 1.9986 + 41792.2) * 1024)
-TRAFFIC_BWD = int((21039.0 * 1.9986 + 36888.7) * 1024)
+# `bench.py --pmc-probe`, each scaled by what the same counter reads for a plain copy of known size
+# (profiles/rmsnorm_fwd_bwd_config2.md).  The figures belong to one state of the kernel sources: TRAFFIC_SOURCES_SHA
+# is the digest of those files when the counters were taken, and `roofline.traffic` is null whenever the files on
+# disk differ (a changed kernel needs new counter runs, not an old number).
+TRAFFIC_FWD = int((16508.05 * 1.99858 + 41793.23) * 1024)    # FETCH_SIZE KiB x copy factor + WRITE_SIZE KiB
+TRAFFIC_BWD = int((21030.51 * 1.99858 + 36865.50) * 1024)
+TRAFFIC_SOURCES = ("norm.hip", "row_kernels.hpp", "row_codec.hpp")
+TRAFFIC_SOURCES_SHA = "6466577f338e8dc6"
+
+
+def sources_sha():
+    import hashlib
+    h = hashlib.sha256()
+    for name in TRAFFIC_SOURCES:
+        with open(os.path.join(ROOT, "hyc-lora_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
 
 
 def algorithmic_bytes(M, H, bits, group, k):
@@ -107,31 +121,155 @@ def time_events(torch, fn, iters, warmup):
     return e0.elapsed_time(e1) / iters
 
 
-def gradw_extra(pkg, torch, wl):
-    """weight-gradient GEMM on the workload's compressed x (configs[2]/[3] shapes): full W and LoRA-A (r = 16)"""
+def time_graph(torch, fn, calls=10, replays=20):
+    """average milliseconds of fn(): `calls` invocations captured into one HIP graph (so that the host cost of the
+    Python wrapper does not space the launches out), replayed `replays` times between two events"""
+    fn()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        fn()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for _ in range(calls):
+            fn()
+    for _ in range(3):
+        graph.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(replays):
+        graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / (calls * replays)
+    del graph
+    return ms
+
+
+def side_bytes(H, bits, group, k):
+    """bytes per token of a channel-compressed activation: packed codes + outlier values + group scales"""
+    return H * bits // 8 + 2 * k + 2 * (H // group)
+
+
+def hbm(nbytes, ms):
+    return {"ms": round(ms, 5), "algorithmic_bytes": int(nbytes), "GBps": round(nbytes / ms / 1e6, 1),
+            "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+
+
+def make_activation(torch, M, H, hot, gain, seed):
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+    x = torch.randn(M, H, generator=gen, device="cuda")
+    x[:, torch.randperm(H, generator=gen, device="cuda")[:hot]] *= gain
+    return x.bfloat16(), gen
+
+
+def time_steady(torch, fn, iters, seconds=0.3):
+    """like time_events, after `seconds` of the same launches: a matrix-core kernel on an idle GPU runs at clocks it
+    does not hold (the first 20 ms read 15-20 % faster than the steady state), so every GEMM leg is timed warm"""
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(20):
+            fn()
+        torch.cuda.synchronize()
+    return time_events(torch, fn, iters, 5)
+
+
+def gradw_extra(pkg, torch, c, shapes=(("full_w", 4096, 100, 30), ("lora_a_r16", 16, 300, 30))):
+    """weight-gradient GEMM dW = dY^T . x_hat on the channel-compressed activation `c`: x_hat decoded inside the GEMM,
+    the staged route (restore x_hat once, then the dense form of the same kernel) and the framework's library GEMM on
+    the restored activation; every leg warmed before it is timed"""
     K, abi = pkg.kernels, pkg._abi
-    lib = wl.lib
-    M, H = wl.M, wl.H
+    lib = abi.load()
+    M, H = c.M, c.H
+    desc = c.desc()
     out = {}
     p = lambda t: ctypes.c_void_p(t.data_ptr()) if t is not None else None
-    for name, N, iters in (("full_w", 4096, 20), ("lora_a_r16", 16, 100)):
+    stream = lambda: ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    xh = K.decompress_channel(c)
+    # chunks of 8 channels that hold more than two outlier channels take the fused GEMM's rare (slow) splice path,
+    # and one such chunk column delays the whole launch: say whether this plan has one
+    seg = H * c.bits // 8
+    idx = c.plan.idx.cpu().long()
+    crowd = int(torch.bincount((idx // seg) * (seg // 8) + (idx % seg) // 8).max()) if idx.numel() else 0
+    for name, N, iters, warm in shapes:
         dy = (0.01 * torch.randn(M, N, device="cuda")).bfloat16()
         dw = torch.empty(N, H, dtype=torch.bfloat16, device="cuda")
         ws_bytes = lib.hyc_gradw_workspace_bytes(M, N, H)
         ws = torch.empty(max(ws_bytes // 4, 1), dtype=torch.float32, device="cuda")
-        args = (p(dy), N, p(wl.c.stored), p(wl.c.vals), p(wl.c.scales), M, N, H, ctypes.byref(wl.desc),
+        args = (p(dy), N, p(c.stored), p(c.vals), p(c.scales), M, N, H, ctypes.byref(desc),
                 ctypes.c_float(1.0), ctypes.c_float(0.0), p(dw), abi.DTYPE_BF16, p(ws))
-        fn = lambda: abi.check(lib.hyc_gradw_gemm(*args, wl._stream()))
-        ms = time_events(torch, fn, iters, 3)
-        xh = K.decompress_channel(wl.c)
-        ms_lib = time_events(torch, lambda: torch.matmul(dy.t(), xh), iters, 3)
-        # the same library's other route: decompress into a scratch matrix, then this kernel on the dense operand
-        ms_staged = time_events(torch, lambda: K.gradw_gemm(dy, wl.c, staged=True), iters, 3)
-        out[name] = {"M": M, "N_out": N, "H": H, "ms": round(ms, 5), "TFLOPs": round(2 * M * N * H / ms / 1e9, 1),
-                     "frac_of_bf16_mfma_peak": round(2 * M * N * H / ms / 1e9 / 2500.0, 4),
-                     "staged_ms": round(ms_staged, 5), "staged_TFLOPs": round(2 * M * N * H / ms_staged / 1e9, 1),
-                     "library_gemm_on_decompressed_ms": round(ms_lib, 5)}
-        del dy, dw, ws, xh
+        fn = lambda: abi.check(lib.hyc_gradw_gemm(*args, stream()))
+        flop = 2.0 * M * N * H
+        ms = time_steady(torch, fn, iters) if N > 64 else time_events(torch, fn, iters, warm)
+        rec = {"M": M, "N_out": N, "H": H, "bits": c.bits, "group": c.group, "most_outlier_channels_in_a_chunk": crowd,
+               "flop": int(flop), "ms": round(ms, 5),
+               "TFLOPs": round(flop / ms / 1e9, 1), "frac_of_bf16_mfma_peak": round(flop / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4)}
+        if N <= 64:
+            # few output rows: the product is bound by reading the compressed activation and dY once
+            nbytes = M * (side_bytes(H, c.bits, c.group, c.plan.k) + 2 * N) + 2 * N * H
+            rec.update({"algorithmic_bytes": int(nbytes), "GBps": round(nbytes / ms / 1e6, 1),
+                        "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)})
+        else:
+            ms_staged = time_steady(torch, lambda: K.gradw_gemm(dy, c, staged=True), iters)
+            ms_dense = time_steady(torch, lambda: K.gradw_gemm(dy, xh), iters)
+            rec.update({"staged_ms": round(ms_staged, 5), "staged_TFLOPs": round(flop / ms_staged / 1e9, 1),
+                        "staged_frac_of_bf16_mfma_peak": round(flop / ms_staged / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
+                        "dense_operand_ms": round(ms_dense, 5), "dense_operand_TFLOPs": round(flop / ms_dense / 1e9, 1),
+                        "dense_operand_frac_of_bf16_mfma_peak": round(flop / ms_dense / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
+                        "default_route": "staged" if N >= K.STAGED_GRADW_MIN_FEATURES else "fused"})
+        ms_lib = (time_steady(torch, lambda: torch.matmul(dy.t(), xh), iters) if N > 64 else
+                  time_events(torch, lambda: torch.matmul(dy.t(), xh), iters, warm))
+        rec["library_gemm_on_decompressed_ms"] = round(ms_lib, 5)
+        out[name] = rec
+        del dy, dw, ws
+    del xh
+    return out
+
+
+def config1_extra(pkg, torch):
+    """BASELINE configs[0] on the GPU: standalone compress + decompress of x [4,512,4096] (41 outlier channels x50,
+    INT4, group 128), and the same at 16x the tokens"""
+    K = pkg.kernels
+    out = {}
+    for tag, M in (("tokens_2048", 2048), ("tokens_32768", 32768)):
+        H, bits, G, k = 4096, 4, 128, 41
+        x, _ = make_activation(torch, M, H, k, 50.0, seed=11)
+        plan = K.select_channels(K.channel_absmax(x), k)
+        c = K.compress_channel(x, plan, bits, G)
+        side = side_bytes(H, bits, G, k)
+        t_c = time_graph(torch, lambda: K.compress_channel(x, plan, bits, G))
+        t_d = time_graph(torch, lambda: K.decompress_channel(c))
+        t_p = time_events(torch, lambda: K.select_channels(K.channel_absmax(x), k), 50, 5)
+        assert torch.equal(K.decompress_channel(K.compress_channel(x, plan, bits, G)), K.decompress_channel(c))
+        out[tag] = {"compress": hbm(M * (2 * H + side), t_c), "decompress": hbm(M * (2 * H + side), t_d),
+                    "round_trip": hbm(2 * M * (2 * H + side), t_c + t_d),
+                    "channel_absmax_and_select_ms": round(t_p, 5)}
+        del x, c
+    return out
+
+
+def config4_extra(pkg, torch):
+    """BASELINE configs[3]: gate / up [4,1024,11008] with 1 % outlier channels x20, INT4 group 128: SiLU backward,
+    the one-pass backward of SiLU(gate)*up, and the down_proj weight gradient (dY [4096,4096], 369 GFLOP) with its
+    LoRA-A (r = 16) companion"""
+    K = pkg.kernels
+    M, H, bits, G = 4096, 11008, 4, 128
+    k = K.num_outlier_channels(H, 0.01)
+    gate, gen = make_activation(torch, M, H, k, 20.0, seed=41)
+    up, _ = make_activation(torch, M, H, k, 20.0, seed=42)
+    act = torch.nn.functional.silu(gate.float()).bfloat16()
+    prod = (act.float() * up.float()).bfloat16()
+    g = (0.02 * torch.randn(M, H, generator=gen, device="cuda")).bfloat16()
+    cg, cu, ca, cp = [K.compress_channel(t, K.select_channels(K.channel_absmax(t), k), bits, G) for t in (gate, up, act, prod)]
+    side = side_bytes(H, bits, G, k)
+    out = {"silu_bwd": hbm(M * (4 * H + side), time_graph(torch, lambda: K.act_bwd("silu", g, cg))),
+           "gated_silu_bwd": hbm(M * (6 * H + 3 * side), time_graph(torch, lambda: K.gated_act_bwd("silu", g, ca, cu, cg))),
+           "silu_fwd_compress": hbm(M * (4 * H + side), time_graph(torch, lambda: K.act_fwd_compress("silu", gate, cg.plan, bits, G)))}
+    del gate, up, act, prod, g, cg, cu, ca
+    out["down_proj"] = gradw_extra(pkg, torch, cp, shapes=(("full_w", 4096, 60, 20), ("lora_a_r16", 16, 300, 30)))
     return out
 
 
@@ -204,7 +342,7 @@ def kernel_tour(pkg, torch, reps=5):
     print(json.dumps({"kernel_tour": True}))
 
 
-def layer_report(pkg, torch, steps=6, attentions=("eager", "flash")):
+def layer_report(pkg, torch, steps=6, attentions=("eager", "flash"), quiet=False):
     """full LLaMA-2-7B-shaped decoder layer (hidden 4096, 32 x 128 heads, intermediate 11008, NF4 base, LoRA r=16 on
     all seven projections), forward + backward, at batch 1 x seq 2048 and batch 4 x seq 1024: what the forward keeps
     for the backward, the peak above the resident weights, and the step time - with every saved activation compressed
@@ -254,7 +392,8 @@ def layer_report(pkg, torch, steps=6, attentions=("eager", "flash")):
             if compress:
                 rec["saved_analytic_bytes"] = int(layer.saved_activation_bytes(B, S))
             out.append(rec)
-            print(json.dumps(rec), flush=True)
+            if not quiet:
+                print(json.dumps(rec), flush=True)
         del layer
         torch.cuda.empty_cache()
     return out
@@ -297,6 +436,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-scaled", action="store_true", help="skip the 16x token-scaled run")
+    ap.add_argument("--no-extras", action="store_true", help="skip the legs of the other BASELINE configurations")
     ap.add_argument("--kernel-tour", action="store_true",
                     help="for rocprofv3 --kernel-trace: run every kernel of the path a few times at the config shapes, then exit")
     ap.add_argument("--pmc-probe", action="store_true",
@@ -343,6 +483,39 @@ def main():
         print(json.dumps({"pmc_probe": True, "copy_bytes_each_way": 2 * M * H, "fwd_bytes": fwd_b, "bwd_bytes": bwd_b}))
         return
 
+    # ---- the other configurations and the long runs first: they also bring the clocks up before the short timed
+    # region (a cold 20-step loop of 15-microsecond kernels reads 10-15 % slower than the same loop on a busy GPU)
+    extra = {}
+    extra["gradw_gemm_int4"] = gradw_extra(pkg, torch, wl.c)
+    if not args.no_extras:
+        extra["config1_compress_decompress"] = config1_extra(pkg, torch)
+        K = pkg.kernels
+        x3, _ = make_activation(torch, M, H, wl.k, 30.0, seed=31)
+        c3 = K.compress_channel(x3, K.select_channels(K.channel_absmax(x3), wl.k), 2, 64)
+        extra["config3_gradw_int2_g64"] = gradw_extra(pkg, torch, c3)
+        del x3, c3
+        extra["config4_mlp_h11008"] = config4_extra(pkg, torch)
+    if not args.no_scaled:
+        # the config-size working set (~150 MB) fits the 256 MB Infinity Cache; 16x the tokens does not
+        Ms = 16 * M
+        wls = Workload(pkg, torch, Ms, H, bits, group, n_hot=20, gain=30.0, seed=1)
+        fs, bs, _ = algorithmic_bytes(Ms, H, bits, group, wls.k)
+        f_ms = time_events(torch, wls.fwd, 60, 10)
+        b_ms = time_events(torch, wls.bwd, 60, 10)
+        bm_ms = time_events(torch, wls.bwd_main, 60, 10)
+        extra["scaled16x"] = {"tokens": Ms, "fwd_ms": round(f_ms, 4), "fwd_GBps": round(fs / f_ms / 1e6, 1),
+                              "bwd_ms": round(b_ms, 4), "bwd_GBps": round(bs / b_ms / 1e6, 1),
+                              "bwd_row_kernel_ms": round(bm_ms, 4),
+                              "fwd_frac_of_hbm_peak": round(fs / f_ms / 1e6 / HBM_PEAK_GBPS, 4),
+                              "bwd_frac_of_hbm_peak": round(bs / b_ms / 1e6 / HBM_PEAK_GBPS, 4),
+                              "bwd_row_kernel_frac_of_hbm_peak": round(bs / bm_ms / 1e6 / HBM_PEAK_GBPS, 4)}
+        del wls
+        torch.cuda.empty_cache()
+    if not args.no_extras:
+        # configs[4]: the decoder layer with the reference's attention wiring, every saved activation compressed / kept bf16
+        extra["config5_decoder_layer"] = layer_report(pkg, torch, steps=4, attentions=("eager",), quiet=True)
+        torch.cuda.empty_cache()
+
     # the step as a HIP graph (three launches; removes the host launch cost from the timed loop)
     wl.step()
     torch.cuda.synchronize()
@@ -354,6 +527,7 @@ def main():
     torch.cuda.current_stream().wait_stream(side)
     with torch.cuda.graph(graph):
         wl.step()
+
     def wall(fn):
         for _ in range(args.warmup):
             fn()
@@ -364,45 +538,42 @@ def main():
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) * 1e3 / args.steps
 
-    # the timed region: K steps between two synchronisations, launched back to back on one stream (the three
-    # kernels of a step are short enough that a graph replay per step costs more than it saves)
+    # per-kernel durations with events on the launch stream, over enough launches for a steady clock; they come
+    # before the timed region so that it starts on a busy GPU
+    n_ev = max(args.steps, 500)
+    fwd_ms = time_events(torch, wl.fwd, n_ev, 50)
+    bwd_ms = time_events(torch, wl.bwd, n_ev, 50)
+    bwd_main_ms = time_events(torch, wl.bwd_main, n_ev, 50)                  # the row kernel alone
+    eager_ms = time_events(torch, wl.step, n_ev, 50)
+
+    # the timed region: W warm-up steps, then exactly K steps between two synchronisations, launched back to back on
+    # one stream (the kernels of a step are short enough that a graph replay per step costs more than it saves)
     ms_step = wall(wl.step)
     ms_graph = wall(graph.replay)
-
-    # eager launches for comparison, and per-kernel durations with events on the launch stream
-    eager_ms = time_events(torch, wl.step, args.steps, args.warmup)
-    fwd_ms = time_events(torch, wl.fwd, args.steps, args.warmup)
-    bwd_ms = time_events(torch, wl.bwd, args.steps, args.warmup)
-    bwd_main_ms = time_events(torch, wl.bwd_main, args.steps, args.warmup)   # k_rmsnorm_bwd_fast alone
+    del graph
 
     value = (fwd_b + bwd_b) / (ms_step * 1e-3) / 1e9
+    fresh = TRAFFIC_SOURCES_SHA != "" and sources_sha() == TRAFFIC_SOURCES_SHA
     if bwd_main_ms >= fwd_ms:
-        dom_name, dom_ms, dom_b, dom_traffic = "hyc::k_rmsnorm_bwd_fast<4,true,true,1024>", bwd_main_ms, bwd_b, TRAFFIC_BWD
+        dom_name, dom_ms, dom_b, dom_traffic = "hyc::k_rmsnorm_bwd_fast<4, true, true, 1024, false>", bwd_main_ms, bwd_b, TRAFFIC_BWD
     else:
-        dom_name, dom_ms, dom_b, dom_traffic = "hyc::k_rmsnorm_fwd_fast<4,16,true,256>", fwd_ms, fwd_b, TRAFFIC_FWD
+        dom_name, dom_ms, dom_b, dom_traffic = "hyc::k_rmsnorm_fwd_fast<4, 16, true, 256, 1>", fwd_ms, fwd_b, TRAFFIC_FWD
     achieved = dom_b / (dom_ms * 1e-3) / 1e9
-    extra = {
+    extra.update({
         "graph_replay_ms_per_step": round(ms_graph, 5), "event_ms_per_step": round(eager_ms, 5),
+        "event_loop_launches": n_ev,
         "fwd_kernel_ms": round(fwd_ms, 5), "fwd_GBps": round(fwd_b / fwd_ms / 1e6, 1),
+        "fwd_frac_of_hbm_peak": round(fwd_b / fwd_ms / 1e6 / HBM_PEAK_GBPS, 4),
         "bwd_kernels_ms": round(bwd_ms, 5), "bwd_GBps": round(bwd_b / bwd_ms / 1e6, 1),
         "bwd_row_kernel_ms": round(bwd_main_ms, 5), "bwd_row_kernel_GBps": round(bwd_b / bwd_main_ms / 1e6, 1),
+        "bwd_row_kernel_frac_of_hbm_peak": round(bwd_b / bwd_main_ms / 1e6 / HBM_PEAK_GBPS, 4),
         "act_mem_bytes_saved_tensor": saved_b + 4 * M, "act_mem_bytes_bf16": 2 * M * H,
         "act_mem_ratio": round(2 * M * H / (saved_b + 4 * M), 3),
-    }
-    extra["gradw_gemm_int4"] = gradw_extra(pkg, torch, wl)
-    if not args.no_scaled:
-        # the config-size working set (~150 MB) fits the 256 MB Infinity Cache; 16x the tokens does not
-        del graph
-        Ms = 16 * M
-        wls = Workload(pkg, torch, Ms, H, bits, group, n_hot=20, gain=30.0, seed=1)
-        fs, bs, _ = algorithmic_bytes(Ms, H, bits, group, wls.k)
-        f_ms = time_events(torch, wls.fwd, 30, 5)
-        b_ms = time_events(torch, wls.bwd, 30, 5)
-        extra["scaled16x"] = {"tokens": Ms, "fwd_ms": round(f_ms, 4), "fwd_GBps": round(fs / f_ms / 1e6, 1),
-                              "bwd_ms": round(b_ms, 4), "bwd_GBps": round(bs / b_ms / 1e6, 1),
-                              "fwd_frac_of_hbm_peak": round(fs / f_ms / 1e6 / HBM_PEAK_GBPS, 4),
-                              "bwd_frac_of_hbm_peak": round(bs / b_ms / 1e6 / HBM_PEAK_GBPS, 4)}
-        del wls
+        "scale_rule": "absmax",
+        "traffic_note": ("HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of `bench.py --pmc-probe` "
+                         "(profiles/rmsnorm_fwd_bwd_config2.md), taken with these kernel sources" if fresh else
+                         "null: the kernel sources differ from the ones the committed counter runs were taken with"),
+    })
     out = {
         "metric": "compress+decompress GB/s", "value": round(value, 2), "unit": "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 5),
@@ -413,7 +584,7 @@ def main():
                    "launch": "fwd + bwd (+ dw column sum) entry points back to back on one stream"},
         "roofline": {"bound": "hbm", "kernel": dom_name, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "algorithmic_bytes": dom_b,
-                     "traffic": dom_traffic},
+                     "traffic": dom_traffic if fresh else None},
         "extra": extra,
     }
     if not args.no_cpu_baseline:
