@@ -78,7 +78,8 @@ class _FlashAttentionAt(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, q_hat, k_hat, v_hat, o_hat, scale, causal=True):
         s = q.shape[-2]
-        mask = torch.ones(s, s, dtype=torch.bool).triu(1) if causal else torch.zeros(s, s, dtype=torch.bool)
+        mask = (torch.ones(s, s, dtype=torch.bool, device=q.device).triu(1) if causal else
+                torch.zeros(s, s, dtype=torch.bool, device=q.device))
         scores = (q @ k.transpose(-2, -1)) * scale
         scores = scores.masked_fill(mask, float("-inf"))
         lse = torch.logsumexp(scores, dim=-1, keepdim=True)
@@ -150,7 +151,7 @@ def decoder_layer(x, params, restored, nh, eps, scaling, cos, sin, quirk=True, p
     q_hat, k_hat, v_hat = (heads(hat(n, rows(t)), nh) for n, t in (("q", q), ("k", k), ("v", v)))
     if attention == "flash":
         with torch.no_grad():
-            mask = torch.ones(s, s, dtype=torch.bool).triu(1)
+            mask = torch.ones(s, s, dtype=torch.bool, device=q.device).triu(1)
             sc = (q @ k.transpose(-2, -1) / math.sqrt(q.shape[-1])).masked_fill(mask, float("-inf"))
             o_exact = rows(torch.softmax(sc, dim=-1) @ v)
         o_hat = heads(hat("o", o_exact), nh)
@@ -158,7 +159,7 @@ def decoder_layer(x, params, restored, nh, eps, scaling, cos, sin, quirk=True, p
     else:
         scores = _value_of(q @ k.transpose(-2, -1), _st(q, q_hat) @ _st(k, k_hat).transpose(-2, -1))
         scores = scores / math.sqrt(q.shape[-1])
-        mask = torch.ones(s, s, dtype=torch.bool).triu(1)
+        mask = torch.ones(s, s, dtype=torch.bool, device=q.device).triu(1)
         scores = scores.masked_fill(mask, torch.finfo(torch.bfloat16).min)
         p_exact = torch.softmax(scores.detach(), dim=-1) if probs is None else probs.float()
         p_hat = hat("p", p_exact)

@@ -223,3 +223,103 @@ def test_training_tracks_the_uncompressed_layer(DL, K):
     assert c[-1] < 0.67 * c[0], (c[0], c[-1])
     assert u[-1] < 0.67 * u[0], (u[0], u[-1])
     assert abs(c[-1] - u[-1]) < 0.15 * u[0], (c[-1], u[-1], u[0])
+
+
+@pytest.mark.parametrize("B,S", [(1, 2048), (4, 1024)])
+def test_layer_at_its_own_size(DL, K, B, S):
+    """The fifth configuration at its real size (hidden 4096, 32 heads x 128, intermediate 11008, NF4 base, LoRA r = 16,
+    1 % outlier channels, INT2 linear inputs, INT4 elsewhere), batch 1 x 2048 and 4 x 1024 tokens, three steps (two
+    calibrating, one steady).  On each step: every compressed site restores, bit for bit on a 48-row sample, what the
+    oracle's compress / decompress gives for the activation the device saw; the kept probabilities are the oracle's
+    set; the layer's output and every gradient are within 1e-2 (relative norm) of the oracle layer evaluated at the
+    restored activations (the oracle, plain fp32 torch, runs on the GPU here: its matrix products at this size take
+    minutes on the host).  After the steps: what a forward keeps matches the analytic count."""
+    cfg = DL.LayerConfig()
+    layer = DL.DecoderLayer(cfg)
+    H, I, nh = cfg.hidden, cfg.intermediate, cfg.heads
+    gen = torch.Generator().manual_seed(B * 1000 + S)
+    P, groups = oracle_params(K, layer)
+    P = {n: t.detach().cuda().requires_grad_(t.requires_grad) for n, t in P.items()}
+    cos, sin = (t.float() for t in DL.rope_tables(S, cfg.head_dim, cfg.rope_theta, "cuda"))
+    rec = {"qkv": {}, "o": {}, "gate_up": {}, "down": {}, "attn": {}}
+    layer.qkv_proj.record, layer.o_proj.record = rec["qkv"], rec["o"]
+    layer.gate_up_proj.record, layer.down_proj.record = rec["gate_up"], rec["down"]
+    layer.attention.record = rec["attn"]
+    grabbed = {}
+    hooks = [layer.input_layernorm.register_forward_hook(lambda m, i, o: grabbed.__setitem__("norm_in", (i[0].detach().clone(), o.grad_fn.saved))),
+             layer.post_attention_layernorm.register_forward_hook(lambda m, i, o: grabbed.__setitem__("norm_post", (i[0].detach().clone(), o.grad_fn.saved))),
+             layer.act.register_forward_hook(lambda m, i, o: grabbed.__setitem__("act", (i[0].detach().clone(), i[1].detach().clone(), o.grad_fn.saved)))]
+    rows = torch.randperm(B * S, generator=gen)[:48].sort().values
+
+    def restore_and_check(x2d, c, bits, group):
+        xh = K.decompress_channel(c)
+        idx = c.plan.idx.cpu().long()
+        r = rows.to(x2d.device)
+        vals, stored, scales = O.hyc_compress(x2d[r].cpu(), idx, bits, group)
+        assert torch.equal(c.stored[r].cpu().view(torch.uint8), stored.view(torch.uint8))
+        assert bits_equal(xh[r].cpu(), O.hyc_decompress(vals, stored, idx, scales, bits, group))
+        return xh
+
+    def err(a, b):
+        return float((a.double() - b.double()).norm() / b.double().norm().clamp_min(1e-30))
+
+    for step in range(3):
+        x = make_input(gen, B, S, H)
+        g = (0.05 * torch.randn(B, S, H, generator=gen)).bfloat16()
+        for p in layer.parameters():
+            p.grad = None
+        xg = x.cuda().requires_grad_(True)
+        y = layer(xg)
+        y.backward(g.cuda())
+        ab, ag, lb, lg = cfg.act_bits, cfg.act_group, cfg.linear_bits, cfg.linear_group
+        R = {}
+        for site in ("norm_in", "norm_post"):
+            xin, c = grabbed[site]
+            R[site] = restore_and_check(xin.reshape(-1, H), c, ab, ag).reshape(B, S, H)
+        for site, key in (("qkv_in", "qkv"), ("o_in", "o"), ("gate_up_in", "gate_up"), ("down_in", "down")):
+            R[site] = restore_and_check(rec[key]["x"], rec[key]["saved"], lb, lg).reshape(B, S, -1)
+        for n, c in zip("qkv", rec["attn"]["saved"]):
+            R[n] = restore_and_check(rec["attn"][n].contiguous(), c, ab, ag).reshape(B, S, H)
+        gate, up, (c_act, c_up, c_gate) = grabbed["act"]
+        R["gate"] = restore_and_check(gate.reshape(-1, I), c_gate, ab, ag).reshape(B, S, I)
+        R["up"] = restore_and_check(up.reshape(-1, I), c_up, ab, ag).reshape(B, S, I)
+        R["act"] = restore_and_check(torch.nn.functional.silu(gate).reshape(-1, I), c_act, ab, ag).reshape(B, S, I)
+        p_dev = rec["attn"]["p"]
+        thr = O.get_statistics_softmax(p_dev, step, cfg.softmax_ratio) if step < 2 else layer.attention.static_value
+        R["p"] = torch.cat([K.softmax_dense(sp) for sp in rec["attn"]["sparse"]]).reshape(p_dev.shape)
+        assert bits_equal(R["p"], O.prune_softmax(p_dev, thr))
+        kept = float((R["p"] > 0).float().mean())
+        assert 0.002 < kept < 0.03, kept
+
+        for t in P.values():
+            t.grad = None
+        xo = x.float().cuda().requires_grad_(True)
+        yo = LO.decoder_layer(xo, P, R, nh, cfg.rms_eps, cfg.lora_alpha / cfg.lora_r, cos, sin, quirk=True, probs=p_dev,
+                              attention="eager")
+        yo.backward(g.float().cuda())
+        errs = {"y": err(y.detach(), yo.detach()), "dx": err(xg.grad, xo.grad),
+                "w_in": err(layer.input_layernorm.weight.grad, P["w_in"].grad),
+                "w_post": err(layer.post_attention_layernorm.weight.grad, P["w_post"].grad)}
+        for n, (mod, i) in groups.items():
+            errs["A_" + n] = err(mod.lora_A[i].grad, P["A_" + n].grad)
+            errs["B_" + n] = err(mod.lora_B[i].grad, P["B_" + n].grad)
+        assert all(v == v and v < 1e-2 for v in errs.values()), (step, errs)
+        del yo, xo, R, p_dev
+        rec["attn"].clear()
+    for h in hooks:
+        h.remove()
+    layer.qkv_proj.record = layer.o_proj.record = layer.gate_up_proj.record = layer.down_proj.record = None
+    layer.attention.record = None
+    assert layer.attention.iteration == 3 and layer.qkv_proj.iteration == 3
+    # what one forward keeps
+    grabbed.clear()
+    del y, xg
+    torch.cuda.synchronize()
+    xg = make_input(gen, B, S, H).cuda().requires_grad_(True)
+    before = torch.cuda.memory_allocated()
+    y = layer(xg)
+    torch.cuda.synchronize()
+    held = torch.cuda.memory_allocated() - before - y.numel() * 2
+    analytic = layer.saved_activation_bytes(B, S)
+    assert 0.9 * analytic < held < 1.25 * analytic, (held, analytic)
+    y.sum().backward()
