@@ -947,11 +947,14 @@ int hyc_gated_act_fwd(int32_t act, const void* gate, int64_t ld_gate, const void
   if ((rc = make_chan_args(d_a, geo, &c_a, &lpg)) || (rc = make_chan_args(d_u, geo, &c_u, &lpg)) ||
       (rc = make_chan_args(d_g, geo, &c_g, &lpg)))
     return rc;
-  // Three encoders side by side: with four segments per thread (2-bit codes) or more than 768 threads per row the
-  // kernel would not fit the register file, so those shapes are left to the separate calls.
-  if (geo.iters != 1 || geo.threads > 768 || (d_a->bits != 4 && d_a->bits != 8) || (lpg != 8 && lpg != 16))
-    return fail(HYC_ENOTSUP, "hyc_gated_act_fwd: needs 4- or 8-bit codes, groups of 64 or 128 channels and rows of at "
-                             "most 768 chunks per segment (use the activation, hyc_compress and a product otherwise)");
+  // Three encoders side by side: the per-thread state grows with the segments a thread holds (four with 2-bit
+  // codes), so the workgroup is capped at 768 threads (512 with 2-bit codes: 256 registers each); longer rows are
+  // left to the separate calls.
+  const int most = d_a->bits == 2 ? 512 : 768;
+  if (geo.iters != 1 || geo.threads > most || (d_a->bits != 2 && d_a->bits != 4 && d_a->bits != 8) || (lpg != 8 && lpg != 16))
+    return fail(HYC_ENOTSUP, "hyc_gated_act_fwd: needs 2-, 4- or 8-bit codes, groups of 64 or 128 channels and rows of at "
+                             "most 768 chunks per segment (512 with 2-bit codes; use the activation, hyc_compress and a "
+                             "product otherwise)");
   if (M == 0) return HYC_OK;
   if (!gate || !up || !h || !stored_a || !stored_u || !stored_g || !scales_a || !scales_u || !scales_g ||
       (d_a->k > 0 && !vals_a) || (d_u->k > 0 && !vals_u) || (d_g->k > 0 && !vals_g))
@@ -972,12 +975,15 @@ int hyc_gated_act_fwd(int32_t act, const void* gate, int64_t ld_gate, const void
 #define HYC_GFWD_T(B_, L_, A_) /* H = 11008: 704 threads, up to 168 registers each */ \
   do { if (geo.threads <= 256) HYC_GFWD(B_, L_, A_, 256); else HYC_GFWD(B_, L_, A_, 768); } while (0)
 #define HYC_GFWD_L(B_, A_) do { if (lpg == 8) HYC_GFWD_T(B_, 8, A_); else HYC_GFWD_T(B_, 16, A_); } while (0)
+#define HYC_GFWD_T2(L_, A_) do { if (geo.threads <= 256) HYC_GFWD(2, L_, A_, 256); else HYC_GFWD(2, L_, A_, 512); } while (0)
 #define HYC_GFWD_B(A_)                                                                                             \
   do {                                                                                                             \
-    if (d_a->bits == 4) HYC_GFWD_L(4, A_); else HYC_GFWD_L(8, A_);                                                \
+    if (d_a->bits == 2) { if (lpg == 8) HYC_GFWD_T2(8, A_); else HYC_GFWD_T2(16, A_); }                            \
+    else if (d_a->bits == 4) HYC_GFWD_L(4, A_); else HYC_GFWD_L(8, A_);                                           \
   } while (0)
   if (act == HYC_ACT_SILU) HYC_GFWD_B(HYC_ACT_SILU); else HYC_GFWD_B(HYC_ACT_GELU_TANH);
 #undef HYC_GFWD_B
+#undef HYC_GFWD_T2
 #undef HYC_GFWD_L
 #undef HYC_GFWD_T
 #undef HYC_GFWD
@@ -1003,10 +1009,11 @@ static int ew_fwd_impl(const char* who, int32_t act, const void* x1, int64_t ld1
   ChanArgs c1 = {}, c2 = {};
   int lpg = 16;
   if ((rc = make_chan_args(d1, geo, &c1, &lpg)) || (two && (rc = make_chan_args(d2, geo, &c2, &lpg)))) return rc;
-  // per-thread state grows with segments x operands: two operands of 2-bit codes do not fit the register file
-  if (geo.iters != 1 || d1->bits == 1 || (two && d1->bits == 2) || (lpg != 8 && lpg != 16))
-    return fail(HYC_ENOTSUP, "%s: needs 2-, 4- or 8-bit codes (4 or 8 for two operands), groups of 64 or 128 channels "
-                             "and rows of at most 1024 chunks per segment (use the separate calls otherwise)", who);
+  // per-thread state grows with segments x operands: two operands of 2-bit codes take a workgroup of at most 512
+  // threads (256 registers each)
+  if (geo.iters != 1 || d1->bits == 1 || (two && d1->bits == 2 && geo.threads > 512) || (lpg != 8 && lpg != 16))
+    return fail(HYC_ENOTSUP, "%s: needs 2-, 4- or 8-bit codes, groups of 64 or 128 channels and rows of at most 1024 "
+                             "chunks per segment (512 for two operands of 2-bit codes; use the separate calls otherwise)", who);
   if (M == 0) return HYC_OK;
   if (!x1 || !y || !stored1 || !scales1 || (d1->k > 0 && !vals1) ||
       (two && (!x2 || !stored2 || !scales2 || (d2->k > 0 && !vals2))))
@@ -1025,7 +1032,10 @@ static int ew_fwd_impl(const char* who, int32_t act, const void* x1, int64_t ld1
                      s1, s2, static_cast<uint16_t*>(y), use_lut)
 #define HYC_EW_T(B_, L_, A_, N_) do { if (geo.threads <= 256) HYC_EW(B_, L_, A_, N_, 256); else HYC_EW(B_, L_, A_, N_, 1024); } while (0)
 #define HYC_EW_L(B_, A_, N_) do { if (lpg == 8) HYC_EW_T(B_, 8, A_, N_); else HYC_EW_T(B_, 16, A_, N_); } while (0)
-  if (two) {
+  if (two && d1->bits == 2) {
+    if (geo.threads <= 256) { if (lpg == 8) HYC_EW(2, 8, ACT_MUL, 2, 256); else HYC_EW(2, 16, ACT_MUL, 2, 256); }
+    else { if (lpg == 8) HYC_EW(2, 8, ACT_MUL, 2, 512); else HYC_EW(2, 16, ACT_MUL, 2, 512); }
+  } else if (two) {
     if (d1->bits == 4) HYC_EW_L(4, ACT_MUL, 2); else HYC_EW_L(8, ACT_MUL, 2);
   } else if (act == HYC_ACT_SILU) {
     if (d1->bits == 2) HYC_EW_L(2, HYC_ACT_SILU, 1); else if (d1->bits == 4) HYC_EW_L(4, HYC_ACT_SILU, 1); else HYC_EW_L(8, HYC_ACT_SILU, 1);

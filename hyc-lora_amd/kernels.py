@@ -566,7 +566,9 @@ def act_fwd_compress_supported(H, bits, group):
 
 
 def hadamard_fwd_compress_supported(H, bits1, group1, bits2, group2):
-    return bits1 == bits2 and group1 == group2 and _row_kernel_fits(H, bits1, group1, (4, 8))
+    """shapes the one-pass product forward covers (two operands of 2-bit codes: at most 512 chunks per segment)"""
+    return (bits1 == bits2 and group1 == group2 and _row_kernel_fits(H, bits1, group1, (2, 4, 8)) and
+            (bits1 != 2 or H * bits1 // 64 <= 512))
 
 
 def act_fwd_compress(act, x2d, plan, bits, group):
@@ -601,7 +603,8 @@ def hadamard_fwd_compress(a2d, b2d, plan_a, plan_b, bits, group):
 
 def gated_act_fwd_supported(H, bits, group):
     """shapes the one-pass forward covers (the rest takes the activation, three compress calls and a product)"""
-    return bits in (4, 8) and group in (64, 128) and H * bits // 64 <= 768 and H % (64 // bits) == 0
+    return (bits in (2, 4, 8) and group in (64, 128) and H * bits // 64 <= (512 if bits == 2 else 768) and
+            H % (64 // bits) == 0)
 
 
 def gated_act_fwd(act, gate2d, up2d, plan_act, plan_up, plan_gate, bits, group):

@@ -229,8 +229,9 @@ int hyc_gated_act_bwd(int32_t act, const void* g, const void* stored_a, const vo
  * and EfficientMemoryHadamard.forward, efficient_hadamard.py:11-53, compute and save), in one pass over gate and up;
  * act(gate) is never written to memory.  gate and up are bf16 [M, H] with row pitches ld_gate, ld_up (elements).  act:
  * HYC_ACT_SILU = F.silu; HYC_ACT_GELU_TANH = the GELU module, whose forward is the erf form (F.gelu) and whose backward
- * is the tanh form.  Same bytes as the separate calls; channel scheme, one code width (4 or 8 bits) and group size (64 or
- * 128) for the three, H * bits / 64 <= 768; HYC_ENOTSUP otherwise (the separate calls cover every shape). */
+ * is the tanh form.  Same bytes as the separate calls; channel scheme, one code width (2, 4 or 8 bits) and group size (64
+ * or 128) for the three, H * bits / 64 <= 768 (<= 512 with 2-bit codes); HYC_ENOTSUP otherwise (the separate calls cover
+ * every shape). */
 int hyc_gated_act_fwd(int32_t act, const void* gate, int64_t ld_gate, const void* up, int64_t ld_up, int64_t M, int64_t H,
                       const hyc_desc* d_a, const hyc_desc* d_u, const hyc_desc* d_g, void* h, void* stored_a, void* vals_a,
                       void* scales_a, void* stored_u, void* vals_u, void* scales_u, void* stored_g, void* vals_g,
@@ -241,9 +242,9 @@ int hyc_gated_act_fwd(int32_t act, const void* gate, int64_t ld_gate, const void
  *   hyc_act_fwd_compress       y = act(x) and x compressed (EfficientMemorySiLU / GELU forward, efficient_silu.py:13-40,
  *                              efficient_gelu.py:13-40; act codes as for hyc_gated_act_fwd); 2-, 4- or 8-bit codes
  *   hyc_hadamard_fwd_compress  y = x1 * x2 and both operands compressed (EfficientMemoryHadamard forward,
- *                              efficient_hadamard.py:11-53); one code width (4 or 8 bits) and group size for both
- * Inputs are bf16 [M, H] with row pitches in elements; groups of 64 or 128 channels, H * bits / 64 <= 1024;
- * HYC_ENOTSUP otherwise. */
+ *                              efficient_hadamard.py:11-53); one code width (2, 4 or 8 bits) and group size for both
+ * Inputs are bf16 [M, H] with row pitches in elements; groups of 64 or 128 channels, H * bits / 64 <= 1024 (<= 512 for
+ * two operands of 2-bit codes); HYC_ENOTSUP otherwise. */
 int hyc_act_fwd_compress(int32_t act, const void* x, int64_t ldx, int64_t M, int64_t H, const hyc_desc* d, void* y,
                          void* stored, void* vals, void* scales, void* stream);
 int hyc_hadamard_fwd_compress(const void* x1, int64_t ld1, const void* x2, int64_t ld2, int64_t M, int64_t H,

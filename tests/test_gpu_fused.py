@@ -232,6 +232,9 @@ def test_gated_forward_activation_matches_the_framework_for_every_bf16_value(K, 
 @pytest.mark.parametrize("act,M,H,bits,group,k", [("silu", 333, 11008, 4, 128, 110), ("gelu", 64, 4096, 4, 128, 41),
                                                   ("silu", 2100, 4096, 4, 64, 41), ("silu", 40, 512, 8, 64, 5),
                                                   ("gelu", 130, 2048, 8, 128, 300),
+                                                  # 2-bit codes: four segments per thread (128 and 344 threads per row)
+                                                  ("silu", 300, 4096, 2, 128, 41), ("gelu", 77, 11008, 2, 64, 110),
+                                                  ("silu", 1030, 11008, 2, 64, 110),
                                                   # three rows of 704 threads per workgroup: the activation table is in use
                                                   ("silu", 2100, 11008, 4, 128, 110), ("gelu", 1600, 11008, 4, 128, 110)])
 def test_gated_forward_equals_the_separate_calls(K, act, M, H, bits, group, k):
@@ -252,8 +255,9 @@ def test_gated_forward_equals_the_separate_calls(K, act, M, H, bits, group, k):
     for got, ref in zip((c_a, c_u, c_g), want):
         assert torch.equal(got.stored.view(torch.uint8), ref.stored.view(torch.uint8))
         assert bits_equal(got.scales, ref.scales) and bits_equal(got.vals, ref.vals)
-    assert not K.gated_act_fwd_supported(4096, 2, 64) and K.gated_act_fwd_supported(11008, 4, 128)
+    assert K.gated_act_fwd_supported(4096, 2, 64) and K.gated_act_fwd_supported(11008, 4, 128)
     assert not K.gated_act_fwd_supported(14336, 4, 128)          # 896 chunks per segment: left to the separate calls
+    assert not K.gated_act_fwd_supported(20480, 2, 64) and not K.gated_act_fwd_supported(4096, 1, 64)
 
 
 @pytest.mark.parametrize("bits,group,M,H,k,wdt,with_bias", [
@@ -328,7 +332,7 @@ def test_activation_forward_with_the_save_fused_in(K, act, M, H, bits, group, k,
 
 
 @pytest.mark.parametrize("M,H,bits,group,k", [(333, 11008, 4, 128, 110), (2100, 4096, 4, 64, 41), (40, 512, 8, 64, 5),
-                                              (9, 2048, 8, 128, 300)])
+                                              (9, 2048, 8, 128, 300), (300, 4096, 2, 128, 41), (1030, 11008, 2, 64, 110)])
 def test_product_forward_with_the_saves_fused_in(K, M, H, bits, group, k):
     gen = torch.Generator().manual_seed(M + H + bits + 1)
     both = torch.randn(M, 2 * H, generator=gen)
@@ -342,7 +346,8 @@ def test_product_forward_with_the_saves_fused_in(K, M, H, bits, group, k):
         ref = K.compress_channel(t, p, bits, group)
         assert torch.equal(got.stored.view(torch.uint8), ref.stored.view(torch.uint8))
         assert bits_equal(got.scales, ref.scales) and bits_equal(got.vals, ref.vals)
-    assert not K.hadamard_fwd_compress_supported(4096, 2, 64, 2, 64) and not K.hadamard_fwd_compress_supported(4096, 4, 64, 8, 64)
+    assert K.hadamard_fwd_compress_supported(4096, 2, 64, 2, 64) and not K.hadamard_fwd_compress_supported(4096, 4, 64, 8, 64)
+    assert not K.hadamard_fwd_compress_supported(20480, 2, 64, 2, 64)
 
 
 def test_rows_beyond_two_gibi_elements(K):
