@@ -52,9 +52,9 @@ def test_gradw_channel(K, bits, group, M, H, N, k):
     xh = K.decompress_channel(c)
     want = dy.float().t() @ xh.cpu().float()
     got32 = K.gradw_gemm(dy.cuda(), c, out_dtype=torch.float32, staged=False).cpu()      # decoded inside the GEMM
-    assert torch.allclose(got32, want, rtol=1e-3, atol=1e-3 * float(want.abs().max()) + 1e-6)
+    assert torch.allclose(got32, want, rtol=1e-3, atol=1e-3)
     got16 = K.gradw_gemm(dy.cuda(), c, out_dtype=torch.bfloat16, staged=False).cpu()
-    assert torch.allclose(got16.float(), want, rtol=1e-2, atol=1e-3 * float(want.abs().max()) + 1e-3)
+    assert torch.allclose(got16.float(), want, rtol=1e-2, atol=1e-3)
     if H % 128 == 0:
         dense = K.gradw_gemm(dy.cuda(), xh, out_dtype=torch.float32).cpu()
         # (also where the few-row kernel folds the group scale of 1- and 2-bit codes into dY: that form is exact)
@@ -65,7 +65,7 @@ def test_gradw_channel(K, bits, group, M, H, N, k):
     # alpha / beta
     base = torch.ones(N, H, dtype=torch.float32, device="cuda")
     out = K.gradw_gemm(dy.cuda(), c, alpha=2.0, out=base, beta=0.5, staged=False).cpu()
-    assert torch.allclose(out, 2.0 * want + 0.5, rtol=1e-3, atol=2e-3 * float(want.abs().max()) + 1e-6)
+    assert torch.allclose(out, 2.0 * want + 0.5, rtol=1e-3, atol=1e-3)
 
 
 def test_gradw_config3_lora_a(K):
@@ -105,7 +105,7 @@ def test_gradw_full_size(K, name, M, N, H, bits, group, k, gain):
     scale = float(want.abs().max())
     for staged in (False, True):
         got = K.gradw_gemm(dy1, c, out_dtype=torch.float32, staged=staged)
-        assert torch.allclose(got, want, rtol=1e-2, atol=1e-3 * scale), (staged, float((got - want).abs().max()), scale)
+        assert torch.allclose(got, want, rtol=1e-2, atol=1e-3), (staged, float((got - want).abs().max()), scale)
     a = K.gradw_gemm(dy1, c, out_dtype=torch.float32, staged=False)
     b = K.gradw_gemm(dy2, c, out_dtype=torch.float32, staged=False)
     both = K.gradw_gemm((dy1.float() + dy2.float()).bfloat16(), c, out_dtype=torch.float32, staged=False)
@@ -392,7 +392,7 @@ def test_rmsnorm_gemma_module(ops, K, mode):
         dx_o, dw_o = O.rmsnorm_bwd(dy, xh, w1, rstd_o)
         assert torch.allclose(xd.grad.cpu().float(), dx_o.float(), rtol=1e-2, atol=1e-3)
         assert mod.weight.grad.dtype == torch.bfloat16
-        assert torch.allclose(mod.weight.grad.cpu().float(), dw_o.float(), rtol=1e-2, atol=2e-3)
+        assert torch.allclose(mod.weight.grad.cpu().float(), dw_o.float(), rtol=1e-2, atol=1e-3)
 
 
 @pytest.mark.parametrize("mode,bits,group", [("ref", 8, 128), ("hyc", 2, 64), ("hyc", 4, 128)])
@@ -413,11 +413,11 @@ def test_linear_module(ops, K, mode, bits, group):
         saved = y.grad_fn.saved
         y.backward(dy.cuda())
         w = lin.weight.detach().cpu()
-        assert torch.allclose(y.detach().cpu().float(), (x.float() @ w.float().t()), rtol=2e-2, atol=2e-2)
+        assert torch.allclose(y.detach().cpu().float(), (x.float() @ w.float().t()), rtol=1e-2, atol=1e-3)
         xh = (K.decompress_threshold(saved) if mode == "ref" else K.decompress_channel(saved)).cpu().reshape(B, S, H)
         dX, dW_lit, dW_f32, _ = O.linear_bwd(dy, xh, w)
-        assert torch.allclose(xd.grad.cpu().float(), dX.float(), rtol=2e-2, atol=2e-3)
-        assert torch.allclose(lin.weight.grad.cpu().float(), dW_f32, rtol=1e-2, atol=1e-3 + 4e-3 * float(dW_f32.abs().max()))
+        assert torch.allclose(xd.grad.cpu().float(), dX.float(), rtol=1e-2, atol=1e-3)
+        assert torch.allclose(lin.weight.grad.cpu().float(), dW_f32, rtol=1e-2, atol=1e-3)
 
 
 @pytest.mark.gpu
@@ -463,7 +463,7 @@ def test_gemm_module(ops, K, mode, bits):
         g = (0.05 * torch.randn(B, nh, S, S, generator=gen)).bfloat16()
         qd, ktd = q.cuda().requires_grad_(True), k.cuda().mT.contiguous().requires_grad_(True)
         y = mod(qd, ktd)
-        assert torch.allclose(y.detach().cpu().float(), q.float() @ k.float().mT, rtol=2e-2, atol=0.3)
+        assert torch.allclose(y.detach().cpu().float(), q.float() @ k.float().mT, rtol=1e-2, atol=1e-3)
         saved = y.grad_fn.saved
         y.backward(g.cuda())
         if mode == "ref":
@@ -482,8 +482,8 @@ def test_gemm_module(ops, K, mode, bits):
         qh, kh = O.hidden_to_head_shape(qh, nh), O.hidden_to_head_shape(kh, nh)
         assert (qh.float() - q.float()).abs().max() < (4.0 if bits == 2 else 2.0)     # sanity only: the right tensor came back
         d1, d2 = O.gemm_bwd(g, qh, kh.mT)
-        assert torch.allclose(qd.grad.cpu().float(), d1, rtol=1e-2, atol=1e-3 + 4e-3 * float(d1.abs().max()))
-        assert torch.allclose(ktd.grad.cpu().float(), d2, rtol=1e-2, atol=1e-3 + 4e-3 * float(d2.abs().max()))
+        assert torch.allclose(qd.grad.cpu().float(), d1, rtol=1e-2, atol=1e-3)
+        assert torch.allclose(ktd.grad.cpu().float(), d2, rtol=1e-2, atol=1e-3)
         assert mod.iteration == call + 1
 
 
@@ -499,7 +499,7 @@ def test_gemm_with_softmax_module(ops, K, mode):
         g = (0.05 * torch.randn(B, nh, S, hd, generator=gen)).bfloat16()
         pd, vd = p.cuda().requires_grad_(True), v.cuda().requires_grad_(True)
         y = mod(pd, vd)
-        assert torch.allclose(y.detach().cpu().float(), p.float() @ v.float(), rtol=2e-2, atol=2e-2)
+        assert torch.allclose(y.detach().cpu().float(), p.float() @ v.float(), rtol=1e-2, atol=1e-3)
         fn = y.grad_fn
         y.backward(g.cuda())
         thr = O.get_statistics_softmax(p, call, 0.1) if call < 2 else mod.static_value_1.cpu()
@@ -509,8 +509,8 @@ def test_gemm_with_softmax_module(ops, K, mode):
         vh = (K.decompress_threshold(c2) if mode == "ref" else K.decompress_channel(c2)).cpu().reshape(B, S, nh * hd)
         vh = O.hidden_to_head_shape(vh, nh)
         d1, d2 = O.gemm_bwd(g, ph, vh)
-        assert torch.allclose(pd.grad.cpu().float(), d1, rtol=1e-2, atol=1e-3 + 4e-3 * float(d1.abs().max()))
-        assert torch.allclose(vd.grad.cpu().float(), d2, rtol=1e-2, atol=1e-3 + 4e-3 * float(d2.abs().max()))
+        assert torch.allclose(pd.grad.cpu().float(), d1, rtol=1e-2, atol=1e-3)
+        assert torch.allclose(vd.grad.cpu().float(), d2, rtol=1e-2, atol=1e-3)
     assert mod.iteration == 3 and mod.static_value_1 is not None
 
 
@@ -760,7 +760,7 @@ def test_linear_with_frozen_weight_saves_nothing(ops, mode):
     y.backward(g)
     assert lin.weight.grad is None
     want = g.float() @ lin.weight.float()
-    assert torch.allclose(x.grad.float(), want, rtol=1e-2, atol=1e-2)
+    assert torch.allclose(x.grad.float(), want, rtol=1e-2, atol=1e-3)
     with torch.no_grad():
         assert lin(x).shape == (2, 32, 64)
 
@@ -817,6 +817,9 @@ def test_flash_attention_module(ops, K, mode, lens, causal):
             restored = [K.decompress_threshold(c).cpu() for c in saved]
         out.backward(dout.cuda())
         out_o, dqkv_o = _attention_oracle(qkv, bounds, restored, causal, dout)
+        # the forward value comes from the framework's own fused attention kernel (not part of this library), which
+        # holds the probabilities in bf16: against the fp32 oracle its output carries their rounding, 2^-8 of values
+        # of order one.  The library's own outputs (the gradients below) are held to rtol 1e-2 / atol 1e-3.
         assert torch.allclose(out.detach().cpu().float(), out_o, rtol=2e-2, atol=2e-2)
         err = float((xg.grad.cpu().float() - dqkv_o).norm() / dqkv_o.norm())
         assert err < 1e-2, (call, err)
