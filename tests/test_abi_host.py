@@ -132,7 +132,8 @@ def test_argument_errors_without_a_gpu(abi):
     assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 4096, null, 4096, 4, 4096, D, D, ctypes.byref(t), null, *nine, null) == abi.ENOTSUP
     assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 4096, null, 4096, 4, 4096, D, ctypes.byref(d2), D, null, *nine, null) == abi.ENOTSUP
     d2b = ctypes.byref(d2)
-    assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 4096, null, 4096, 4, 4096, d2b, d2b, d2b, null, *nine, null) == abi.ENOTSUP  # 2-bit codes
+    assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 4096, null, 4096, 4, 4096, d2b, d2b, d2b, null, *nine, null) == abi.EFAULT   # 2-bit codes: covered
+    assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 20480, null, 20480, 4, 20480, d2b, d2b, d2b, null, *nine, null) == abi.ENOTSUP  # ... to 512 chunks
     assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 14336, null, 14336, 4, 14336, D, D, D, null, *nine, null) == abi.ENOTSUP    # 896 chunks
     assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 4000, null, 4096, 4, 4096, D, D, D, null, *nine, null) == abi.EINVAL   # pitch < H
     assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 8192, null, 4100, 4, 4096, D, D, D, null, *nine, null) == abi.EINVAL   # pitch % 8
@@ -148,7 +149,8 @@ def test_argument_errors_without_a_gpu(abi):
     assert lib.hyc_act_fwd_compress(abi.ACT_GELU_TANH, null, 4096, 0, 4096, D, null, null, null, null, null) == 0
     assert lib.hyc_hadamard_fwd_compress(null, 4096, null, 4096, 4, 4096, D, None, null, *six, null) == abi.EFAULT
     assert lib.hyc_hadamard_fwd_compress(null, 4096, null, 4096, 4, 4096, D, ctypes.byref(d2), null, *six, null) == abi.ENOTSUP
-    assert lib.hyc_hadamard_fwd_compress(null, 4096, null, 4096, 4, 4096, d2b, d2b, null, *six, null) == abi.ENOTSUP   # two 2-bit operands
+    assert lib.hyc_hadamard_fwd_compress(null, 4096, null, 4096, 4, 4096, d2b, d2b, null, *six, null) == abi.EFAULT    # two 2-bit operands: covered
+    assert lib.hyc_hadamard_fwd_compress(null, 20480, null, 20480, 4, 20480, d2b, d2b, null, *six, null) == abi.ENOTSUP  # ... to 512 chunks
     assert lib.hyc_hadamard_fwd_compress(null, 4096, null, 4100, 4, 4096, D, D, null, *six, null) == abi.EINVAL
     assert lib.hyc_hadamard_fwd_compress(null, 4096, null, 4096, 4, 4096, D, D, null, *six, null) == abi.EFAULT
     assert lib.hyc_layernorm_fwd_compress(null, null, null, 0, 1e-5, 4, 4096, None, null, null, null, null, null, null, null, null) == abi.EFAULT
