@@ -1069,6 +1069,40 @@ k_gradw_big(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_o
       b_at[u] = row * BP + 8 * cc;
     }
   }
+  // Chunks with more than two outlier channels are rare, but one of them must not slow the launch down: the third
+  // and fourth outlier value of ONE such chunk per thread are requested like everything else (in the stage before
+  // they are needed; their cache line arrived with the first two) and written over the decoded chunk in LDS.  What
+  // that does not cover (a fifth value, a second such chunk in a thread, 8-bit codes, whose register budget is
+  // spent) takes patch_more() below; both conditions are wave-uniform.
+  constexpr bool FASTX = SRC == 0 && BITS != 8;
+  constexpr int UROW = (THREADS / CPR) * BP;               // elements between a thread's chunks u and u + 1 in an LDS buffer
+  bool hasx = false, has4 = false, slow = false;
+  int xat2 = 0, xat3 = 0;                                  // LDS element offsets (chunk u = 0) of the two values
+  uint32_t vx2 = NOWHERE, vx3 = NOWHERE;                   // their byte offsets in vals, token row 0 of the stage
+  if (SRC == 0) {
+#pragma unroll
+    for (int i = 0; i < NST; ++i) {
+      const int n = __popc(co.m8[i]);
+      if (n > 2) {
+        if (FASTX && !hasx) {
+          hasx = true;
+          uint32_t m = co.m8[i];
+          m &= m - 1; m &= m - 1;
+          xat2 = b_at[i] + (__ffs(m) - 1);
+          vx2 = (uint32_t)((item0 / CPR) * kk2) + co.vb[i] + 4u;
+          m &= m - 1;
+          has4 = m != 0;
+          if (has4) { xat3 = b_at[i] + (__ffs(m) - 1); vx3 = vx2 + 2u; }
+          slow = slow || n > 4;
+        } else {
+          slow = true;
+        }
+      }
+    }
+  }
+  const bool slow_any = __ballot(slow) != 0;
+  const BufferRsrc rs_x = make_rsrc(SRC == 0 && ca.k ? vals + m_begin * (int64_t)ca.k : nullptr,
+                                    __builtin_amdgcn_readfirstlane((uint32_t)(m_end - m_begin) * kk2));
   // the resources of the next stage to request
   const char* pa = reinterpret_cast<const char*>(dy + m_begin * ldy);
   const char* pb = reinterpret_cast<const char*>(stored) + m_begin * (int64_t)b_pitch;
@@ -1180,6 +1214,7 @@ k_gradw_big(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_o
     constexpr float OFFV = (BITS == 8) ? 128.f : (float)Q<BITS>::OFF;
     uint32_t cw[NCH][2], res[NCH][4];
     float sc[NCH], ns[NCH];
+    uint32_t xv2[B_PER], xv3[B_PER];
     auto slot = [&](auto tno) __attribute__((always_inline)) {
       constexpr int t = decltype(tno)::value;
       __builtin_amdgcn_sched_barrier(0);
@@ -1188,6 +1223,14 @@ k_gradw_big(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_o
         acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(t < 16 ? fa0[a] : fa1[a], t < 16 ? fb0[b] : fb1[b], acc[a][b], 0, 0, 0);
       }
       if constexpr (t < 8) read_frag(HYC_AS(B), HYC_BS(B), 16, t, fa1, fb1);
+      if constexpr (FASTX && (t == 1 || t == 2)) {                      // (unconditional: lanes without such a chunk ask for nothing)
+        const uint32_t xoff = (uint32_t)(m1 - m_begin) * kk2;
+#pragma unroll
+        for (int u = 0; u < B_PER; ++u) {
+          if (t == 1) xv2[u] = load_b16(rs_x, vx2 + xoff + (uint32_t)(u * (THREADS / CPR)) * kk2);
+          else xv3[u] = load_b16(rs_x, vx3 + xoff + (uint32_t)(u * (THREADS / CPR)) * kk2);
+        }
+      }
       if constexpr (SRC == 0 && t < 16) {                               // two elements of chunk c of stage s+1
         constexpr int c = t >> 2, w = t & 3, u = c / NST, i = c % NST;
         if constexpr (w == 0) {
@@ -1219,7 +1262,16 @@ k_gradw_big(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_o
         else
           *reinterpret_cast<uint4*>(&HYC_BS(NB)[b_at[c]]) = Rd.b[c];
         if constexpr (t == 23 && SRC == 0) {
-          if (co.more_pairs) patch_more(HYC_BS(NB), m1);
+          if (co.more_pairs) {
+            if (FASTX && hasx) {
+#pragma unroll
+              for (int u = 0; u < B_PER; ++u) {
+                HYC_BS(NB)[xat2 + u * UROW] = (uint16_t)xv2[u];
+                if (has4) HYC_BS(NB)[xat3 + u * UROW] = (uint16_t)xv3[u];
+              }
+            }
+            if (!FASTX || slow_any) patch_more(HYC_BS(NB), m1);
+          }
         }
       }
       if constexpr (t == 24) __syncthreads();                           // buffer NB is complete, buffer B read for the last time

@@ -68,6 +68,28 @@ def test_gradw_channel(K, bits, group, M, H, N, k):
     assert torch.allclose(out, 2.0 * want + 0.5, rtol=1e-3, atol=1e-3)
 
 
+@pytest.mark.parametrize("bits,group", [(4, 128), (2, 64), (1, 64), (8, 128)])
+@pytest.mark.parametrize("hot", [[8, 9, 10], [40, 41, 42, 43, 300], [16, 17, 18, 600, 601, 602, 603], [64, 65, 66, 67, 68, 900],
+                                 [0, 1, 2, 3, 4, 5, 6, 7, 512, 513, 514]])
+def test_gradw_crowded_chunks(K, bits, group, hot):
+    """chunks of eight channels with three, four and more outlier channels (and two such chunks in one thread's
+    reach) in the 256-feature kernel: the product with the codes decoded inside equals the product with the restored
+    activation"""
+    M, H, N = 300, 1024, 256
+    gen = torch.Generator().manual_seed(len(hot) + bits)
+    x = torch.randn(M, H, generator=gen)
+    x[:, hot] *= 25.0
+    x = x.bfloat16().cuda()
+    dy = (0.05 * torch.randn(M, N, generator=gen)).bfloat16().cuda()
+    plan = K.select_channels(K.channel_absmax(x), len(hot))
+    assert plan.idx.cpu().tolist() == sorted(hot)
+    c = K.compress_channel(x, plan, bits, group)
+    xh = K.decompress_channel(c)
+    dense = K.gradw_gemm(dy, xh, out_dtype=torch.float32)
+    fused = K.gradw_gemm(dy, c, out_dtype=torch.float32, staged=False)
+    assert torch.allclose(fused, dense, rtol=1e-5, atol=1e-5 * float(dense.abs().max()))
+
+
 def test_gradw_config3_lora_a(K):
     """BASELINE config 3: X [4,1024,4096] as 1 % bf16 outliers + INT2 group 64; grad_A = (s * dY @ B)^T @ x_hat, r = 16"""
     M, H, r = 4096, 4096, 16
