@@ -15,9 +15,11 @@ Each function cites the reference lines it follows.  Two families:
   rest is quantised with a scale per (token, group of G channels).  The reference
   holds no implementation of the channel selection rule; the functions below are
   composed from the reference's primitives (zero-out, divide, round, clamp,
-  offset, half-split packing).  PARITY UNPINNED BY THE REFERENCE for the selection
-  rule and for the group-scale granularity; pinned for quantise / pack / unpack /
-  dequantise, which are shared with the ``ref_*`` family.
+  offset, half-split packing).  Quantise / pack / unpack / dequantise are shared
+  with the ``ref_*`` family and pinned with it; the group scales (both rules, see
+  hyc_group_scales) are pinned by an integer model, invariants and the special case
+  that reduces to the reference's per-token scheme (below).  The selection rule has
+  no counterpart in the reference to pin against.
 
 Pinning status (see tests/test_oracle_*.py):
 * pack / unpack                - brute force over all byte values, pure Python loops
@@ -34,7 +36,14 @@ Pinning status (see tests/test_oracle_*.py):
 * rope_fwd / rope_bwd          - complex-number form of the rotation; float64 torch.autograd
 * philox4x32_10 / dropout_*    - Random123 known-answer vectors for the generator; keep fraction; the mask
                                  mapping itself restates triton 3.6.0's tl.rand: parity unpinned by reference outputs
-* hyc_select_channels / hyc group scales - parity unpinned (no reference code)
+* hyc group scales (hyc_group_scales, rules "range" and "absmax")
+                               - integer model of bf16(bf16(a) / levels) in exact rationals with round-half-even
+                                 on tiny inputs; range rule: a group's min and max land 2^b - 1 codes apart (+-1);
+                                 absmax rule: the extreme element takes the extreme code and every element is
+                                 within half a step; group = H, k = 0 with the range rule = ref_compress with the
+                                 golden-pinned per-token scale, byte for byte
+* hyc_select_channels          - brute force on small inputs, ties, idempotence; no reference code exists for the
+                                 channel rule, so there are no reference outputs to pin it to
 * nf4_quantize / nf4_dequantize - parity unpinned (bitsandbytes is not in the reference tree); checked against
                                  the published level table: nearest level by exact distance, round trips
 """
