@@ -229,6 +229,21 @@ def gradw_extra(pkg, torch, c, shapes=(("full_w", 4096, 100, 30), ("lora_a_r16",
     return out
 
 
+def hbm_yardstick(torch):
+    """what the framework's own streaming kernels reach on this GPU in this run, on tensors that do not fit the
+    Infinity Cache (512 MiB each): a device copy (1 read + 1 write per byte) and c = a + b (2 reads + 1 write)"""
+    n = 256 << 20                                               # bf16 elements: 512 MiB per tensor
+    a = torch.empty(n, dtype=torch.bfloat16, device="cuda").normal_()
+    b = torch.empty_like(a).normal_()
+    c = torch.empty_like(a)
+    t_copy = time_events(torch, lambda: c.copy_(a), 20, 3)
+    t_add = time_events(torch, lambda: torch.add(a, b, out=c), 20, 3)
+    out = {"tensor_bytes": 2 * n, "copy": hbm(4 * n, t_copy), "add": hbm(6 * n, t_add)}
+    del a, b, c
+    torch.cuda.empty_cache()
+    return out
+
+
 def config1_extra(pkg, torch):
     """BASELINE configs[0] on the GPU: standalone compress + decompress of x [4,512,4096] (41 outlier channels x50,
     INT4, group 128), and the same at 16x the tokens"""
@@ -496,6 +511,7 @@ def main():
         del x3, c3
         extra["config4_mlp_h11008"] = config4_extra(pkg, torch)
     if not args.no_scaled:
+        extra["hbm_yardstick"] = hbm_yardstick(torch)
         # the config-size working set (~150 MB) fits the 256 MB Infinity Cache; 16x the tokens does not
         Ms = 16 * M
         wls = Workload(pkg, torch, Ms, H, bits, group, n_hot=20, gain=30.0, seed=1)
