@@ -873,15 +873,9 @@ static inline int norm_geom(int cps, NormGeom* n) {
   return HYC_OK;
 }
 
-#ifndef BWD_FAST_SLOTS_MAX
-#define BWD_FAST_SLOTS_MAX 4
-#endif
-#ifndef HYC_BWD_BIG
-#define HYC_BWD_BIG 1024
-#endif
-#ifndef BWD_SLOTS_SMALL
-#define BWD_SLOTS_SMALL 1
-#endif
+constexpr int BWD_FAST_SLOTS_MAX = 4;      // row slots per workgroup of the fast backward kernel, at most
+constexpr int BWD_FAST_THREADS_MAX = 1024; // ... and its thread bound (the static LDS queue is sized by it)
+constexpr int BWD_SLOTS_SMALL = 1;         // row slots per workgroup of the generic backward kernel on narrow rows
 // backward launch shape: slots per workgroup and rows per workgroup
 struct BwdShape {
   int slots, threads, rpb;
@@ -901,8 +895,8 @@ static inline BwdShape bwd_shape(int64_t M, int bits, int cps, const NormGeom& n
     // weight row (dynamic); 160 KB per workgroup on gfx950
     int fs0 = 1024 / b.fast_T;
     if (fs0 > BWD_FAST_SLOTS_MAX) fs0 = BWD_FAST_SLOTS_MAX;
-    const int64_t maxt = fs0 * b.fast_T <= 256 ? 256 : HYC_BWD_BIG, nseg = bits == 8 ? 1 : 2;
-    if (fs0 * b.fast_T > HYC_BWD_BIG) b.fast_ok = false;
+    const int64_t maxt = fs0 * b.fast_T <= 256 ? 256 : BWD_FAST_THREADS_MAX, nseg = bits == 8 ? 1 : 2;
+    if (fs0 * b.fast_T > BWD_FAST_THREADS_MAX) b.fast_ok = false;
     const int64_t H = (int64_t)cps * 64 / bits;
     const int64_t lds = RING_D * maxt * nseg * 16 + 1024 + H * 4;
     b.fast_ok = b.fast_ok && lds <= 160 * 1024;
@@ -1126,13 +1120,13 @@ static int norm_bwd_impl(const void* dy, const void* stored, const void* vals, c
     const int key_ = (wf32 ? 4 : 0) + (c2_quirk ? 2 : 0) + (fthreads <= 256 ? 0 : 1);        \
     switch (key_) {                                                                           \
       case 0: HYC_BWD_FAST(B_, false, false, 256); break;                                     \
-      case 1: HYC_BWD_FAST(B_, false, false, HYC_BWD_BIG); break;                                    \
+      case 1: HYC_BWD_FAST(B_, false, false, BWD_FAST_THREADS_MAX); break;                                    \
       case 2: HYC_BWD_FAST(B_, false, true, 256); break;                                      \
-      case 3: HYC_BWD_FAST(B_, false, true, HYC_BWD_BIG); break;                                     \
+      case 3: HYC_BWD_FAST(B_, false, true, BWD_FAST_THREADS_MAX); break;                                     \
       case 4: HYC_BWD_FAST(B_, true, false, 256); break;                                      \
-      case 5: HYC_BWD_FAST(B_, true, false, HYC_BWD_BIG); break;                                     \
+      case 5: HYC_BWD_FAST(B_, true, false, BWD_FAST_THREADS_MAX); break;                                     \
       case 6: HYC_BWD_FAST(B_, true, true, 256); break;                                       \
-      default: HYC_BWD_FAST(B_, true, true, HYC_BWD_BIG); break;                                     \
+      default: HYC_BWD_FAST(B_, true, true, BWD_FAST_THREADS_MAX); break;                                     \
     }                                                                                         \
   } while (0)
       if (dense_fast) {
@@ -1143,13 +1137,13 @@ static int norm_bwd_impl(const void* dy, const void* stored, const void* vals, c
                      static_cast<uint16_t*>(dx), dw_partials)
         switch ((wf32 ? 4 : 0) + (c2_quirk ? 2 : 0) + (fthreads <= 256 ? 0 : 1)) {
           case 0: HYC_BWD_DENSE(false, false, 256); break;
-          case 1: HYC_BWD_DENSE(false, false, HYC_BWD_BIG); break;
+          case 1: HYC_BWD_DENSE(false, false, BWD_FAST_THREADS_MAX); break;
           case 2: HYC_BWD_DENSE(false, true, 256); break;
-          case 3: HYC_BWD_DENSE(false, true, HYC_BWD_BIG); break;
+          case 3: HYC_BWD_DENSE(false, true, BWD_FAST_THREADS_MAX); break;
           case 4: HYC_BWD_DENSE(true, false, 256); break;
-          case 5: HYC_BWD_DENSE(true, false, HYC_BWD_BIG); break;
+          case 5: HYC_BWD_DENSE(true, false, BWD_FAST_THREADS_MAX); break;
           case 6: HYC_BWD_DENSE(true, true, 256); break;
-          default: HYC_BWD_DENSE(true, true, HYC_BWD_BIG); break;
+          default: HYC_BWD_DENSE(true, true, BWD_FAST_THREADS_MAX); break;
         }
 #undef HYC_BWD_DENSE
       }
