@@ -645,9 +645,8 @@ static int direct_splits_max(int64_t M, int64_t N_out, int64_t H) {
 // Large output (N_out > 32), first form: workgroup tile 128 (n) x 256 (h), four waves of 64 x 128, two LDS stages.
 // While the MFMAs of stage s run, the global loads of stage s+1 are in flight; they are written into the other LDS
 // buffer after the MFMAs have been issued, and one barrier per stage separates the two.  128 accumulator registers
-// per lane and two waves per SIMD.  It is launched for a dense activation whose tile grid is too small for the
-// 256-feature form below (the template still carries the eight-wave and channel-scheme variants it was written with;
-// k_gradw_big has taken their place).
+// per lane and two waves per SIMD.  For a dense activation whose tile grid is too small for the 256-feature form
+// below.
 // ------------------------------------------------------------------------------------------------
 constexpr int WK = 32;      // tokens per stage
 constexpr int WN = 128;     // dY features per workgroup of this form (the second form takes 2 * WN)
@@ -662,25 +661,21 @@ struct WideRegs {            // one stage of global data per thread
   uint32_t o0[B_PER][NSEG], o1[B_PER][NSEG];   // ... and the first two outlier values of the chunk
 };
 
-template <int BITS, int SRC, int WNT>
-__global__ void __launch_bounds__(2 * WNT) __attribute__((amdgpu_waves_per_eu(2)))
+// dense activation only (x = bf16 [M, H]); grid: x = n-tile, y = h-tile, z = token split
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
 k_gradw_wide(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_out, int64_t H,
-             const uint8_t* __restrict__ stored, const uint16_t* __restrict__ vals, const uint16_t* __restrict__ scales,
-             ChanArgs ca, int CPS, int64_t tokens_per_split, float alpha, float beta,
+             const uint16_t* __restrict__ x, int64_t tokens_per_split, float alpha, float beta,
              void* __restrict__ out, int out_f32, float* __restrict__ partial) {
-  constexpr int NSEG = (SRC == 0) ? Q<BITS>::NSEG : 1;
-  constexpr int HS = WH / NSEG;               // columns of the tile that come from one segment
-  constexpr int CPR = HS / 8;                 // packed 8-byte chunks (channel scheme) / 16-byte chunks (dense) per token row and segment
-  constexpr int THREADS = 2 * WNT;            // waves: WNT/64 along n x 2 along h, 64 x 128 each
-  constexpr int AP = WNT + WPAD, BP = WH + WPAD;
+  constexpr int CPR = WH / 8;                 // 16-byte chunks per token row of the x tile
+  constexpr int THREADS = 2 * WN;             // four waves: 2 along n x 2 along h, 64 x 128 each
+  constexpr int AP = WN + WPAD, BP = WH + WPAD;
   __shared__ __align__(16) uint16_t As[2][WK * AP];
   __shared__ __align__(16) uint16_t Bs[2][WK * BP];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int64_t n0 = (int64_t)blockIdx.x * WNT;
-  const int64_t SEG = (SRC == 0) ? (int64_t)CPS * 8 : H;
-  const int64_t j0 = (int64_t)blockIdx.y * HS;          // first column of the tile inside each segment
+  const int64_t n0 = (int64_t)blockIdx.x * WN;
+  const int64_t j0 = (int64_t)blockIdx.y * WH;
   const int64_t m_begin = (int64_t)blockIdx.z * tokens_per_split;
   const int64_t m_end = m_begin + tokens_per_split < M ? m_begin + tokens_per_split : M;
   const int wn = (wave >> 1) * 64, wh = (wave & 1) * 128;
@@ -693,114 +688,45 @@ k_gradw_wide(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
 
-  constexpr int A_PER = WK * WNT / 8 / THREADS;           // 16-byte chunks of the dY stage per thread (2)
-  constexpr int B_ITEMS = WK * CPR;
-  constexpr int B_PER = (B_ITEMS + THREADS - 1) / THREADS;
-  static_assert(B_ITEMS % THREADS == 0 || B_ITEMS < THREADS, "items per stage");
-  // Narrow codes give fewer packed words per stage than threads: PARTS threads then share a word, NST segments each.
-  constexpr int PARTS = (SRC == 0 && B_ITEMS < THREADS) ? THREADS / B_ITEMS : 1;
-  constexpr int NST = NSEG / PARTS;                       // segments a thread decodes
-  static_assert(NSEG % PARTS == 0 && (PARTS == 1 || PARTS * B_ITEMS == THREADS), "threads per packed word");
-  const int seg0 = (PARTS > 1 ? tid / B_ITEMS : 0) * NST; // first of them
-  const int item0 = PARTS > 1 ? tid % B_ITEMS : tid;      // the thread's first item
-  constexpr bool b_thread = true;
-  typedef WideRegs<NST, A_PER, B_PER> Regs;
-  // A thread decodes the same chunk column of every row it touches (THREADS is a multiple of CPR), so its outlier
-  // work is static: selectors that splice up to two outlier values into a decoded chunk, as in the row kernels.
-  ChunkOutliers<NST> co;
-  {
-    uint32_t pw[NST];
-#pragma unroll
-    for (int i = 0; i < NST; ++i)
-      pw[i] = (SRC == 0) ? ca.plan[(seg0 + i) * CPS + (int)(j0 / 8) + item0 % CPR] : 0u;
-    co.init(pw);
-  }
-
+  constexpr int A_PER = WK * WN / 8 / THREADS;            // 16-byte chunks of the dY stage per thread (2)
+  constexpr int B_PER = WK * CPR / THREADS;               // ... and of the x stage (4)
+  typedef WideRegs<1, A_PER, B_PER> Regs;
   // Every operand of the token loop is read through a buffer resource that spans exactly this workgroup's token
-  // range: the hardware drops what lies beyond it (rows past m_end, features past N_out, outlier slots a chunk
-  // does not have) and returns zeros, so nothing is clamped, predicated or branched on, and the address of a load
-  // is a per-thread constant.
-  const uint32_t gpr = (uint32_t)ca.groups_per_row, kk2 = 2u * (uint32_t)ca.k;
-  const uint32_t b_pitch = (SRC == 0) ? (uint32_t)SEG : 2u * (uint32_t)H;          // bytes per token of the x operand
-  uint32_t va[A_PER], vb[B_PER], vs[B_PER][NST], vo0[B_PER][NST], vo1[B_PER][NST];
+  // range: the hardware drops what lies beyond it (rows past m_end, features past N_out) and returns zeros, so
+  // nothing is clamped, predicated or branched on, and the address of a load is a per-thread constant.
+  const uint32_t b_pitch = 2u * (uint32_t)H;
+  uint32_t va[A_PER], vb[B_PER];
 #pragma unroll
   for (int u = 0; u < A_PER; ++u) {
     const int idx = tid + u * THREADS;
-    const int row = idx / (WNT / 8), cc = idx % (WNT / 8);
+    const int row = idx / (WN / 8), cc = idx % (WN / 8);
     va[u] = n0 + 8 * cc < N_out ? 2u * ((uint32_t)row * (uint32_t)ldy + (uint32_t)n0 + 8u * cc) : NOWHERE;
   }
 #pragma unroll
   for (int u = 0; u < B_PER; ++u) {
-    const int idx = item0 + u * THREADS;
-    const int row = idx / CPR, cc = idx % CPR;
-    if (SRC == 0) {
-      const int c = (int)(j0 / 8) + cc;
-      vb[u] = (uint32_t)row * b_pitch + 8u * c;
-#pragma unroll
-      for (int i = 0; i < NST; ++i) {
-        vs[u][i] = 2u * ((uint32_t)row * gpr + (uint32_t)(((seg0 + i) * CPS + c) >> ca.chunk_to_group_shift));
-        vo0[u][i] = co.has0[i] ? (uint32_t)row * kk2 + co.vb[i] : NOWHERE;
-        vo1[u][i] = co.has1[i] ? (uint32_t)row * kk2 + co.vb[i] + 2u : NOWHERE;
-      }
-    } else {
-      vb[u] = (uint32_t)row * b_pitch + 2u * ((uint32_t)j0 + 8u * cc);
-    }
+    const int idx = tid + u * THREADS;
+    vb[u] = (uint32_t)(idx / CPR) * b_pitch + 2u * ((uint32_t)j0 + 8u * (idx % CPR));
   }
   auto fetch = [&](Regs& R, int64_t m0) __attribute__((always_inline)) {
     // the resources of a stage start at its first token (scalar arithmetic), so the per-thread offsets never change
     const uint32_t left = (uint32_t)(m_end - m0);
     const BufferRsrc rs_a = make_rsrc(dy + m0 * ldy, left * 2u * (uint32_t)ldy);
-    const BufferRsrc rs_b = make_rsrc(stored + m0 * (int64_t)b_pitch, left * b_pitch);
+    const BufferRsrc rs_b = make_rsrc(x + m0 * H, left * b_pitch);
 #pragma unroll
     for (int u = 0; u < A_PER; ++u) R.a[u] = load_b128(rs_a, va[u]);
-    if (SRC == 0) {
-      const BufferRsrc rs_s = make_rsrc(scales + m0 * (int64_t)gpr, left * 2u * gpr);
-      const BufferRsrc rs_o = make_rsrc(ca.k ? vals + m0 * (int64_t)ca.k : nullptr, left * kk2);
 #pragma unroll
-      for (int u = 0; u < B_PER; ++u) {
-        const uint2 pk = load_b64(rs_b, vb[u]);
-        R.b[u] = make_uint4(pk.x, pk.y, 0, 0);
-#pragma unroll
-        for (int i = 0; i < NST; ++i) {
-          R.s[u][i] = load_b16(rs_s, vs[u][i]);
-          R.o0[u][i] = load_b16(rs_o, vo0[u][i]);
-          R.o1[u][i] = load_b16(rs_o, vo1[u][i]);
-        }
-      }
-    } else {
-#pragma unroll
-      for (int u = 0; u < B_PER; ++u) R.b[u] = load_b128(rs_b, vb[u]);
-    }
+    for (int u = 0; u < B_PER; ++u) R.b[u] = load_b128(rs_b, vb[u]);
   };
-  // (chunks with more than two outlier channels: the remaining pairs, rare, loaded in place)
-  auto finish_chunk = [&](uint4 r, int i, int cc, int64_t m) __attribute__((always_inline)) {
-    if (co.more_pairs)
-      r = splice_more(r, co.more_pairs, ca.plan[(seg0 + i) * CPS + (int)(j0 / 8) + cc], vals + (m < m_end ? m : m_end - 1) * ca.k, true, 1.f);
-    return r;
-  };
-  // decode one stage of registers (tokens mb ..) into LDS buffer `buf`
-  auto stash = [&](int buf, const Regs& R, int64_t mb) __attribute__((always_inline)) {
+  auto stash = [&](int buf, const Regs& R) __attribute__((always_inline)) {
 #pragma unroll
     for (int u = 0; u < A_PER; ++u) {
       const int idx = tid + u * THREADS;
-      const int row = idx / (WNT / 8), cc = idx % (WNT / 8);
-      *reinterpret_cast<uint4*>(&As[buf][row * AP + 8 * cc]) = R.a[u];
+      *reinterpret_cast<uint4*>(&As[buf][(idx / (WN / 8)) * AP + 8 * (idx % (WN / 8))]) = R.a[u];
     }
-    if (b_thread) {
 #pragma unroll
-      for (int u = 0; u < B_PER; ++u) {
-        const int idx = item0 + u * THREADS;
-        const int row = idx / CPR, cc = idx % CPR;
-        if (SRC == 0) {
-#pragma unroll
-          for (int i = 0; i < NST; ++i)
-            *reinterpret_cast<uint4*>(&Bs[buf][row * BP + (seg0 + i) * HS + 8 * cc]) = finish_chunk(
-                co.splice_value(i, dequant8_fast<BITS>(R.b[u].x, R.b[u].y, seg0 + i, bf_to_f((uint16_t)R.s[u][i])), R.o0[u][i],
-                                R.o1[u][i]), i, cc, mb + row);
-        } else {
-          *reinterpret_cast<uint4*>(&Bs[buf][row * BP + 8 * cc]) = R.b[u];
-        }
-      }
+    for (int u = 0; u < B_PER; ++u) {
+      const int idx = tid + u * THREADS;
+      *reinterpret_cast<uint4*>(&Bs[buf][(idx / CPR) * BP + 8 * (idx % CPR)]) = R.b[u];
     }
   };
   // The 16 MFMAs of a stage run as 8 pairs (k sub-step t/4, column tile t%4; both row tiles of the wave).  Operand
@@ -827,106 +753,23 @@ k_gradw_wide(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_
     }
   };
 
-  // Three stages in flight: stage s in LDS under the MFMAs, stage s+1 in registers being decoded into the other
-  // LDS buffer in the shadow of those MFMAs, stage s+2 on its way from memory.  One barrier per stage.
+  // Three stages in flight: stage s in LDS under the MFMAs, stage s+1 in registers on its way into the other LDS
+  // buffer, stage s+2 on its way from memory.  One barrier per stage.
   if (m_begin < m_end) {
     Regs R0, R1;
     int64_t m0 = m_begin;
     fetch(R0, m0);
-    stash(0, R0, m0);
+    stash(0, R0);
     if (m0 + WK < m_end) fetch(R0, m0 + WK);
-    // steady state: the next three stages exist, so nothing is conditional and the decode of stage s+1 shares a
-    // basic block with the MFMAs of stage s (the scheduling groups below interleave them)
-    // One MFMA takes 8 passes; the wave issues in order, so the decode is cut into 16 pieces (two elements each:
-    // convert, scale, round, pack) and one piece follows each of the stage's 16 MFMAs.
-    auto overlap = [&](int buf, const Regs& R, int64_t mb) __attribute__((always_inline)) {
-      constexpr int NP = B_PER * NST * 4;                               // two-element pieces of a thread's decode
-      constexpr bool PIECES = SRC == 0 && (NP == 16 || NP == 8);        // 2-, 4- and 8-bit codes
-      constexpr int EVERY = PIECES ? 16 / NP : 1;                       // MFMAs per piece
-      if (!PIECES) {
-        stash(buf ^ 1, R, mb);
-        mfma_stage(buf);
-      } else {
-        constexpr uint32_t REP = (BITS == 8) ? 0x80808080u : Q<BITS>::CODE_MASK * 0x01010101u;
-        constexpr float OFFV = (BITS == 8) ? 128.f : (float)Q<BITS>::OFF;
-        uint32_t cw[B_PER][NST][2], res[B_PER][NST][4];
-        float sc[B_PER][NST], ns[B_PER][NST];
-#pragma unroll
-        for (int u = 0; u < B_PER; ++u)
-#pragma unroll
-          for (int i = 0; i < NST; ++i) {
-            cw[u][i][0] = (BITS == 8) ? R.b[u].x ^ REP : (R.b[u].x >> ((seg0 + i) * BITS)) & REP;
-            cw[u][i][1] = (BITS == 8) ? R.b[u].y ^ REP : (R.b[u].y >> ((seg0 + i) * BITS)) & REP;
-            sc[u][i] = bf_to_f((uint16_t)R.s[u][i]);
-            ns[u][i] = -OFFV * sc[u][i];
-          }
-        // the pair schedule of mfma_stage, with one decode piece after every (EVERY-th) MFMA
-        int piece = 0;
-        bf16x8_t af[2][2], bq[4];
-        af[0][0] = frag32(As[buf], AP, wn, 0);
-        af[0][1] = frag32(As[buf], AP, wn + 32, 0);
-        bq[0] = frag32(Bs[buf], BP, wh, 0);
-        bq[1] = frag32(Bs[buf], BP, wh + 32, 0);
-#pragma unroll
-        for (int t = 0; t < 8; ++t) {
-          const int k = t >> 2, b = t & 3;
-          __builtin_amdgcn_sched_barrier(0);
-          if (t + 2 < 8) bq[(t + 2) & 3] = frag32(Bs[buf], BP, wh + 32 * ((t + 2) & 3), 16 * ((t + 2) >> 2));
-          if (t == 1) {
-            af[1][0] = frag32(As[buf], AP, wn, 16);
-            af[1][1] = frag32(As[buf], AP, wn + 32, 16);
-          }
-#pragma unroll
-          for (int a = 0; a < 2; ++a) {
-            __builtin_amdgcn_sched_barrier(0);
-            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[k][a], bq[t & 3], acc[a][b], 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
-            if ((2 * t + a) % EVERY == 0) {
-              const int u = piece / (4 * NST), i = (piece / 4) % NST, w = piece % 4;
-              const uint32_t src = cw[u][i][w >> 1] >> (16 * (w & 1));
-              const float f0 = __builtin_fmaf((float)(src & 0xFFu), sc[u][i], ns[u][i]);
-              const float f1 = __builtin_fmaf((float)((src >> 8) & 0xFFu), sc[u][i], ns[u][i]);
-              res[u][i][w] = pack_bf16(f0, f1);
-              ++piece;
-            }
-          }
-        }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int u = 0; u < A_PER; ++u) {
-          const int idx = tid + u * THREADS;
-          const int row = idx / (WNT / 8), cc = idx % (WNT / 8);
-          *reinterpret_cast<uint4*>(&As[buf ^ 1][row * AP + 8 * cc]) = R.a[u];
-        }
-#pragma unroll
-        for (int u = 0; u < B_PER; ++u) {
-          const int idx = item0 + u * THREADS;
-          const int row = idx / CPR, cc = idx % CPR;
-#pragma unroll
-          for (int i = 0; i < NST; ++i)
-            *reinterpret_cast<uint4*>(&Bs[buf ^ 1][row * BP + (seg0 + i) * HS + 8 * cc]) = finish_chunk(
-                co.splice_value(i, make_uint4(res[u][i][0], res[u][i][1], res[u][i][2], res[u][i][3]), R.o0[u][i], R.o1[u][i]),
-                i, cc, mb + row);
-        }
-      }
-    };
-    for (; m0 + 3 * WK < m_end; m0 += 2 * WK) {
-      fetch(R1, m0 + 2 * WK);
-      __syncthreads();                                    // buffer 0 is complete; buffer 1 is no longer read
-      overlap(0, R0, m0 + WK);
-      fetch(R0, m0 + 3 * WK);
-      __syncthreads();
-      overlap(1, R1, m0 + 2 * WK);
-    }
     for (; m0 < m_end; m0 += 2 * WK) {
       if (m0 + 2 * WK < m_end) fetch(R1, m0 + 2 * WK);
       __syncthreads();                                    // buffer 0 is complete; buffer 1 is no longer read
-      if (m0 + WK < m_end) stash(1, R0, m0 + WK);
+      if (m0 + WK < m_end) stash(1, R0);
       mfma_stage(0);
       if (m0 + WK < m_end) {
         if (m0 + 3 * WK < m_end) fetch(R0, m0 + 3 * WK);
         __syncthreads();
-        if (m0 + 2 * WK < m_end) stash(0, R1, m0 + 2 * WK);
+        if (m0 + 2 * WK < m_end) stash(0, R1);
         mfma_stage(1);
       }
     }
@@ -938,9 +781,7 @@ k_gradw_wide(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_
   for (int a = 0; a < 2; ++a)
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
-      const int hl = wh + 32 * b + (lane & 31);              // column inside the tile
-      const int64_t hs = j0 + (hl % HS);                     // column inside its segment
-      const int64_t h = (int64_t)(hl / HS) * SEG + hs;
+      const int64_t h = j0 + wh + 32 * b + (lane & 31);
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int64_t n = n0 + wn + 32 * a + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
@@ -1519,16 +1360,15 @@ int hyc_gradw_gemm(const void* dy, int64_t ldy, const void* stored, const void* 
   const bool fits32 = (tps + WK) * pitch_max < ((int64_t)1 << 31);
   if (wide && fits32) {
     const dim3 wgrid((unsigned)((N_out + wnt - 1) / wnt), (unsigned)(H / WH), (unsigned)splits);
-#define HYC_WIDE_W(B_, S_, W_)                                                                                    \
-  hipLaunchKernelGGL((k_gradw_wide<B_, S_, W_>), wgrid, dim3(2 * W_), 0, st, static_cast<const uint16_t*>(dy), ldy, M, \
-                     N_out, H, static_cast<const uint8_t*>(stored), static_cast<const uint16_t*>(vals),          \
-                     static_cast<const uint16_t*>(scales), ca, g.cps, tps, alpha, beta, out, of32, partial)
+#define HYC_WIDE()                                                                                               \
+  hipLaunchKernelGGL(k_gradw_wide, wgrid, dim3(2 * WN), 0, st, static_cast<const uint16_t*>(dy), ldy, M, N_out, H, \
+                     static_cast<const uint16_t*>(stored), tps, alpha, beta, out, of32, partial)
 #define HYC_BIG(B_, S_)                                                                                            \
   hipLaunchKernelGGL((k_gradw_big<B_, S_>), wgrid, dim3(256), 0, st, static_cast<const uint16_t*>(dy), ldy, M,     \
                      N_out, H, static_cast<const uint8_t*>(stored), static_cast<const uint16_t*>(vals),          \
                      static_cast<const uint16_t*>(scales), ca, g.cps, tps, alpha, beta, out, of32, partial)
     if (wnt == WN) {
-      HYC_WIDE_W(4, 2, WN);
+      HYC_WIDE();
     } else if (chan) {
       switch (d->bits) {
         case 1: HYC_BIG(1, 0); break;
@@ -1540,7 +1380,7 @@ int hyc_gradw_gemm(const void* dy, int64_t ldy, const void* stored, const void* 
       HYC_BIG(4, 2);
     }
 #undef HYC_BIG
-#undef HYC_WIDE_W
+#undef HYC_WIDE
   } else {
 #define HYC_GEMM(B_, S_, N_)                                                                                     \
   hipLaunchKernelGGL((k_gradw<B_, S_, N_>), grid, dim3(256), 0, st, static_cast<const uint16_t*>(dy), ldy, M, N_out, H, \
