@@ -184,54 +184,64 @@ k_act_bwd_fast(const uint16_t* __restrict__ g, const uint8_t* __restrict__ store
   for (int i = 0; i < NSEG; ++i) plan[i] = ca.plan[i * CPS + c];
   ChunkOutliers<NSEG> co;
   co.init(plan);
+  // Every memory instruction of the row loop is an unconditional buffer operation: a row past the end gets a resource
+  // of zero bytes (loads return zeros, stores are dropped), an outlier slot the chunk does not have gets an offset
+  // beyond every resource.  No branch surrounds a load, so the compiler's waits are sized for the steady state.
   const int64_t stride = gridDim.x;
   int64_t row = blockIdx.x;
-  const uint16_t* gp = g + row * H + 8 * c;
-  uint16_t* dxp = dx + row * H + 8 * c;
-  const uint8_t* sp = stored + row * SEG + 8 * c;
-  const uint16_t* vp = vals + row * ca.k;
-  const uint16_t* scp = scales + row * ca.groups_per_row + (c >> ca.chunk_to_group_shift);
-  const int64_t xstep = stride * H, sstep = stride * SEG, vstep = stride * ca.k, scstep = stride * ca.groups_per_row;
-  uint2 pk = make_uint2(0, 0);
-  uint4 graw[NSEG];
-  uint32_t sc[NSEG];   // one register each: a packed pair would be assembled right after the load and stall on it
-  uint32_t o0[NSEG], o1[NSEG];
-  if (row < M) {
-    pk = *reinterpret_cast<const uint2*>(sp);
+  const uint32_t row_b = 2u * (uint32_t)H, seg_b = 2u * (uint32_t)SEG, gpr_b = 2u * (uint32_t)ca.groups_per_row;
+  const uint32_t val_b = 2u * (uint32_t)ca.k;
+  const uint32_t xo = 16u * (uint32_t)c, so = 8u * (uint32_t)c;
+  uint32_t sco[NSEG], vo0[NSEG], vo1[NSEG];
 #pragma unroll
-    for (int i = 0; i < NSEG; ++i) { graw[i] = *reinterpret_cast<const uint4*>(gp + i * SEG); sc[i] = scp[i * seg_groups]; }
-    co.request(vp, o0, o1);
+  for (int i = 0; i < NSEG; ++i) {
+    sco[i] = 2u * (uint32_t)((c >> ca.chunk_to_group_shift) + i * seg_groups);
+    vo0[i] = co.has0[i] ? co.vb[i] : NOWHERE;
+    vo1[i] = co.has1[i] ? co.vb[i] + 2u : NOWHERE;
   }
-  for (; row < M; row += stride) {
-    uint2 pk_n = make_uint2(0, 0);
+  auto row_of = [&](const void* base, int64_t r, uint32_t bytes) __attribute__((always_inline)) {
+    return make_rsrc(static_cast<const char*>(base) + r * (int64_t)bytes, r < M ? bytes : 0u);
+  };
+  uint2 pk;
+  uint4 graw[NSEG];
+  uint32_t sc[NSEG], o0[NSEG], o1[NSEG];
+  auto request = [&](int64_t r, uint2& pk_, uint4 (&g_)[NSEG], uint32_t (&sc_)[NSEG], uint32_t (&o0_)[NSEG],
+                     uint32_t (&o1_)[NSEG]) __attribute__((always_inline)) {
+    const BufferRsrc rs_g = row_of(g, r, row_b), rs_s = row_of(stored, r, (uint32_t)SEG);
+    const BufferRsrc rs_c = row_of(scales, r, gpr_b), rs_v = row_of(vals, r, val_b);
+    pk_ = load_b64(rs_s, so);
+#pragma unroll
+    for (int i = 0; i < NSEG; ++i) {
+      g_[i] = load_b128(rs_g, xo + (uint32_t)i * seg_b);
+      sc_[i] = load_b16(rs_c, sco[i]);
+      o0_[i] = load_b16(rs_v, vo0[i]);
+      o1_[i] = load_b16(rs_v, vo1[i]);
+    }
+  };
+  request(row, pk, graw, sc, o0, o1);
+  const int64_t steps = row < M ? (M - row + stride - 1) / stride : 0;
+  for (int64_t step = 0; step < steps; ++step, row += stride) {
+    uint2 pk_n;
     uint4 g_n[NSEG];
     uint32_t sc_n[NSEG], o0_n[NSEG], o1_n[NSEG];
-    if (row + stride < M) {
-      pk_n = *reinterpret_cast<const uint2*>(sp + sstep);
-#pragma unroll
-      for (int i = 0; i < NSEG; ++i) {
-        g_n[i] = *reinterpret_cast<const uint4*>(gp + xstep + i * SEG);
-        sc_n[i] = scp[scstep + i * seg_groups];
-      }
-      co.request(vp + vstep, o0_n, o1_n);
-    }
+    request(row + stride, pk_n, g_n, sc_n, o0_n, o1_n);
+    const BufferRsrc rs_o = row_of(dx, row, row_b);
 #pragma unroll
     for (int i = 0; i < NSEG; ++i) {
       float xv[8], gv[8], o[8];
       const float sf = bf_to_f((uint16_t)sc[i]);
       uint4 r = co.splice(i, dequant8<BITS>(pk.x, pk.y, i, sf), o0[i], o1[i], sf);
-      if (co.more_pairs) r = splice_more(r, co.more_pairs, ca.plan[i * CPS + c], vp, true, sf);
+      if (co.more_pairs) r = splice_more(r, co.more_pairs, ca.plan[i * CPS + c], vals + row * ca.k, true, sf);
       unpack8(graw[i], gv);
       if (!(HAS_LUT && use_lut && lut_grad8(lut, r, gv, o))) {
         unpack8(r, xv);
         act_grad8<ACT>(xv, gv, o);
       }
-      store_stream(dxp + i * SEG, pack8(o));
+      store_b128_stream(rs_o, xo + (uint32_t)i * seg_b, pack8(o));
     }
     pk = pk_n;
 #pragma unroll
     for (int i = 0; i < NSEG; ++i) { graw[i] = g_n[i]; sc[i] = sc_n[i]; o0[i] = o0_n[i]; o1[i] = o1_n[i]; }
-    gp += xstep; dxp += xstep; sp += sstep; vp += vstep; scp += scstep;
   }
 }
 
