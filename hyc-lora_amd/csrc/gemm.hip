@@ -1049,13 +1049,46 @@ k_gradw_big(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_o
   };
   // One stage: the MFMAs on LDS buffer B; the register set Rd (stage s+1, tokens m1 ..) goes to buffer B+1 on the
   // way and the set Rf is requested anew (stage s+3).
-  auto stage = [&](auto bno, const Regs& Rd, Regs& Rf, int64_t m1) __attribute__((always_inline)) {
+  // What the decode of a stage needs before its first piece - the code bytes of each chunk isolated, its scale as a
+  // float and the offset term - is prepared in the last eight slots of the stage before (they are the lightest), as
+  // are the requests for the further outlier values of a crowded chunk; both live across the stage boundary.
+  constexpr uint32_t REP = (BITS == 8) ? 0x80808080u : Q<BITS>::CODE_MASK * 0x01010101u;
+  constexpr float OFFV = (BITS == 8) ? 128.f : (float)Q<BITS>::OFF;
+  uint32_t cw[NCH][2];
+  float sc[NCH], ns[NCH];
+  uint32_t xv2[B_PER], xv3[B_PER];
+  auto prepare_codes = [&](const Regs& R, int c) __attribute__((always_inline)) {
+    const int u = c / NST, i = c % NST;
+    cw[c][0] = (BITS == 8) ? R.b[u].x ^ REP : (R.b[u].x >> ((seg0 + i) * BITS)) & REP;
+    cw[c][1] = (BITS == 8) ? R.b[u].y ^ REP : (R.b[u].y >> ((seg0 + i) * BITS)) & REP;
+    asm volatile("" : "+v"(cw[c][0]), "+v"(cw[c][1]));                  // (keeps the byte-wise conversions of the pieces)
+  };
+  auto prepare_scale = [&](const Regs& R, int c) __attribute__((always_inline)) {
+    sc[c] = bf_to_f((uint16_t)R.s[c / NST][c % NST]);
+    ns[c] = -OFFV * sc[c];
+  };
+  auto request_extras = [&](int64_t mb, int which) __attribute__((always_inline)) {   // (lanes without a crowded chunk ask for nothing)
+    const uint32_t xoff = (uint32_t)(mb - m_begin) * kk2;
+#pragma unroll
+    for (int u = 0; u < B_PER; ++u) {
+      if (which == 0) xv2[u] = load_b16(rs_x, vx2 + xoff + (uint32_t)(u * (THREADS / CPR)) * kk2);
+      else xv3[u] = load_b16(rs_x, vx3 + xoff + (uint32_t)(u * (THREADS / CPR)) * kk2);
+    }
+  };
+  // One wait per group of registers instead of one per use: naming them all in an empty asm makes the compiler wait
+  // for the last of them here, and the uses that follow need no wait of their own.
+  auto arrived_a = [&](Regs& R) __attribute__((always_inline)) {
+    asm volatile("" : "+v"(R.a[0].x), "+v"(R.a[1].x), "+v"(R.a[2].x), "+v"(R.a[3].x));   // (one word stands for its load)
+  };
+  auto arrived_frags = [&](bf16x8_t (&fa)[4], bf16x8_t (&fb)[4]) __attribute__((always_inline)) {
+    asm volatile("" : "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[3]));
+    asm volatile("" : "+v"(fb[0]), "+v"(fb[1]), "+v"(fb[2]), "+v"(fb[3]));
+  };
+  // Rd: decoded and written to LDS in this stage (stage s+1); Rf: requested anew (stage s+3); Rn: decoded in the next
+  // stage (stage s+2; its codes and scales are prepared at the end of this one)
+  auto stage = [&](auto bno, Regs& Rd, Regs& Rf, const Regs& Rn, int64_t m1) __attribute__((always_inline)) {
     constexpr int B = decltype(bno)::value, NB = (B + 1) % NBUF;
-    constexpr uint32_t REP = (BITS == 8) ? 0x80808080u : Q<BITS>::CODE_MASK * 0x01010101u;
-    constexpr float OFFV = (BITS == 8) ? 128.f : (float)Q<BITS>::OFF;
-    uint32_t cw[NCH][2], res[NCH][4];
-    float sc[NCH], ns[NCH];
-    uint32_t xv2[B_PER], xv3[B_PER];
+    uint32_t res[NCH][4];
     auto slot = [&](auto tno) __attribute__((always_inline)) {
       constexpr int t = decltype(tno)::value;
       __builtin_amdgcn_sched_barrier(0);
@@ -1064,23 +1097,8 @@ k_gradw_big(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_o
         acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(t < 16 ? fa0[a] : fa1[a], t < 16 ? fb0[b] : fb1[b], acc[a][b], 0, 0, 0);
       }
       if constexpr (t < 8) read_frag(HYC_AS(B), HYC_BS(B), 16, t, fa1, fb1);
-      if constexpr (FASTX && (t == 1 || t == 2)) {                      // (unconditional: lanes without such a chunk ask for nothing)
-        const uint32_t xoff = (uint32_t)(m1 - m_begin) * kk2;
-#pragma unroll
-        for (int u = 0; u < B_PER; ++u) {
-          if (t == 1) xv2[u] = load_b16(rs_x, vx2 + xoff + (uint32_t)(u * (THREADS / CPR)) * kk2);
-          else xv3[u] = load_b16(rs_x, vx3 + xoff + (uint32_t)(u * (THREADS / CPR)) * kk2);
-        }
-      }
       if constexpr (SRC == 0 && t < 16) {                               // two elements of chunk c of stage s+1
-        constexpr int c = t >> 2, w = t & 3, u = c / NST, i = c % NST;
-        if constexpr (w == 0) {
-          cw[c][0] = (BITS == 8) ? Rd.b[u].x ^ REP : (Rd.b[u].x >> ((seg0 + i) * BITS)) & REP;
-          cw[c][1] = (BITS == 8) ? Rd.b[u].y ^ REP : (Rd.b[u].y >> ((seg0 + i) * BITS)) & REP;
-          asm volatile("" : "+v"(cw[c][0]), "+v"(cw[c][1]));            // (keeps the byte-wise conversions below)
-          sc[c] = bf_to_f((uint16_t)Rd.s[u][i]);
-          ns[c] = -OFFV * sc[c];
-        }
+        constexpr int c = t >> 2, w = t & 3;
         const uint32_t src = cw[c][w >> 1];
         const float f0 = __builtin_fmaf((float)((src >> (16 * (w & 1))) & 0xFFu), sc[c], ns[c]);
         const float f1 = __builtin_fmaf((float)((src >> (16 * (w & 1) + 8)) & 0xFFu), sc[c], ns[c]);
@@ -1090,6 +1108,10 @@ k_gradw_big(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_o
         constexpr int j0_ = (t - 8) * NLOAD / 8, j1_ = (t - 7) * NLOAD / 8;
         for_each_slot([&](auto jno) __attribute__((always_inline)) { request(Rf, j0_ + decltype(jno)::value); },
                       std::make_integer_sequence<int, j1_ - j0_>{});
+      }
+      if constexpr (t == 16) {
+        arrived_a(Rd);
+        arrived_frags(fa1, fb1);
       }
       if constexpr (t >= 16 && t < 20) {
         *reinterpret_cast<uint4*>(&HYC_AS(NB)[a_at[t - 16]]) = Rd.a[t - 16];
@@ -1117,6 +1139,10 @@ k_gradw_big(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_o
       }
       if constexpr (t == 24) __syncthreads();                           // buffer NB is complete, buffer B read for the last time
       if constexpr (t >= 24) read_frag(HYC_AS(NB), HYC_BS(NB), 0, t - 24, fa0, fb0);
+      if constexpr (SRC == 0 && t >= 24) {                              // for the next stage's decode
+        if constexpr ((t & 1) == 0) prepare_codes(Rn, (t - 24) >> 1); else prepare_scale(Rn, (t - 24) >> 1);
+        if constexpr (FASTX && (t == 26 || t == 27)) request_extras(m1 + WK, t - 26);
+      }
     };
     for_each_slot(slot, std::make_integer_sequence<int, 32>{});
     __builtin_amdgcn_sched_barrier(0);
@@ -1133,10 +1159,15 @@ k_gradw_big(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_o
 #pragma unroll
     for (int q = 0; q < 8; ++q) read_frag(HYC_AS(0), HYC_BS(0), 0, q, fa0, fb0);
     int64_t m1 = m_begin + WK;
+    if (SRC == 0) {
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) { prepare_codes(R1, c); prepare_scale(R1, c); }
+      if (FASTX) { request_extras(m1, 0); request_extras(m1, 1); }
+    }
     for (int64_t s = 0; s < nstages; s += 3) {                         // a stage past the end holds zeros
-      stage(StageNo<0>{}, R1, R0, m1);
-      stage(StageNo<1>{}, R2, R1, m1 + WK);
-      stage(StageNo<2>{}, R0, R2, m1 + 2 * WK);
+      stage(StageNo<0>{}, R1, R0, R2, m1);
+      stage(StageNo<1>{}, R2, R1, R0, m1 + WK);
+      stage(StageNo<2>{}, R0, R2, R1, m1 + 2 * WK);
       m1 += 3 * WK;
     }
   }
