@@ -805,15 +805,16 @@ k_gradw_wide(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_
 // Large output, second form: workgroup tile 256 (n) x 256 (h) on FOUR waves of 128 x 128, one per SIMD.  A wave's 256
 // fp32 accumulators live in the accumulation registers (the compiler puts them there by itself at one wave per SIMD),
 // which leaves the 256 ordinary registers to operand fragments and to the data of the next three stages.  Against the
-// 64 x 128 wave tile this halves the operand bytes read from LDS per MFMA (8 fragments per 16 MFMAs instead of 6 per
-// 8) - the traffic that bounds the eight-wave form.  With a single wave per SIMD nothing but the wave's own next
-// instructions can fill the 32 cycles of an MFMA (eight issue slots: the MFMA and seven others), so a stage of 32
-// tokens is laid out by hand as 32 slots, one MFMA each:
+// 64 x 128 wave tile of the first form this halves the operand bytes read from LDS per MFMA (8 fragments per 16
+// MFMAs instead of 6 per 8).  With a single wave per SIMD nothing but the wave's own next instructions can fill the
+// 32 cycles of an MFMA (eight issue slots: the MFMA and seven others; measured: up to six ordinary VALU instructions
+// hide under one), so a stage of 32 tokens is laid out by hand as 32 slots, one MFMA each:
 //   slots  0- 7  read the fragments of the stage's second 16 tokens
 //   slots  0-15  decode stage s+1 (two elements per slot; its registers were requested two stages ago)
 //   slots  8-15  request stage s+3 into the register set that held stage s
 //   slots 16-23  write stage s+1 to the next LDS buffer, move the buffer resources on
-//   slot  24     the stage's one barrier; slots 24-31 read the fragments of the first 16 tokens of stage s+1
+//   slot  24     the stage's one barrier; slots 24-31 read the fragments of the first 16 tokens of stage s+1 and
+//                prepare the decode of stage s+2 (code bytes, scales)
 // ------------------------------------------------------------------------------------------------
 template <int V> struct StageNo { static constexpr int value = V; };
 // f(StageNo<0>), f(StageNo<1>), ... : a loop whose bodies are separate instantiations (no unroll threshold applies)
