@@ -525,6 +525,14 @@ def main():
                               "fwd_frac_of_hbm_peak": round(fs / f_ms / 1e6 / HBM_PEAK_GBPS, 4),
                               "bwd_frac_of_hbm_peak": round(bs / b_ms / 1e6 / HBM_PEAK_GBPS, 4),
                               "bwd_row_kernel_frac_of_hbm_peak": round(bs / bm_ms / 1e6 / HBM_PEAK_GBPS, 4)}
+        if not args.no_extras:
+            # the trained shape of the weight gradient (LoRA-A, 16 features) on the same 16x activation: INT4 with
+            # 128-channel groups (what the fused norm saved) and INT2 with 64-channel groups (configs[2]'s width)
+            lora = (("lora_a_r16", 16, 100, 20),)
+            extra["scaled16x"]["gradw_int4_g128"] = gradw_extra(pkg, torch, wls.c, shapes=lora)["lora_a_r16"]
+            c2s = pkg.kernels.compress_channel(wls.x, wls.plan, 2, 64)
+            extra["scaled16x"]["gradw_int2_g64"] = gradw_extra(pkg, torch, c2s, shapes=lora)["lora_a_r16"]
+            del c2s
         del wls
         torch.cuda.empty_cache()
     if not args.no_extras:

@@ -195,6 +195,27 @@ k_gradw(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_out, 
 constexpr int DK = 32;     // tokens per step = one MFMA k-step
 
 typedef float floatx4_t __attribute__((ext_vector_type(4)));
+typedef float floatx2_t __attribute__((ext_vector_type(2)));
+
+// Buffer loads with a scalar offset on top of the lane's: the hardware checks the SUM of both offsets against the
+// size of the resource, so a row selected through the scalar offset is dropped (reads zeros) when it lies past the end.
+__device__ __forceinline__ uint2 load_b64(BufferRsrc r, uint32_t off, uint32_t scalar_off) {
+  const u32x2_t v = __builtin_amdgcn_raw_buffer_load_b64(r, (int)off, (int)scalar_off, 0);
+  return make_uint2(v.x, v.y);
+}
+__device__ __forceinline__ uint32_t load_b16(BufferRsrc r, uint32_t off, uint32_t scalar_off) {
+  return (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(r, (int)off, (int)scalar_off, 0);
+}
+
+// Codes to floats, two per instruction.  A byte below 17 read as an FP8 number (E4M3, bias 7) is that integer times
+// 2^-9: the exponent fields 0 and 1 share one step.  The scaled packed conversion multiplies by a power of two on
+// its way (it takes the exponent of its scale operand), so with 2^9 the two bytes of one half of `w` come out as the
+// floats of their integer values: exact, and half the instructions of one conversion per byte.  Serves every code
+// width whose codes stay below 16.
+template <bool HIGH_HALF>
+__device__ __forceinline__ floatx2_t small_bytes_to_float(uint32_t w) {
+  return __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(w, 512.f, HIGH_HALF);
+}
 
 struct DirectArgs {
   const uint16_t* dy; int64_t ldy, M, N_out, H;
@@ -222,7 +243,7 @@ struct DirectRegs {          // what one lane loads for one step: a packed word 
 //     so the bit pattern of 2^BITS with the code in the top mantissa bits IS the number 2^BITS + code.  One byte
 //     permute picks the lane's byte of two tokens' words, one shift and one and-or put the code field of a segment
 //     under that pattern: 1 + 1/(2 SPT) operations per element plus 40 per segment and step for hi and lo (the fma
-//     form takes 3.9 per element).  The surplus 2^BITS + OFF per element is removed at the end through two more MFMAs
+//     form takes 2.9 per element, half of them conversions, which issue at a lower rate).  The surplus 2^BITS + OFF per element is removed at the end through two more MFMAs
 //     per step whose B operand is all ones (sum_t A[n, t] in every column): dW -= (2^BITS + OFF) * that sum.
 //     Products are exact and fp32-accumulated either way; the partial sums are at most 6 times larger than the
 //     result's terms, so nothing is lost to cancellation.
@@ -255,7 +276,7 @@ __device__ __forceinline__ void gradw_direct_tile(const DirectArgs& A, float* re
   const int hsel = l16 / LC;                                                     // which of the R byte subsets (0 when R <= 1)
   const int c = MAINT ? (hy - sgrp * c_tiles) * LC + (l16 % LC) : 0;             // chunk inside the segment
   const int q = MAINT ? 0 : hy * 16 + l16;                                       // outlier number
-  const int shs = (BITS == 8) ? 0 : seg * BITS;
+  const int shs = (BITS == 8 || SPT == Q<BITS>::NSEG) ? 0 : seg * BITS;   // a tile of all segments starts at bit 0
   const int64_t m_begin = (int64_t)blockIdx.z * A.tokens_per_split;
   const int64_t m_end = m_begin + A.tokens_per_split < A.M ? m_begin + A.tokens_per_split : A.M;
 
@@ -313,53 +334,27 @@ __device__ __forceinline__ void gradw_direct_tile(const DirectArgs& A, float* re
     for (int g = 0; g < (FOLD ? SPT : 1); ++g) accs[g][a] = (floatx4_t){0.f, 0.f, 0.f, 0.f};
   }
 
-  // Every load is unconditional: lanes past the last chunk / outlier / feature read their neighbour's data (the
-  // results are dropped at the write-out), tokens past the end read the last token with a zeroed dY operand.
+  // Every load is unconditional.  Lanes past the last chunk / outlier / feature read their neighbour's data (the
+  // results are dropped at the write-out).  The buffer resources of a step span exactly its valid tokens, token e of
+  // a lane's eight sits in the scalar offset (the hardware checks the sum of both offsets against the size), so
+  // tokens past the end of the range read zeros: a zero dY operand, a zero scale.
   auto fetch = [&](int64_t m0, DirectRegs<SPT>& Rg, uint32_t (&ar)[NT][8]) __attribute__((always_inline)) {
-    const int left = (int)(m_end - m0 < DK ? m_end - m0 : DK);                  // valid tokens of the step
-    const char* ab = asrc + m0 * dy_b;
-    const char* bb = bsrc + m0 * tok_b;
-    const char* sb = ssrc + m0 * sc_b;
-    if (left == DK) {                                                            // all steps but the last: scalar base + lane offset
-      uint32_t bo = boff, so[SPT], ao[NT];
-      asm volatile("" : "+v"(bo));                                               // keep them 32-bit values of this block
+    const uint32_t left = (uint32_t)(m_end - m0 < DK ? m_end - m0 : DK);        // valid tokens of the step
+    const BufferRsrc rs_a = make_rsrc(asrc + m0 * dy_b, left * (uint32_t)dy_b);
+    const BufferRsrc rs_b = make_rsrc(bsrc + m0 * tok_b, left * (uint32_t)tok_b);
+    const BufferRsrc rs_s = make_rsrc(ssrc + m0 * sc_b, left * (uint32_t)sc_b);
 #pragma unroll
-      for (int g = 0; g < SPT; ++g) { so[g] = soff[g]; asm volatile("" : "+v"(so[g])); }
+    for (int e = 0; e < 8; ++e) {
+      if (MAINT) {
+        const uint2 w = load_b64(rs_b, boff, (uint32_t)e * (uint32_t)tok_b);
+        Rg.blo[e] = w.x; Rg.bhi[e] = w.y;
 #pragma unroll
-      for (int a = 0; a < NT; ++a) { ao[a] = aoff[a]; asm volatile("" : "+v"(ao[a])); }
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        if (MAINT) {
-          const uint2 w = *reinterpret_cast<const uint2*>(bb + bo);
-          Rg.blo[e] = w.x; Rg.bhi[e] = w.y;
-#pragma unroll
-          for (int g = 0; g < SPT; ++g) Rg.sc[g][e] = *reinterpret_cast<const uint16_t*>(sb + so[g]);
-        } else {
-          Rg.blo[e] = *reinterpret_cast<const uint16_t*>(bb + bo);
-        }
-#pragma unroll
-        for (int a = 0; a < NT; ++a) ar[a][e] = *reinterpret_cast<const uint16_t*>(ab + ao[a]);
-        bb += tok_b; sb += sc_b; ab += dy_b;
+        for (int g = 0; g < SPT; ++g) Rg.sc[g][e] = load_b16(rs_s, soff[g], (uint32_t)e * (uint32_t)sc_b);
+      } else {
+        Rg.blo[e] = load_b16(rs_b, boff, (uint32_t)e * (uint32_t)tok_b);
       }
-    } else {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int t = 8 * kq + e;
-        const int tc = t < left ? t : left - 1;
-        if (MAINT) {
-          const uint2 w = *reinterpret_cast<const uint2*>(bb + tc * tok_b + lane_b);
-          Rg.blo[e] = w.x; Rg.bhi[e] = w.y;
-#pragma unroll
-          for (int g = 0; g < SPT; ++g) Rg.sc[g][e] = *reinterpret_cast<const uint16_t*>(sb + tc * sc_b + lane_s[g]);
-        } else {
-          Rg.blo[e] = *reinterpret_cast<const uint16_t*>(bb + tc * tok_b + lane_b);
-        }
-#pragma unroll
-        for (int a = 0; a < NT; ++a) {
-          const uint32_t v = *reinterpret_cast<const uint16_t*>(ab + tc * dy_b + lane_a[a]);
-          ar[a][e] = t < left ? v : 0u;
-        }
-      }
+      for (int a = 0; a < NT; ++a) ar[a][e] = load_b16(rs_a, aoff[a], (uint32_t)e * (uint32_t)dy_b);
     }
   };
   auto step = [&](DirectRegs<SPT>& Rg, uint32_t (&ar)[NT][8]) __attribute__((always_inline)) {
@@ -457,21 +452,45 @@ __device__ __forceinline__ void gradw_direct_tile(const DirectArgs& A, float* re
           // segment seg + g's code of every byte, as a byte
           clo[e] = (BITS == 8) ? Rg.blo[e] ^ 0x80808080u : (Rg.blo[e] >> (shs + g * BITS)) & REP;
           chi[e] = (BITS == 8) ? Rg.bhi[e] ^ 0x80808080u : (Rg.bhi[e] >> (shs + g * BITS)) & REP;
+          // opaque from here on: each code then costs one byte-to-float conversion; left visible, the compiler folds
+          // this mask into one bit-field extract per code ahead of the conversion
+          asm volatile("" : "+v"(clo[e]), "+v"(chi[e]));
         }
+        if (BITS <= 4) {
+          // two neighbouring bytes of a token's word per conversion; a fragment register wants two tokens of one byte
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          uint32_t wj[4];
+          for (int j = 0; j < 8; j += 2) {
+            uint32_t w0[4], w1[4];
 #pragma unroll
-          for (int e = 0; e < 8; e += 2) {
-            float f[2];
+            for (int e = 0; e < 8; e += 2) {
+              floatx2_t p[2];
 #pragma unroll
-            for (int d = 0; d < 2; ++d) {
-              const uint32_t w = (j < 4) ? clo[e + d] : chi[e + d];
-              f[d] = __builtin_fmaf((float)((w >> (8 * (j & 3))) & 0xFFu), s[e + d], ns[e + d]);
+              for (int d = 0; d < 2; ++d) {
+                const uint32_t w = (j < 4) ? clo[e + d] : chi[e + d];
+                p[d] = (j & 2) ? small_bytes_to_float<true>(w) : small_bytes_to_float<false>(w);
+              }
+              w0[e >> 1] = pack_bf16(__builtin_fmaf(p[0].x, s[e], ns[e]), __builtin_fmaf(p[1].x, s[e + 1], ns[e + 1]));
+              w1[e >> 1] = pack_bf16(__builtin_fmaf(p[0].y, s[e], ns[e]), __builtin_fmaf(p[1].y, s[e + 1], ns[e + 1]));
             }
-            wj[e >> 1] = pack_bf16(f[0], f[1]);
+            bfrag[j] = __builtin_bit_cast(bf16x8_t, (u32x4_t){w0[0], w0[1], w0[2], w0[3]});
+            bfrag[j + 1] = __builtin_bit_cast(bf16x8_t, (u32x4_t){w1[0], w1[1], w1[2], w1[3]});
           }
-          bfrag[j] = __builtin_bit_cast(bf16x8_t, (u32x4_t){wj[0], wj[1], wj[2], wj[3]});
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            uint32_t wj[4];
+#pragma unroll
+            for (int e = 0; e < 8; e += 2) {
+              float f[2];
+#pragma unroll
+              for (int d = 0; d < 2; ++d) {
+                const uint32_t w = (j < 4) ? clo[e + d] : chi[e + d];
+                f[d] = __builtin_fmaf((float)((w >> (8 * (j & 3))) & 0xFFu), s[e + d], ns[e + d]);
+              }
+              wj[e >> 1] = pack_bf16(f[0], f[1]);
+            }
+            bfrag[j] = __builtin_bit_cast(bf16x8_t, (u32x4_t){wj[0], wj[1], wj[2], wj[3]});
+          }
         }
 #pragma unroll
         for (int a = 0; a < NT; ++a)
@@ -600,25 +619,28 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) k
 }
 
 // How a shape is laid on the kernel: R (see above) from the group width, SPT from the registers the accumulators of
-// NT x SPT x 8/R tiles leave, LC chunks per tile.
-struct DirectPlan { int r, spt, lc; };
+// NT x SPT x 8/R tiles leave, LC chunks per tile, and how many workgroups of the variant a CU holds at once (three
+// where it needs at most 168 registers per lane, else two).
+struct DirectPlan { int r, spt, lc, per_cu; };
 static DirectPlan direct_plan(int bits, int lpg, int64_t N_out) {
   DirectPlan p;
   const int nseg = 8 / bits, nt = N_out <= 16 ? 1 : 2;
   p.r = (bits > 2 || lpg < 8) ? 0 : (lpg >= 16 ? 1 : (nt == 1 ? 2 : 0));
-  p.spt = p.r == 0 ? 1 : (nt == 1 ? 2 : 1);
+  // 4-bit codes, one feature tile: both segments of a packed word in one tile, so every word is loaded once
+  p.spt = p.r == 0 ? (bits == 4 && nt == 1 ? 2 : 1) : (nt == 1 ? 2 : 1);
   if (p.spt > nseg) p.spt = nseg;
   p.lc = p.r == 2 ? 8 : 16;
+  p.per_cu = (nt == 1 && p.r != 1 && !(p.r == 0 && p.spt == 2)) ? 3 : 2;
   return p;
 }
 
 // The streaming kernel serves N_out <= DIRECT_MAX_N.  Token splits: as many as keep the whole grid resident at once
-// (two workgroups per CU, DIRECT_BLOCKS in all).  The kernel is bound by its decode work, so a grid a little over that
-// leaves most of the chip idle during a second round (65 536 x 4096 INT4: 560 workgroups 88 us, 490 workgroups 65 us).
+// (256 CUs x the plan's workgroups per CU).  The kernel is bound by its decode work, so a grid a little over that
+// leaves most of the chip idle during a second round (65 536 x 4096 INT4, two per CU: 560 workgroups 88 us, 490
+// workgroups 65 us).
 constexpr int64_t DIRECT_MAX_N = 32;
-constexpr int64_t DIRECT_BLOCKS = 512;
-static int direct_splits(int64_t M, int64_t y_tiles) {
-  int64_t s = DIRECT_BLOCKS / (y_tiles > 0 ? y_tiles : 1);
+static int direct_splits(int64_t M, int64_t y_tiles, int per_cu) {
+  int64_t s = (int64_t)256 * per_cu / (y_tiles > 0 ? y_tiles : 1);
   const int64_t max_by_tokens = (M + 8 * DK - 1) / (8 * DK);      // at least two steps per wave
   if (s > max_by_tokens) s = max_by_tokens;
   if (s < 1) s = 1;
@@ -635,7 +657,7 @@ static int direct_splits_max(int64_t M, int64_t N_out, int64_t H) {
   int best = 1;
   for (int bits = 1; bits <= 8; bits *= 2)
     for (int lpg = 4; lpg <= 16; lpg *= 2) {
-      const int sp = direct_splits(M, direct_y_tiles(H, bits, lpg, 0, N_out));
+      const int sp = direct_splits(M, direct_y_tiles(H, bits, lpg, 0, N_out), direct_plan(bits, lpg, N_out).per_cu);
       if (sp > best) best = sp;
     }
   return best;
@@ -1101,9 +1123,14 @@ k_gradw_big(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_o
       if constexpr (SRC == 0 && t < 16) {                               // two elements of chunk c of stage s+1
         constexpr int c = t >> 2, w = t & 3;
         const uint32_t src = cw[c][w >> 1];
-        const float f0 = __builtin_fmaf((float)((src >> (16 * (w & 1))) & 0xFFu), sc[c], ns[c]);
-        const float f1 = __builtin_fmaf((float)((src >> (16 * (w & 1) + 8)) & 0xFFu), sc[c], ns[c]);
-        res[c][w] = pack_bf16(f0, f1);
+        float c0, c1;
+        if constexpr (BITS <= 4) {                                      // both codes of the half-word in one conversion
+          const floatx2_t p = (w & 1) ? small_bytes_to_float<true>(src) : small_bytes_to_float<false>(src);
+          c0 = p.x; c1 = p.y;
+        } else {
+          c0 = (float)((src >> (16 * (w & 1))) & 0xFFu); c1 = (float)((src >> (16 * (w & 1) + 8)) & 0xFFu);
+        }
+        res[c][w] = pack_bf16(__builtin_fmaf(c0, sc[c], ns[c]), __builtin_fmaf(c1, sc[c], ns[c]));
       }
       if constexpr (t >= 8 && t < 16) {
         constexpr int j0_ = (t - 8) * NLOAD / 8, j1_ = (t - 7) * NLOAD / 8;
@@ -1329,7 +1356,7 @@ int hyc_gradw_gemm(const void* dy, int64_t ldy, const void* stored, const void* 
     const DirectPlan pl = direct_plan(d->bits, lpg, N_out);
     const int c_tiles = (g.cps + pl.lc - 1) / pl.lc, o_tiles = (d->k + 15) / 16;
     const int y_tiles = (g.nseg / pl.spt) * c_tiles + o_tiles;
-    const int splits = M > 0 ? direct_splits(M, y_tiles) : 1;
+    const int splits = M > 0 ? direct_splits(M, y_tiles, pl.per_cu) : 1;
     if (splits > 1 && !workspace) return fail(HYC_EFAULT, "hyc_gradw_gemm: workspace of hyc_gradw_workspace_bytes() bytes required");
     if (splits > 1 && !aligned16(workspace)) return fail(HYC_EINVAL, "hyc_gradw_gemm: workspace must be 16-byte aligned");
     int64_t tps = (M + splits - 1) / splits;
@@ -1353,7 +1380,7 @@ int hyc_gradw_gemm(const void* dy, int64_t ldy, const void* stored, const void* 
     switch (d->bits) {
       case 1: HYC_DIRECT(1); break;
       case 2: HYC_DIRECT(2); break;
-      case 4: if (nt == 1) HYC_DIRECT_K(4, 1, 1, 0); else HYC_DIRECT_K(4, 2, 1, 0); break;
+      case 4: if (nt == 1) HYC_DIRECT_K(4, 1, 2, 0); else HYC_DIRECT_K(4, 2, 1, 0); break;
       default: if (nt == 1) HYC_DIRECT_K(8, 1, 1, 0); else HYC_DIRECT_K(8, 2, 1, 0); break;
     }
 #undef HYC_DIRECT_K

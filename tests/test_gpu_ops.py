@@ -90,6 +90,23 @@ def test_gradw_crowded_chunks(K, bits, group, hot):
     assert torch.allclose(fused, dense, rtol=1e-5, atol=1e-5 * float(dense.abs().max()))
 
 
+@pytest.mark.parametrize("bits,group,M,N", [(4, 128, 333, 16), (2, 64, 1000, 16), (8, 128, 97, 24), (4, 128, 300, 256)])
+def test_gradw_column_slice_of_dy(K, bits, group, M, N):
+    """dY handed over as a column slice of a wider matrix (row pitch above its width), with a ragged token count: the
+    same bits as with a contiguous copy"""
+    H = 1024
+    x, gen = make_x(bits + M, M, H, 10, 20.0)
+    wide = (0.05 * torch.randn(M, N + 24, generator=gen)).bfloat16().cuda()
+    dy = wide[:, 8:8 + N]
+    assert dy.stride(0) == N + 24 and not dy.is_contiguous()
+    xd = x.cuda()
+    c = K.compress_channel(xd, K.select_channels(K.channel_absmax(xd), 10), bits, group)
+    got = K.gradw_gemm(dy, c, out_dtype=torch.float32, staged=False)
+    assert torch.equal(got, K.gradw_gemm(dy.contiguous(), c, out_dtype=torch.float32, staged=False))
+    want = dy.float().t() @ K.decompress_channel(c).float()
+    assert torch.allclose(got, want, rtol=1e-3, atol=1e-3)
+
+
 def test_gradw_config3_lora_a(K):
     """BASELINE config 3: X [4,1024,4096] as 1 % bf16 outliers + INT2 group 64; grad_A = (s * dY @ B)^T @ x_hat, r = 16"""
     M, H, r = 4096, 4096, 16
