@@ -195,7 +195,6 @@ k_gradw(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_out, 
 constexpr int DK = 32;     // tokens per step = one MFMA k-step
 
 typedef float floatx4_t __attribute__((ext_vector_type(4)));
-typedef float floatx2_t __attribute__((ext_vector_type(2)));
 
 // Buffer loads with a scalar offset on top of the lane's: the hardware checks the SUM of both offsets against the
 // size of the resource, so a row selected through the scalar offset is dropped (reads zeros) when it lies past the end.

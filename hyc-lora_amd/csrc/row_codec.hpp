@@ -294,6 +294,24 @@ __device__ __forceinline__ void codes8(const float (&v)[8], float s, uint32_t& l
   }
 }
 
+// The eight byte values of two words as floats.  Codes below 16 (1-, 2- and 4-bit) go two per instruction: a byte
+// below 17 read as an FP8 number (E4M3, bias 7) is that integer times 2^-9 (the exponent fields 0 and 1 share one
+// step), and the scaled packed conversion multiplies by a power of two on its way (it takes the exponent of its scale
+// operand), so with 2^9 the two bytes of a half-word come out as the floats of their integer values, exactly.
+template <int BITS>
+__device__ __forceinline__ void codes8_to_float(uint32_t a, uint32_t b, float (&c)[8]) {
+  if (BITS <= 4) {
+    const floatx2_t p0 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(a, 512.f, false);
+    const floatx2_t p1 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(a, 512.f, true);
+    const floatx2_t p2 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(b, 512.f, false);
+    const floatx2_t p3 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(b, 512.f, true);
+    c[0] = p0.x; c[1] = p0.y; c[2] = p1.x; c[3] = p1.y; c[4] = p2.x; c[5] = p2.y; c[6] = p3.x; c[7] = p3.y;
+  } else {
+    c[0] = (float)(a & 0xFFu); c[1] = (float)((a >> 8) & 0xFFu); c[2] = (float)((a >> 16) & 0xFFu); c[3] = (float)(a >> 24);
+    c[4] = (float)(b & 0xFFu); c[5] = (float)((b >> 8) & 0xFFu); c[6] = (float)((b >> 16) & 0xFFu); c[7] = (float)(b >> 24);
+  }
+}
+
 // Dequantised values of segment `seg` of a packed word, as four packed bf16 pairs:
 // x_hat = bf16((code - OFF) * s); (code - OFF) * s is exact in fp32, so one fma and one rounding.
 template <int BITS>
@@ -302,11 +320,11 @@ __device__ __forceinline__ uint4 dequant8(uint32_t lo, uint32_t hi, int seg, flo
   uint32_t a, b;
   if (BITS == 8) { a = lo ^ REP; b = hi ^ REP; }             // int8 -> biased unsigned (q + 128)
   else { a = (lo >> (seg * BITS)) & REP; b = (hi >> (seg * BITS)) & REP; }
-  // opaque from here on: the four codes of a word are then converted by v_cvt_f32_ubyte0..3, one instruction each
-  // (left to itself the compiler extracts every field from the packed word first: two instructions per code)
+  // opaque from here on: the codes of a word are then converted straight from its bytes (left to itself the
+  // compiler extracts every field from the packed word first: two instructions per code)
   asm volatile("" : "+v"(a), "+v"(b));
-  float c[8] = {(float)(a & 0xFFu), (float)((a >> 8) & 0xFFu), (float)((a >> 16) & 0xFFu), (float)(a >> 24),
-                (float)(b & 0xFFu), (float)((b >> 8) & 0xFFu), (float)((b >> 16) & 0xFFu), (float)(b >> 24)};
+  float c[8];
+  codes8_to_float<BITS>(a, b, c);
   constexpr float OFFV = (BITS == 8) ? 128.f : (float)Q<BITS>::OFF;
   if (__builtin_expect(s < 1e30f, 1)) {
     const float ns = -OFFV * s;
@@ -330,8 +348,8 @@ __device__ __forceinline__ uint4 dequant8_fast(uint32_t lo, uint32_t hi, int seg
   if (BITS == 8) { a = lo ^ REP; b = hi ^ REP; }
   else { a = (lo >> (seg * BITS)) & REP; b = (hi >> (seg * BITS)) & REP; }
   asm volatile("" : "+v"(a), "+v"(b));                       // see dequant8
-  float c[8] = {(float)(a & 0xFFu), (float)((a >> 8) & 0xFFu), (float)((a >> 16) & 0xFFu), (float)(a >> 24),
-                (float)(b & 0xFFu), (float)((b >> 8) & 0xFFu), (float)((b >> 16) & 0xFFu), (float)(b >> 24)};
+  float c[8];
+  codes8_to_float<BITS>(a, b, c);
   constexpr float OFFV = (BITS == 8) ? 128.f : (float)Q<BITS>::OFF;
   const float ns = -OFFV * s;
 #pragma unroll
