@@ -177,7 +177,7 @@ def time_steady(torch, fn, iters, seconds=0.3):
     return time_events(torch, fn, iters, 5)
 
 
-def gradw_extra(pkg, torch, c, shapes=(("full_w", 4096, 100, 30), ("lora_a_r16", 16, 300, 30))):
+def gradw_extra(pkg, torch, c, shapes=(("full_w", 4096, 100, 30), ("lora_a_r16", 16, 300, 30), ("lora_a_r64", 64, 300, 30))):
     """weight-gradient GEMM dW = dY^T . x_hat on the channel-compressed activation `c`: x_hat decoded inside the GEMM,
     the staged route (restore x_hat once, then the dense form of the same kernel) and the framework's library GEMM on
     the restored activation; every leg warmed before it is timed"""
@@ -284,7 +284,7 @@ def config4_extra(pkg, torch):
            "gated_silu_bwd": hbm(M * (6 * H + 3 * side), time_graph(torch, lambda: K.gated_act_bwd("silu", g, ca, cu, cg))),
            "silu_fwd_compress": hbm(M * (4 * H + side), time_graph(torch, lambda: K.act_fwd_compress("silu", gate, cg.plan, bits, G)))}
     del gate, up, act, prod, g, cg, cu, ca
-    out["down_proj"] = gradw_extra(pkg, torch, cp, shapes=(("full_w", 4096, 60, 20), ("lora_a_r16", 16, 300, 30)))
+    out["down_proj"] = gradw_extra(pkg, torch, cp, shapes=(("full_w", 4096, 60, 20), ("lora_a_r16", 16, 300, 30), ("lora_a_r64", 64, 300, 30)))
     return out
 
 

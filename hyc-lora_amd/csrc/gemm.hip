@@ -177,7 +177,8 @@ k_gradw(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_out, 
 
 
 // ------------------------------------------------------------------------------------------------
-// Few output rows (N_out <= 32: the LoRA-A shape, dW [r, H]): a streaming kernel without LDS tiles.
+// Few output rows (N_out <= 128: the LoRA-A shapes, dW [r, H], 32 features per workgroup): a streaming kernel without
+// LDS tiles.
 //
 // v_mfma_f32_16x16x32_bf16: per lane 8 consecutive tokens of ONE row (A, a feature of dY) or ONE column (B, a
 // channel of x_hat); lane L holds row/column L mod 16 and tokens 8*(L/16) .. +7 of the 32-token step.  A lane
@@ -637,9 +638,12 @@ static DirectPlan direct_plan(int bits, int lpg, int64_t N_out) {
 // (256 CUs x the plan's workgroups per CU).  The kernel is bound by its decode work, so a grid a little over that
 // leaves most of the chip idle during a second round (65 536 x 4096 INT4, two per CU: 560 workgroups 88 us, 490
 // workgroups 65 us).
-constexpr int64_t DIRECT_MAX_N = 32;
-static int direct_splits(int64_t M, int64_t y_tiles, int per_cu) {
-  int64_t s = (int64_t)256 * per_cu / (y_tiles > 0 ? y_tiles : 1);
+// More than 32 features run as blockIdx.x tiles of 32 that decode the packed words again: up to four such tiles
+// that still beats staging the tile in LDS for a product this thin.
+constexpr int64_t DIRECT_MAX_N = 128;
+static int64_t direct_x_tiles(int64_t N_out) { return N_out <= 32 ? 1 : (N_out + 31) / 32; }
+static int direct_splits(int64_t M, int64_t yx_tiles, int per_cu) {
+  int64_t s = (int64_t)256 * per_cu / (yx_tiles > 0 ? yx_tiles : 1);
   const int64_t max_by_tokens = (M + 8 * DK - 1) / (8 * DK);      // at least two steps per wave
   if (s > max_by_tokens) s = max_by_tokens;
   if (s < 1) s = 1;
@@ -656,7 +660,7 @@ static int direct_splits_max(int64_t M, int64_t N_out, int64_t H) {
   int best = 1;
   for (int bits = 1; bits <= 8; bits *= 2)
     for (int lpg = 4; lpg <= 16; lpg *= 2) {
-      const int sp = direct_splits(M, direct_y_tiles(H, bits, lpg, 0, N_out), direct_plan(bits, lpg, N_out).per_cu);
+      const int sp = direct_splits(M, direct_y_tiles(H, bits, lpg, 0, N_out) * direct_x_tiles(N_out), direct_plan(bits, lpg, N_out).per_cu);
       if (sp > best) best = sp;
     }
   return best;
@@ -1355,7 +1359,8 @@ int hyc_gradw_gemm(const void* dy, int64_t ldy, const void* stored, const void* 
     const DirectPlan pl = direct_plan(d->bits, lpg, N_out);
     const int c_tiles = (g.cps + pl.lc - 1) / pl.lc, o_tiles = (d->k + 15) / 16;
     const int y_tiles = (g.nseg / pl.spt) * c_tiles + o_tiles;
-    const int splits = M > 0 ? direct_splits(M, y_tiles, pl.per_cu) : 1;
+    const int x_tiles = (int)direct_x_tiles(N_out);
+    const int splits = M > 0 ? direct_splits(M, (int64_t)y_tiles * x_tiles, pl.per_cu) : 1;
     if (splits > 1 && !workspace) return fail(HYC_EFAULT, "hyc_gradw_gemm: workspace of hyc_gradw_workspace_bytes() bytes required");
     if (splits > 1 && !aligned16(workspace)) return fail(HYC_EINVAL, "hyc_gradw_gemm: workspace must be 16-byte aligned");
     int64_t tps = (M + splits - 1) / splits;
@@ -1363,7 +1368,7 @@ int hyc_gradw_gemm(const void* dy, int64_t ldy, const void* stored, const void* 
     if (tps < DK) tps = DK;
     float* partial = splits > 1 ? static_cast<float*>(workspace) : nullptr;
     const int nt = N_out <= 16 ? 1 : 2;
-    const dim3 grid(1, (unsigned)y_tiles, (unsigned)splits);
+    const dim3 grid((unsigned)x_tiles, (unsigned)y_tiles, (unsigned)splits);
     const int of32 = out_dtype == HYC_DTYPE_F32;
     DirectArgs da = {static_cast<const uint16_t*>(dy), ldy, M, N_out, H, static_cast<const uint8_t*>(stored),
                      static_cast<const uint16_t*>(vals), static_cast<const uint16_t*>(scales), ca, g.cps, c_tiles, tps,

@@ -39,7 +39,10 @@ GEMM_CASES = [(4, 128, 200, 512, 16, 5), (2, 64, 300, 2048, 512, 20), (1, 64, 20
               (2, 128, 333, 2048, 16, 20), (2, 128, 257, 2048, 32, 20), (2, 256, 190, 1024, 24, 10), (1, 128, 200, 2048, 16, 20),
               (1, 64, 130, 1024, 8, 10), (2, 64, 77, 11008, 16, 110), (2, 64, 2100, 1024, 32, 10), (2, 64, 31, 512, 16, 0),
               # 256-feature tiles: fewer tokens than the stages in flight, and a tile grid small enough for token splits
-              (2, 64, 40, 1024, 256, 10), (4, 128, 8200, 1024, 256, 10), (8, 128, 8192, 512, 264, 5)]
+              (2, 64, 40, 1024, 256, 10), (4, 128, 8200, 1024, 256, 10), (8, 128, 8192, 512, 264, 5),
+              # 33 to 128 output rows: the few-row kernel in tiles of 32 features (the last one partial)
+              (4, 128, 300, 2048, 64, 20), (8, 128, 130, 1024, 96, 10), (4, 128, 4100, 1024, 128, 10), (2, 128, 520, 2048, 72, 20),
+              (2, 64, 333, 1024, 64, 10), (1, 128, 200, 2048, 104, 20)]
 
 
 @pytest.mark.parametrize("bits,group,M,H,N,k", GEMM_CASES)
