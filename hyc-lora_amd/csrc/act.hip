@@ -4,6 +4,7 @@
 //   Hadamard  dx1 = g*x2, dx2 = x1*g                          operators/efficient_hadamard.py:62-66
 // Every intermediate is rounded to bf16 exactly where the reference's torch expression rounds it (each
 // torch op on bf16 tensors computes in fp32 and rounds once; Python scalars enter as fp32).
+#include <stdlib.h>
 #include "abi_util.hpp"
 #include "row_kernels.hpp"
 
@@ -126,6 +127,17 @@ static_assert(LUT_N <= LUT_NEG, "the sign bit is or-ed into the index");
 // wants rows x threads of a workgroup above a threshold: measured on 4096-row inputs, 512 pays for the activation
 // backward (H = 4096: SiLU 23.8 -> 21.7 us, GELU 40.6 -> 32.9) but not for the forward and gated kernels, whose direct
 // evaluation is cheaper next to their other work (they start at 1024, i.e. at 8192 rows of 4096 channels).
+// Workgroups of the row kernels whose loop takes one row per iteration: `cap` resident ones, or one per `rows_each`
+// rows when that is more.  The kernels without a derivative table (nothing to amortise per workgroup) run faster on
+// short loops that the dispatcher balances: measured on 4096 x 11008 / 16 384 x 11008, INT4: activation forward + save
+// 44.1 -> 39.3 / 179 -> 161 us at four rows each, product forward + two saves 60.0 -> 54.7 / 291 -> 232 us at two,
+// product backward 245 -> 226 us at four (the table kernels lose: gated backward 65 -> 84 us at two rows each).
+static int row_loop_grid(int64_t M, int64_t cap, int rows_each) {
+  int64_t g = M / rows_each;
+  if (g < cap) g = cap;
+  if (g > M) g = M;
+  return (int)g;
+}
 static inline int lut_pays(int64_t M, int grid, int threads, int64_t least) {
   const int64_t rows_per_wg = (M + grid - 1) / grid;
   return rows_per_wg * threads >= least;
@@ -857,7 +869,7 @@ int hyc_hadamard_bwd(const void* g, const void* stored1, const void* vals1, cons
       if (!aligned16(g) || !aligned16(dx1) || !aligned16(dx2) || !aligned8(stored1) || !aligned8(stored2))
         return fail(HYC_EINVAL, "hyc_hadamard_bwd: g, dx must be 16-byte aligned, stored 8-byte");
       const int64_t cap = 256 * (geo.threads >= 512 ? 3 : 8);
-      const int grid = (int)(M < cap ? M : cap);
+      const int grid = row_loop_grid(M, cap, 4);
       hipStream_t st = begin_launch(stream);
 #define HYC_HAD(B_, MT_)                                                                                           \
   hipLaunchKernelGGL((k_hadamard_bwd_fast<B_, MT_>), dim3(grid), dim3(geo.threads), 0, st,                         \
@@ -975,7 +987,7 @@ int hyc_gated_act_fwd(int32_t act, const void* gate, int64_t ld_gate, const void
   const GatedFwdSite su = {c_u, static_cast<uint8_t*>(stored_u), static_cast<uint16_t*>(vals_u), static_cast<uint16_t*>(scales_u)};
   const GatedFwdSite sg = {c_g, static_cast<uint8_t*>(stored_g), static_cast<uint16_t*>(vals_g), static_cast<uint16_t*>(scales_g)};
   const int64_t cap = 256 * (geo.threads >= 512 ? 3 : 8);
-  const int grid = (int)(M < cap ? M : cap);
+  const int grid = geo.threads >= 512 ? row_loop_grid(M, cap, 4) : (int)(M < cap ? M : cap);
   hipStream_t st = begin_launch(stream);
   const int use_lut = lut_pays(M, grid, geo.threads, LUT_PAYS_OTHER);
 #define HYC_GFWD(B_, L_, A_, MT_)                                                                                  \
@@ -1033,7 +1045,7 @@ static int ew_fwd_impl(const char* who, int32_t act, const void* x1, int64_t ld1
   const GatedFwdSite s1 = {c1, static_cast<uint8_t*>(stored1), static_cast<uint16_t*>(vals1), static_cast<uint16_t*>(scales1)};
   const GatedFwdSite s2 = {c2, static_cast<uint8_t*>(stored2), static_cast<uint16_t*>(vals2), static_cast<uint16_t*>(scales2)};
   const int64_t cap = 256 * (geo.threads >= 512 ? 3 : 8);
-  const int grid = (int)(M < cap ? M : cap);
+  const int grid = row_loop_grid(M, cap, two ? 2 : 4);
   hipStream_t st = begin_launch(stream);
   const int use_lut = !two && lut_pays(M, grid, geo.threads, LUT_PAYS_OTHER);
 #define HYC_EW(B_, L_, A_, N_, MT_)                                                                                \
