@@ -103,11 +103,15 @@ __device__ __forceinline__ void queue_read(uint32_t addr, uint32_t after, uint4 
 // rows per wave in the forward kernel's queue: three, or two where three would not leave room (long rows of 2-bit codes)
 constexpr int fwd_queue_depth(int maxt, int nseg) { return RING_D * maxt * nseg * 16 <= 128 * 1024 ? RING_D : 2; }
 
-template <int BITS, int LPGT, bool WF32, int MAXT, int RULE>
-__global__ void __launch_bounds__(MAXT)
-k_rmsnorm_fwd_fast(const uint16_t* __restrict__ x, const void* __restrict__ w, float eps, int64_t M, int64_t H,
-                   int CPS, ChanArgs ca, uint16_t* __restrict__ y, float* __restrict__ rstd_out, uint8_t* __restrict__ stored,
-                   uint16_t* __restrict__ vals, uint16_t* __restrict__ scales) {
+// LN: LayerNorm with the two-pass statistics of operators/efficient_layernorm.py:15-61 (mean = sum(x)/H, var =
+// sum((x - mean)^2)/H, y = ((x - mean)*rstd)*w + b): the row is in registers, so the second pass costs one more
+// workgroup reduction and no memory traffic.
+template <int BITS, int LPGT, bool WF32, int MAXT, int RULE, bool LN>
+__device__ __forceinline__ void
+norm_fwd_fast_rows(const uint16_t* __restrict__ x, const void* __restrict__ w, const void* __restrict__ bias, float eps,
+                   int64_t M, int64_t H, int CPS, const ChanArgs& ca, uint16_t* __restrict__ y, float* __restrict__ mean_out,
+                   float* __restrict__ rstd_out, uint8_t* __restrict__ stored, uint16_t* __restrict__ vals,
+                   uint16_t* __restrict__ scales) {
   constexpr int NSEG = Q<BITS>::NSEG;
   constexpr int D = fwd_queue_depth(MAXT, NSEG);                      // rows in the queue
   __shared__ float red[2][16];
@@ -137,17 +141,18 @@ k_rmsnorm_fwd_fast(const uint16_t* __restrict__ x, const void* __restrict__ w, f
   const uint32_t qlane = lds_offset(queue) + (uint32_t)(wave * (NSEG * 1024)) + 16u * (uint32_t)(c & 63);
 
   uint32_t km[NSEG][4];                                            // AND masks that zero the outlier channels
-  float wv[NSEG][8];
+  float wv[NSEG][8], bv[LN ? NSEG : 1][8];
   {
     uint32_t plan[NSEG];
 #pragma unroll
     for (int i = 0; i < NSEG; ++i) {
       plan[i] = 0;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) wv[i][j] = 0.f;
+      for (int j = 0; j < 8; ++j) { wv[i][j] = 0.f; if (LN) bv[LN ? i : 0][j] = 0.f; }
       if (active) {
         plan[i] = ca.plan[i * CPS + c];
         load_w8t<WF32>(w, (int64_t)i * SEG + 8 * c, wv[i]);
+        if (LN && bias) load_w8t<WF32>(bias, (int64_t)i * SEG + 8 * c, bv[LN ? i : 0]);
       }
     }
     ChunkOutliers<NSEG> co;
@@ -182,6 +187,7 @@ k_rmsnorm_fwd_fast(const uint16_t* __restrict__ x, const void* __restrict__ w, f
   {
     const BufferRsrc nothing = make_rsrc(x, 0u);
     store_b32(nothing, NOWHERE, 0u);                                 // stands for: rstd
+    if (LN) store_b32(nothing, NOWHERE + 4u, 0u);                    // mean
     store_b64(nothing, NOWHERE + 8u, 0u, 0u);                        // the packed word
 #pragma unroll
     for (int i = 0; i < NSEG; ++i) store_b16(nothing, NOWHERE + 2u * (i + 1), (uint16_t)0);   // NSEG scales
@@ -211,7 +217,7 @@ k_rmsnorm_fwd_fast(const uint16_t* __restrict__ x, const void* __restrict__ w, f
       float v[8];
       unpack8(raw[i], v);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) ss = __builtin_fmaf(v[j], v[j], ss);
+      for (int j = 0; j < 8; ++j) ss = LN ? ss + v[j] : __builtin_fmaf(v[j], v[j], ss);
       unpack8(make_uint4(raw[i].x & km[i][0], raw[i].y & km[i][1], raw[i].z & km[i][2], raw[i].w & km[i][3]), v);
       uint32_t cl, ch;
       const float s = quant_seg<BITS, LPGT, RULE>(v, LPGT, cl, ch, false);
@@ -233,6 +239,27 @@ k_rmsnorm_fwd_fast(const uint16_t* __restrict__ x, const void* __restrict__ w, f
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     float tot = red[parity][0];
     for (int i = 1; i < nw; ++i) tot += red[parity][i];
+    float mean = 0.f;
+    if (LN) {
+      // second pass over the registers; its partial sums take the other buffer (a wave can only write that one again
+      // after the next row's first barrier, which every wave reaches after it has read this row's values)
+      mean = tot * invH;
+      float var = 0.f;
+#pragma unroll
+      for (int i = 0; i < NSEG; ++i) {
+        float v[8];
+        unpack8(raw[i], v);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) { const float dlt = v[j] - mean; var = __builtin_fmaf(dlt, dlt, var); }
+      }
+      parity ^= 1;
+      var = wave_sum(active ? var : 0.f);
+      if ((c & 63) == 0) red[parity][wave] = var;
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      tot = red[parity][0];
+      for (int i = 1; i < nw; ++i) tot += red[parity][i];
+      store_b32(row_of(mean_out, row, 4u), ro, __float_as_uint(mean));
+    }
     const float rstd = 1.0f / __builtin_sqrtf(tot * invH + eps);
     store_b32(row_of(rstd_out, row, 4u), ro, __float_as_uint(rstd));
     const BufferRsrc rs_y = row_of(y, row, row_b);
@@ -241,11 +268,28 @@ k_rmsnorm_fwd_fast(const uint16_t* __restrict__ x, const void* __restrict__ w, f
       float v[8];
       unpack8(raw[i], v);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) v[j] = (v[j] * rstd) * wv[i][j];
+      for (int j = 0; j < 8; ++j) v[j] = LN ? ((v[j] - mean) * rstd) * wv[i][j] + bv[LN ? i : 0][j] : (v[j] * rstd) * wv[i][j];
       store_b128_stream(rs_y, xo + (uint32_t)i * seg_b, pack8(v));
     }
     st_b = st_b >= (D - 1) * STAGE_B ? 0 : st_b + STAGE_B;
   }
+}
+
+template <int BITS, int LPGT, bool WF32, int MAXT, int RULE>
+__global__ void __launch_bounds__(MAXT)
+k_rmsnorm_fwd_fast(const uint16_t* __restrict__ x, const void* __restrict__ w, float eps, int64_t M, int64_t H,
+                   int CPS, ChanArgs ca, uint16_t* __restrict__ y, float* __restrict__ rstd_out, uint8_t* __restrict__ stored,
+                   uint16_t* __restrict__ vals, uint16_t* __restrict__ scales) {
+  norm_fwd_fast_rows<BITS, LPGT, WF32, MAXT, RULE, false>(x, w, nullptr, eps, M, H, CPS, ca, y, nullptr, rstd_out, stored, vals, scales);
+}
+
+template <int BITS, int LPGT, bool WF32, int MAXT, int RULE>
+__global__ void __launch_bounds__(MAXT)
+k_layernorm_fwd_fast(const uint16_t* __restrict__ x, const void* __restrict__ w, const void* __restrict__ bias, float eps,
+                     int64_t M, int64_t H, int CPS, ChanArgs ca, uint16_t* __restrict__ y, float* __restrict__ mean_out,
+                     float* __restrict__ rstd_out, uint8_t* __restrict__ stored, uint16_t* __restrict__ vals,
+                     uint16_t* __restrict__ scales) {
+  norm_fwd_fast_rows<BITS, LPGT, WF32, MAXT, RULE, true>(x, w, bias, eps, M, H, CPS, ca, y, mean_out, rstd_out, stored, vals, scales);
 }
 
 // two float4 at LDS byte addresses `addr` and `addr + second`
@@ -997,21 +1041,23 @@ static int norm_fwd_impl(const void* x, const void* w, const void* bias, int32_t
   hipStream_t st = begin_launch(stream);
   const uint16_t* xp = static_cast<const uint16_t*>(x);
   // fast path: every lane owns one chunk per segment, group width known at compile time
-  if (!ln && d->mode == HYC_MODE_CHANNEL && n.iters == 1 && (lpg == 8 || lpg == 16) && d->bits != 1) {
+  if (d->mode == HYC_MODE_CHANNEL && n.iters == 1 && (lpg == 8 || lpg == 16) && d->bits != 1) {
     uint16_t* yp = static_cast<uint16_t*>(y);
     uint8_t* stp = static_cast<uint8_t*>(stored);
     uint16_t* vp = static_cast<uint16_t*>(vals);
     uint16_t* scp = static_cast<uint16_t*>(scales);
-#define HYC_FWD_FAST(B_, L_, W_, MT_)                                                                              \
+#define HYC_FWD_FAST_R(B_, L_, W_, MT_, R_)                                                                        \
   do {                                                                                                             \
     const size_t qb_ = (size_t)fwd_queue_depth(MT_, Q<B_>::NSEG) * n.T * Q<B_>::NSEG * 16;                         \
-    if (ca.absmax)                                                                                                 \
-      hipLaunchKernelGGL((k_rmsnorm_fwd_fast<B_, L_, W_, MT_, SCALE_ABSMAX>), dim3(grid), dim3(n.T), qb_, st, xp, w, eps, M, H, \
-                         g.cps, ca, yp, rstd, stp, vp, scp);                                                       \
+    if (ln)                                                                                                        \
+      hipLaunchKernelGGL((k_layernorm_fwd_fast<B_, L_, W_, MT_, R_>), dim3(grid), dim3(n.T), qb_, st, xp, w, bias, eps, M, H, \
+                         g.cps, ca, yp, mean, rstd, stp, vp, scp);                                                 \
     else                                                                                                           \
-      hipLaunchKernelGGL((k_rmsnorm_fwd_fast<B_, L_, W_, MT_, SCALE_RANGE>), dim3(grid), dim3(n.T), qb_, st, xp, w, eps, M, H, \
+      hipLaunchKernelGGL((k_rmsnorm_fwd_fast<B_, L_, W_, MT_, R_>), dim3(grid), dim3(n.T), qb_, st, xp, w, eps, M, H, \
                          g.cps, ca, yp, rstd, stp, vp, scp);                                                       \
   } while (0)
+#define HYC_FWD_FAST(B_, L_, W_, MT_)                                                                              \
+  do { if (ca.absmax) HYC_FWD_FAST_R(B_, L_, W_, MT_, SCALE_ABSMAX); else HYC_FWD_FAST_R(B_, L_, W_, MT_, SCALE_RANGE); } while (0)
 #define HYC_FWD_FAST_W(B_, L_)                                                        \
   do {                                                                                \
     if (n.T <= 256) { if (wf32) HYC_FWD_FAST(B_, L_, true, 256); else HYC_FWD_FAST(B_, L_, false, 256); }  \
@@ -1027,7 +1073,8 @@ static int norm_fwd_impl(const void* x, const void* w, const void* bias, int32_t
     }
 #undef HYC_FWD_FAST_W
 #undef HYC_FWD_FAST
-    return check_launch("hyc_rmsnorm_fwd_compress");
+#undef HYC_FWD_FAST_R
+    return check_launch(ln ? "hyc_layernorm_fwd_compress" : "hyc_rmsnorm_fwd_compress");
   }
 #define HYC_FWD_K(KERNEL_)                                                                                         \
   hipLaunchKernelGGL(KERNEL_, dim3(grid), dim3(n.T), 0, st, xp, w, bias, wf32, eps, M, H, g.cps,                   \

@@ -263,7 +263,8 @@ def test_gated_forward_equals_the_separate_calls(K, act, M, H, bits, group, k):
 @pytest.mark.parametrize("bits,group,M,H,k,wdt,with_bias", [
     (4, 64, 80, 768, 8, torch.float32, True), (4, 128, 33, 1024, 10, torch.bfloat16, True),
     (2, 64, 2100, 4096, 41, torch.float32, False), (8, 32, 9, 512, 5, torch.bfloat16, True),
-    (1, 64, 17, 1024, 0, torch.float32, True), (4, 128, 20, 11008, 110, torch.float32, True)])
+    (1, 64, 17, 1024, 0, torch.float32, True), (4, 128, 20, 11008, 110, torch.float32, True),
+    (4, 128, 9000, 768, 8, torch.float32, True), (8, 128, 5000, 1024, 10, torch.bfloat16, False)])   # many rows per workgroup
 def test_layernorm_forward_channel(K, bits, group, M, H, k, wdt, with_bias):
     """one pass = the reference's two-pass statistics and y (efficient_layernorm.py:15-61) plus hyc_compress of x"""
     gen = torch.Generator().manual_seed(bits + M + H)
