@@ -229,41 +229,22 @@ struct DirectRegs {          // what one lane loads for one step: a packed word 
   uint32_t blo[8], bhi[8], sc[SPT][8];
 };
 
-// MAINT: true = a tile of LC chunks of SPT segments, decoded from the same packed words (which are then read once
+// MAINT: true = a tile of 16 chunks of SPT segments, decoded from the same packed words (which are then read once
 //        per SPT segments); false = a tile of 16 outlier channels (bf16 values, nothing to decode)
 // NT = 16-row tiles of dY features (N_out <= 16*NT)
-// R:  0 = every lane applies its own group scale: x_hat = bf16((code - OFF) * s), LC = 16 chunks per tile.
-//     1, 2 = 1- and 2-bit codes with the scale folded into dY.  code - OFF is one of {-2, -1, 0, 1}, so
-//     x_hat = (code - OFF) * s is exact: nothing is rounded, and dW[n, h] = sum_t (dY[t, n] * s[t]) * (code[t, h] - OFF)
-//     is the same sum whenever all 16 columns of an MFMA lie in ONE scale group.  R lanes share a chunk and take
-//     every R-th byte of its packed word, so a tile is LC = 16/R chunks: group >= 128 channels: R = 1, 64 channels:
-//     R = 2.  (4-bit codes do round x_hat to bf16, which a folded scale cannot reproduce: they keep R = 0.)
-//     The A operand becomes dY * s, exactly, as two bf16 terms hi + lo (the product of two 8-bit significands has 16
-//     bits); the B operand is the integer code - OFF, which needs no arithmetic at all: bf16 has 8 significant bits,
-//     so the bit pattern of 2^BITS with the code in the top mantissa bits IS the number 2^BITS + code.  One byte
-//     permute picks the lane's byte of two tokens' words, one shift and one and-or put the code field of a segment
-//     under that pattern: 1 + 1/(2 SPT) operations per element plus 40 per segment and step for hi and lo (the fma
-//     form takes 2.9 per element, half of them conversions, which issue at a lower rate).  The surplus 2^BITS + OFF per element is removed at the end through two more MFMAs
-//     per step whose B operand is all ones (sum_t A[n, t] in every column): dW -= (2^BITS + OFF) * that sum.
-//     Products are exact and fp32-accumulated either way; the partial sums are at most 6 times larger than the
-//     result's terms, so nothing is lost to cancellation.
-template <int BITS, int NT, bool MAINT, int SPT, int R>
+// Every lane applies its own group scale: x_hat = bf16((code - OFF) * s), exactly what hyc_decompress writes.  (An
+// earlier form folded the scale of 1- and 2-bit codes into dY, where code - OFF is exact, and fed the integer codes
+// to the MFMAs as bf16 bit patterns; since the codes are converted two per instruction the plain form is as fast
+// - 2-bit codes, 64-channel groups, 65 536 x 4096: 55.0 us folded, 41.8 us plain - and it went.)
+template <int BITS, int NT, bool MAINT, int SPT>
 __device__ __forceinline__ void gradw_direct_tile(const DirectArgs& A, float* red, int hy, int64_t n0) {
-  static_assert(R == 0 || (BITS <= 2 && MAINT && (R == 1 || R == 2)), "the folded form serves 1- and 2-bit codes");
-  constexpr bool FOLD = R > 0;
-  constexpr int RR = FOLD ? R : 1;
-  constexpr int LC = 16 / RR;                                                    // chunks per tile
-  constexpr int NJ = 8 / RR;                                                     // MFMAs (16 channels each) per segment
+  constexpr int LC = 16;                                                         // chunks per tile
+  constexpr int NJ = 8;                                                          // MFMAs (16 channels each) per segment
   constexpr uint32_t CMASK = (BITS == 8) ? 0xFFu : Q<BITS>::CODE_MASK;
   constexpr uint32_t REP = CMASK * 0x01010101u;
   constexpr float OFFV = (BITS == 8) ? 128.f : (float)Q<BITS>::OFF;
   constexpr int NB = MAINT ? NJ * SPT : 1;                                       // 16-column MFMA tiles per wave
   constexpr int RP = 17;                                                         // padded pitch of the reduction buffer
-  // folded form: bf16 pattern of 2^BITS, the code field's place under it, what to take off again
-  constexpr int FSH = 7 - (BITS & 7);                                            // code -> top mantissa bits
-  constexpr uint32_t FMAGIC = ((uint32_t)(127 + BITS) << 7) * 0x00010001u;
-  constexpr uint32_t FMASK = ((CMASK << FSH) & 0x7Fu) * 0x00010001u;
-  constexpr float FCORR = (float)(1 << (BITS & 7)) + OFFV;
   const ChanArgs& ca = A.ca;
   const int CPS = A.CPS, c_tiles = A.c_tiles;
   const int64_t ldy = A.ldy, N_out = A.N_out, H = A.H;
@@ -273,8 +254,7 @@ __device__ __forceinline__ void gradw_direct_tile(const DirectArgs& A, float* re
   const int l16 = lane & 15, kq = lane >> 4;                                     // column / token quarter
   const int sgrp = MAINT ? hy / c_tiles : 0;                                     // group of SPT segments
   const int seg = sgrp * SPT;                                                    // its first segment
-  const int hsel = l16 / LC;                                                     // which of the R byte subsets (0 when R <= 1)
-  const int c = MAINT ? (hy - sgrp * c_tiles) * LC + (l16 % LC) : 0;             // chunk inside the segment
+  const int c = MAINT ? (hy - sgrp * c_tiles) * LC + l16 : 0;                    // chunk inside the segment
   const int q = MAINT ? 0 : hy * 16 + l16;                                       // outlier number
   const int shs = (BITS == 8 || SPT == Q<BITS>::NSEG) ? 0 : seg * BITS;   // a tile of all segments starts at bit 0
   const int64_t m_begin = (int64_t)blockIdx.z * A.tokens_per_split;
@@ -325,14 +305,10 @@ __device__ __forceinline__ void gradw_direct_tile(const DirectArgs& A, float* re
   }
 
   floatx4_t acc[NT][NB];
-  floatx4_t accs[FOLD ? SPT : 1][NT];                                            // folded form: sum_t A[n, t] per segment
 #pragma unroll
-  for (int a = 0; a < NT; ++a) {
+  for (int a = 0; a < NT; ++a)
 #pragma unroll
     for (int b = 0; b < NB; ++b) acc[a][b] = (floatx4_t){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int g = 0; g < (FOLD ? SPT : 1); ++g) accs[g][a] = (floatx4_t){0.f, 0.f, 0.f, 0.f};
-  }
 
   // Every load is unconditional.  Lanes past the last chunk / outlier / feature read their neighbour's data (the
   // results are dropped at the write-out).  The buffer resources of a step span exactly its valid tokens, token e of
@@ -358,83 +334,6 @@ __device__ __forceinline__ void gradw_direct_tile(const DirectArgs& A, float* re
     }
   };
   auto step = [&](DirectRegs<SPT>& Rg, uint32_t (&ar)[NT][8]) __attribute__((always_inline)) {
-    if (FOLD) {
-      uint32_t magic = FMAGIC;
-      asm volatile("" : "+v"(magic));                  // in a vector register, so that (x & mask) | magic is one v_and_or_b32
-      const bf16x8_t ones = __builtin_bit_cast(bf16x8_t, (u32x4_t){0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u});
-      // A operands of segment g: dY * s is a product of two 8-bit significands, so it is exactly hi + lo with
-      // hi = bf16(dY * s) and lo = dY * s - hi, both bf16; their row sums through the all-ones B operand
-      auto make_a = [&](int g, bf16x8_t (&ahi)[NT], bf16x8_t (&alo)[NT]) __attribute__((always_inline)) {
-        float sg[8];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) sg[e] = bf_to_f((uint16_t)Rg.sc[g][e]);
-#pragma unroll
-        for (int a = 0; a < NT; ++a) {
-          uint32_t wh[4], wl[4];
-#pragma unroll
-          for (int e = 0; e < 8; e += 2) {
-            const float p0 = __uint_as_float(ar[a][e] << 16) * sg[e], p1 = __uint_as_float(ar[a][e + 1] << 16) * sg[e + 1];
-            wh[e >> 1] = pack_bf16(p0, p1);
-            wl[e >> 1] = pack_bf16(p0 - bf_lo(wh[e >> 1]), p1 - bf_hi(wh[e >> 1]));
-          }
-          ahi[a] = __builtin_bit_cast(bf16x8_t, (u32x4_t){wh[0], wh[1], wh[2], wh[3]});
-          alo[a] = __builtin_bit_cast(bf16x8_t, (u32x4_t){wl[0], wl[1], wl[2], wl[3]});
-          accs[g][a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ahi[a], ones, accs[g][a], 0, 0, 0);
-          accs[g][a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(alo[a], ones, accs[g][a], 0, 0, 0);
-        }
-      };
-      // B operands: for byte slot jj of the lane, the raw bytes of two tokens side by side ...
-      auto make_d = [&](int jj, uint32_t (&d)[4]) __attribute__((always_inline)) {
-        const uint32_t sel = 0x0C040C00u + (uint32_t)(RR * (jj % (4 / RR)) + hsel) * 0x00010001u;
-#pragma unroll
-        for (int ep = 0; ep < 4; ++ep) {
-          const uint32_t w0 = (jj < NJ / 2) ? Rg.blo[2 * ep] : Rg.bhi[2 * ep];
-          const uint32_t w1 = (jj < NJ / 2) ? Rg.blo[2 * ep + 1] : Rg.bhi[2 * ep + 1];
-          d[ep] = __builtin_amdgcn_perm(w1, w0, sel);                            // [byte of token 2ep, 0, byte of token 2ep+1, 0]
-          if (SPT != Q<BITS>::NSEG) d[ep] >>= shs;                               // first segment of the tile to bit 0
-        }
-      };
-      // ... then the code field of segment g under the bf16 pattern, and the MFMAs of (g, jj)
-      auto mfmas = [&](int g, int jj, const uint32_t (&d)[4], const bf16x8_t (&ahi)[NT], const bf16x8_t (&alo)[NT])
-                       __attribute__((always_inline)) {
-        const int sh = FSH - g * BITS;                                           // compile-time after unrolling
-        const int shl = sh > 0 ? sh : 0, shr = sh < 0 ? -sh : 0;
-        uint32_t w[4];
-#pragma unroll
-        for (int ep = 0; ep < 4; ++ep) w[ep] = (((d[ep] << shl) >> shr) & FMASK) | magic;
-        const bf16x8_t bf = __builtin_bit_cast(bf16x8_t, (u32x4_t){w[0], w[1], w[2], w[3]});
-#pragma unroll
-        for (int a = 0; a < NT; ++a) {
-          acc[a][g * NJ + jj] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ahi[a], bf, acc[a][g * NJ + jj], 0, 0, 0);
-          acc[a][g * NJ + jj] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(alo[a], bf, acc[a][g * NJ + jj], 0, 0, 0);
-        }
-      };
-      // whichever of the two intermediate sets is smaller stays live across the other loop
-      if (SPT * NT * 8 <= NJ * 4) {
-        bf16x8_t ahi[SPT][NT], alo[SPT][NT];
-#pragma unroll
-        for (int g = 0; g < SPT; ++g) make_a(g, ahi[g], alo[g]);
-#pragma unroll
-        for (int jj = 0; jj < NJ; ++jj) {
-          uint32_t d[4];
-          make_d(jj, d);
-#pragma unroll
-          for (int g = 0; g < SPT; ++g) mfmas(g, jj, d, ahi[g], alo[g]);
-        }
-      } else {
-        uint32_t d[NJ][4];
-#pragma unroll
-        for (int jj = 0; jj < NJ; ++jj) make_d(jj, d[jj]);
-#pragma unroll
-        for (int g = 0; g < SPT; ++g) {
-          bf16x8_t ahi[NT], alo[NT];
-          make_a(g, ahi, alo);
-#pragma unroll
-          for (int jj = 0; jj < NJ; ++jj) mfmas(g, jj, d[jj], ahi, alo);
-        }
-      }
-      return;
-    }
     bf16x8_t af[NT];
 #pragma unroll
     for (int a = 0; a < NT; ++a)
@@ -522,15 +421,6 @@ __device__ __forceinline__ void gradw_direct_tile(const DirectArgs& A, float* re
       if (m0 + 3 * WS < m_end) fetch(m0 + 3 * WS, R1, a1);
     }
   }
-  if (FOLD) {                                                                    // take the 2^BITS + OFF per element off again
-#pragma unroll
-    for (int a = 0; a < NT; ++a)
-#pragma unroll
-      for (int b = 0; b < NB; ++b)
-#pragma unroll
-        for (int v = 0; v < 4; ++v) acc[a][b][v] = __builtin_fmaf(-FCORR, accs[b / NJ][a][v], acc[a][b][v]);
-  }
-
   // ---- the four waves add up in LDS: (wave 0 + wave 2) in one half of `red`, (wave 1 + wave 3) in the other, the
   // two halves are added by the write-out; layout of a half [row n][tile b][lane] with a padded pitch ----
   // lane holds column (lane mod 16) and rows 4*(lane/16) + v of each 16x16 tile
@@ -566,13 +456,12 @@ __device__ __forceinline__ void gradw_direct_tile(const DirectArgs& A, float* re
   // ---- write-out by all threads, neighbouring threads = neighbouring channels ----
   const float alpha = A.alpha, beta = A.beta;
   if (!wo_in) return;
-  // channel = (segment tg of the tile, chunk tcl of the tile, byte tb of the packed word): MFMA tile 8/R*tg + tb/R,
-  // lane (tb mod R) * LC + tcl
+  // channel = (segment tg of the tile, chunk tcl of the tile, byte tb of the packed word): MFMA tile 8*tg + tb, lane tcl
   if (wo_vec) {                                        // partial sums of a main tile: 16-byte stores, 4 channels per thread
     constexpr int NSTEP4 = 256 / (COLS / 4);
     int ro[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) ro[i] = (wo_tg * NJ + (wo_tb + i) / RR) * RP + ((wo_tb + i) % RR) * LC + wo_tcl;
+    for (int i = 0; i < 4; ++i) ro[i] = (wo_tg * NJ + wo_tb + i) * RP + wo_tcl;
     const uint32_t m4 = (wo_pword >> wo_tb) & 0xFu;    // outlier channels belong to the outlier tiles
     for (int nl = tid / (COLS / 4); nl < 16 * NT && n0 + nl < N_out; nl += NSTEP4) {
       float v[4];
@@ -589,7 +478,7 @@ __device__ __forceinline__ void gradw_direct_tile(const DirectArgs& A, float* re
     return;
   }
   if (MAINT && ((wo_pword >> wo_tb) & 1u)) return;
-  const int rb = MAINT ? wo_tg * NJ + wo_tb / RR : 0, rl = MAINT ? (wo_tb % RR) * LC + wo_tcl : tid % COLS;
+  const int rb = MAINT ? wo_tg * NJ + wo_tb : 0, rl = MAINT ? wo_tcl : tid % COLS;
   for (int nl = tid / COLS; nl < 16 * NT && n0 + nl < N_out; nl += 256 / COLS) {
     const float val = red[(nl * NB + rb) * RP + rl] + red[HALF + (nl * NB + rb) * RP + rl];
     const int64_t n = n0 + nl;
@@ -607,30 +496,26 @@ __device__ __forceinline__ void gradw_direct_tile(const DirectArgs& A, float* re
 
 // one launch: blockIdx.y < (NSEG / SPT) * c_tiles are the tiles of quantised channels, the rest the outlier tiles
 // (two waves per SIMD at least: with 256 registers or fewer the accumulators stay in ordinary vector registers)
-template <int BITS, int NT, int SPT, int R>
+template <int BITS, int NT, int SPT>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) k_gradw_direct(DirectArgs A) {
   static_assert(Q<BITS>::NSEG % SPT == 0, "segments per tile must divide the segments of a packed word");
-  constexpr int NB = (R > 0 ? 8 / R : 8) * SPT;
+  constexpr int NB = 8 * SPT;
   __shared__ float red[2 * 16 * NT * NB * 17];
   const int main_tiles = (Q<BITS>::NSEG / SPT) * A.c_tiles;
   const int64_t n0 = (int64_t)blockIdx.x * (16 * NT);                            // first feature of the workgroup
-  if ((int)blockIdx.y < main_tiles) gradw_direct_tile<BITS, NT, true, SPT, R>(A, red, (int)blockIdx.y, n0);
-  else gradw_direct_tile<BITS, NT, false, 1, 0>(A, red, (int)blockIdx.y - main_tiles, n0);
+  if ((int)blockIdx.y < main_tiles) gradw_direct_tile<BITS, NT, true, SPT>(A, red, (int)blockIdx.y, n0);
+  else gradw_direct_tile<BITS, NT, false, 1>(A, red, (int)blockIdx.y - main_tiles, n0);
 }
 
-// How a shape is laid on the kernel: R (see above) from the group width, SPT from the registers the accumulators of
-// NT x SPT x 8/R tiles leave, LC chunks per tile, and how many workgroups of the variant a CU holds at once (three
-// where it needs at most 168 registers per lane, else two).
-struct DirectPlan { int r, spt, lc, per_cu; };
-static DirectPlan direct_plan(int bits, int lpg, int64_t N_out) {
+// How a shape is laid on the kernel: SPT segments of a packed word per tile (two with one feature tile, so that every
+// word is loaded once; the accumulators of two feature tiles leave room for one), and how many workgroups of the
+// variant a CU holds at once (three where it needs at most 168 registers per lane, else two).
+struct DirectPlan { int spt, per_cu; };
+static DirectPlan direct_plan(int bits, int64_t N_out) {
   DirectPlan p;
   const int nseg = 8 / bits, nt = N_out <= 16 ? 1 : 2;
-  p.r = (bits > 2 || lpg < 8) ? 0 : (lpg >= 16 ? 1 : (nt == 1 ? 2 : 0));
-  // 4-bit codes, one feature tile: both segments of a packed word in one tile, so every word is loaded once
-  p.spt = p.r == 0 ? (bits == 4 && nt == 1 ? 2 : 1) : (nt == 1 ? 2 : 1);
-  if (p.spt > nseg) p.spt = nseg;
-  p.lc = p.r == 2 ? 8 : 16;
-  p.per_cu = (nt == 1 && p.r != 1 && !(p.r == 0 && p.spt == 2)) ? 3 : 2;
+  p.spt = nt == 1 && nseg >= 2 ? 2 : 1;
+  p.per_cu = (nt == 1 && p.spt == 1) ? 3 : 2;
   return p;
 }
 
@@ -650,19 +535,18 @@ static int direct_splits(int64_t M, int64_t yx_tiles, int per_cu) {
   if (s > 64) s = 64;
   return (int)s;
 }
-static int64_t direct_y_tiles(int64_t H, int bits, int lpg, int k, int64_t N_out) {
-  const DirectPlan p = direct_plan(bits, lpg, N_out);
+static int64_t direct_y_tiles(int64_t H, int bits, int k, int64_t N_out) {
+  const DirectPlan p = direct_plan(bits, N_out);
   const int64_t cps = (H * bits + 63) / 64;
-  return (8 / bits / p.spt) * ((cps + p.lc - 1) / p.lc) + (k + 15) / 16;
+  return (8 / bits / p.spt) * ((cps + 15) / 16) + (k + 15) / 16;
 }
-// the most splits any code width and group width can ask for (the workspace query does not know them)
+// the most splits any code width can ask for (the workspace query does not know it)
 static int direct_splits_max(int64_t M, int64_t N_out, int64_t H) {
   int best = 1;
-  for (int bits = 1; bits <= 8; bits *= 2)
-    for (int lpg = 4; lpg <= 16; lpg *= 2) {
-      const int sp = direct_splits(M, direct_y_tiles(H, bits, lpg, 0, N_out) * direct_x_tiles(N_out), direct_plan(bits, lpg, N_out).per_cu);
-      if (sp > best) best = sp;
-    }
+  for (int bits = 1; bits <= 8; bits *= 2) {
+    const int sp = direct_splits(M, direct_y_tiles(H, bits, 0, N_out) * direct_x_tiles(N_out), direct_plan(bits, N_out).per_cu);
+    if (sp > best) best = sp;
+  }
   return best;
 }
 
@@ -1356,8 +1240,8 @@ int hyc_gradw_gemm(const void* dy, int64_t ldy, const void* stored, const void* 
   if (chan && N_out <= DIRECT_MAX_N) {
     if (M > 0 && (!dy || !stored || !scales || (d->k > 0 && !vals))) return fail(HYC_EFAULT, "hyc_gradw_gemm: null buffer");
     if (M > 0 && !aligned8(stored)) return fail(HYC_EINVAL, "hyc_gradw_gemm: stored must be 8-byte aligned");
-    const DirectPlan pl = direct_plan(d->bits, lpg, N_out);
-    const int c_tiles = (g.cps + pl.lc - 1) / pl.lc, o_tiles = (d->k + 15) / 16;
+    const DirectPlan pl = direct_plan(d->bits, N_out);
+    const int c_tiles = (g.cps + 15) / 16, o_tiles = (d->k + 15) / 16;
     const int y_tiles = (g.nseg / pl.spt) * c_tiles + o_tiles;
     const int x_tiles = (int)direct_x_tiles(N_out);
     const int splits = M > 0 ? direct_splits(M, (int64_t)y_tiles * x_tiles, pl.per_cu) : 1;
@@ -1373,19 +1257,13 @@ int hyc_gradw_gemm(const void* dy, int64_t ldy, const void* stored, const void* 
     DirectArgs da = {static_cast<const uint16_t*>(dy), ldy, M, N_out, H, static_cast<const uint8_t*>(stored),
                      static_cast<const uint16_t*>(vals), static_cast<const uint16_t*>(scales), ca, g.cps, c_tiles, tps,
                      alpha, beta, out, of32, partial};
-#define HYC_DIRECT_K(B_, N_, S_, R_) hipLaunchKernelGGL((k_gradw_direct<B_, N_, S_, R_>), grid, dim3(256), 0, st, da)
-#define HYC_DIRECT(B_)                                                                                 \
-  do {                                                                                                 \
-    constexpr int NS = 8 / B_;                         /* the SPT of direct_plan() */                  \
-    if (pl.r == 0) { if (nt == 1) HYC_DIRECT_K(B_, 1, 1, 0); else HYC_DIRECT_K(B_, 2, 1, 0); }         \
-    else if (pl.r == 1) { if (nt == 1) HYC_DIRECT_K(B_, 1, (NS < 2 ? NS : 2), 1); else HYC_DIRECT_K(B_, 2, 1, 1); } \
-    else HYC_DIRECT_K(B_, 1, (NS < 2 ? NS : 2), 2);     /* direct_plan() keeps R = 2 to N_out <= 16 */ \
-  } while (0)
+#define HYC_DIRECT_K(B_, N_, S_) hipLaunchKernelGGL((k_gradw_direct<B_, N_, S_>), grid, dim3(256), 0, st, da)
+#define HYC_DIRECT(B_) do { if (nt == 1) HYC_DIRECT_K(B_, 1, (B_ < 8 ? 2 : 1)); else HYC_DIRECT_K(B_, 2, 1); } while (0)   /* direct_plan() */
     switch (d->bits) {
       case 1: HYC_DIRECT(1); break;
       case 2: HYC_DIRECT(2); break;
-      case 4: if (nt == 1) HYC_DIRECT_K(4, 1, 2, 0); else HYC_DIRECT_K(4, 2, 1, 0); break;
-      default: if (nt == 1) HYC_DIRECT_K(8, 1, 1, 0); else HYC_DIRECT_K(8, 2, 1, 0); break;
+      case 4: HYC_DIRECT(4); break;
+      default: HYC_DIRECT(8); break;
     }
 #undef HYC_DIRECT_K
 #undef HYC_DIRECT

@@ -34,8 +34,8 @@ def make_x(seed, M, H, n_hot, gain):
 GEMM_CASES = [(4, 128, 200, 512, 16, 5), (2, 64, 300, 2048, 512, 20), (1, 64, 200, 2048, 256, 20), (8, 128, 150, 1024, 264, 30), (4, 32, 100, 512, 256, 300), (4, 128, 4096, 4096, 16, 41), (2, 64, 1000, 4096, 16, 41),
               (4, 128, 333, 1024, 256, 10), (8, 128, 130, 512, 136, 5), (1, 64, 96, 1024, 40, 10),
               (2, 64, 257, 2048, 128, 20), (4, 128, 64, 11008, 32, 110), (4, 128, 520, 1024, 4096, 10),
-              # few output rows with the scale folded into dY: group 128 / 256 (16 chunks per tile), group 64 (8 chunks,
-              # two lanes per chunk), one and two 16-row tiles of dY, ragged token counts, a partial last tile
+              # few output rows, 1- and 2-bit codes (two segments of a packed word per tile): groups of 64 / 128 / 256
+              # channels, one and two 16-row tiles of dY, ragged token counts, a partial last tile
               (2, 128, 333, 2048, 16, 20), (2, 128, 257, 2048, 32, 20), (2, 256, 190, 1024, 24, 10), (1, 128, 200, 2048, 16, 20),
               (1, 64, 130, 1024, 8, 10), (2, 64, 77, 11008, 16, 110), (2, 64, 2100, 1024, 32, 10), (2, 64, 31, 512, 16, 0),
               # 256-feature tiles: fewer tokens than the stages in flight, and a tile grid small enough for token splits
@@ -60,7 +60,6 @@ def test_gradw_channel(K, bits, group, M, H, N, k):
     assert torch.allclose(got16.float(), want, rtol=1e-2, atol=1e-3)
     if H % 128 == 0:
         dense = K.gradw_gemm(dy.cuda(), xh, out_dtype=torch.float32).cpu()
-        # (also where the few-row kernel folds the group scale of 1- and 2-bit codes into dY: that form is exact)
         assert torch.allclose(dense, got32, rtol=1e-5, atol=1e-5 * float(want.abs().max()))
         # the staged route (restore once, then the same kernel on the dense operand) is what wide outputs default to
         assert torch.equal(K.gradw_gemm(dy.cuda(), c, out_dtype=torch.float32, staged=True).cpu(), dense)
