@@ -355,7 +355,8 @@ static inline int row_grid(int64_t M, int threads) {
 
 // Long inputs: one workgroup per two rows.  The row loops take one row per iteration with the next one requested
 // ahead; short loops that the dispatcher balances beat both the default grid and a grid of exactly the resident
-// workgroups (65 536 x 4096 INT4: compress 141 -> 121 us, decompress 102 -> 96 us; 16 384 x 11008: 93 -> 83, 71 -> 66).
+// workgroups (65 536 x 4096 INT4: compress 141 -> 121 us, decompress 102 -> 96 us; 16 384 x 11008: 93 -> 83, 71 -> 66;
+// threshold scheme, 16 384 x 4096: 36.5 -> 30.7 and 47.0 -> 38.7 us).
 static int long_input_grid(int64_t M, int dflt) {
   const int64_t g = M / 2;
   return g > dflt ? (int)g : dflt;
@@ -440,7 +441,7 @@ int hyc_compress_rows(const void* x, int64_t ldx, int64_t M, int64_t H, const hy
     if (M == 0) return HYC_OK;
     if (!x || !stored) return fail(HYC_EFAULT, "hyc_compress: null buffer");
     if (!aligned16(x) || !aligned8(stored)) return fail(HYC_EINVAL, "hyc_compress: x must be 16-byte and stored 8-byte aligned");
-    const int grid = row_grid(M, g.threads);
+    const int grid = long_input_grid(M, row_grid(M, g.threads));
     HYC_DISPATCH_BITS(d->bits,
       if (perchan) hipLaunchKernelGGL((k_compress_thr<B, true>), dim3(grid), dim3(g.threads), 0, st,
                                       static_cast<const uint16_t*>(x), M, H, g.cps, g.iters, a,
@@ -501,7 +502,7 @@ int hyc_decompress(const void* stored, const void* vals, const void* scales, int
     if (!stored || !xhat) return fail(HYC_EFAULT, "hyc_decompress: null buffer");
     if (!a.row_ptr) return fail(HYC_EFAULT, "hyc_decompress: threshold mode needs csr_row_ptr");
     if (!aligned16(xhat) || !aligned8(stored)) return fail(HYC_EINVAL, "hyc_decompress: xhat must be 16-byte and stored 8-byte aligned");
-    const int grid = row_grid(M, g.threads);
+    const int grid = long_input_grid(M, row_grid(M, g.threads));
     const size_t lds = (size_t)H * 2;
     HYC_DISPATCH_BITS(d->bits,
       if (perchan) hipLaunchKernelGGL((k_decompress_thr<B, true>), dim3(grid), dim3(g.threads), lds, st,
