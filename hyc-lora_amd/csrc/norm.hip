@@ -306,18 +306,18 @@ __device__ __forceinline__ void lds_read_8f(uint32_t addr, uint32_t second, floa
 // LDS at the end, in slot order, so a workgroup writes one fp32 partial row.
 // DENSE: `stored` is the restored activation itself (bf16 [M, H]; what a threshold-scheme caller hands over after
 // hyc_decompress), read with the chunk mapping of 4-bit codes; nothing is decoded.
-template <int BITS, bool WF32, bool QUIRK, int MAXT, bool DENSE = false>
-__global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(4, 8)))
-k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ stored, const uint16_t* __restrict__ vals,
+// D: rows per wave in the queue (three; two for rows so long that the weight row leaves no room for a third stage)
+template <int BITS, bool WF32, bool QUIRK, int MAXT, bool DENSE, int D>
+__device__ __forceinline__ void
+norm_bwd_fast_rows(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ stored, const uint16_t* __restrict__ vals,
                    const uint16_t* __restrict__ scales, const void* __restrict__ w, const float* __restrict__ rstd,
-                   const float* __restrict__ mean, int64_t M, int64_t H, int T, int CPS, int slots, int steps, ChanArgs ca,
+                   const float* __restrict__ mean, int64_t M, int64_t H, int T, int CPS, int slots, int steps, const ChanArgs& ca,
                    uint16_t* __restrict__ dx, float* __restrict__ dw_partials) {
   // A thread decodes at most two segments of its packed word: with four segments (2-bit codes) two threads share
   // a word, which keeps the per-thread state (and so the occupancy) the same for every bit width.
   constexpr int NSEG = Q<BITS>::NSEG > 2 ? 2 : Q<BITS>::NSEG;         // segments per thread
   constexpr int PARTS = Q<BITS>::NSEG / NSEG;                         // threads per packed word
   constexpr int STAGE_B = MAXT * NSEG * 16;                           // bytes of one queue stage of the workgroup
-  constexpr int D = RING_D;                                           // rows in the queue
   __shared__ float red[2][4][2][16];                                  // [parity][slot][value][wave]
   __shared__ __align__(16) uint4 queue[D * MAXT * NSEG];              // [stage][wave][segment][lane]: dy chunks on their way in
   // dynamic LDS: the weight row as fp32 [segment][half chunk][CPS] float4 (read again for every row: sixteen
@@ -421,7 +421,7 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
   }
   __builtin_amdgcn_sched_barrier(0);
   request_dy(row, 0);
-  request_dy(row + stride, STAGE_B);
+  if (D > 2) request_dy(row + stride, STAGE_B);
   __builtin_amdgcn_sched_barrier(0);
   request_codes(row);
   __builtin_amdgcn_sched_barrier(0);
@@ -446,7 +446,7 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
   // previous row's stores; entering the loop must look the same, or the waits at the top of the loop would be sized
   // for the first row and drain the queue on every row.  So: a request for a row past the end (zeros into the stage
   // that the first iteration requests next) and as many stores to nowhere (dropped before they reach memory).
-  request_dy(M, (D - 1) * STAGE_B);
+  if (D > 2) request_dy(M, (D - 1) * STAGE_B);
 #pragma unroll
   for (int i = 0; i < NSEG; ++i)   // (distinct offsets: identical stores would be folded into one)
     store_b128_stream(make_rsrc(dx, 0u), NOWHERE + 16u * i, make_uint4(0, 0, 0, 0));
@@ -500,10 +500,16 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
     // The row is decoded: its registers take the next row's codes, scales and outliers now, and the row after that
     // goes into the queue stage that was read two rows ago.  Order matters, see above.
     __builtin_amdgcn_sched_barrier(0);
+    if (D == 2) {
+      // a queue of two: the next row's entry takes the stage that was just read, and it must be OLDER than the next
+      // row's registers, whose use vouches for it
+      request_dy(row + stride, st_b >= STAGE_B ? st_b - STAGE_B : st_b + STAGE_B);
+      __builtin_amdgcn_sched_barrier(0);
+    }
     request_codes(row + stride);
     request_outliers(row + stride);
     __builtin_amdgcn_sched_barrier(0);
-    request_dy(row + (D - 1) * stride, st_b >= STAGE_B ? st_b - STAGE_B : st_b + (D - 1) * STAGE_B);
+    if (D > 2) request_dy(row + (D - 1) * stride, st_b >= STAGE_B ? st_b - STAGE_B : st_b + (D - 1) * STAGE_B);
     __builtin_amdgcn_sched_barrier(0);
     // two sums per slot, one barrier
     p1 = wave_sum(p1);
@@ -561,6 +567,26 @@ k_rmsnorm_bwd_fast(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ 
     }
   }
 }
+
+#define HYC_NORM_BWD_FAST_PARAMS                                                                                      \
+  const uint16_t* __restrict__ dy, const uint8_t* __restrict__ stored, const uint16_t* __restrict__ vals,              \
+  const uint16_t* __restrict__ scales, const void* __restrict__ w, const float* __restrict__ rstd,                     \
+  const float* __restrict__ mean, int64_t M, int64_t H, int T, int CPS, int slots, int steps, ChanArgs ca,             \
+  uint16_t* __restrict__ dx, float* __restrict__ dw_partials
+template <int BITS, bool WF32, bool QUIRK, int MAXT, bool DENSE = false>
+__global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(4, 8)))
+k_rmsnorm_bwd_fast(HYC_NORM_BWD_FAST_PARAMS) {
+  norm_bwd_fast_rows<BITS, WF32, QUIRK, MAXT, DENSE, RING_D>(dy, stored, vals, scales, w, rstd, mean, M, H, T, CPS, slots, steps, ca,
+                                                              dx, dw_partials);
+}
+// rows of 1024 chunks per segment (16 384 channels of 4-bit codes): a queue of two stages beside the 64 KB weight row
+template <int BITS, bool WF32, bool QUIRK>
+__global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 8)))
+k_rmsnorm_bwd_fast_long(HYC_NORM_BWD_FAST_PARAMS) {
+  norm_bwd_fast_rows<BITS, WF32, QUIRK, 1024, false, 2>(dy, stored, vals, scales, w, rstd, mean, M, H, T, CPS, slots, steps, ca,
+                                                        dx, dw_partials);
+}
+#undef HYC_NORM_BWD_FAST_PARAMS
 
 // ------------------------------------------------------------------------------------------------
 // forward: y, rstd, and x compressed.  MODE 0 = channel, 1 = threshold.  One workgroup = one row at a time.
@@ -927,6 +953,7 @@ struct BwdShape {
   int fast_slots;      // fast path: row slots per workgroup and workgroups (= partial rows)
   int fast_T;          //   threads per row slot (two threads share a packed word of 2-bit codes)
   bool fast_ok;
+  bool fast_long;      //   rows so long that the queue holds two stages, not three
   int64_t fast_P;
 };
 static inline BwdShape bwd_shape(int64_t M, int bits, int cps, const NormGeom& n) {
@@ -934,6 +961,7 @@ static inline BwdShape bwd_shape(int64_t M, int bits, int cps, const NormGeom& n
   const int parts = bits == 2 ? 2 : 1;
   b.fast_T = ((parts * cps + 63) / 64) * 64;
   b.fast_ok = n.iters == 1 && bits != 1 && b.fast_T <= 1024;
+  b.fast_long = false;
   if (b.fast_ok) {
     // LDS of the fast kernel: the dy queue and the row sums (static, sized by the kernel's thread bound) and the
     // weight row (dynamic); 160 KB per workgroup on gfx950
@@ -943,7 +971,9 @@ static inline BwdShape bwd_shape(int64_t M, int bits, int cps, const NormGeom& n
     if (fs0 * b.fast_T > BWD_FAST_THREADS_MAX) b.fast_ok = false;
     const int64_t H = (int64_t)cps * 64 / bits;
     const int64_t lds = RING_D * maxt * nseg * 16 + 1024 + H * 4;
-    b.fast_ok = b.fast_ok && lds <= 160 * 1024;
+    // (a queue of two stages where three do not fit: one row slot of 1024 threads)
+    b.fast_long = b.fast_ok && lds > 160 * 1024 && maxt == 1024 && 2 * maxt * nseg * 16 + 1024 + H * 4 <= 160 * 1024;
+    b.fast_ok = b.fast_ok && (lds <= 160 * 1024 || b.fast_long);
   }
   b.slots = n.T <= 256 ? BWD_SLOTS_SMALL : 1;
   b.threads = b.slots * n.T;
@@ -1007,7 +1037,7 @@ int64_t hyc_rmsnorm_bwd_partial_rows(int64_t M, int64_t H, const hyc_desc* d) {
   NormGeom n;
   if (row_geom(H, d->bits, &g) || norm_geom(g.cps, &n)) return 0;
   const BwdShape b = bwd_shape(M, d->bits, g.cps, n);
-  return ((d->mode == HYC_MODE_CHANNEL || (d->mode == HYC_MODE_DENSE && d->bits == 4)) && b.fast_ok) ? b.fast_P : b.P;
+  return ((d->mode == HYC_MODE_CHANNEL && b.fast_ok) || (d->mode == HYC_MODE_DENSE && d->bits == 4 && b.fast_ok && !b.fast_long)) ? b.fast_P : b.P;
 }
 
 static int norm_fwd_impl(const void* x, const void* w, const void* bias, int32_t w_dtype, float eps, int64_t M, int64_t H,
@@ -1144,7 +1174,7 @@ static int norm_bwd_impl(const void* dy, const void* stored, const void* vals, c
   const bool wf32 = w_dtype == HYC_DTYPE_F32;
   const BwdShape b = bwd_shape(M, d->bits, g.cps, n);
   // the dense source takes the fast kernel through the chunk mapping of 4-bit codes (two half rows per thread)
-  const bool dense_fast = d->mode == HYC_MODE_DENSE && d->bits == 4 && b.fast_ok;
+  const bool dense_fast = d->mode == HYC_MODE_DENSE && d->bits == 4 && b.fast_ok && !b.fast_long;
   const bool fast = (d->mode == HYC_MODE_CHANNEL && b.fast_ok) || dense_fast;
   const int64_t used_P = fast ? b.fast_P : b.P;
   if (M > 0) {
@@ -1196,6 +1226,21 @@ static int norm_bwd_impl(const void* dy, const void* stored, const void* vals, c
           default: HYC_BWD_DENSE(true, true, BWD_FAST_THREADS_MAX); break;
         }
 #undef HYC_BWD_DENSE
+      }
+      else if (b.fast_long) {
+#define HYC_BWD_LONG(B_, W_, Q_)                                                                                   \
+  hipLaunchKernelGGL((k_rmsnorm_bwd_fast_long<B_, W_, Q_>), dim3((unsigned)b.fast_P), dim3(fthreads), flds, st, gp, \
+                     static_cast<const uint8_t*>(stored), static_cast<const uint16_t*>(vals),                     \
+                     static_cast<const uint16_t*>(scales), w, rstd, mean, M, H, b.fast_T, g.cps, b.fast_slots, fsteps, ca, \
+                     static_cast<uint16_t*>(dx), dw_partials)
+#define HYC_BWD_LONG_WQ(B_)                                                                                        \
+  do {                                                                                                             \
+    if (wf32) { if (c2_quirk) HYC_BWD_LONG(B_, true, true); else HYC_BWD_LONG(B_, true, false); }                  \
+    else { if (c2_quirk) HYC_BWD_LONG(B_, false, true); else HYC_BWD_LONG(B_, false, false); }                     \
+  } while (0)
+        if (d->bits == 2) HYC_BWD_LONG_WQ(2); else if (d->bits == 4) HYC_BWD_LONG_WQ(4); else HYC_BWD_LONG_WQ(8);
+#undef HYC_BWD_LONG_WQ
+#undef HYC_BWD_LONG
       }
       else if (d->bits == 2) HYC_BWD_FAST_WQ(2);
       else if (d->bits == 4) HYC_BWD_FAST_WQ(4);

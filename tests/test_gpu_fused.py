@@ -41,7 +41,9 @@ NORM_CASES = [(4, 128, 96, 4096, 41, torch.float32), (4, 128, 96, 4096, 41, torc
               (8, 128, 12, 11008, 110, torch.float32),
               # more rows than workgroups: every workgroup walks several rows with the next one requested ahead
               (4, 128, 2300, 4096, 41, torch.float32), (4, 64, 1100, 11008, 110, torch.bfloat16),
-              (2, 64, 2300, 4096, 41, torch.bfloat16)]
+              (2, 64, 2300, 4096, 41, torch.bfloat16),
+              # the longest rows of 4-bit codes: the backward's queue holds two stages beside the 64 KB weight row
+              (4, 128, 700, 16384, 164, torch.float32)]
 
 
 @pytest.mark.parametrize("rule", ["absmax", "range"])
