@@ -311,7 +311,7 @@ template <int BITS, bool WF32, bool QUIRK, int MAXT, bool DENSE, int D>
 __device__ __forceinline__ void
 norm_bwd_fast_rows(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ stored, const uint16_t* __restrict__ vals,
                    const uint16_t* __restrict__ scales, const void* __restrict__ w, const float* __restrict__ rstd,
-                   const float* __restrict__ mean, int64_t M, int64_t H, int T, int CPS, int slots, int steps, const ChanArgs& ca,
+                   const float* __restrict__ mean, int64_t M, int64_t H, int T, int CPS, int slots, int steps, ChanArgs ca,
                    uint16_t* __restrict__ dx, float* __restrict__ dw_partials) {
   // A thread decodes at most two segments of its packed word: with four segments (2-bit codes) two threads share
   // a word, which keeps the per-thread state (and so the occupancy) the same for every bit width.
