@@ -138,6 +138,15 @@ static int row_loop_grid(int64_t M, int64_t cap, int rows_each) {
   if (g > M) g = M;
   return (int)g;
 }
+// A row of the gated kernels that is too long for one workgroup (their per-thread state caps the workgroup at `most`
+// threads) is shared by 2 to 4 workgroups of whole waves.  Returns the number of workgroups per row, 0 if none fits.
+static int gated_row_parts(int cps, int most) {
+  if (cps <= most) return 1;
+  for (int n = 2; n <= 4; ++n)
+    if (cps % n == 0 && (cps / n) % 64 == 0 && cps / n <= most) return n;
+  return 0;
+}
+
 static inline int lut_pays(int64_t M, int grid, int threads, int64_t least) {
   const int64_t rows_per_wg = (M + grid - 1) / grid;
   return rows_per_wg * threads >= least;
@@ -410,7 +419,9 @@ k_gated_act_bwd_fast(const uint16_t* __restrict__ g, const uint8_t* __restrict__
     lut_fill<ACT>(lut);
     __syncthreads();
   }
-  const int c = threadIdx.x;
+  // (a row too long for one workgroup's registers is shared by gridDim.y workgroups of whole waves: nothing in this
+  // kernel looks beyond a scale group)
+  const int c = (int)(blockIdx.y * blockDim.x + threadIdx.x);
   if (c >= CPS) return;                                 // tail of the last wave
   const int64_t SEG = (int64_t)CPS * 8;
   const int64_t stride = gridDim.x;
@@ -526,7 +537,7 @@ k_gated_act_fwd_fast(const uint16_t* __restrict__ gate, int64_t ldg, const uint1
     lut_fill_value<ACT>(lut);
     __syncthreads();
   }
-  const int c = threadIdx.x;
+  const int c = (int)(blockIdx.y * blockDim.x + threadIdx.x);   // (gridDim.y workgroups of whole waves share a long row)
   if (c >= CPS) return;                                 // tail of the last wave; scale groups never straddle it
   const int64_t SEG = (int64_t)CPS * 8;
   const bool leader = (c & (LPGT - 1)) == 0;
@@ -918,12 +929,18 @@ int hyc_gated_act_bwd(int32_t act, const void* g, const void* stored_a, const vo
     return fail(HYC_EFAULT, "hyc_gated_act_bwd: null buffer");
   if (!aligned16(g) || !aligned16(d_gate) || !aligned16(d_up) || !aligned8(stored_a) || !aligned8(stored_u) || !aligned8(stored_g))
     return fail(HYC_EINVAL, "hyc_gated_act_bwd: g, d_gate, d_up must be 16-byte aligned, stored 8-byte");
-  const int64_t cap = 256 * (geo.threads >= 512 ? 3 : 8);
-  const int grid = (int)(M < cap ? M : cap);
+  // rows of more than 768 chunks: two workgroups of the 768-thread variant per row where the row divides into whole
+  // waves (the 1024-thread variant has 128 registers per thread and spills: 4096 x 14336, 113 us against 85)
+  const int parts0 = geo.threads > 768 ? gated_row_parts(geo.cps, 768) : 1;
+  const int parts = parts0 > 1 ? parts0 : 1;          // (no division into whole waves: the 1024-thread variant)
+  const int threads = parts > 1 ? geo.cps / parts : geo.threads;
+  const int64_t cap = 256 * (threads * parts >= 512 ? 3 : 8) / parts;
+  const int gx = (int)(M < cap ? M : cap);
+  const dim3 grid((unsigned)gx, (unsigned)(parts > 1 ? parts : 1));
   hipStream_t st = begin_launch(stream);
-  const int use_lut = lut_pays(M, grid, geo.threads, LUT_PAYS_OTHER);
+  const int use_lut = lut_pays(M, gx, threads, LUT_PAYS_OTHER);
 #define HYC_GATED(B_, A_, MT_)                                                                                     \
-  hipLaunchKernelGGL((k_gated_act_bwd_fast<B_, A_, MT_>), dim3(grid), dim3(geo.threads), 0, st,                    \
+  hipLaunchKernelGGL((k_gated_act_bwd_fast<B_, A_, MT_>), grid, dim3(threads), 0, st,                              \
                      static_cast<const uint16_t*>(g), static_cast<const uint8_t*>(stored_a),                       \
                      static_cast<const uint16_t*>(vals_a), static_cast<const uint16_t*>(scales_a), c_a,            \
                      static_cast<const uint8_t*>(stored_u), static_cast<const uint16_t*>(vals_u),                  \
@@ -932,8 +949,8 @@ int hyc_gated_act_bwd(int32_t act, const void* g, const void* stored_a, const vo
                      geo.cps, static_cast<uint16_t*>(d_gate), static_cast<uint16_t*>(d_up), use_lut)
 #define HYC_GATED_T(B_, A_)                                                       \
   do {                                                                            \
-    if (geo.threads <= 256) HYC_GATED(B_, A_, 256);                               \
-    else if (geo.threads <= 768) HYC_GATED(B_, A_, 768); /* H = 11008: 704 threads, 168 registers each */ \
+    if (threads <= 256) HYC_GATED(B_, A_, 256);                                   \
+    else if (threads <= 768) HYC_GATED(B_, A_, 768); /* H = 11008: 704 threads, 168 registers each */ \
     else HYC_GATED(B_, A_, 1024);                                                 \
   } while (0)
 #define HYC_GATED_B(A_)                                                           \
@@ -973,10 +990,12 @@ int hyc_gated_act_fwd(int32_t act, const void* gate, int64_t ld_gate, const void
   // codes), so the workgroup is capped at 768 threads (512 with 2-bit codes: 256 registers each); longer rows are
   // left to the separate calls.
   const int most = d_a->bits == 2 ? 512 : 768;
-  if (geo.iters != 1 || geo.threads > most || (d_a->bits != 2 && d_a->bits != 4 && d_a->bits != 8) || (lpg != 8 && lpg != 16))
+  const int parts = geo.iters == 1 ? (geo.threads > most ? gated_row_parts(geo.cps, most) : 1) : 0;
+  if (parts == 0 || (d_a->bits != 2 && d_a->bits != 4 && d_a->bits != 8) || (lpg != 8 && lpg != 16))
     return fail(HYC_ENOTSUP, "hyc_gated_act_fwd: needs 2-, 4- or 8-bit codes, groups of 64 or 128 channels and rows of at "
-                             "most 768 chunks per segment (512 with 2-bit codes; use the activation, hyc_compress and a "
-                             "product otherwise)");
+                             "most 768 chunks per segment (512 with 2-bit codes), or up to 1024 that divide into 2 to 4 "
+                             "such parts of whole waves (use the activation, hyc_compress and a product otherwise)");
+  const int threads = parts > 1 ? geo.cps / parts : geo.threads;
   if (M == 0) return HYC_OK;
   if (!gate || !up || !h || !stored_a || !stored_u || !stored_g || !scales_a || !scales_u || !scales_g ||
       (d_a->k > 0 && !vals_a) || (d_u->k > 0 && !vals_u) || (d_g->k > 0 && !vals_g))
@@ -986,18 +1005,19 @@ int hyc_gated_act_fwd(int32_t act, const void* gate, int64_t ld_gate, const void
   const GatedFwdSite sa = {c_a, static_cast<uint8_t*>(stored_a), static_cast<uint16_t*>(vals_a), static_cast<uint16_t*>(scales_a)};
   const GatedFwdSite su = {c_u, static_cast<uint8_t*>(stored_u), static_cast<uint16_t*>(vals_u), static_cast<uint16_t*>(scales_u)};
   const GatedFwdSite sg = {c_g, static_cast<uint8_t*>(stored_g), static_cast<uint16_t*>(vals_g), static_cast<uint16_t*>(scales_g)};
-  const int64_t cap = 256 * (geo.threads >= 512 ? 3 : 8);
-  const int grid = geo.threads >= 512 ? row_loop_grid(M, cap, 4) : (int)(M < cap ? M : cap);
+  const int64_t cap = 256 * (threads * parts >= 512 ? 3 : 8) / parts;
+  const int gx = threads * parts >= 512 ? row_loop_grid(M, cap, 4) : (int)(M < cap ? M : cap);
+  const dim3 grid((unsigned)gx, (unsigned)parts);
   hipStream_t st = begin_launch(stream);
-  const int use_lut = lut_pays(M, grid, geo.threads, LUT_PAYS_OTHER);
+  const int use_lut = lut_pays(M, gx, threads, LUT_PAYS_OTHER);
 #define HYC_GFWD(B_, L_, A_, MT_)                                                                                  \
-  hipLaunchKernelGGL((k_gated_act_fwd_fast<B_, L_, A_, MT_>), dim3(grid), dim3(geo.threads), 0, st,                \
+  hipLaunchKernelGGL((k_gated_act_fwd_fast<B_, L_, A_, MT_>), grid, dim3(threads), 0, st,                          \
                      static_cast<const uint16_t*>(gate), ld_gate, static_cast<const uint16_t*>(up), ld_up, M, H,   \
                      geo.cps, sa, su, sg, static_cast<uint16_t*>(h), use_lut)
 #define HYC_GFWD_T(B_, L_, A_) /* H = 11008: 704 threads, up to 168 registers each */ \
-  do { if (geo.threads <= 256) HYC_GFWD(B_, L_, A_, 256); else HYC_GFWD(B_, L_, A_, 768); } while (0)
+  do { if (threads <= 256) HYC_GFWD(B_, L_, A_, 256); else HYC_GFWD(B_, L_, A_, 768); } while (0)
 #define HYC_GFWD_L(B_, A_) do { if (lpg == 8) HYC_GFWD_T(B_, 8, A_); else HYC_GFWD_T(B_, 16, A_); } while (0)
-#define HYC_GFWD_T2(L_, A_) do { if (geo.threads <= 256) HYC_GFWD(2, L_, A_, 256); else HYC_GFWD(2, L_, A_, 512); } while (0)
+#define HYC_GFWD_T2(L_, A_) do { if (threads <= 256) HYC_GFWD(2, L_, A_, 256); else HYC_GFWD(2, L_, A_, 512); } while (0)
 #define HYC_GFWD_B(A_)                                                                                             \
   do {                                                                                                             \
     if (d_a->bits == 2) { if (lpg == 8) HYC_GFWD_T2(8, A_); else HYC_GFWD_T2(16, A_); }                            \
