@@ -139,11 +139,12 @@ static int row_loop_grid(int64_t M, int64_t cap, int rows_each) {
   return (int)g;
 }
 // A row of the gated kernels that is too long for one workgroup (their per-thread state caps the workgroup at `most`
-// threads) is shared by 2 to 4 workgroups of whole waves.  Returns the number of workgroups per row, 0 if none fits.
-static int gated_row_parts(int cps, int most) {
+// threads) is shared by 2 to 4 workgroups, each a whole number of scale groups (lpg chunks).  Returns the number of
+// workgroups per row, 0 if none fits.
+static int gated_row_parts(int cps, int most, int lpg) {
   if (cps <= most) return 1;
   for (int n = 2; n <= 4; ++n)
-    if (cps % n == 0 && (cps / n) % 64 == 0 && cps / n <= most) return n;
+    if (cps % n == 0 && (cps / n) % lpg == 0 && ((cps / n + 63) / 64) * 64 <= most) return n;
   return 0;
 }
 
@@ -411,18 +412,18 @@ k_gated_act_bwd_fast(const uint16_t* __restrict__ g, const uint8_t* __restrict__
                      const uint16_t* __restrict__ s_a, ChanArgs c_a, const uint8_t* __restrict__ st_u,
                      const uint16_t* __restrict__ v_u, const uint16_t* __restrict__ s_u, ChanArgs c_u,
                      const uint8_t* __restrict__ st_g, const uint16_t* __restrict__ v_g, const uint16_t* __restrict__ s_g,
-                     ChanArgs c_g, int64_t M, int64_t H, int CPS, uint16_t* __restrict__ d_gate, uint16_t* __restrict__ d_up,
-                     int use_lut) {
+                     ChanArgs c_g, int64_t M, int64_t H, int CPS, int cps_wg, uint16_t* __restrict__ d_gate,
+                     uint16_t* __restrict__ d_up, int use_lut) {
   constexpr int NSEG = Q<BITS>::NSEG;
   __shared__ uint16_t lut[LUT_NEG + LUT_N];             // the activation's derivative, see lut_fill
   if (use_lut) {
     lut_fill<ACT>(lut);
     __syncthreads();
   }
-  // (a row too long for one workgroup's registers is shared by gridDim.y workgroups of whole waves: nothing in this
-  // kernel looks beyond a scale group)
-  const int c = (int)(blockIdx.y * blockDim.x + threadIdx.x);
-  if (c >= CPS) return;                                 // tail of the last wave
+  // (a row too long for one workgroup's registers is shared by gridDim.y workgroups of cps_wg chunks each, a whole
+  // number of scale groups: nothing in this kernel looks beyond a scale group)
+  const int c = (int)blockIdx.y * cps_wg + (int)threadIdx.x;
+  if ((int)threadIdx.x >= cps_wg) return;               // tail of the last wave
   const int64_t SEG = (int64_t)CPS * 8;
   const int64_t stride = gridDim.x;
   int64_t row = blockIdx.x;
@@ -529,7 +530,7 @@ struct GatedFwdSite {       // one compressed output
 template <int BITS, int LPGT, int ACT, int MAXT>
 __global__ void __launch_bounds__(MAXT)
 k_gated_act_fwd_fast(const uint16_t* __restrict__ gate, int64_t ldg, const uint16_t* __restrict__ up, int64_t ldu, int64_t M,
-                     int64_t H, int CPS, GatedFwdSite sa, GatedFwdSite su, GatedFwdSite sg, uint16_t* __restrict__ h,
+                     int64_t H, int CPS, int cps_wg, GatedFwdSite sa, GatedFwdSite su, GatedFwdSite sg, uint16_t* __restrict__ h,
                      int use_lut) {
   constexpr int NSEG = Q<BITS>::NSEG;
   __shared__ uint16_t lut[LUT_NEG + LUT_N];
@@ -537,8 +538,8 @@ k_gated_act_fwd_fast(const uint16_t* __restrict__ gate, int64_t ldg, const uint1
     lut_fill_value<ACT>(lut);
     __syncthreads();
   }
-  const int c = (int)(blockIdx.y * blockDim.x + threadIdx.x);   // (gridDim.y workgroups of whole waves share a long row)
-  if (c >= CPS) return;                                 // tail of the last wave; scale groups never straddle it
+  const int c = (int)blockIdx.y * cps_wg + (int)threadIdx.x;    // (gridDim.y workgroups of cps_wg chunks share a long row)
+  if ((int)threadIdx.x >= cps_wg) return;               // tail of the last wave; scale groups never straddle it
   const int64_t SEG = (int64_t)CPS * 8;
   const bool leader = (c & (LPGT - 1)) == 0;
   const int shift = sa.ca.chunk_to_group_shift;         // the three sites share the group width
@@ -931,9 +932,9 @@ int hyc_gated_act_bwd(int32_t act, const void* g, const void* stored_a, const vo
     return fail(HYC_EINVAL, "hyc_gated_act_bwd: g, d_gate, d_up must be 16-byte aligned, stored 8-byte");
   // rows of more than 768 chunks: two workgroups of the 768-thread variant per row where the row divides into whole
   // waves (the 1024-thread variant has 128 registers per thread and spills: 4096 x 14336, 113 us against 85)
-  const int parts0 = geo.threads > 768 ? gated_row_parts(geo.cps, 768) : 1;
+  const int parts0 = geo.threads > 768 ? gated_row_parts(geo.cps, 768, lpg) : 1;
   const int parts = parts0 > 1 ? parts0 : 1;          // (no division into whole waves: the 1024-thread variant)
-  const int threads = parts > 1 ? geo.cps / parts : geo.threads;
+  const int cps_wg = geo.cps / parts, threads = parts > 1 ? ((cps_wg + 63) / 64) * 64 : geo.threads;
   const int64_t cap = 256 * (threads * parts >= 512 ? 3 : 8) / parts;
   const int gx = (int)(M < cap ? M : cap);
   const dim3 grid((unsigned)gx, (unsigned)(parts > 1 ? parts : 1));
@@ -946,7 +947,7 @@ int hyc_gated_act_bwd(int32_t act, const void* g, const void* stored_a, const vo
                      static_cast<const uint8_t*>(stored_u), static_cast<const uint16_t*>(vals_u),                  \
                      static_cast<const uint16_t*>(scales_u), c_u, static_cast<const uint8_t*>(stored_g),           \
                      static_cast<const uint16_t*>(vals_g), static_cast<const uint16_t*>(scales_g), c_g, M, H,      \
-                     geo.cps, static_cast<uint16_t*>(d_gate), static_cast<uint16_t*>(d_up), use_lut)
+                     geo.cps, cps_wg, static_cast<uint16_t*>(d_gate), static_cast<uint16_t*>(d_up), use_lut)
 #define HYC_GATED_T(B_, A_)                                                       \
   do {                                                                            \
     if (threads <= 256) HYC_GATED(B_, A_, 256);                                   \
@@ -990,12 +991,12 @@ int hyc_gated_act_fwd(int32_t act, const void* gate, int64_t ld_gate, const void
   // codes), so the workgroup is capped at 768 threads (512 with 2-bit codes: 256 registers each); longer rows are
   // left to the separate calls.
   const int most = d_a->bits == 2 ? 512 : 768;
-  const int parts = geo.iters == 1 ? (geo.threads > most ? gated_row_parts(geo.cps, most) : 1) : 0;
+  const int parts = geo.iters == 1 ? (geo.threads > most ? gated_row_parts(geo.cps, most, lpg) : 1) : 0;
   if (parts == 0 || (d_a->bits != 2 && d_a->bits != 4 && d_a->bits != 8) || (lpg != 8 && lpg != 16))
     return fail(HYC_ENOTSUP, "hyc_gated_act_fwd: needs 2-, 4- or 8-bit codes, groups of 64 or 128 channels and rows of at "
                              "most 768 chunks per segment (512 with 2-bit codes), or up to 1024 that divide into 2 to 4 "
-                             "such parts of whole waves (use the activation, hyc_compress and a product otherwise)");
-  const int threads = parts > 1 ? geo.cps / parts : geo.threads;
+                             "such parts of whole scale groups (use the activation, hyc_compress and a product otherwise)");
+  const int cps_wg = geo.cps / parts, threads = parts > 1 ? ((cps_wg + 63) / 64) * 64 : geo.threads;
   if (M == 0) return HYC_OK;
   if (!gate || !up || !h || !stored_a || !stored_u || !stored_g || !scales_a || !scales_u || !scales_g ||
       (d_a->k > 0 && !vals_a) || (d_u->k > 0 && !vals_u) || (d_g->k > 0 && !vals_g))
@@ -1013,7 +1014,7 @@ int hyc_gated_act_fwd(int32_t act, const void* gate, int64_t ld_gate, const void
 #define HYC_GFWD(B_, L_, A_, MT_)                                                                                  \
   hipLaunchKernelGGL((k_gated_act_fwd_fast<B_, L_, A_, MT_>), grid, dim3(threads), 0, st,                          \
                      static_cast<const uint16_t*>(gate), ld_gate, static_cast<const uint16_t*>(up), ld_up, M, H,   \
-                     geo.cps, sa, su, sg, static_cast<uint16_t*>(h), use_lut)
+                     geo.cps, cps_wg, sa, su, sg, static_cast<uint16_t*>(h), use_lut)
 #define HYC_GFWD_T(B_, L_, A_) /* H = 11008: 704 threads, up to 168 registers each */ \
   do { if (threads <= 256) HYC_GFWD(B_, L_, A_, 256); else HYC_GFWD(B_, L_, A_, 768); } while (0)
 #define HYC_GFWD_L(B_, A_) do { if (lpg == 8) HYC_GFWD_T(B_, 8, A_); else HYC_GFWD_T(B_, 16, A_); } while (0)

@@ -605,10 +605,10 @@ def gated_act_fwd_supported(H, bits, group):
     """shapes the one-pass forward covers (the rest takes the activation, three compress calls and a product)"""
     if bits not in (2, 4, 8) or group not in (64, 128) or H % (64 // bits) != 0:
         return False
-    chunks, most = H * bits // 64, 512 if bits == 2 else 768
-    # one workgroup per row, or 2 to 4 workgroups of whole waves for rows of up to 1024 chunks
-    return chunks <= most or (chunks <= 1024 and any(chunks % n == 0 and (chunks // n) % 64 == 0 and chunks // n <= most
-                                                     for n in (2, 3, 4)))
+    chunks, most, lpg = H * bits // 64, 512 if bits == 2 else 768, group // 8
+    # one workgroup per row, or 2 to 4 workgroups (whole scale groups each) for rows of up to 1024 chunks
+    return chunks <= most or (chunks <= 1024 and any(chunks % n == 0 and (chunks // n) % lpg == 0 and
+                                                     -(-(chunks // n) // 64) * 64 <= most for n in (2, 3, 4)))
 
 
 def gated_act_fwd(act, gate2d, up2d, plan_act, plan_up, plan_gate, bits, group):

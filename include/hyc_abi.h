@@ -231,7 +231,7 @@ int hyc_gated_act_bwd(int32_t act, const void* g, const void* stored_a, const vo
  * HYC_ACT_SILU = F.silu; HYC_ACT_GELU_TANH = the GELU module, whose forward is the erf form (F.gelu) and whose backward
  * is the tanh form.  Same bytes as the separate calls; channel scheme, one code width (2, 4 or 8 bits) and group size (64
  * or 128) for the three, H * bits / 64 <= 768 (<= 512 with 2-bit codes), or up to 1024 when it divides by 2, 3 or 4 into
- * such parts that are multiples of 64 (H = 14336 and 16384 with 4-bit codes do); HYC_ENOTSUP otherwise (the separate
+ * such parts of whole scale groups (H = 13824, 14336 and 16384 with 4-bit codes do); HYC_ENOTSUP otherwise (the separate
  * calls cover every shape). */
 int hyc_gated_act_fwd(int32_t act, const void* gate, int64_t ld_gate, const void* up, int64_t ld_up, int64_t M, int64_t H,
                       const hyc_desc* d_a, const hyc_desc* d_u, const hyc_desc* d_g, void* h, void* stored_a, void* vals_a,

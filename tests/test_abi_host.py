@@ -134,9 +134,10 @@ def test_argument_errors_without_a_gpu(abi):
     d2b = ctypes.byref(d2)
     assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 4096, null, 4096, 4, 4096, d2b, d2b, d2b, null, *nine, null) == abi.EFAULT   # 2-bit codes: covered
     assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 20480, null, 20480, 4, 20480, d2b, d2b, d2b, null, *nine, null) == abi.EFAULT   # 640 chunks: two parts of 320
-    assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 22016, null, 22016, 4, 22016, d2b, d2b, d2b, null, *nine, null) == abi.ENOTSUP  # 688 chunks: above 512, no whole waves
+    assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 32832, null, 32832, 4, 32832, d2b, d2b, d2b, null, *nine, null) == abi.ENOTSUP  # 1026 chunks: row too long
     assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 14336, null, 14336, 4, 14336, D, D, D, null, *nine, null) == abi.EFAULT     # 896 chunks: two workgroups per row
-    assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 13824, null, 13824, 4, 13824, D, D, D, null, *nine, null) == abi.ENOTSUP    # 864 chunks: no division into whole waves
+    assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 13824, null, 13824, 4, 13824, D, D, D, null, *nine, null) == abi.EFAULT     # 864 chunks: two parts of 27 groups
+    assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 12544, null, 12544, 4, 12544, D, D, D, null, *nine, null) == abi.ENOTSUP    # 784 chunks = 49 groups: no 2 to 4 equal parts
     assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 4000, null, 4096, 4, 4096, D, D, D, null, *nine, null) == abi.EINVAL   # pitch < H
     assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 8192, null, 4100, 4, 4096, D, D, D, null, *nine, null) == abi.EINVAL   # pitch % 8
     assert lib.hyc_gated_act_fwd(abi.ACT_SILU, null, 8192, null, 8192, 4, 4096, D, D, D, null, *nine, null) == abi.EFAULT

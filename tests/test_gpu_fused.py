@@ -178,7 +178,8 @@ def test_hadamard_bwd(K, M, H, b1, g1, b2, g2):
 @pytest.mark.parametrize("M,H,bits,group", [(40, 4096, 4, 128), (2100, 11008, 2, 64), (33, 2048, 8, 64),
                                             (2100, 11008, 4, 128),       # three 704-thread rows per workgroup: derivative table
                                             (900, 14336, 4, 128), (70, 16384, 4, 64),   # two workgroups per row
-                                            (50, 13824, 4, 128)])        # 864 chunks: one workgroup of 1024 threads
+                                            (50, 13824, 4, 128), (300, 13824, 4, 64),   # 864 chunks: two workgroups of 432 threads
+                                            (40, 12544, 4, 128)])        # 784 chunks: one workgroup of 1024 threads
 def test_gated_act_bwd_equals_the_two_steps(K, act, M, H, bits, group):
     """one pass over (act(gate), up, gate) = hadamard backward followed by the activation backward, bit for bit"""
     k = K.num_outlier_channels(H, 0.01)
@@ -243,7 +244,9 @@ def test_gated_forward_activation_matches_the_framework_for_every_bf16_value(K, 
                                                   ("silu", 2100, 11008, 4, 128, 110), ("gelu", 1600, 11008, 4, 128, 110),
                                                   # rows of 896 and 1024 chunks: two workgroups per row
                                                   ("silu", 700, 14336, 4, 128, 143), ("gelu", 130, 16384, 4, 64, 164),
-                                                  ("silu", 90, 28672, 2, 128, 287)])
+                                                  ("silu", 90, 28672, 2, 128, 287),
+                                                  # 864 chunks: two workgroups of 432 threads, the last wave partly filled
+                                                  ("gelu", 210, 13824, 4, 128, 138), ("silu", 130, 13824, 4, 64, 138)])
 def test_gated_forward_equals_the_separate_calls(K, act, M, H, bits, group, k):
     """one pass = F.silu / F.gelu, three hyc_compress calls and a product, bit for bit; gate and up are column slices of
     one wider matrix, as a fused gate/up projection hands them over"""
@@ -264,8 +267,9 @@ def test_gated_forward_equals_the_separate_calls(K, act, M, H, bits, group, k):
         assert bits_equal(got.scales, ref.scales) and bits_equal(got.vals, ref.vals)
     assert K.gated_act_fwd_supported(4096, 2, 64) and K.gated_act_fwd_supported(11008, 4, 128)
     assert K.gated_act_fwd_supported(14336, 4, 128)              # 896 chunks per segment: two workgroups per row
-    assert not K.gated_act_fwd_supported(13824, 4, 128)          # 864 chunks: no division into whole waves, separate calls
-    assert not K.gated_act_fwd_supported(22016, 2, 64) and not K.gated_act_fwd_supported(4096, 1, 64)
+    assert K.gated_act_fwd_supported(13824, 4, 128)              # 864 chunks: two parts of 27 scale groups
+    assert not K.gated_act_fwd_supported(12544, 4, 128)          # 784 chunks = 49 groups: no 2 to 4 equal parts, separate calls
+    assert not K.gated_act_fwd_supported(32832, 2, 64) and not K.gated_act_fwd_supported(4096, 1, 64)
 
 
 @pytest.mark.parametrize("bits,group,M,H,k,wdt,with_bias", [
