@@ -268,7 +268,7 @@ def config1_extra(pkg, torch):
 
 def config4_extra(pkg, torch):
     """BASELINE configs[3]: gate / up [4,1024,11008] with 1 % outlier channels x20, INT4 group 128: SiLU backward,
-    the one-pass backward of SiLU(gate)*up, and the down_proj weight gradient (dY [4096,4096], 369 GFLOP) with its
+    the one-pass backward and forward of SiLU(gate)*up, the forwards with their saves, and the down_proj weight gradient (dY [4096,4096], 369 GFLOP) with its
     LoRA-A (r = 16) companion"""
     K = pkg.kernels
     M, H, bits, G = 4096, 11008, 4, 128
@@ -282,7 +282,10 @@ def config4_extra(pkg, torch):
     side = side_bytes(H, bits, G, k)
     out = {"silu_bwd": hbm(M * (4 * H + side), time_graph(torch, lambda: K.act_bwd("silu", g, cg))),
            "gated_silu_bwd": hbm(M * (6 * H + 3 * side), time_graph(torch, lambda: K.gated_act_bwd("silu", g, ca, cu, cg))),
-           "silu_fwd_compress": hbm(M * (4 * H + side), time_graph(torch, lambda: K.act_fwd_compress("silu", gate, cg.plan, bits, G)))}
+           "silu_fwd_compress": hbm(M * (4 * H + side), time_graph(torch, lambda: K.act_fwd_compress("silu", gate, cg.plan, bits, G))),
+           # SiLU(gate) * up and the three saves (act(gate), up, gate) in one pass: reads gate and up, writes the product
+           "gated_silu_fwd": hbm(M * (6 * H + 3 * side), time_graph(torch, lambda: K.gated_act_fwd("silu", gate, up, ca.plan, cu.plan, cg.plan, bits, G))),
+           "product_fwd_compress": hbm(M * (6 * H + 2 * side), time_graph(torch, lambda: K.hadamard_fwd_compress(act, up, ca.plan, cu.plan, bits, G)))}
     del gate, up, act, prod, g, cg, cu, ca
     out["down_proj"] = gradw_extra(pkg, torch, cp, shapes=(("full_w", 4096, 60, 20), ("lora_a_r16", 16, 300, 30), ("lora_a_r64", 64, 300, 30)))
     return out
