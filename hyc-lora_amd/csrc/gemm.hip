@@ -749,9 +749,24 @@ k_gradw_big(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_o
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int64_t n0 = (int64_t)blockIdx.x * TN;
+  // Which tile: workgroups are dealt to the 8 XCDs in turn (workgroup L of a launch runs on XCD L mod 8) and every XCD
+  // has an L2 of its own, so XCD q takes a contiguous run of tiles in an order that walks 4 feature tiles by all
+  // channel tiles: its workgroups then share 4 dY panels and a short run of x_hat panels instead of 2 and all of them
+  // (1-4 % on real operands: 4096 x 4096 x 11008 dense 328 -> 320 us, INT2 4096^3 138 -> 132 us).
+  int tile_n = (int)blockIdx.x, tile_h = (int)blockIdx.y;
+  {
+    const int gx = (int)gridDim.x, gy = (int)gridDim.y, T = gx * gy;
+    if (T % 8 == 0 && gx % 4 == 0) {
+      const int L = tile_n + gx * tile_h;
+      const int t = (L % 8) * (T / 8) + L / 8;
+      const int band = t / (4 * gy), r = t - band * (4 * gy);
+      tile_n = band * 4 + r % 4;
+      tile_h = r / 4;
+    }
+  }
+  const int64_t n0 = (int64_t)tile_n * TN;
   const int64_t SEG = (SRC == 0) ? (int64_t)CPS * 8 : H;
-  const int64_t j0 = (int64_t)blockIdx.y * HS;          // first column of the tile inside each segment
+  const int64_t j0 = (int64_t)tile_h * HS;              // first column of the tile inside each segment
   const int64_t m_begin = (int64_t)blockIdx.z * tokens_per_split;
   const int64_t m_end = m_begin + tokens_per_split < M ? m_begin + tokens_per_split : M;
   const int wn = (wave >> 1) * 128, wh = (wave & 1) * 128;
