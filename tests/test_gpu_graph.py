@@ -93,3 +93,74 @@ def test_replays_equal_the_eager_sequence(pkg, M, H, bits, group, r):
         assert torch.isfinite(noise)
         for got, ref in zip(seq.outputs(), want):
             assert torch.equal(got.view(torch.uint8), ref.view(torch.uint8)), "replay %d" % rep
+
+
+def _channel_tensors(c):
+    return [c.stored, c.vals, c.scales]
+
+
+@pytest.mark.parametrize("M,H,bits,group", [(520, 2048, 4, 128), (1030, 4096, 2, 64)])
+def test_the_other_channel_entry_points_replay(pkg, M, H, bits, group):
+    """compress / decompress, the one-pass forwards (activation, product, gated), their backwards, LayerNorm forward
+    and backward and the wide weight gradient (codes decoded in the kernel, and the restored operand) through the
+    package's wrappers: their output tensors come from the graph's memory pool, the kernels are the captured ones"""
+    K = pkg.kernels
+    gen = torch.Generator(device="cuda").manual_seed(11)
+    k = K.num_outlier_channels(H, 0.01)
+
+    def mk(scale):
+        t = scale * torch.randn(M, H, generator=gen, device="cuda")
+        t[:, torch.randperm(H, generator=gen, device="cuda")[:k]] *= 20.0
+        return t.bfloat16()
+
+    gate, up, g = mk(1.0), mk(1.0), mk(0.02)
+    dyN = (0.01 * torch.randn(M, 256, generator=gen, device="cuda")).bfloat16()
+    w = 1 + 0.1 * torch.randn(H, generator=gen, device="cuda")
+    b = 0.1 * torch.randn(H, generator=gen, device="cuda")
+    plans = [K.select_channels(K.channel_absmax(t), k) for t in (torch.nn.functional.silu(gate), up, gate)]
+    gated = K.gated_act_fwd_supported(H, bits, group)
+    product = K.hadamard_fwd_compress_supported(H, bits, group, bits, group)
+
+    def run():
+        out = []
+        c = K.compress_channel(gate, plans[2], bits, group)
+        out += _channel_tensors(c) + [K.decompress_channel(c)]
+        y, cx = K.act_fwd_compress("gelu", gate, plans[2], bits, group)
+        out += [y] + _channel_tensors(cx) + [K.act_bwd("gelu", g, cx)]
+        if product:
+            y, ca, cb = K.hadamard_fwd_compress(gate, up, plans[2], plans[1], bits, group)
+            out += [y] + _channel_tensors(ca) + _channel_tensors(cb) + list(K.hadamard_bwd(g, ca, cb))
+        if gated:
+            h, c_act, c_up, c_gate = K.gated_act_fwd("silu", gate, up, plans[0], plans[1], plans[2], bits, group)
+            out += [h] + _channel_tensors(c_act) + _channel_tensors(c_up) + _channel_tensors(c_gate)
+            out += list(K.gated_act_bwd("silu", g, c_act, c_up, c_gate))
+        y, mean, rstd, cl = K.layernorm_fwd_compress_channel(gate, w, b, 1e-5, plans[2], bits, group)
+        out += [y, mean, rstd] + _channel_tensors(cl) + list(K.layernorm_bwd(g, cl, w, mean, rstd))
+        out += [K.gradw_gemm(dyN, c, staged=False), K.gradw_gemm(dyN, c, staged=True)]
+        return out
+
+    want = [t.clone() for t in run()]
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        got = run()
+    for rep in range(3):
+        if rep == 1:                                    # fresh input in the same buffers
+            gate.mul_(-0.75)
+            g.mul_(2.0)
+            want = [t.clone() for t in run()]
+        for t in got:
+            t.view(torch.uint8).fill_(0xA5)
+        noise = torch.randn(1 << 16, device="cuda").cumsum(0).sum()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.isfinite(noise)
+        assert len(got) == len(want)
+        for i, (a, r) in enumerate(zip(got, want)):
+            assert torch.equal(a.view(torch.uint8), r.view(torch.uint8)), "replay %d, output %d" % (rep, i)
