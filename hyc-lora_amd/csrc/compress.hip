@@ -4,6 +4,7 @@
 
 #include "abi_util.hpp"
 #include "row_kernels.hpp"
+#include "wave_scan.hpp"
 
 namespace hyc {
 
@@ -273,9 +274,9 @@ k_decompress_thr(const uint8_t* __restrict__ stored, int64_t M, int64_t H, int C
 
 // ---- outliers as CSR ------------------------------------------------------------------------------
 // 8-bit mask of the elements of chunk cc (plain column order) that exceed the threshold
-__device__ __forceinline__ uint32_t hot_mask8(const uint16_t* xr, int64_t cc, int64_t H, int64_t s_pos,
-                                              const ThrArgs& a, uint4& raw, float (&v)[8]) {
-  raw = *reinterpret_cast<const uint4*>(xr + 8 * cc);
+// (`raw` = the chunk as loaded)
+__device__ __forceinline__ uint32_t hot_mask8_of(const uint4& raw, int64_t cc, int64_t H, int64_t s_pos,
+                                                 const ThrArgs& a, float (&v)[8]) {
   unpack8(raw, v);
   if (a.rank > 0) {
     float b[8];
@@ -287,6 +288,11 @@ __device__ __forceinline__ uint32_t hot_mask8(const uint16_t* xr, int64_t cc, in
 #pragma unroll
   for (int j = 0; j < 8; ++j) m |= (__builtin_fabsf(v[j]) > a.thr) ? (1u << j) : 0u;
   return m;
+}
+__device__ __forceinline__ uint32_t hot_mask8(const uint16_t* xr, int64_t cc, int64_t H, int64_t s_pos,
+                                              const ThrArgs& a, uint4& raw, float (&v)[8]) {
+  raw = *reinterpret_cast<const uint4*>(xr + 8 * cc);
+  return hot_mask8_of(raw, cc, H, s_pos, a, v);
 }
 
 // one wave per row, 4 rows per workgroup
@@ -313,36 +319,39 @@ k_outlier_count(const uint16_t* __restrict__ x, int64_t M, int64_t H, ThrArgs a,
 __global__ void __launch_bounds__(256)
 k_outlier_fill(const uint16_t* __restrict__ x, int64_t M, int64_t H, ThrArgs a, const int32_t* __restrict__ row_ptr,
                int32_t* __restrict__ cols, uint16_t* __restrict__ vals) {
+  __shared__ uint32_t stage_all[4][STAGE_CAP];
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= M) return;                                  // whole waves leave together
+  uint32_t* stage = stage_all[threadIdx.x >> 6];
   const uint16_t* xr = x + row * H;
   const int64_t s_pos = row % a.S;
   const int64_t nch = H / 8;
-  int running = row_ptr[row];
+  const int64_t base = row_ptr[row];
+  int32_t* cols_row = cols + base;
+  uint16_t* vals_row = vals + base;
+  int running = 0;
+  uint4 next = lane < nch ? *reinterpret_cast<const uint4*>(xr + 8 * lane) : make_uint4(0, 0, 0, 0);
   for (int64_t c0 = 0; c0 < nch; c0 += 64) {
     const int64_t cc = c0 + lane;
-    uint4 raw; float v[8];
+    const uint4 raw = next;
+    if (cc + 64 < nch) next = *reinterpret_cast<const uint4*>(xr + 8 * (cc + 64));   // the next chunk is on its way
+    float v[8];
     uint32_t m = 0;
-    if (cc < nch) m = hot_mask8(xr, cc, H, s_pos, a, raw, v);
+    if (cc < nch) m = hot_mask8_of(raw, cc, H, s_pos, a, v);
     const int cnt = __popc(m);
-    int incl = cnt;                                      // inclusive scan over the wave
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-      const int t = __shfl_up(incl, d, 64);
-      if (lane >= d) incl += t;
-    }
+    const int incl = wave_inclusive_scan(cnt);           // prefix sum over the wave
     int pos = running + incl - cnt;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       if ((m >> j) & 1u) {
-        cols[pos] = (int32_t)(8 * cc + j);
-        vals[pos] = f_to_bf(v[j]);                       // the value after the base was removed
+        stage_entry(stage, pos, (int)(8 * cc + j), f_to_bf(v[j]), cols_row, vals_row);   // the value after the base was removed
         ++pos;
       }
     }
-    running += __shfl(incl, 63, 64);
+    running += __builtin_amdgcn_readlane(incl, 63);
   }
+  stage_flush(stage, running, cols_row, vals_row);
 }
 
 // ---- launch helpers -------------------------------------------------------------------------------

@@ -5,6 +5,7 @@
 //   dense     yh as a dense matrix (what true_decompress_softmax returns)
 // Reference: operators/efficient_softmax.py:10-45, operators/compress_function.py:264-275.
 #include "abi_util.hpp"
+#include "wave_scan.hpp"
 
 namespace hyc {
 
@@ -176,45 +177,47 @@ k_softmax_count(const uint16_t* __restrict__ y, int64_t rows, int64_t N, float t
   if (lane == 0) counts[row] = (int32_t)total;
 }
 
-// one wave per row: ordered compaction of the kept entries
+// one wave per row: ordered compaction of the kept entries (prefix sum over the lanes, entries staged in LDS and
+// stored as contiguous runs)
 __global__ void __launch_bounds__(256)
 k_softmax_fill(const uint16_t* __restrict__ y, int64_t rows, int64_t N, float thr, const int32_t* __restrict__ row_ptr,
                int32_t* __restrict__ cols, uint16_t* __restrict__ vals) {
+  __shared__ uint32_t stage_all[4][STAGE_CAP];
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (row >= rows) return;
+  if (row >= rows) return;                               // whole waves leave together
+  uint32_t* stage = stage_all[threadIdx.x >> 6];
   const uint16_t* yr = y + row * N;
   const int64_t nch = N / 8;
-  int running = row_ptr[row];
+  const int64_t base = row_ptr[row];
+  int32_t* cols_row = cols + base;
+  uint16_t* vals_row = vals + base;
+  int running = 0;
+  uint4 next = lane < nch ? *reinterpret_cast<const uint4*>(yr + 8 * lane) : make_uint4(0, 0, 0, 0);
   for (int64_t c0 = 0; c0 < nch; c0 += 64) {
     const int64_t c = c0 + lane;
-    uint4 raw = make_uint4(0, 0, 0, 0);
+    const uint4 raw = next;
+    if (c + 64 < nch) next = *reinterpret_cast<const uint4*>(yr + 8 * (c + 64));   // the next chunk is on its way
     float v[8];
     uint32_t m = 0;
     if (c < nch) {
-      raw = *reinterpret_cast<const uint4*>(yr + 8 * c);
       unpack8(raw, v);
 #pragma unroll
       for (int j = 0; j < 8; ++j) m |= (v[j] > thr) ? (1u << j) : 0u;
     }
     const int cnt = __popc(m);
-    int incl = cnt;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-      const int t = __shfl_up(incl, d, 64);
-      if (lane >= d) incl += t;
-    }
+    const int incl = wave_inclusive_scan(cnt);
     int pos = running + incl - cnt;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       if ((m >> j) & 1u) {
-        cols[pos] = (int32_t)(8 * c + j);
-        vals[pos] = f_to_bf(v[j]);
+        stage_entry(stage, pos, (int)(8 * c + j), f_to_bf(v[j]), cols_row, vals_row);
         ++pos;
       }
     }
-    running += __shfl(incl, 63, 64);
+    running += __builtin_amdgcn_readlane(incl, 63);
   }
+  stage_flush(stage, running, cols_row, vals_row);
 }
 
 // the same for rows of up to 4096 entries with every load of the row issued up front (CPL chunks per lane)
@@ -222,16 +225,21 @@ template <int CPL>
 __global__ void __launch_bounds__(256)
 k_softmax_fill_wave(const uint16_t* __restrict__ y, int64_t rows, int64_t N, float thr, const int32_t* __restrict__ row_ptr,
                     int32_t* __restrict__ cols, uint16_t* __restrict__ vals) {
+  __shared__ uint32_t stage_all[4][STAGE_CAP];
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= rows) return;
+  uint32_t* stage = stage_all[threadIdx.x >> 6];
   const uint16_t* yr = y + row * N;
   const int nch = (int)(N / 8);
   uint4 raw[CPL];
 #pragma unroll
   for (int u = 0; u < CPL; ++u)
     raw[u] = lane + 64 * u < nch ? *reinterpret_cast<const uint4*>(yr + 8 * (lane + 64 * u)) : make_uint4(0, 0, 0, 0);
-  int running = row_ptr[row];
+  const int64_t base = row_ptr[row];
+  int32_t* cols_row = cols + base;
+  uint16_t* vals_row = vals + base;
+  int running = 0;
 #pragma unroll
   for (int u = 0; u < CPL; ++u) {
     const int c = lane + 64 * u;
@@ -243,25 +251,20 @@ k_softmax_fill_wave(const uint16_t* __restrict__ y, int64_t rows, int64_t N, flo
       for (int j = 0; j < 8; ++j) m |= (v[j] > thr) ? (1u << j) : 0u;
     }
     const int cnt = __popc(m);
-    int incl = cnt;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-      const int t = __shfl_up(incl, d, 64);
-      if (lane >= d) incl += t;
-    }
+    const int incl = wave_inclusive_scan(cnt);
     int pos = running + incl - cnt;
     if (m) {
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         if ((m >> j) & 1u) {
-          cols[pos] = (int32_t)(8 * c + j);
-          vals[pos] = f_to_bf(v[j]);
+          stage_entry(stage, pos, 8 * c + j, f_to_bf(v[j]), cols_row, vals_row);
           ++pos;
         }
       }
     }
-    running += __shfl(incl, 63, 64);
+    running += __builtin_amdgcn_readlane(incl, 63);
   }
+  stage_flush(stage, running, cols_row, vals_row);
 }
 
 // one wave per row; the output row is assembled in LDS (zeros + kept entries) and written out coalesced.

@@ -204,6 +204,25 @@ def _coo_of(c, S):
     return torch.stack([rows // S, rows % S, c.cols.cpu().long()]), c.vals.cpu()
 
 
+@pytest.mark.parametrize("H,ratio", [(4096, 0.45), (8192, 0.3), (2048, 0.999)])
+def test_threshold_rows_with_more_outliers_than_a_wave_stages(K, H, ratio):
+    """a low threshold keeps more than 1024 outlier elements per row: the first 1024 leave through the wave's staging
+    row in LDS, the rest go to memory one by one; order and values must be the reference's either way"""
+    B, S, bits = 2, 9, 4
+    gen = torch.Generator().manual_seed(H)
+    x = torch.randn(B, S, H, generator=gen).bfloat16()
+    thr, L, R, scale = O.get_statistics(x, 0, ratio, 1.0, bits, "per-token", 0)
+    coo, stored, _ = O.ref_compress(x, thr, scale, bits, 1.0, L, R)
+    coo = coo.coalesce()
+    c = K.compress_threshold(x.reshape(-1, H).cuda(), S, float(thr), scale.cuda(), bits)
+    rp = c.row_ptr.cpu()
+    assert int((rp[1:] - rp[:-1]).max()) > 1024
+    idx, vals = _coo_of(c, S)
+    assert torch.equal(idx, coo.indices())
+    assert bits_equal(vals, coo.values())
+    assert bits_equal(K.decompress_threshold(c).cpu().reshape(B, S, H), O.ref_decompress(coo, stored, bits, scale, L=L, R=R))
+
+
 @pytest.mark.parametrize("bits", [1, 2, 4, 8])
 @pytest.mark.parametrize("method", ["per-tensor", "per-channel", "per-token"])
 @pytest.mark.parametrize("rank", [0, 2])

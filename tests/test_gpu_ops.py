@@ -182,6 +182,27 @@ def test_softmax_kernels(K, shape):
     assert (dx.float() == want.float()).float().mean() > 0.995
 
 
+@pytest.mark.parametrize("shape,keep", [((1, 1, 9, 4096), 0.5), ((1, 2, 5, 8192), 0.4), ((2, 1, 6, 2048), 1.0), ((1, 1, 70, 2048), 0.0)])
+def test_softmax_rows_with_many_or_no_kept_entries(K, shape, keep):
+    """rows that keep more entries than a wave stages in LDS (1024) spill the rest straight to memory; rows that keep
+    everything or nothing are the two ends of that path"""
+    gen = torch.Generator().manual_seed(int(1000 * keep) + shape[-1])
+    y = torch.softmax((2 * torch.randn(*shape, generator=gen)).bfloat16().float(), dim=-1).bfloat16()
+    if keep == 1.0:
+        thr = 0.0                                        # strict comparison: every positive probability stays
+    elif keep == 0.0:
+        thr = 2.0
+    else:
+        thr = float(torch.quantile(y.float().flatten(), 1 - keep))
+    sp = K.softmax_sparsify(y.cuda(), thr)
+    coo_o = O.true_compress_softmax(y, torch.tensor(thr)).coalesce()
+    coo = K.sparse_rows_to_coo(sp).coalesce()
+    assert torch.equal(coo.indices().cpu(), coo_o.indices()) and bits_equal(coo.values().cpu(), coo_o.values())
+    if keep >= 0.4:
+        assert int((sp.row_ptr[1:] - sp.row_ptr[:-1]).max()) > 1024
+    assert torch.equal(K.softmax_dense(sp).cpu(), O.true_decompress_softmax(coo_o))
+
+
 def test_softmax_golden(K, golden_softmax):
     gs = golden_softmax
     y, thr = from_bits(gs["y"]), from_bits(gs["thr"])
