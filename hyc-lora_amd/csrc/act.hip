@@ -801,9 +801,14 @@ static int launch_act(const void* g, const void* stored, const void* vals, const
     return fail(HYC_EINVAL, "%s: g, dx must be 16-byte aligned, stored 8-byte (16 when dense)", who);
   const int64_t cap = 256 * (geo.threads >= 512 ? 3 : 8);
   int grid = (int)(M < cap ? M : cap);
-  // narrow rows (two waves or fewer per workgroup): fewer workgroups with four rows or more each, so that the derivative
-  // table pays (4096 x 4096 INT2: GELU 40 -> 25 us, SiLU 25 -> 19 us)
-  if (ACT != ACT_MUL && geo.threads * geo.iters <= 128 && M >= 4096 && grid > 1024) grid = 1024;
+  // Every workgroup of the activation kernels fills its own derivative table, so workgroups of four waves or fewer get
+  // more rows each instead of the chip more workgroups: about two waves per SIMD (4096 x 4096 INT2, 128 threads, 2048
+  // -> 1024 workgroups: GELU 40 -> 25 us, SiLU 25 -> 19 us; INT4, 256 threads, 2048 -> 512: GELU 27.6 -> 17.3 us, SiLU
+  // 17.6 -> 15.2 us, and 232 -> 221 us at 65 536 rows; H = 5120, 320 threads, 2048 -> 768: 36.0 -> 21.2 / 24.6 -> 18.6 us)
+  if (ACT != ACT_MUL && geo.iters == 1) {
+    const int fewer = geo.threads <= 128 ? 1024 : geo.threads <= 256 ? 512 : 768;
+    if (grid > fewer) grid = fewer;
+  }
   hipStream_t st = begin_launch(stream);
   const int use_lut = lut_pays(M, grid, geo.threads * geo.iters, LUT_PAYS_BWD);
   if (d->mode == HYC_MODE_CHANNEL && geo.iters == 1 && d->bits != 1) {
@@ -935,7 +940,10 @@ int hyc_gated_act_bwd(int32_t act, const void* g, const void* stored_a, const vo
   const int parts0 = geo.threads > 768 ? gated_row_parts(geo.cps, 768, lpg) : 1;
   const int parts = parts0 > 1 ? parts0 : 1;          // (no division into whole waves: the 1024-thread variant)
   const int cps_wg = geo.cps / parts, threads = parts > 1 ? ((cps_wg + 63) / 64) * 64 : geo.threads;
-  const int64_t cap = 256 * (threads * parts >= 512 ? 3 : 8) / parts;
+  // (workgroups of fewer than eight waves: fewer of them with more rows each, as for the activation backward - INT4,
+  // 4096 x 4096, 2048 -> 768 workgroups: 30.7 -> 24.9 us; H = 5120, 2048 -> 512: 55.8 -> 44.0 us; INT2, 2048 -> 1024: 37.6 -> 33.7 us)
+  // (from 32 768 rows on the tables are paid for either way and the resident grid is 2 % ahead: 394 against 403 us at 65 536)
+  const int64_t cap = threads * parts >= 512 ? 768 / parts : M >= 32768 ? 2048 : threads <= 128 ? 1024 : threads <= 256 ? 768 : 512;
   const int gx = (int)(M < cap ? M : cap);
   const dim3 grid((unsigned)gx, (unsigned)(parts > 1 ? parts : 1));
   hipStream_t st = begin_launch(stream);
