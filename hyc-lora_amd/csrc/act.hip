@@ -572,6 +572,11 @@ k_gated_act_fwd_fast(const uint16_t* __restrict__ gate, int64_t ldg, const uint1
   uint16_t* hp = h + row * H + 8 * c;
   const int64_t gstep = stride * ldg, ustep = stride * ldu, hstep = stride * H, sstep = stride * SEG, scstep = stride * gpr;
   int64_t soff = row * SEG + 8 * c, scoff = row * gpr + (c >> shift);
+  // outlier channels, kept verbatim: thread c copies channel idx[c] of each site (+ CPS, ... when a site has more of
+  // them than the row has threads); the index is read once, the element at the top of the row's iteration
+  const bool ga = c < sa.ca.k, gu = c < su.ca.k, gg = c < sg.ca.k;
+  const int ia = ga ? sa.ca.idx[c] : 0, iu = gu ? su.ca.idx[c] : 0, ig = gg ? sg.ca.idx[c] : 0;
+  uint16_t oa = 0, ou = 0, og = 0;
   uint4 graw[NSEG], uraw[NSEG];
   if (row < M) {
 #pragma unroll
@@ -581,6 +586,9 @@ k_gated_act_fwd_fast(const uint16_t* __restrict__ gate, int64_t ldg, const uint1
     }
   }
   for (; row < M; row += stride) {
+    // (by every lane, and ahead of the next row's requests: a branch around a load ends in a full wait, and loads
+    // return in order, so the wait for these at the end of the row leaves the next row's in flight)
+    oa = grow[ia]; ou = urow[iu]; og = grow[ig];
     uint4 g_n[NSEG], u_n[NSEG];
     if (row + stride < M) {
 #pragma unroll
@@ -622,11 +630,19 @@ k_gated_act_fwd_fast(const uint16_t* __restrict__ gate, int64_t ldg, const uint1
     *reinterpret_cast<uint2*>(sa.stored + soff) = make_uint2(lo_a, hi_a);
     *reinterpret_cast<uint2*>(su.stored + soff) = make_uint2(lo_u, hi_u);
     *reinterpret_cast<uint2*>(sg.stored + soff) = make_uint2(lo_g, hi_g);
-    // outlier channels, kept verbatim: thread t copies channel idx[t] (+ CPS, ...) of each site
-    for (int t = c; t < sa.ca.k; t += CPS)
-      sa.vals[row * sa.ca.k + t] = f_to_bf(act_value<ACT>(bf_to_f(grow[sa.ca.idx[t]])));
-    for (int t = c; t < su.ca.k; t += CPS) su.vals[row * su.ca.k + t] = urow[su.ca.idx[t]];
-    for (int t = c; t < sg.ca.k; t += CPS) sg.vals[row * sg.ca.k + t] = grow[sg.ca.idx[t]];
+    if (ga) {
+      sa.vals[row * sa.ca.k + c] = f_to_bf(act_value<ACT>(bf_to_f(oa)));
+      for (int t = c + CPS; t < sa.ca.k; t += CPS)
+        sa.vals[row * sa.ca.k + t] = f_to_bf(act_value<ACT>(bf_to_f(grow[sa.ca.idx[t]])));
+    }
+    if (gu) {
+      su.vals[row * su.ca.k + c] = ou;
+      for (int t = c + CPS; t < su.ca.k; t += CPS) su.vals[row * su.ca.k + t] = urow[su.ca.idx[t]];
+    }
+    if (gg) {
+      sg.vals[row * sg.ca.k + c] = og;
+      for (int t = c + CPS; t < sg.ca.k; t += CPS) sg.vals[row * sg.ca.k + t] = grow[sg.ca.idx[t]];
+    }
 #pragma unroll
     for (int i = 0; i < NSEG; ++i) { graw[i] = g_n[i]; uraw[i] = u_n[i]; }
     grow += gstep; urow += ustep; hp += hstep; soff += sstep; scoff += scstep;
@@ -676,6 +692,11 @@ k_ew_fwd_fast(const uint16_t* __restrict__ x1, int64_t ld1, const uint16_t* __re
   uint16_t* yp = y + row * H + 8 * c;
   const int64_t step1 = stride * ld1, step2 = stride * ld2, ystep = stride * H, sstep = stride * SEG, scstep = stride * gpr;
   int64_t soff = row * SEG + 8 * c, scoff = row * gpr + (c >> shift);
+  // outlier channels, kept verbatim: thread c copies channel idx[c] of each operand (+ CPS, ... when there are more of
+  // them than the row has threads); the index is read once, the element at the top of the row's iteration
+  const bool g1 = c < s1.ca.k, g2 = NIN == 2 && c < s2.ca.k;
+  const int i1 = g1 ? s1.ca.idx[c] : 0, i2 = g2 ? s2.ca.idx[c] : 0;
+  uint16_t ov1 = 0, ov2 = 0;
   uint4 raw[NIN][NSEG];
   if (row < M) {
 #pragma unroll
@@ -685,6 +706,10 @@ k_ew_fwd_fast(const uint16_t* __restrict__ x1, int64_t ld1, const uint16_t* __re
     }
   }
   for (; row < M; row += stride) {
+    // (by every lane, and ahead of the next row's requests: a branch around a load ends in a full wait, and loads
+    // return in order, so the wait for these at the end of the row leaves the next row's in flight)
+    ov1 = r1[i1];
+    if (NIN == 2) ov2 = r2[i2];
     uint4 nxt[NIN][NSEG];
     if (row + stride < M) {
 #pragma unroll
@@ -725,9 +750,14 @@ k_ew_fwd_fast(const uint16_t* __restrict__ x1, int64_t ld1, const uint16_t* __re
     }
     *reinterpret_cast<uint2*>(s1.stored + soff) = make_uint2(lo[0], hi[0]);
     if (NIN == 2) *reinterpret_cast<uint2*>(s2.stored + soff) = make_uint2(lo[NIN - 1], hi[NIN - 1]);
-    for (int t = c; t < s1.ca.k; t += CPS) s1.vals[row * s1.ca.k + t] = r1[s1.ca.idx[t]];
-    if (NIN == 2)
-      for (int t = c; t < s2.ca.k; t += CPS) s2.vals[row * s2.ca.k + t] = r2[s2.ca.idx[t]];
+    if (g1) {
+      s1.vals[row * s1.ca.k + c] = ov1;
+      for (int t = c + CPS; t < s1.ca.k; t += CPS) s1.vals[row * s1.ca.k + t] = r1[s1.ca.idx[t]];
+    }
+    if (g2) {
+      s2.vals[row * s2.ca.k + c] = ov2;
+      for (int t = c + CPS; t < s2.ca.k; t += CPS) s2.vals[row * s2.ca.k + t] = r2[s2.ca.idx[t]];
+    }
 #pragma unroll
     for (int n = 0; n < NIN; ++n)
 #pragma unroll
