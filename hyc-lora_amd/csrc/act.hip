@@ -973,7 +973,10 @@ int hyc_gated_act_bwd(int32_t act, const void* g, const void* stored_a, const vo
   // (workgroups of fewer than eight waves: fewer of them with more rows each, as for the activation backward - INT4,
   // 4096 x 4096, 2048 -> 768 workgroups: 30.7 -> 24.9 us; H = 5120, 2048 -> 512: 55.8 -> 44.0 us; INT2, 2048 -> 1024: 37.6 -> 33.7 us)
   // (from 32 768 rows on the tables are paid for either way and the resident grid is 2 % ahead: 394 against 403 us at 65 536)
-  const int64_t cap = threads * parts >= 512 ? 768 / parts : M >= 32768 ? 2048 : threads <= 128 ? 1024 : threads <= 256 ? 768 : 512;
+  // Rows of eight waves or more: a CU holds one such workgroup at a time, so one per CU (and row part) with all its
+  // rows beats three or four that each fill a table and start from an empty pipeline (4096 x 11008: 64.6 -> 60.1 us,
+  // 2048 rows: 39.5 -> 32.8; the same at 16 384 rows; a grid that is not a multiple of the 256 CUs loses up to 15 %).
+  const int64_t cap = threads * parts >= 512 ? 256 : M >= 32768 ? 2048 : threads <= 128 ? 1024 : threads <= 256 ? 768 : 512;
   const int gx = (int)(M < cap ? M : cap);
   const dim3 grid((unsigned)gx, (unsigned)(parts > 1 ? parts : 1));
   hipStream_t st = begin_launch(stream);
@@ -1045,7 +1048,9 @@ int hyc_gated_act_fwd(int32_t act, const void* gate, int64_t ld_gate, const void
   const GatedFwdSite su = {c_u, static_cast<uint8_t*>(stored_u), static_cast<uint16_t*>(vals_u), static_cast<uint16_t*>(scales_u)};
   const GatedFwdSite sg = {c_g, static_cast<uint8_t*>(stored_g), static_cast<uint16_t*>(vals_g), static_cast<uint16_t*>(scales_g)};
   const int64_t cap = 256 * (threads * parts >= 512 ? 3 : 8) / parts;
-  const int gx = threads * parts >= 512 ? row_loop_grid(M, cap, 4) : (int)(M < cap ? M : cap);
+  // (rows of eight waves or more: one workgroup per CU and row part, as in the gated backward - 4096 x 11008:
+  // 85.7 -> 79.1 us, 4096 x 14336: 124.9 -> 107.5, 2048 x 11008: 48.3 -> 40.0, 16 384 x 11008: 339 -> 321)
+  const int gx = threads * parts >= 512 ? (int)(M < 256 ? M : 256) : (int)(M < cap ? M : cap);
   const dim3 grid((unsigned)gx, (unsigned)parts);
   hipStream_t st = begin_launch(stream);
   const int use_lut = lut_pays(M, gx, threads, LUT_PAYS_OTHER);
@@ -1104,7 +1109,10 @@ static int ew_fwd_impl(const char* who, int32_t act, const void* x1, int64_t ld1
   const GatedFwdSite s1 = {c1, static_cast<uint8_t*>(stored1), static_cast<uint16_t*>(vals1), static_cast<uint16_t*>(scales1)};
   const GatedFwdSite s2 = {c2, static_cast<uint8_t*>(stored2), static_cast<uint16_t*>(vals2), static_cast<uint16_t*>(scales2)};
   const int64_t cap = 256 * (geo.threads >= 512 ? 3 : 8);
-  const int grid = row_loop_grid(M, cap, two ? 2 : 4);
+  int grid = row_loop_grid(M, cap, two ? 2 : 4);
+  // (the erf form of GELU is the most expensive table to fill: wide rows take two workgroups per CU - 4096 x 11008:
+  // 43.3 -> 39.4 us, 2048 rows: 25.8 -> 23.8, 16 384 rows: 176 -> 167; SiLU and the product keep the short loops)
+  if (!two && act == HYC_ACT_GELU_TANH && geo.threads >= 512 && grid > 512) grid = 512;
   hipStream_t st = begin_launch(stream);
   const int use_lut = !two && lut_pays(M, grid, geo.threads, LUT_PAYS_OTHER);
 #define HYC_EW(B_, L_, A_, N_, MT_)                                                                                \
