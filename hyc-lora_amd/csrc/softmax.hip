@@ -63,7 +63,8 @@ k_softmax_fwd(const uint16_t* __restrict__ x, int64_t rows, int64_t N, float thr
 // reductions only (no barrier), exp evaluated once per element, the next row requested before this one is processed.
 // CAUSAL: row r belongs to query position r % period and sees columns 0..position only; the rest of the row is
 // neither read (x may hold anything there) nor exponentiated, and comes out as exact zeros.
-template <int CPL, bool CAUSAL>
+// FULL: the row is exactly 512 CPL entries, every lane owns CPL chunks and nothing is predicated on that.
+template <int CPL, bool CAUSAL, bool FULL>
 __global__ void __launch_bounds__(256)
 k_softmax_fwd_wave(const uint16_t* x, int64_t rows, int64_t N, float thr, uint16_t* y,   // y may be x (in place)
                    int32_t* __restrict__ counts, int64_t period) {
@@ -74,7 +75,7 @@ k_softmax_fwd_wave(const uint16_t* x, int64_t rows, int64_t N, float thr, uint16
   int64_t row = (int64_t)blockIdx.x * 4 + wave;
   bool on[CPL];
 #pragma unroll
-  for (int u = 0; u < CPL; ++u) on[u] = lane + 64 * u < nch;
+  for (int u = 0; u < CPL; ++u) on[u] = FULL || lane + 64 * u < nch;
   // last visible column of the current row (everything when not causal); rows advance by a fixed stride, so the
   // position advances by stride mod period with one conditional subtraction
   const int per = CAUSAL ? (int)period : 1;
@@ -327,11 +328,13 @@ int hyc_softmax_fwd(const void* x, int64_t rows, int64_t N, float threshold, voi
     // one row per wave: a capped grid whose waves loop over rows is 6-15 % slower (the dispatcher balances short waves better)
     const int64_t blocks = (rows + 3) / 4, cap = blocks;
     const dim3 grid((unsigned)(blocks < cap ? blocks : cap));
-#define HYC_SMW(C_)                                                                                                \
-  hipLaunchKernelGGL((k_softmax_fwd_wave<C_, false>), grid, dim3(256), 0, st, static_cast<const uint16_t*>(x), rows, N, \
+#define HYC_SMW_F(C_, F_)                                                                                          \
+  hipLaunchKernelGGL((k_softmax_fwd_wave<C_, false, F_>), grid, dim3(256), 0, st, static_cast<const uint16_t*>(x), rows, N, \
                      thr, static_cast<uint16_t*>(y), counts, (int64_t)1)
+#define HYC_SMW(C_) do { if ((C_) > 1 && N == 512 * (C_)) HYC_SMW_F(C_, true); else HYC_SMW_F(C_, false); } while (0)
     if (cpl <= 1) HYC_SMW(1); else if (cpl <= 2) HYC_SMW(2); else if (cpl <= 4) HYC_SMW(4); else HYC_SMW(8);
 #undef HYC_SMW
+#undef HYC_SMW_F
   } else if (x) {
     const int64_t cap = 256 * 8;
     hipLaunchKernelGGL(k_softmax_fwd, dim3((unsigned)(rows < cap ? rows : cap)), dim3(256), 0, st,
@@ -359,11 +362,13 @@ int hyc_softmax_causal_fwd(const void* x, int64_t rows, int64_t N, int64_t perio
   const int cpl = (int)((N / 8 + 63) / 64);
   const int64_t blocks = (rows + 3) / 4, cap = blocks;        // one row per wave, see hyc_softmax_fwd
   const dim3 grid((unsigned)(blocks < cap ? blocks : cap));
-#define HYC_SMC(C_)                                                                                               \
-  hipLaunchKernelGGL((k_softmax_fwd_wave<C_, true>), grid, dim3(256), 0, st, static_cast<const uint16_t*>(x), rows, N, \
+#define HYC_SMC_F(C_, F_)                                                                                         \
+  hipLaunchKernelGGL((k_softmax_fwd_wave<C_, true, F_>), grid, dim3(256), 0, st, static_cast<const uint16_t*>(x), rows, N, \
                      thr, static_cast<uint16_t*>(y), counts, period)
+#define HYC_SMC(C_) do { if ((C_) > 1 && N == 512 * (C_)) HYC_SMC_F(C_, true); else HYC_SMC_F(C_, false); } while (0)
   if (cpl <= 1) HYC_SMC(1); else if (cpl <= 2) HYC_SMC(2); else if (cpl <= 4) HYC_SMC(4); else HYC_SMC(8);
 #undef HYC_SMC
+#undef HYC_SMC_F
   return check_launch("hyc_softmax_causal_fwd");
 }
 
