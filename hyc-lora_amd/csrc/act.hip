@@ -804,7 +804,7 @@ k_act_bwd(const uint16_t* __restrict__ g, const uint8_t* __restrict__ stored, co
           }
           unpack8(graw[i], gv);
           if (!(HAS_LUT && use_lut && lut_grad8(lut, xr, gv, o))) act_grad8<ACT>(xv, gv, o);
-          *reinterpret_cast<uint4*>(dx + row * H + col) = pack8(o);
+          store_stream(dx + row * H + col, pack8(o));
         }
       }
     }

@@ -54,7 +54,7 @@ k_decompress_chan(const uint8_t* __restrict__ stored, const uint16_t* __restrict
         const uint2 w = *reinterpret_cast<const uint2*>(sr + 8 * c);
 #pragma unroll
         for (int i = 0; i < NSEG; ++i) {
-          *reinterpret_cast<uint4*>(xr + i * SEG + 8 * c) = decode_chan_pk<BITS>(w.x, w.y, i, c, CPS, a, vr, scr);
+          store_stream(xr + i * SEG + 8 * c, decode_chan_pk<BITS>(w.x, w.y, i, c, CPS, a, vr, scr));
         }
       }
     }

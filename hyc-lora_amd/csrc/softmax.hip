@@ -50,7 +50,7 @@ k_softmax_fwd(const uint16_t* __restrict__ x, int64_t rows, int64_t N, float thr
         v[j] = bfr(expf(v[j] - m) / l);
         kept += (v[j] > thr) ? 1 : 0;
       }
-      *reinterpret_cast<uint4*>(yr + 8 * c) = pack8(v);
+      store_stream(yr + 8 * c, pack8(v));
     }
     if (counts) {
       const float total = block_sum((float)kept, red);
