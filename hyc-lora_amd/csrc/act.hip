@@ -148,6 +148,12 @@ static int gated_row_parts(int cps, int most, int lpg) {
   return 0;
 }
 
+// the packed code word of a row chunk: written once, read again only in the backward pass
+__device__ __forceinline__ void store_codes(uint8_t* p, uint32_t lo, uint32_t hi) {
+  const u32x2_t t = {lo, hi};
+  __builtin_nontemporal_store(t, reinterpret_cast<u32x2_t*>(p));
+}
+
 static inline int lut_pays(int64_t M, int grid, int threads, int64_t least) {
   const int64_t rows_per_wg = (M + grid - 1) / grid;
   return rows_per_wg * threads >= least;
@@ -627,9 +633,9 @@ k_gated_act_fwd_fast(const uint16_t* __restrict__ gate, int64_t ldg, const uint1
       if (leader) sg.scales[scoff + i * seg_groups] = f_to_bf(s);
       if (BITS == 8) { lo_g = cl; hi_g = ch; } else { lo_g |= cl << (i * BITS); hi_g |= ch << (i * BITS); }
     }
-    *reinterpret_cast<uint2*>(sa.stored + soff) = make_uint2(lo_a, hi_a);
-    *reinterpret_cast<uint2*>(su.stored + soff) = make_uint2(lo_u, hi_u);
-    *reinterpret_cast<uint2*>(sg.stored + soff) = make_uint2(lo_g, hi_g);
+    store_codes(sa.stored + soff, lo_a, hi_a);
+    store_codes(su.stored + soff, lo_u, hi_u);
+    store_codes(sg.stored + soff, lo_g, hi_g);
     if (ga) {
       sa.vals[row * sa.ca.k + c] = f_to_bf(act_value<ACT>(bf_to_f(oa)));
       for (int t = c + CPS; t < sa.ca.k; t += CPS)
@@ -748,8 +754,8 @@ k_ew_fwd_fast(const uint16_t* __restrict__ x1, int64_t ld1, const uint16_t* __re
         if (BITS == 8) { lo[n] = cl; hi[n] = ch; } else { lo[n] |= cl << (i * BITS); hi[n] |= ch << (i * BITS); }
       }
     }
-    *reinterpret_cast<uint2*>(s1.stored + soff) = make_uint2(lo[0], hi[0]);
-    if (NIN == 2) *reinterpret_cast<uint2*>(s2.stored + soff) = make_uint2(lo[NIN - 1], hi[NIN - 1]);
+    store_codes(s1.stored + soff, lo[0], hi[0]);
+    if (NIN == 2) store_codes(s2.stored + soff, lo[NIN - 1], hi[NIN - 1]);
     if (g1) {
       s1.vals[row * s1.ca.k + c] = ov1;
       for (int t = c + CPS; t < s1.ca.k; t += CPS) s1.vals[row * s1.ca.k + t] = r1[s1.ca.idx[t]];

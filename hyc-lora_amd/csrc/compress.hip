@@ -120,7 +120,7 @@ k_compress_chan_fast(const uint16_t* __restrict__ x, int64_t M, int64_t H /* row
       if (BITS == 8) { lo = cl; hi = ch; }
       else { lo |= cl << (i * BITS); hi |= ch << (i * BITS); }
     }
-    *reinterpret_cast<uint2*>(sp) = make_uint2(lo, hi);
+    { const u32x2_t t = {lo, hi}; __builtin_nontemporal_store(t, reinterpret_cast<u32x2_t*>(sp)); }   // (read again only in the backward pass)
     if (gather) {
       vp[c] = o;
       for (int t = c + CPS; t < a.k; t += CPS) vp[t] = xrow[a.idx[t]];   // only when k exceeds the workgroup size
