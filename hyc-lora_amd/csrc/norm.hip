@@ -206,9 +206,17 @@ norm_fwd_fast_rows(const uint16_t* __restrict__ x, const void* __restrict__ w, c
     // ahead; one with a short queue) goes into the stage that was read one row ago
     store_b16(rs_v, vo, (uint16_t)og);
     __builtin_amdgcn_sched_barrier(0);
-    og = request_outlier(row + stride);
-    __builtin_amdgcn_sched_barrier(0);
-    request(row + (D - 1) * stride, st_b >= STAGE_B ? st_b - STAGE_B : st_b + (D - 1) * STAGE_B);
+    if (D > 2) {
+      og = request_outlier(row + stride);
+      __builtin_amdgcn_sched_barrier(0);
+      request(row + (D - 1) * stride, st_b >= STAGE_B ? st_b - STAGE_B : st_b + (D - 1) * STAGE_B);
+    } else {
+      // a queue of two: the next row's entry is requested here, so it has to be older than the register that will
+      // vouch for it (with three stages that entry went out one row earlier)
+      request(row + stride, st_b >= STAGE_B ? st_b - STAGE_B : st_b + STAGE_B);
+      __builtin_amdgcn_sched_barrier(0);
+      og = request_outlier(row + stride);
+    }
     __builtin_amdgcn_sched_barrier(0);
     float ss = 0.f;
     uint32_t lo = 0, hi = 0;
@@ -1288,7 +1296,7 @@ int hyc_rmsnorm_bwd(const void* dy, const void* stored, const void* vals, const 
 // device holds its own copy of the array) and kept.
 static __device__ __align__(256) float scratch[HYC_RMSNORM_BWD_STATIC_MAX_FLOATS];
 
-static int static_scratch(float** out) {
+static int static_scratch(float** out, hipStream_t stream) {
   static std::atomic<float*> per_device[64];
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
@@ -1296,6 +1304,17 @@ static int static_scratch(float** out) {
   if (dev < 0 || dev >= 64) return fail(HYC_ENOTSUP, "hyc_rmsnorm_bwd_static: device ordinal %d (0..63 are covered)", dev);
   float* p = per_device[dev].load(std::memory_order_acquire);
   if (!p) {
+    // asking the runtime for the address is not a stream operation: under a capture it could fail or end the capture,
+    // so a first call that arrives there is refused instead (any earlier call on this device, M = 0 included, avoids it)
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    e = hipStreamIsCapturing(stream, &cap);
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      return fail(HYC_ELAUNCH, "hyc_rmsnorm_bwd_static: hipStreamIsCapturing: %s", hipGetErrorString(e));
+    }
+    if (cap != hipStreamCaptureStatusNone)
+      return fail(HYC_EINVAL, "hyc_rmsnorm_bwd_static: the first call on a device resolves the workspace address and must be "
+                  "made outside a stream capture (a call with M = 0 is enough)");
     void* sym = nullptr;
     e = hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch));
     if (e != hipSuccess || !sym) {
@@ -1320,8 +1339,9 @@ int hyc_rmsnorm_bwd_static(const void* dy, const void* stored, const void* vals,
                 "use hyc_rmsnorm_bwd with a caller workspace", (long long)rows, (long long)H,
                 (long long)HYC_RMSNORM_BWD_STATIC_MAX_FLOATS);
   float* partials = nullptr;
-  const int rc = static_scratch(&partials);
+  const int rc = static_scratch(&partials, static_cast<hipStream_t>(stream));
   if (rc) return rc;
+  if (M == 0) return HYC_OK;                     // nothing to do: the call has resolved the workspace address
   return norm_bwd_impl(dy, stored, vals, scales, w, w_dtype, rstd, nullptr, M, H, d, c2_quirk, dx, partials, dw, stream);
 }
 

@@ -378,7 +378,7 @@ struct ChanArgs {           // HYC_MODE_CHANNEL
   int k;                    // outlier channels
   int groups_per_row;       // H / G
   int chunk_to_group_shift; // log2(G/8)
-  int absmax;               // group scale rule: 0 = (max - min) / (2^b - 1), 1 = max|x| / (2^(b-1) - 1)
+  int absmax;               // group scale rule: 0 = bf16(bf16(max - min) / (2^b - 1)), 1 = bf16(bf16(2 max|x|) / (2^b - 1)) (1-bit: max|x|)
 };
 
 struct ThrArgs {            // HYC_MODE_THRESHOLD

@@ -55,18 +55,21 @@ def _need_weight(w, H):
 
 def threshold_value(t):
     """Python float of a threshold.  A device tensor costs one host round trip the first time; the float is then kept
-    on the tensor object, so the frozen threshold of a calibrated module (the same 0-d tensor call after call) is
-    read back once, not at every step.  (A caller that changes such a tensor in place must drop `_hyc_float`.)"""
+    on the tensor object together with the tensor's version counter, so the frozen threshold of a calibrated module
+    (the same 0-d tensor call after call) is read back once, not at every step, and an in-place update of the tensor
+    (`copy_`, `mul_`, a restored state) is seen.  The read-back is a synchronisation: the calibration calls of a module
+    must run outside a stream capture."""
     if not isinstance(t, torch.Tensor):
         return float(t)
-    v = getattr(t, "_hyc_float", None)
-    if v is None:
-        v = float(t)
+    cached = getattr(t, "_hyc_float", None)
+    version = t._version
+    if cached is None or cached[0] != version:
+        cached = (version, float(t))
         try:
-            t._hyc_float = v
+            t._hyc_float = cached
         except AttributeError:
             pass
-    return v
+    return cached[1]
 
 
 def num_outlier_channels(H, ratio):
@@ -146,8 +149,11 @@ def _check_plan(plan, device=None):
                              "calibration state to the GPU (load_calibration_state does)" % name)
         if t.dtype != torch.int32 or not t.is_contiguous() or t.numel() != n:
             raise ValueError("%s must be a contiguous int32 tensor of %d elements" % (name, n))
-        if device is not None and t.device != device:
-            raise ValueError("%s lives on %s, the activation on %s" % (name, t.device, device))
+        if device is not None:
+            want = torch.device(device)
+            index = want.index if want.index is not None else torch.cuda.current_device()
+            if t.device.type != want.type or t.device.index != index:
+                raise ValueError("%s lives on %s, the activation on %s" % (name, t.device, device))
     if plan.scale_rule not in SCALE_RULES:
         raise ValueError("scale_rule must be 'absmax' or 'range', got %r" % (plan.scale_rule,))
 

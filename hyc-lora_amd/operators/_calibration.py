@@ -147,6 +147,8 @@ def load_calibration_state(model, state, strict=True, device=None):
                     site.plan = K.ChannelPlan(val["H"], val["k"], place(val["idx"]).to(torch.int32).contiguous(),
                                               place(val["plan"]).to(torch.int32).contiguous(),
                                               val.get("scale_rule", "range"))
+                    # a site that is still calibrating plans again on its next call: with the rule it was saved with
+                    site.scale_rule = site.plan.scale_rule
     if strict and unknown:
         raise KeyError("no memory-efficient module named %s" % ", ".join(unknown))
     return unknown

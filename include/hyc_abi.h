@@ -185,7 +185,9 @@ int hyc_rmsnorm_bwd(const void* dy, const void* stored, const void* vals, const 
  * fp32; with 2- or 4-bit codes every width up to 16384 channels fits at any M: at most 256 rows), HYC_EINVAL beyond; dw must not be
  * NULL.  Each GPU the library runs on holds its own 16 MiB array until the process ends; every call on a GPU uses that
  * GPU's array, so two calls that overlap on one GPU (different streams) race: serialise them or use hyc_rmsnorm_bwd.
- * The first call on a device asks the runtime for the array's address (no allocation, but make it outside a capture). */
+ * The array used is the CURRENT device's: the current device must be the one that owns `stream` and the buffers.  The
+ * first call on a device asks the runtime for the array's address (no allocation); that call must come outside a stream
+ * capture (HYC_EINVAL under one) - a call with M = 0 does it and launches nothing. */
 #define HYC_RMSNORM_BWD_STATIC_MAX_FLOATS (4 * 1024 * 1024)
 int hyc_rmsnorm_bwd_static(const void* dy, const void* stored, const void* vals, const void* scales, const void* w,
                            int32_t w_dtype, const float* rstd, int64_t M, int64_t H, const hyc_desc* d, int32_t c2_quirk,

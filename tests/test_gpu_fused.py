@@ -300,6 +300,34 @@ def test_layernorm_forward_channel(K, bits, group, M, H, k, wdt, with_bias):
         K.layernorm_fwd_compress_channel(xd, w.cuda(), torch.zeros(H - 8, dtype=wdt, device="cuda"), 1e-5, plan, bits, group)
 
 
+@pytest.mark.parametrize("rule", ["absmax", "range"])
+@pytest.mark.parametrize("group,M,H,k", [(64, 2100, 11008, 110), (128, 2051, 13824, 138), (64, 2300, 16384, 164)])
+def test_long_rows_of_2bit_codes_with_several_rows_per_workgroup(K, group, M, H, k, rule):
+    """Rows of 2-bit codes with more than 256 chunks per segment travel through a queue of two stages (three do not fit
+    the LDS); with more rows than workgroups every workgroup walks several rows, so the entry of the next row is
+    requested while the current one is encoded.  RMSNorm and LayerNorm forward, codes / scales / outlier values bit for
+    bit against the oracle."""
+    x, gen = make_x(H + M, M, H, k // 2, 30.0)
+    x = (x.float() + 0.25).bfloat16()
+    w = 1 + 0.1 * torch.randn(H, generator=gen)
+    b = 0.1 * torch.randn(H, generator=gen)
+    xd = x.cuda()
+    plan = K.select_channels(K.channel_absmax(xd), k, rule)
+    idx = plan.idx.cpu()
+    vals, stored, scales = O.hyc_compress(x, idx, 2, group, rule)
+    y, rstd, c = K.rmsnorm_fwd_compress_channel(xd, w.cuda(), 1e-6, plan, 2, group)
+    y_o, rstd_o = O.rmsnorm_fwd(x, w, 1e-6)
+    assert torch.allclose(rstd.cpu(), rstd_o, rtol=2e-6, atol=0)
+    assert bf16_ulp_diff(y.cpu(), y_o).max() <= 1
+    assert torch.equal(c.stored.cpu(), stored) and bits_equal(c.scales.cpu(), scales) and bits_equal(c.vals.cpu(), vals)
+    y, mean, rstd, c = K.layernorm_fwd_compress_channel(xd, w.cuda(), b.cuda(), 1e-5, plan, 2, group)
+    y_o, mean_o, rstd_o = O.layernorm_fwd(x, w, b, 1e-5)
+    assert torch.allclose(mean.cpu(), mean_o, rtol=1e-5, atol=1e-6) and torch.allclose(rstd.cpu(), rstd_o, rtol=1e-5, atol=0)
+    diff = (y.cpu().float() - y_o.float()).abs()
+    assert bool(((bf16_ulp_diff(y.cpu(), y_o) <= 1) | (diff <= 2e-3)).all())
+    assert torch.equal(c.stored.cpu(), stored) and bits_equal(c.scales.cpu(), scales) and bits_equal(c.vals.cpu(), vals)
+
+
 @pytest.mark.parametrize("bits,method,rank", [(8, "per-channel", 2), (4, "per-token", 0), (2, "per-tensor", 0)])
 def test_layernorm_forward_threshold(K, bits, method, rank):
     B, S, H = 2, 24, 768

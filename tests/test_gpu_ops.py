@@ -601,6 +601,29 @@ def test_calibration_state_resume(ops, mode):
     assert torch.equal(grads[0], grads[1]) and b[0].iteration == 3
 
 
+def test_calibration_state_resume_during_calibration(ops):
+    """a state saved after ONE calibration call: the restored module plans again on its next call, and it does so with
+    the scale rule of the saved state, not with its constructor's default; what it writes out again names that rule"""
+    gen = torch.Generator().manual_seed(43)
+    kw = dict(outlier_ratio=0.02, sub_outlier_ratio=1.0, sub_outlier_bit=4, sub_outlier_quantize_method="per-channel", rank=0)
+    a = torch.nn.Sequential(ops.EfficientMemorySiLU(mode="hyc", group_size=64, scale_rule="range", **kw))
+    xs = [(0.5 + torch.randn(2, 32, 512, generator=gen)).bfloat16().cuda() for _ in range(3)]
+    a(xs[0].clone().requires_grad_(True))
+    b = torch.nn.Sequential(ops.EfficientMemorySiLU(mode="hyc", group_size=64, **kw))       # default rule: "absmax"
+    ops.load_calibration_state(b, ops.calibration_state(a))
+    assert b[0].iteration == 1 and b[0].site.scale_rule == "range"
+    g = torch.ones_like(xs[0])
+    for x in xs[1:]:
+        grads = []
+        for m in (a, b):
+            xi = x.clone().requires_grad_(True)
+            m(xi).backward(g)
+            grads.append(xi.grad)
+        assert torch.equal(grads[0], grads[1])
+    assert b[0].site.plan.scale_rule == "range"
+    assert ops.calibration_state(b)["0"]["site"]["scale_rule"] == "range"
+
+
 # ------------------------------------------------------------------ NF4 frozen base
 @pytest.mark.parametrize("shape", [(64,), (128, 192), (4096, 512)])
 def test_nf4_kernels(K, shape):
