@@ -13,7 +13,7 @@ MODE_CHANNEL, MODE_THRESHOLD, MODE_DENSE = 0, 1, 2
 DTYPE_BF16, DTYPE_F32 = 0, 1
 ACT_SILU, ACT_GELU_TANH = 0, 1
 SCALE_RANGE, SCALE_ABSMAX = 0, 1
-ABI_VERSION = 2
+ABI_VERSION = 3
 RMSNORM_BWD_STATIC_MAX_FLOATS = 4 * 1024 * 1024
 EINVAL, EFAULT, ENOTSUP, ELAUNCH = -22, -14, -95, -5
 
@@ -72,6 +72,7 @@ SIGNATURES = {
                                           c_ptr] + [c_ptr] * 6 + [c_ptr]),
     "hyc_softmax_fwd": (c_i32, [c_ptr, c_i64, c_i64, c_f32, c_ptr, c_ptr, c_ptr]),
     "hyc_softmax_causal_fwd": (c_i32, [c_ptr, c_i64, c_i64, c_i64, c_f32, c_ptr, c_ptr, c_ptr]),
+    "hyc_csr_offsets": (c_i32, [c_ptr, c_i64, c_i64, c_ptr, c_ptr, c_ptr]),
     "hyc_softmax_fill": (c_i32, [c_ptr, c_i64, c_i64, c_f32, c_ptr, c_ptr, c_ptr, c_ptr]),
     "hyc_softmax_bwd": (c_i32, [c_ptr, c_i64, c_i64, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr]),
     "hyc_softmax_dense": (c_i32, [c_i64, c_i64, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr]),

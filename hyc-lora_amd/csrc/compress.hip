@@ -328,6 +328,7 @@ k_outlier_fill(const uint16_t* __restrict__ x, int64_t M, int64_t H, ThrArgs a, 
   const int64_t s_pos = row % a.S;
   const int64_t nch = H / 8;
   const int64_t base = row_ptr[row];
+  const int limit = (int)(row_ptr[row + 1] - base);        // the row's room in cols / vals
   int32_t* cols_row = cols + base;
   uint16_t* vals_row = vals + base;
   int running = 0;
@@ -345,13 +346,13 @@ k_outlier_fill(const uint16_t* __restrict__ x, int64_t M, int64_t H, ThrArgs a, 
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       if ((m >> j) & 1u) {
-        stage_entry(stage, pos, (int)(8 * cc + j), f_to_bf(v[j]), cols_row, vals_row);   // the value after the base was removed
+        stage_entry(stage, pos, limit, (int)(8 * cc + j), f_to_bf(v[j]), cols_row, vals_row);   // the value after the base was removed
         ++pos;
       }
     }
     running += __builtin_amdgcn_readlane(incl, 63);
   }
-  stage_flush(stage, running, cols_row, vals_row);
+  stage_flush(stage, running, limit, cols_row, vals_row);
 }
 
 // ---- launch helpers -------------------------------------------------------------------------------

@@ -178,6 +178,41 @@ k_softmax_count(const uint16_t* __restrict__ y, int64_t rows, int64_t N, float t
   if (lane == 0) counts[row] = (int32_t)total;
 }
 
+// Row offsets of a CSR structure from the per-row counts, in one workgroup: row_ptr[r] = min(capacity, counts[0] + ... +
+// counts[r - 1]) for r = 0 .. rows, and the uncut total.  A thread adds a run of consecutive counts, the runs are
+// scanned over the workgroup (64-bit: the total may exceed what the buffers hold), then every thread writes its run.
+constexpr int OFFS_THREADS = 1024;
+__global__ void __launch_bounds__(OFFS_THREADS)
+k_csr_offsets(const int32_t* __restrict__ counts, int64_t rows, int64_t capacity, int32_t* __restrict__ row_ptr,
+              int64_t* __restrict__ total) {
+  __shared__ long long wave_sum_[OFFS_THREADS / 64];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t per = (rows + OFFS_THREADS - 1) / OFFS_THREADS;
+  const int64_t i0 = (int64_t)tid * per, i1 = i0 + per < rows ? i0 + per : rows;
+  long long mine = 0;
+  for (int64_t i = i0; i < i1; ++i) mine += counts[i];
+  long long incl = mine;                                    // inclusive scan over the wave
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const long long up = __shfl_up(incl, d);
+    if (lane >= d) incl += up;
+  }
+  if (lane == 63) wave_sum_[wave] = incl;
+  __syncthreads();
+  long long before = 0, all = 0;
+#pragma unroll
+  for (int w = 0; w < OFFS_THREADS / 64; ++w) { const long long t = wave_sum_[w]; all += t; before += w < wave ? t : 0; }
+  long long run = before + incl - mine;
+  for (int64_t i = i0; i < i1; ++i) {
+    row_ptr[i] = (int32_t)(run < capacity ? run : capacity);
+    run += counts[i];
+  }
+  if (tid == 0) {
+    row_ptr[rows] = (int32_t)(all < capacity ? all : capacity);
+    if (total) *total = all;
+  }
+}
+
 // one wave per row: ordered compaction of the kept entries (prefix sum over the lanes, entries staged in LDS and
 // stored as contiguous runs)
 __global__ void __launch_bounds__(256)
@@ -191,6 +226,7 @@ k_softmax_fill(const uint16_t* __restrict__ y, int64_t rows, int64_t N, float th
   const uint16_t* yr = y + row * N;
   const int64_t nch = N / 8;
   const int64_t base = row_ptr[row];
+  const int limit = (int)(row_ptr[row + 1] - base);        // the row's room in cols / vals
   int32_t* cols_row = cols + base;
   uint16_t* vals_row = vals + base;
   int running = 0;
@@ -212,13 +248,13 @@ k_softmax_fill(const uint16_t* __restrict__ y, int64_t rows, int64_t N, float th
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       if ((m >> j) & 1u) {
-        stage_entry(stage, pos, (int)(8 * c + j), f_to_bf(v[j]), cols_row, vals_row);
+        stage_entry(stage, pos, limit, (int)(8 * c + j), f_to_bf(v[j]), cols_row, vals_row);
         ++pos;
       }
     }
     running += __builtin_amdgcn_readlane(incl, 63);
   }
-  stage_flush(stage, running, cols_row, vals_row);
+  stage_flush(stage, running, limit, cols_row, vals_row);
 }
 
 // the same for rows of up to 4096 entries with every load of the row issued up front (CPL chunks per lane)
@@ -238,6 +274,7 @@ k_softmax_fill_wave(const uint16_t* __restrict__ y, int64_t rows, int64_t N, flo
   for (int u = 0; u < CPL; ++u)
     raw[u] = lane + 64 * u < nch ? *reinterpret_cast<const uint4*>(yr + 8 * (lane + 64 * u)) : make_uint4(0, 0, 0, 0);
   const int64_t base = row_ptr[row];
+  const int limit = (int)(row_ptr[row + 1] - base);        // the row's room in cols / vals
   int32_t* cols_row = cols + base;
   uint16_t* vals_row = vals + base;
   int running = 0;
@@ -258,14 +295,14 @@ k_softmax_fill_wave(const uint16_t* __restrict__ y, int64_t rows, int64_t N, flo
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         if ((m >> j) & 1u) {
-          stage_entry(stage, pos, 8 * c + j, f_to_bf(v[j]), cols_row, vals_row);
+          stage_entry(stage, pos, limit, 8 * c + j, f_to_bf(v[j]), cols_row, vals_row);
           ++pos;
         }
       }
     }
     running += __builtin_amdgcn_readlane(incl, 63);
   }
-  stage_flush(stage, running, cols_row, vals_row);
+  stage_flush(stage, running, limit, cols_row, vals_row);
 }
 
 // one wave per row; the output row is assembled in LDS (zeros + kept entries) and written out coalesced.
@@ -371,6 +408,14 @@ int hyc_softmax_causal_fwd(const void* x, int64_t rows, int64_t N, int64_t perio
 #undef HYC_SMC
 #undef HYC_SMC_F
   return check_launch("hyc_softmax_causal_fwd");
+}
+
+int hyc_csr_offsets(const int32_t* counts, int64_t rows, int64_t capacity, int32_t* row_ptr, int64_t* total, void* stream) {
+  if (rows < 0) return fail(HYC_EINVAL, "hyc_csr_offsets: rows=%lld", (long long)rows);
+  if (!row_ptr || (rows > 0 && !counts)) return fail(HYC_EFAULT, "hyc_csr_offsets: null buffer");
+  if (capacity < 0 || capacity > 0x7FFFFFFFll) capacity = 0x7FFFFFFFll;          // row_ptr is int32
+  hipLaunchKernelGGL(k_csr_offsets, dim3(1), dim3(OFFS_THREADS), 0, begin_launch(stream), counts, rows, capacity, row_ptr, total);
+  return check_launch("hyc_csr_offsets");
 }
 
 int hyc_softmax_fill(const void* y, int64_t rows, int64_t N, float threshold, const int32_t* row_ptr, int32_t* cols,

@@ -21,23 +21,27 @@ __device__ __forceinline__ int wave_inclusive_scan(int v) {
 
 // The kept entries (column, bf16 bits) of one row, in column order.  The first STAGE_CAP of them wait in the wave's
 // staging row (one 32-bit word each: column in the low half, value in the high half; columns stay below 65 536) and
-// leave through flush(); entries beyond that go to memory one by one.
+// leave through flush(); entries beyond that go to memory one by one.  `limit` = the room the row has in cols / vals
+// (row_ptr[row + 1] - row_ptr[row]): it equals the row's count unless the caller's offsets were cut off at the capacity
+// of its buffers, in which case the entries past it are dropped (the caller learns of it from the total it asked for).
 constexpr int STAGE_CAP = 1024;
 
-__device__ __forceinline__ void stage_entry(uint32_t* stage, int pos, int col, uint16_t bits, int32_t* cols_row, uint16_t* vals_row) {
+__device__ __forceinline__ void stage_entry(uint32_t* stage, int pos, int limit, int col, uint16_t bits, int32_t* cols_row,
+                                            uint16_t* vals_row) {
   if (pos < STAGE_CAP) {
     stage[pos] = (uint32_t)col | ((uint32_t)bits << 16);
-  } else {
+  } else if (pos < limit) {
     cols_row[pos] = col;
     vals_row[pos] = bits;
   }
 }
 
 // `count` = entries of the row; every lane of the wave calls this after the last stage_entry() of the row
-__device__ __forceinline__ void stage_flush(const uint32_t* stage, int count, int32_t* cols_row, uint16_t* vals_row) {
+__device__ __forceinline__ void stage_flush(const uint32_t* stage, int count, int limit, int32_t* cols_row, uint16_t* vals_row) {
   __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");   // the other lanes' staging writes before these reads
   __builtin_amdgcn_wave_barrier();
   const int lane = threadIdx.x & 63;
+  count = count < limit ? count : limit;
   const int n = count < STAGE_CAP ? count : STAGE_CAP;
   for (int e = lane; e < n; e += 64) {
     const uint32_t w = stage[e];

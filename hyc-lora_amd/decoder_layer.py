@@ -282,7 +282,8 @@ class _AttentionFunc(torch.autograd.Function):
                 p, _ = K.softmax_fwd(scores, causal_period=s, inplace=True)
                 kept.append(p)                                     # kept whole, in bf16
             elif not calibrating:
-                p, sp = K.softmax_fwd(scores, K.threshold_value(mod.static_value), causal_period=s, inplace=True)
+                p, sp = K.softmax_fwd(scores, K.threshold_value(mod.static_value), causal_period=s, inplace=True,
+                                      budget=K.kept_budget(mod.static_value))
                 kept.append(sp)
             else:
                 p, _ = K.softmax_fwd(scores, causal_period=s, inplace=True)

@@ -72,6 +72,106 @@ def threshold_value(t):
     return cached[1]
 
 
+class KeptBudget:
+    """Room for the sparse side data (kept softmax probabilities, element outliers) of one calibrated site, so that its
+    steady-state calls never wait for the GPU.
+
+    The reference reads the number of kept entries back on every call (`to_sparse()`, compress_function.py:153, :269)
+    before it can allocate them.  Here a call that has a budget allocates `capacity(rows)` entries - 1.25 x the largest
+    kept fraction seen so far, plus a little - cuts the row offsets off at that capacity on the device (hyc_csr_offsets)
+    and leaves the true total in a device word.  Entries past the capacity are dropped, which must not go unnoticed: the
+    total travels to pinned host memory behind the kernels, and the next call of the site that finds it arrived checks
+    it (`poll`), raises if entries were dropped and grows the budget.  `sync_check()` does the same at once.
+    """
+    MARGIN = 1.25
+
+    def __init__(self):
+        self.per_row = -1.0        # largest kept entries per row seen (negative: nothing seen yet)
+        self._pending = []         # (event, pinned int64 scalar, capacity, rows) of calls not checked yet
+        self._spare = []           # pinned scalars to use again
+
+    @property
+    def ready(self):
+        return self.per_row >= 0.0
+
+    def observe(self, nnz, rows):
+        self.per_row = max(self.per_row, nnz / max(rows, 1))
+
+    def capacity(self, rows):
+        return int(self.per_row * self.MARGIN * rows) + rows // 8 + 1024
+
+    def watch(self, total, capacity, rows):
+        """keep an eye on `total` (int64 device scalar of a call that was given `capacity`)"""
+        if torch.cuda.is_current_stream_capturing():
+            return                                  # a captured call is checked by whoever replays it (SparseRows.total)
+        host = self._spare.pop() if self._spare else torch.empty((), dtype=torch.int64, pin_memory=True)
+        host.copy_(total, non_blocking=True)
+        done = torch.cuda.Event()
+        done.record()
+        self._pending.append((done, host, capacity, rows))
+
+    def _check(self, host, capacity, rows):
+        n = int(host)
+        self._spare.append(host)
+        self.observe(n, rows)
+        if n > capacity:
+            raise RuntimeError("a compressed activation kept %d sparse entries but its buffers were sized for %d "
+                               "(1.25 x the largest share seen before): the entries beyond were dropped and the "
+                               "gradients computed from that call are not exact.  The budget has been raised; "
+                               "repeat the step." % (n, capacity))
+
+    def poll(self):
+        """check the calls whose totals have arrived; never waits (and asks nothing of the runtime during a capture)"""
+        if torch.cuda.is_current_stream_capturing():
+            return
+        while self._pending and self._pending[0][0].query():
+            _, host, capacity, rows = self._pending.pop(0)
+            self._check(host, capacity, rows)
+
+    def sync_check(self):
+        """wait for every watched call and check it"""
+        while self._pending:
+            done, host, capacity, rows = self._pending.pop(0)
+            done.synchronize()
+            self._check(host, capacity, rows)
+
+
+def kept_budget(threshold):
+    """The KeptBudget that travels with a threshold tensor (created on first use; None for a plain number).  A site that
+    is still calibrating measures a fresh threshold tensor on every call, so each of its calls finds a new budget and
+    sizes its buffers exactly; the frozen threshold of a calibrated site is the same tensor call after call, so its
+    first steady-state call reads the total back once and the later ones do not."""
+    if not isinstance(threshold, torch.Tensor):
+        return None
+    budget = getattr(threshold, "_hyc_budget", None)
+    if budget is None:
+        budget = KeptBudget()
+        try:
+            threshold._hyc_budget = budget
+        except AttributeError:
+            return None
+    return budget
+
+
+def _csr_offsets(lib, counts, rows, budget):
+    """(row_ptr, nnz to allocate, total) from per-row counts.  Without a budget, or with one that has seen nothing yet,
+    the total is read back (one host round trip) and the buffers are exact; otherwise nothing waits."""
+    dev = counts.device
+    row_ptr = torch.empty(rows + 1, dtype=torch.int32, device=dev)
+    total = torch.empty((), dtype=torch.int64, device=dev)
+    if budget is not None and budget.ready:
+        budget.poll()
+        cap = budget.capacity(rows)
+        check(lib.hyc_csr_offsets(_p(counts), rows, cap, _p(row_ptr), _p(total), _stream()))
+        budget.watch(total, cap, rows)
+        return row_ptr, cap, total
+    check(lib.hyc_csr_offsets(_p(counts), rows, -1, _p(row_ptr), _p(total), _stream()))
+    nnz = int(total.item())
+    if budget is not None:
+        budget.observe(nnz, rows)
+    return row_ptr, nnz, total
+
+
 def num_outlier_channels(H, ratio):
     """k = floor(ratio*H + 1/2)"""
     import math
@@ -298,9 +398,10 @@ def fit_rows(L, S):
     return out
 
 
-def compress_threshold(x2d, S, threshold, scale, bits, L=None, R=None):
+def compress_threshold(x2d, S, threshold, scale, bits, L=None, R=None, budget=None):
     """codes + CSR outliers of x [M,H] (row m is sequence position m mod S).  One host read-back
-    (the outlier total) sizes the CSR arrays, as `.to_sparse()` does in the reference."""
+    (the outlier total) sizes the CSR arrays, as `.to_sparse()` does in the reference; with a KeptBudget that has seen
+    a call they are sized ahead of time and nothing waits."""
     _need(x2d, BF16, "x")
     _need(scale, BF16, "scale")
     M, H = x2d.shape
@@ -314,9 +415,7 @@ def compress_threshold(x2d, S, threshold, scale, bits, L=None, R=None):
     counts = torch.empty(M, dtype=torch.int32, device=dev)
     d = threshold_desc(threshold, scale, bits, S, H, L, R)
     check(lib.hyc_compress(_p(x2d), M, H, ctypes.byref(d), _p(stored), None, None, _p(counts), _stream()))
-    row_ptr = torch.zeros(M + 1, dtype=torch.int32, device=dev)
-    torch.cumsum(counts, 0, out=row_ptr[1:])
-    nnz = int(row_ptr[-1].item())
+    row_ptr, nnz, _ = _csr_offsets(lib, counts, M, budget)
     cols = torch.empty(nnz, dtype=torch.int32, device=dev)
     vals = torch.empty(nnz, dtype=BF16, device=dev)
     check(lib.hyc_ref_outlier_fill(_p(x2d), M, H, ctypes.byref(d), _p(row_ptr), _p(cols) if nnz else None,
@@ -370,7 +469,7 @@ def rmsnorm_fwd_compress_channel(x2d, w, eps, plan, bits, group):
     return y, rstd, c
 
 
-def rmsnorm_fwd_compress_threshold(x2d, w, eps, S, threshold, scale, bits, L=None, R=None):
+def rmsnorm_fwd_compress_threshold(x2d, w, eps, S, threshold, scale, bits, L=None, R=None, budget=None):
     """-> (y, rstd, ThresholdCompressed of x)"""
     _need(x2d, BF16, "x")
     _need(scale, BF16, "scale")
@@ -388,9 +487,7 @@ def rmsnorm_fwd_compress_threshold(x2d, w, eps, S, threshold, scale, bits, L=Non
     d = threshold_desc(threshold, scale, bits, S, H, L, R)
     check(lib.hyc_rmsnorm_fwd_compress(_p(x2d), _p(w), _wdtype(w), float(eps), M, H, ctypes.byref(d), _p(y), _p(rstd),
                                        _p(stored), None, None, _p(counts), _stream()))
-    row_ptr = torch.zeros(M + 1, dtype=torch.int32, device=dev)
-    torch.cumsum(counts, 0, out=row_ptr[1:])
-    nnz = int(row_ptr[-1].item())
+    row_ptr, nnz, _ = _csr_offsets(lib, counts, M, budget)
     cols = torch.empty(nnz, dtype=torch.int32, device=dev)
     vals = torch.empty(nnz, dtype=BF16, device=dev)
     check(lib.hyc_ref_outlier_fill(_p(x2d), M, H, ctypes.byref(d), _p(row_ptr), _p(cols) if nnz else None,
@@ -429,7 +526,7 @@ def layernorm_fwd_compress_channel(x2d, w, bias, eps, plan, bits, group):
     return y, mean, rstd, c
 
 
-def layernorm_fwd_compress_threshold(x2d, w, bias, eps, S, threshold, scale, bits, L=None, R=None):
+def layernorm_fwd_compress_threshold(x2d, w, bias, eps, S, threshold, scale, bits, L=None, R=None, budget=None):
     """-> (y, mean, rstd, ThresholdCompressed of x)"""
     _need(x2d, BF16, "x")
     _need(scale, BF16, "scale")
@@ -449,9 +546,7 @@ def layernorm_fwd_compress_threshold(x2d, w, bias, eps, S, threshold, scale, bit
     d = threshold_desc(threshold, scale, bits, S, H, L, R)
     check(lib.hyc_layernorm_fwd_compress(_p(x2d), _p(w), _p(bias), _wdtype(w), float(eps), M, H, ctypes.byref(d), _p(y),
                                          _p(mean), _p(rstd), _p(stored), None, None, _p(counts), _stream()))
-    row_ptr = torch.zeros(M + 1, dtype=torch.int32, device=dev)
-    torch.cumsum(counts, 0, out=row_ptr[1:])
-    nnz = int(row_ptr[-1].item())
+    row_ptr, nnz, _ = _csr_offsets(lib, counts, M, budget)
     cols = torch.empty(nnz, dtype=torch.int32, device=dev)
     vals = torch.empty(nnz, dtype=BF16, device=dev)
     check(lib.hyc_ref_outlier_fill(_p(x2d), M, H, ctypes.byref(d), _p(row_ptr), _p(cols) if nnz else None,
@@ -681,30 +776,31 @@ def gradw_gemm(dy2d, src, out_dtype=BF16, alpha=1.0, out=None, beta=0.0, staged=
 class SparseRows:
     """probabilities above the threshold, CSR over the flattened leading dims"""
     row_ptr: torch.Tensor   # int32 [rows+1]
-    cols: torch.Tensor      # int32 [nnz]
+    cols: torch.Tensor      # int32 [nnz] (or the capacity a KeptBudget provided: row_ptr says what is in use)
     vals: torch.Tensor      # bf16 [nnz]
     shape: tuple
+    total: Optional[torch.Tensor] = None   # int64 0-d on the device: the entries above the threshold (> cols.numel(): some were dropped)
 
     @property
     def rows(self):
         return self.row_ptr.numel() - 1
 
 
-def _csr_from_counts(lib, y2d, threshold, counts):
+def _csr_from_counts(lib, y2d, threshold, counts, budget=None):
     rows, N = y2d.shape
     dev = y2d.device
-    row_ptr = torch.zeros(rows + 1, dtype=torch.int32, device=dev)
-    torch.cumsum(counts, 0, out=row_ptr[1:])
-    nnz = int(row_ptr[-1].item())
+    row_ptr, nnz, total = _csr_offsets(lib, counts, rows, budget)
     cols = torch.empty(nnz, dtype=torch.int32, device=dev)
     vals = torch.empty(nnz, dtype=BF16, device=dev)
     check(lib.hyc_softmax_fill(_p(y2d), rows, N, float(threshold), _p(row_ptr), _p(cols) if nnz else None,
                                _p(vals) if nnz else None, _stream()))
-    return row_ptr, cols, vals
+    return row_ptr, cols, vals, total
 
 
-def softmax_fwd(x, threshold=None, causal_period=None, inplace=False):
+def softmax_fwd(x, threshold=None, causal_period=None, inplace=False, budget=None):
     """y = softmax(x, -1) bf16; with a threshold also the kept entries (y > bf16(threshold)) as SparseRows.
+    budget: the site's KeptBudget (see there): once it has seen a call, the kept entries are sized ahead of time and the
+    call returns without waiting for the GPU.
     causal_period = S applies the causal mask of S query positions inside the kernel (row r is position r % S).
     inplace: y overwrites x (rows of at most 4096 entries: a row is held in registers before anything is written)."""
     _need(x, BF16, "x")
@@ -723,20 +819,20 @@ def softmax_fwd(x, threshold=None, causal_period=None, inplace=False):
         check(lib.hyc_softmax_causal_fwd(_p(x2), rows, N, int(causal_period), thr, _p(y), _p(counts), _stream()))
     if threshold is None:
         return y.reshape(x.shape), None
-    row_ptr, cols, vals = _csr_from_counts(lib, y, threshold, counts)
-    return y.reshape(x.shape), SparseRows(row_ptr, cols, vals, tuple(x.shape))
+    row_ptr, cols, vals, total = _csr_from_counts(lib, y, threshold, counts, budget)
+    return y.reshape(x.shape), SparseRows(row_ptr, cols, vals, tuple(x.shape), total)
 
 
-def softmax_sparsify(y, threshold):
-    """kept entries of already computed probabilities"""
+def softmax_sparsify(y, threshold, budget=None):
+    """kept entries of already computed probabilities (budget: as for softmax_fwd)"""
     _need(y, BF16, "y")
     N = y.shape[-1]
     y2 = y.reshape(-1, N)
     lib = _abi.load()
     counts = torch.empty(y2.shape[0], dtype=torch.int32, device=y.device)
     check(lib.hyc_softmax_fwd(None, y2.shape[0], N, float(threshold), _p(y2), _p(counts), _stream()))
-    row_ptr, cols, vals = _csr_from_counts(lib, y2, threshold, counts)
-    return SparseRows(row_ptr, cols, vals, tuple(y.shape))
+    row_ptr, cols, vals, total = _csr_from_counts(lib, y2, threshold, counts, budget)
+    return SparseRows(row_ptr, cols, vals, tuple(y.shape), total)
 
 
 def softmax_bwd(g, sp: SparseRows, inplace=False):

@@ -79,8 +79,10 @@ def _check_quantised(sub_outlier_bit, sub_outlier_ratio):
         raise NotImplementedError("sub_outlier_bit == 16 (no quantisation) is outside the accelerated path")
 
 
-def compress_to_csr(x, outlier, scale, sub_outlier_bit, sub_outlier_ratio, L, R):
-    """the kernels' own container (codes + CSR outliers); x is [B,S,H] or [B,nh,S,hd]"""
+def compress_to_csr(x, outlier, scale, sub_outlier_bit, sub_outlier_ratio, L, R, exact=False):
+    """the kernels' own container (codes + CSR outliers); x is [B,S,H] or [B,nh,S,hd].  exact: size the outlier arrays by
+    reading their total back (what a conversion to COO needs); otherwise a frozen threshold tensor sizes them ahead
+    of time from its second use on (kernels.KeptBudget)."""
     _check_quantised(sub_outlier_bit, sub_outlier_ratio)
     if x.dim() == 4:
         x = head_to_hidden_shape(x)
@@ -88,7 +90,8 @@ def compress_to_csr(x, outlier, scale, sub_outlier_bit, sub_outlier_ratio, L, R)
     S, H = x.shape[-2], x.shape[-1]
     rank0 = L is None or not bool(L.shape[-1]) or (L.shape[-1] == 16 and getattr(L, "_hyc_zero", False))
     c = K.compress_threshold(x.reshape(-1, H), S, K.threshold_value(outlier), scale.contiguous(), sub_outlier_bit,
-                             None if rank0 else L.contiguous(), None if rank0 else R.contiguous())
+                             None if rank0 else L.contiguous(), None if rank0 else R.contiguous(),
+                             budget=None if exact else K.kept_budget(outlier))
     return c, tuple(x.shape)
 
 
@@ -119,7 +122,7 @@ def true_divide_outlier_suboutlier_svd_compress(x: torch.Tensor, outlier: float,
                                                 sub_outlier_ratio: float = 1., L: torch.Tensor = None,
                                                 R: torch.Tensor = None):
     """-> (outliers as a sparse COO bf16 tensor, packed codes [B,S,H*bit/8] uint8 (int8 [B,S,H] for 8 bits), scale)"""
-    c, shape = compress_to_csr(x, outlier, scale, sub_outlier_bit, sub_outlier_ratio, L, R)
+    c, shape = compress_to_csr(x, outlier, scale, sub_outlier_bit, sub_outlier_ratio, L, R, exact=True)
     return csr_to_coo(c, shape), c.stored.reshape(shape[:-1] + (c.stored.shape[-1],)), scale
 
 

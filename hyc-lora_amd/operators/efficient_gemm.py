@@ -136,7 +136,7 @@ class EfficientMemoryGEMMWithSoftmaxFunc(torch.autograd.Function):
         o1 = get_statistics_softmax(x1, iteration, outlier_ratio_1) if iteration < 2 else static_value_1
         o2, L2, R2, s2 = _calibrated(x2, iteration, static_value_2, outlier_ratio_2, sub_outlier_ratio_2,
                                      sub_outlier_bit_2, sub_outlier_quantize_method_2, rank)
-        ctx.sparse = K.softmax_sparsify(x1.contiguous(), K.threshold_value(o1))
+        ctx.sparse = K.softmax_sparsify(x1.contiguous(), K.threshold_value(o1), budget=K.kept_budget(o1))
         c2, shape2 = compress_to_csr(x2, o2, s2, sub_outlier_bit_2, sub_outlier_ratio_2,
                                      L2 if rank > 0 else None, R2 if rank > 0 else None)
         ctx.saved = (c2, shape2)
@@ -158,7 +158,7 @@ class _ChannelGEMMWithSoftmaxFunc(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x1, x2, threshold, plan2, bits2, group):
         r2, (b, s2, nh) = _as_hidden_rows(x2)
-        ctx.sparse = K.softmax_sparsify(x1.contiguous(), threshold)
+        ctx.sparse = K.softmax_sparsify(x1.contiguous(), K.threshold_value(threshold), budget=K.kept_budget(threshold))
         ctx.saved = K.compress_channel(r2, plan2, bits2, group)
         ctx.geom = (b, s2, nh)
         return x1 @ x2
@@ -199,7 +199,7 @@ class EfficientMemoryGEMMWithSoftmax(torch.nn.Module):
                 o1 = self.static_value_1
             r2, _ = _as_hidden_rows(x2)
             p2 = self.site_2.channel_plan(r2, self.iteration)
-            result = _ChannelGEMMWithSoftmaxFunc.apply(x1, x2, K.threshold_value(o1), p2, self.sub_outlier_bit_2, self.group_size)
+            result = _ChannelGEMMWithSoftmaxFunc.apply(x1, x2, o1, p2, self.sub_outlier_bit_2, self.group_size)
             self.iteration += 1
             return result
         result, o1, o2, L2, R2, s2 = EfficientMemoryGEMMWithSoftmaxFunc.apply(

@@ -57,7 +57,7 @@ class EfficientMemoryLayerNormFunc(torch.autograd.Function):
             w, b = _affine(weight, bias)
             y, mean, rstd, c = K.layernorm_fwd_compress_threshold(
                 x2, w, b, eps, x.shape[-2], K.threshold_value(outlier), scale.contiguous(), sub_outlier_bit,
-                L.contiguous() if rank > 0 else None, R.contiguous() if rank > 0 else None)
+                L.contiguous() if rank > 0 else None, R.contiguous() if rank > 0 else None, budget=K.kept_budget(outlier))
         else:
             y, mean, rstd = _forward_stats(x2, weight, bias, eps)
             c, _ = compress_to_csr(x, outlier, scale, sub_outlier_bit, sub_outlier_ratio, L if rank > 0 else None,

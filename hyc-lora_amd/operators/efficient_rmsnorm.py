@@ -29,7 +29,7 @@ def _ref_forward(ctx, x, outlier_ratio, sub_outlier_ratio, sub_outlier_bit, sub_
     y, rstd, c = K.rmsnorm_fwd_compress_threshold(x2, _effective_weight(weight, weight_offset), eps, S, K.threshold_value(outlier),
                                                   scale.contiguous(), sub_outlier_bit,
                                                   L.contiguous() if rank > 0 else None,
-                                                  R.contiguous() if rank > 0 else None)
+                                                  R.contiguous() if rank > 0 else None, budget=K.kept_budget(outlier))
     ctx.saved = c
     ctx.rstd = rstd
     ctx.weight = weight

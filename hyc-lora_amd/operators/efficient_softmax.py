@@ -1,8 +1,9 @@
 """Softmax over the last dimension whose backward runs from the few probabilities above a calibrated threshold.
 
 Mirror of the reference's operators/efficient_softmax.py:10-75 (same class names, `apply` signature, `iteration` /
-`static_value` attributes).  Steady state is one kernel for y plus the per-row counts of kept entries and one kernel
-that writes them as CSR (int32 column, bf16 value); the backward reads the incoming gradient once:
+`static_value` attributes).  Steady state is one kernel for y plus the per-row counts of kept entries, one for the row
+offsets and one that writes the kept entries as CSR (int32 column, bf16 value), with no host round trip from the
+second steady-state call on (kernels.KeptBudget); the backward reads the incoming gradient once:
 dx = (g - sum_j g_j * p_j) * p with p zero outside the kept set.
 """
 import torch
@@ -22,7 +23,7 @@ class EfficientMemorySoftmaxFunc(torch.autograd.Function):
         scores = x.contiguous()
         if iteration >= _CALIBRATION_CALLS:
             threshold = static_value
-            probs, ctx.kept = K.softmax_fwd(scores, K.threshold_value(threshold))
+            probs, ctx.kept = K.softmax_fwd(scores, K.threshold_value(threshold), budget=K.kept_budget(threshold))
         else:
             # the threshold of this call comes from its own probabilities, so they are needed before the pruning
             probs, _ = K.softmax_fwd(scores)

@@ -66,7 +66,7 @@
 extern "C" {
 #endif
 
-#define HYC_ABI_VERSION 2
+#define HYC_ABI_VERSION 3
 
 /* error codes (negative errno values) */
 #define HYC_OK 0
@@ -161,7 +161,8 @@ int hyc_decompress(const void* stored, const void* vals, const void* scales, int
 /* ---- threshold-mode outliers as CSR ---------------------------------------------------------- */
 /* counts[m] = #{c : |x[m,c] - base[m,c]| > threshold} */
 int hyc_ref_outlier_count(const void* x, int64_t M, int64_t H, const hyc_desc* d, int32_t* counts, void* stream);
-/* row_ptr int32 [M+1] = exclusive prefix sums of the counts; fills cols / vals in ascending column order */
+/* row_ptr int32 [M+1] = exclusive prefix sums of the counts (or hyc_csr_offsets with a capacity: row m then keeps its
+ * first row_ptr[m+1] - row_ptr[m] outliers); fills cols / vals in ascending column order */
 int hyc_ref_outlier_fill(const void* x, int64_t M, int64_t H, const hyc_desc* d, const int32_t* row_ptr,
                          int32_t* cols, void* vals, void* stream);
 
@@ -264,7 +265,16 @@ int hyc_softmax_fwd(const void* x, int64_t rows, int64_t N, float threshold, voi
  * out as exact zeros.  1 <= period <= N <= 4096. */
 int hyc_softmax_causal_fwd(const void* x, int64_t rows, int64_t N, int64_t period, float threshold, void* y,
                            int32_t* counts, void* stream);
-/* the kept probabilities as CSR: row_ptr int32 [rows+1] (exclusive prefix sums of counts), cols ascending per row */
+/* Row offsets from per-row counts (of hyc_softmax_fwd, hyc_ref_outlier_count or the fused forwards), without the host:
+ * row_ptr int32 [rows+1], row_ptr[r] = min(capacity, counts[0] + ... + counts[r-1]); *total (int64, may be NULL) = the
+ * uncut sum.  capacity = the entries the caller's cols / vals buffers hold (negative: no limit).  With the offsets cut
+ * off at a capacity, the fill entry points keep the first row_ptr[r+1] - row_ptr[r] entries of row r and drop the rest,
+ * and every consumer reads exactly what was kept; total > capacity tells the caller that entries were dropped.  This is
+ * what lets a calibrated caller size cols / vals ahead of time (e.g. 1.25 x the kept fraction it measured) instead of
+ * reading the total back before it allocates, as the reference's to_sparse() does (compress_function.py:153, :269). */
+int hyc_csr_offsets(const int32_t* counts, int64_t rows, int64_t capacity, int32_t* row_ptr, int64_t* total, void* stream);
+/* the kept probabilities as CSR: row_ptr int32 [rows+1] (exclusive prefix sums of counts, or hyc_csr_offsets), cols
+ * ascending per row; row r receives its first row_ptr[r+1] - row_ptr[r] kept entries */
 int hyc_softmax_fill(const void* y, int64_t rows, int64_t N, float threshold, const int32_t* row_ptr, int32_t* cols,
                      void* vals, void* stream);
 /* dx = (g - sum_j g_j*yh_j) * yh, yh = the CSR probabilities (zero elsewhere); dx may be g itself (in place) */

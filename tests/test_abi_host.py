@@ -33,7 +33,7 @@ def test_every_declared_symbol_is_exported_and_bound(abi):
         assert hasattr(lib, n), n
         assert n in abi.SIGNATURES, "no ctypes prototype for " + n
     assert sorted(abi.SIGNATURES) == names
-    assert lib.hyc_abi_version() == 2
+    assert lib.hyc_abi_version() == 3
 
 
 def test_desc_layout_matches_header(abi):

@@ -164,3 +164,54 @@ def test_the_other_channel_entry_points_replay(pkg, M, H, bits, group):
         assert len(got) == len(want)
         for i, (a, r) in enumerate(zip(got, want)):
             assert torch.equal(a.view(torch.uint8), r.view(torch.uint8)), "replay %d, output %d" % (rep, i)
+
+
+def test_softmax_module_replays_once_calibrated(pkg):
+    """EfficientMemorySoftmax forward + backward from its fourth call on never waits for the GPU (the kept entries are
+    sized from the site's budget, kernels.KeptBudget), so the pair can be captured; replays on fresh scores and
+    gradients equal the eager module bit for bit, and the device-side total shows that nothing was dropped."""
+    ops, K = pkg.operators, pkg.kernels
+    gen = torch.Generator(device="cuda").manual_seed(21)
+    shape = (2, 4, 256, 256)
+    mk = lambda s: (s * torch.randn(*shape, generator=gen, device="cuda")).bfloat16()
+    mod = ops.EfficientMemorySoftmax(outlier_ratio=0.02)
+    for _ in range(3):                                   # two calibration calls, one steady call that measures the budget
+        x = mk(3.0).requires_grad_(True)
+        mod(x).backward(mk(0.1))
+    assert mod.iteration == 3 and K.kept_budget(mod.static_value).ready
+    x, g = mk(3.0), mk(0.1)
+
+    def run():
+        xi = x.detach().clone().requires_grad_(True)
+        y = mod(xi)
+        kept = y.grad_fn.kept
+        y.backward(g)
+        return [y.detach(), xi.grad, kept.row_ptr, kept.total.view(1)]
+
+    def eager():
+        y, sp = K.softmax_fwd(x, K.threshold_value(mod.static_value))
+        return [y, K.softmax_bwd(g, sp), sp.row_ptr, sp.total.view(1)]
+
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        got = run()
+    for rep in range(3):
+        if rep:
+            x.copy_(mk(2.0 + rep))
+            g.copy_(mk(0.1 * rep))
+        want = [t.clone() for t in eager()]
+        for t in got[:2]:
+            t.view(torch.uint8).fill_(0xA5)
+        noise = torch.randn(1 << 16, device="cuda").cumsum(0).sum()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.isfinite(noise)
+        for i, (a, r) in enumerate(zip(got, want)):
+            assert torch.equal(a.view(torch.uint8), r.view(torch.uint8)), "replay %d, output %d" % (rep, i)

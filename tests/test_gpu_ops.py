@@ -182,6 +182,73 @@ def test_softmax_kernels(K, shape):
     assert (dx.float() == want.float()).float().mean() > 0.995
 
 
+def test_softmax_kept_entries_sized_ahead_of_time(K):
+    """A site's second call with the same threshold tensor sizes the kept entries from its budget and never reads the
+    total back: same offsets, same entries, same gradient as the exact call, and the true total in a device word.
+    With a budget that is too small the rows are cut off where the buffers end, every consumer sees exactly what was
+    kept, and the check that follows the call raises."""
+    gen = torch.Generator().manual_seed(5)
+    shape = (2, 3, 70, 1024)
+    thr = torch.tensor(0.004)
+    budget = K.kept_budget(thr)
+    assert budget is K.kept_budget(thr) and not budget.ready and K.kept_budget(0.5) is None
+    outs = []
+    for call in range(3):
+        x = (3 * torch.randn(*shape, generator=gen)).bfloat16().cuda()
+        g = (0.1 * torch.randn(*shape, generator=gen)).bfloat16().cuda()
+        y, sp = K.softmax_fwd(x, K.threshold_value(thr), budget=budget)
+        y2, exact = K.softmax_fwd(x, K.threshold_value(thr))
+        nnz = exact.cols.numel()
+        assert budget.ready and int(sp.total) == nnz == int(exact.total)
+        assert torch.equal(sp.row_ptr, exact.row_ptr) and torch.equal(sp.cols[:nnz], exact.cols) and bits_equal(sp.vals[:nnz], exact.vals)
+        assert (sp.cols.numel() == nnz) == (call == 0)          # the first call measured, the later ones provided room
+        assert bits_equal(K.softmax_bwd(g, sp), K.softmax_bwd(g, exact)) and bits_equal(K.softmax_dense(sp), K.softmax_dense(exact))
+        outs.append(sp)
+    budget.sync_check()                                          # nothing was dropped
+    # too small a budget: the offsets stop at the capacity
+    small = K.KeptBudget()
+    small.observe(nnz // 3, exact.rows)
+    small.MARGIN = 1.0
+    cap = small.capacity(exact.rows)
+    assert cap < nnz
+    y, cut = K.softmax_fwd(x, K.threshold_value(thr), budget=small)
+    assert int(cut.total) == nnz and int(cut.row_ptr[-1]) == cap and cut.cols.numel() == cap
+    assert torch.equal(cut.row_ptr, exact.row_ptr.clamp(max=cap))
+    assert torch.equal(cut.cols, exact.cols[:cap]) and bits_equal(cut.vals, exact.vals[:cap])
+    dense, want = K.softmax_dense(cut), K.softmax_dense(exact)
+    rows_kept = int((exact.row_ptr[1:] <= cap).sum())             # these rows are whole
+    assert bits_equal(dense.view(-1, shape[-1])[:rows_kept], want.view(-1, shape[-1])[:rows_kept])
+    assert int((dense.view(-1, shape[-1])[rows_kept + 1:] != 0).sum()) == 0
+    with pytest.raises(RuntimeError, match="dropped"):
+        small.sync_check()
+    assert small.capacity(exact.rows) >= nnz                      # the budget has grown
+
+
+@pytest.mark.parametrize("bits,method", [(4, "per-channel"), (8, "per-tensor")])
+def test_threshold_outliers_sized_ahead_of_time(K, bits, method):
+    """the element outliers of the reference scheme through a budget: the second call with the same threshold tensor
+    allocates ahead of time and restores the same activation as the exact call"""
+    gen = torch.Generator().manual_seed(bits)
+    B, S, H = 2, 48, 1024
+    thr = None
+    for call in range(3):
+        x = torch.randn(B, S, H, generator=gen)
+        x[..., :5] *= 12
+        x = x.bfloat16()
+        if thr is None:
+            torch.manual_seed(0)
+            thr, L, R, scale = O.get_statistics(x, 0, 0.01, 1.0, bits, method, 0)
+            thr_d, scale_d = thr.cuda(), scale.cuda()
+        x2 = x.reshape(-1, H).cuda()
+        c = K.compress_threshold(x2, S, K.threshold_value(thr_d), scale_d, bits, budget=K.kept_budget(thr_d))
+        e = K.compress_threshold(x2, S, K.threshold_value(thr_d), scale_d, bits)
+        nnz = e.cols.numel()
+        assert (c.cols.numel() == nnz) == (call == 0)
+        assert torch.equal(c.row_ptr, e.row_ptr) and torch.equal(c.cols[:nnz], e.cols) and bits_equal(c.vals[:nnz], e.vals)
+        assert torch.equal(c.stored, e.stored) and bits_equal(K.decompress_threshold(c), K.decompress_threshold(e))
+    K.kept_budget(thr_d).sync_check()
+
+
 @pytest.mark.parametrize("shape,keep", [((1, 1, 9, 4096), 0.5), ((1, 2, 5, 8192), 0.4), ((2, 1, 6, 2048), 1.0), ((1, 1, 70, 2048), 0.0)])
 def test_softmax_rows_with_many_or_no_kept_entries(K, shape, keep):
     """rows that keep more entries than a wave stages in LDS (1024) spill the rest straight to memory; rows that keep
