@@ -51,6 +51,14 @@ def rel_err(a, b):
     return float((a.double() - b.double()).norm() / b.double().norm().clamp_min(1e-30))
 
 
+def outside_tolerance(a, b, rtol=1e-2, atol=1e-3):
+    """share of the elements of `a` that miss |a - b| <= rtol |b| + atol max|b| (the bound of rtol 1e-2 / atol 1e-3 with
+    the absolute part on the scale of the tensor: gradients of different tensors differ by orders of magnitude)"""
+    a, b = a.double(), b.double()
+    bound = rtol * b.abs() + atol * b.abs().max()
+    return float(((a - b).abs() > bound).double().mean())
+
+
 def check_grads(layer, groups, xg, P, xo, tol):
     errs = {"dx": rel_err(xg.grad.cpu(), xo.grad)}
     for n, (mod, i) in groups.items():
@@ -60,6 +68,15 @@ def check_grads(layer, groups, xg, P, xo, tol):
     errs["w_post"] = rel_err(layer.post_attention_layernorm.weight.grad.cpu(), P["w_post"].grad)
     bad = {k: v for k, v in errs.items() if not v < tol}
     assert not bad, bad
+    # element by element (a norm would hide a handful of wrong elements): every element within rtol 1e-2 plus 1e-2 of
+    # the tensor's largest element (see test_layer_at_its_own_size for why the absolute part follows the scale)
+    pairs = {"dx": (xg.grad.cpu(), xo.grad), "w_in": (layer.input_layernorm.weight.grad.cpu(), P["w_in"].grad),
+             "w_post": (layer.post_attention_layernorm.weight.grad.cpu(), P["w_post"].grad)}
+    for n, (mod, i) in groups.items():
+        pairs["A_" + n] = (mod.lora_A[i].grad.cpu(), P["A_" + n].grad)
+        pairs["B_" + n] = (mod.lora_B[i].grad.cpu(), P["B_" + n].grad)
+    wrong = {n: outside_tolerance(a, b, 1e-2, 1e-2) for n, (a, b) in pairs.items()}
+    assert not any(wrong.values()), {n: v for n, v in wrong.items() if v}
     return errs
 
 
@@ -304,6 +321,26 @@ def test_layer_at_its_own_size(DL, K, B, S):
             errs["A_" + n] = err(mod.lora_A[i].grad, P["A_" + n].grad)
             errs["B_" + n] = err(mod.lora_B[i].grad, P["B_" + n].grad)
         assert all(v == v and v < 1e-2 for v in errs.values()), (step, errs)
+        # ... and element by element: a norm would hide a handful of wrong elements
+        pairs = {"y": (y.detach(), yo.detach()), "dx": (xg.grad, xo.grad),
+                 "w_in": (layer.input_layernorm.weight.grad, P["w_in"].grad),
+                 "w_post": (layer.post_attention_layernorm.weight.grad, P["w_post"].grad)}
+        for n, (mod, i) in groups.items():
+            pairs["A_" + n] = (mod.lora_A[i].grad, P["A_" + n].grad)
+            pairs["B_" + n] = (mod.lora_B[i].grad, P["B_" + n].grad)
+        # The tensors here are not of unit scale (max |ref| between 1.5 and 300), so the absolute part of rtol 1e-2 /
+        # atol 1e-3 is taken relative to the largest element of the reference.  The device computes the forward in
+        # bf16 and the oracle in fp32, so the two backward passes start from activations that differ by a bf16
+        # rounding per operator: sums over thousands of tokens of such terms land within 1e-3 of the tensor's scale of
+        # each other only on average, and the elements that are small against that scale miss the tight bound by a
+        # little (a share of the elements, largest for the dB, whose second operand h = x A^T carries the forward's
+        # rounding twice).  Hence two bounds: EVERY element within rtol 1e-2 + 1e-2 of the scale (one wrong element
+        # fails this), and the share outside the tight bound limited per kind of tensor.
+        worst = {n: outside_tolerance(a, b, 1e-2, 1e-2) for n, (a, b) in pairs.items()}
+        assert not any(worst.values()), (step, {n: v for n, v in worst.items() if v})
+        outside = {n: outside_tolerance(a, b, 1e-2, 1e-3) for n, (a, b) in pairs.items()}
+        limit = lambda n: 0.25 if n.startswith("B_") else 0.15 if n.startswith(("A_", "w_")) else 0.05 if n == "dx" else 1e-4
+        assert all(v <= limit(n) for n, v in outside.items()), (step, outside)
         del yo, xo, R, p_dev
         rec["attn"].clear()
     for h in hooks:
