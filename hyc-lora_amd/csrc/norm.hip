@@ -908,31 +908,37 @@ k_rmsnorm_bwd(const uint16_t* __restrict__ dy, const uint8_t* __restrict__ store
 }
 
 // dw[c] = sum_p partials[p, c] in a fixed order: 32 columns x 8 row lanes per workgroup, each lane sums rows
-// p = lane, lane+8, ... and the 8 lane sums are added in lane order.
+// p = lane, lane+8, ... and the 8 lane sums are added in lane order.  The kernel is one round trip to memory long, so
+// a lane asks for all of its rows at once (32 loads in flight cover the 256 partial rows of the fast backward; rows
+// past the end lie beyond the buffer resource and read zeros).
 __global__ void __launch_bounds__(256)
 k_colsum(const float* __restrict__ partials, int64_t P, int64_t H, void* __restrict__ dw, bool wf32) {
   __shared__ float part[8][33];
+  constexpr int BATCH = 32;
   const int cx = threadIdx.x & 31, lane = threadIdx.x >> 5;
   const int64_t c = (int64_t)blockIdx.x * 32 + cx;
-  float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
-  if (c < H) {
-    int64_t p = lane;
-    for (; p + 24 < P; p += 32) {
-      s0 += partials[p * H + c];
-      s1 += partials[(p + 8) * H + c];
-      s2 += partials[(p + 16) * H + c];
-      s3 += partials[(p + 24) * H + c];
-    }
-    for (; p < P; p += 8) s0 += partials[p * H + c];
+  float s = 0.f;
+  for (int64_t p0 = 0; p0 < P; p0 += 8 * BATCH) {
+    // rows p0 .. of the partial matrix as one resource (a batch spans at most 256 rows of at most 256 KB)
+    const int64_t rows = P - p0 < 8 * BATCH ? P - p0 : 8 * BATCH;
+    const BufferRsrc rs = make_rsrc(partials + p0 * H, (uint32_t)(rows * H * 4));
+    const uint32_t off = c < H ? (uint32_t)((lane * H + c) * 4) : NOWHERE;
+    float t[BATCH];
+#pragma unroll
+    for (int i = 0; i < BATCH; ++i) t[i] = __uint_as_float(load_b32(rs, off + (uint32_t)i * (uint32_t)(8 * H * 4)));
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+#pragma unroll
+    for (int i = 0; i < BATCH; i += 4) { s0 += t[i]; s1 += t[i + 1]; s2 += t[i + 2]; s3 += t[i + 3]; }
+    s += (s0 + s1) + (s2 + s3);
   }
-  part[lane][cx] = (s0 + s1) + (s2 + s3);
+  part[lane][cx] = s;
   __syncthreads();
   if (lane == 0 && c < H) {
-    float s = 0.f;
+    float tot = 0.f;
 #pragma unroll
-    for (int l = 0; l < 8; ++l) s += part[l][cx];
-    if (wf32) static_cast<float*>(dw)[c] = s;
-    else static_cast<uint16_t*>(dw)[c] = f_to_bf(s);
+    for (int l = 0; l < 8; ++l) tot += part[l][cx];
+    if (wf32) static_cast<float*>(dw)[c] = tot;
+    else static_cast<uint16_t*>(dw)[c] = f_to_bf(tot);
   }
 }
 
