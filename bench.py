@@ -395,7 +395,7 @@ def kernel_tour(pkg, torch, reps=5):
     print(json.dumps({"kernel_tour": True}))
 
 
-def layer_report(pkg, torch, steps=6, attentions=("eager", "flash"), quiet=False):
+def layer_report(pkg, torch, steps=6, attentions=("eager", "flash"), quiet=False, compressions=(True, False)):
     """full LLaMA-2-7B-shaped decoder layer (hidden 4096, 32 x 128 heads, intermediate 11008, NF4 base, LoRA r=16 on
     all seven projections), forward + backward, at batch 1 x seq 2048 and batch 4 x seq 1024: what the forward keeps
     for the backward, the peak above the resident weights, and the step time - with every saved activation compressed
@@ -404,7 +404,7 @@ def layer_report(pkg, torch, steps=6, attentions=("eager", "flash"), quiet=False
     attention kernel around compressed q, k, v and output."""
     DL = importlib.import_module("hyc-lora_amd.decoder_layer")
     out = []
-    for compress, attention in [(c, a) for c in (True, False) for a in attentions]:
+    for compress, attention in [(c, a) for c in compressions for a in attentions]:
         layer = DL.DecoderLayer(DL.LayerConfig(compress=compress, attention=attention))
         torch.cuda.synchronize()
         for (B, S) in ((1, 2048), (4, 1024)):
@@ -496,6 +496,8 @@ def main():
                     help="for rocprofv3 --pmc: 5x a plain 32 MiB device copy, 5x fwd, 5x bwd, then exit")
     ap.add_argument("--layer-report", action="store_true",
                     help="full decoder layer (the fifth BASELINE configuration): saved bytes, peak memory, step time; then exit")
+    ap.add_argument("--layer-compress", choices=["on", "off", "both"], default="both",
+                    help="with --layer-report: the layer with compressed activations, the same layer keeping bf16, or both")
     ap.add_argument("--layer-attention", choices=["eager", "flash", "both"], default="both",
                     help="with --layer-report: which attention form(s) of the layer to run")
     args = ap.parse_args()
@@ -519,7 +521,8 @@ def main():
         return
     if args.layer_report:
         del wl
-        layer_report(pkg, torch, attentions=("eager", "flash") if args.layer_attention == "both" else (args.layer_attention,))
+        layer_report(pkg, torch, attentions=("eager", "flash") if args.layer_attention == "both" else (args.layer_attention,),
+                     compressions={"on": (True,), "off": (False,), "both": (True, False)}[args.layer_compress])
         return
     if args.pmc_probe:
         dst = torch.empty_like(wl.x)

@@ -179,37 +179,65 @@ k_softmax_count(const uint16_t* __restrict__ y, int64_t rows, int64_t N, float t
 }
 
 // Row offsets of a CSR structure from the per-row counts, in one workgroup: row_ptr[r] = min(capacity, counts[0] + ... +
-// counts[r - 1]) for r = 0 .. rows, and the uncut total.  A thread adds a run of consecutive counts, the runs are
-// scanned over the workgroup (64-bit: the total may exceed what the buffers hold), then every thread writes its run.
-constexpr int OFFS_THREADS = 1024;
+// counts[r - 1]) for r = 0 .. rows, and the uncut total.  The kernel is as long as its trips to memory, so a thread
+// asks for all it can hold at once: 32 768 counts are one round of eight 16-byte loads per thread (sub-tile j =
+// counts 4096 j .. 4096 j + 4095, four neighbouring counts per thread: loads and stores contiguous across the wave).
+// The thread sums of every sub-tile are scanned over the wave (DPP), the wave totals of all sub-tiles meet in LDS behind
+// one barrier, and a 64-bit carry runs through the sub-tiles and on to the next 32 768 counts (the total may exceed
+// what the buffers hold).  VEC: counts and row_ptr are 16-byte aligned.
+constexpr int OFFS_THREADS = 1024, OFFS_SUB = 8, OFFS_TILE = OFFS_THREADS * 4;
+template <bool VEC>
 __global__ void __launch_bounds__(OFFS_THREADS)
 k_csr_offsets(const int32_t* __restrict__ counts, int64_t rows, int64_t capacity, int32_t* __restrict__ row_ptr,
               int64_t* __restrict__ total) {
-  __shared__ long long wave_sum_[OFFS_THREADS / 64];
+  __shared__ int tot[OFFS_SUB][OFFS_THREADS / 64];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int64_t per = (rows + OFFS_THREADS - 1) / OFFS_THREADS;
-  const int64_t i0 = (int64_t)tid * per, i1 = i0 + per < rows ? i0 + per : rows;
-  long long mine = 0;
-  for (int64_t i = i0; i < i1; ++i) mine += counts[i];
-  long long incl = mine;                                    // inclusive scan over the wave
+  long long carry = 0;
+  for (int64_t base = 0; base < rows; base += (int64_t)OFFS_SUB * OFFS_TILE) {
+    int c[OFFS_SUB][4], sum[OFFS_SUB], incl[OFFS_SUB];
 #pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    const long long up = __shfl_up(incl, d);
-    if (lane >= d) incl += up;
-  }
-  if (lane == 63) wave_sum_[wave] = incl;
-  __syncthreads();
-  long long before = 0, all = 0;
+    for (int j = 0; j < OFFS_SUB; ++j) {
+      const int64_t i = base + (int64_t)j * OFFS_TILE + 4 * tid;
+      if (VEC && i + 3 < rows) {
+        const int4 v = *reinterpret_cast<const int4*>(counts + i);
+        c[j][0] = v.x; c[j][1] = v.y; c[j][2] = v.z; c[j][3] = v.w;
+      } else {
 #pragma unroll
-  for (int w = 0; w < OFFS_THREADS / 64; ++w) { const long long t = wave_sum_[w]; all += t; before += w < wave ? t : 0; }
-  long long run = before + incl - mine;
-  for (int64_t i = i0; i < i1; ++i) {
-    row_ptr[i] = (int32_t)(run < capacity ? run : capacity);
-    run += counts[i];
+        for (int e = 0; e < 4; ++e) c[j][e] = i + e < rows ? counts[i + e] : 0;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < OFFS_SUB; ++j) {
+      sum[j] = (c[j][0] + c[j][1]) + (c[j][2] + c[j][3]);
+      incl[j] = wave_inclusive_scan(sum[j]);
+      if (lane == 63) tot[j][wave] = incl[j];
+    }
+    __syncthreads();
+    long long run = carry;                                  // entries before sub-tile j
+#pragma unroll
+    for (int j = 0; j < OFFS_SUB; ++j) {
+      int before = 0, all = 0;
+#pragma unroll
+      for (int w = 0; w < OFFS_THREADS / 64; ++w) { const int t = tot[j][w]; all += t; before += w < wave ? t : 0; }
+      long long at = run + before + incl[j] - sum[j];
+      const int64_t i = base + (int64_t)j * OFFS_TILE + 4 * tid;
+      int o[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { o[e] = (int32_t)(at < capacity ? at : capacity); at += c[j][e]; }
+      if (VEC && i + 3 < rows) {
+        *reinterpret_cast<int4*>(row_ptr + i) = make_int4(o[0], o[1], o[2], o[3]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) if (i + e < rows) row_ptr[i + e] = o[e];
+      }
+      run += all;
+    }
+    carry = run;
+    __syncthreads();                                        // tot is written again by the next round
   }
   if (tid == 0) {
-    row_ptr[rows] = (int32_t)(all < capacity ? all : capacity);
-    if (total) *total = all;
+    row_ptr[rows] = (int32_t)(carry < capacity ? carry : capacity);
+    if (total) *total = carry;
   }
 }
 
@@ -414,7 +442,10 @@ int hyc_csr_offsets(const int32_t* counts, int64_t rows, int64_t capacity, int32
   if (rows < 0) return fail(HYC_EINVAL, "hyc_csr_offsets: rows=%lld", (long long)rows);
   if (!row_ptr || (rows > 0 && !counts)) return fail(HYC_EFAULT, "hyc_csr_offsets: null buffer");
   if (capacity < 0 || capacity > 0x7FFFFFFFll) capacity = 0x7FFFFFFFll;          // row_ptr is int32
-  hipLaunchKernelGGL(k_csr_offsets, dim3(1), dim3(OFFS_THREADS), 0, begin_launch(stream), counts, rows, capacity, row_ptr, total);
+  if (aligned16(counts) && aligned16(row_ptr))
+    hipLaunchKernelGGL(k_csr_offsets<true>, dim3(1), dim3(OFFS_THREADS), 0, begin_launch(stream), counts, rows, capacity, row_ptr, total);
+  else
+    hipLaunchKernelGGL(k_csr_offsets<false>, dim3(1), dim3(OFFS_THREADS), 0, begin_launch(stream), counts, rows, capacity, row_ptr, total);
   return check_launch("hyc_csr_offsets");
 }
 
