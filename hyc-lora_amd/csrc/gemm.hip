@@ -236,8 +236,11 @@ struct DirectRegs {          // what one lane loads for one step: a packed word 
 // earlier form folded the scale of 1- and 2-bit codes into dY, where code - OFF is exact, and fed the integer codes
 // to the MFMAs as bf16 bit patterns; since the codes are converted two per instruction the plain form is as fast
 // - 2-bit codes, 64-channel groups, 65 536 x 4096: 55.0 us folded, 41.8 us plain - and it went.)
-template <int BITS, int NT, bool MAINT, int SPT>
+// NW = waves per workgroup (4 or 8): the waves share the workgroup's token range step by step, so with eight a wave has
+//      half as many steps to walk and the token range needs half as many splits across workgroups
+template <int BITS, int NT, bool MAINT, int SPT, int NW>
 __device__ __forceinline__ void gradw_direct_tile(const DirectArgs& A, float* red, int hy, int64_t n0) {
+  constexpr int NTHR = 64 * NW;
   constexpr int LC = 16;                                                         // chunks per tile
   constexpr int NJ = 8;                                                          // MFMAs (16 channels each) per segment
   constexpr uint32_t CMASK = (BITS == 8) ? 0xFFu : Q<BITS>::CODE_MASK;
@@ -289,7 +292,7 @@ __device__ __forceinline__ void gradw_direct_tile(const DirectArgs& A, float* re
   static_assert(COLS <= 256, "one thread per channel of the tile");
   const int mode = A.partial != nullptr ? 0 : (A.out_f32 ? 1 : 2);
   const bool wo_vec = MAINT && mode == 0;                                        // 4 channels per thread (the workspace is 16-byte aligned)
-  const int wo_col = wo_vec ? (tid % (COLS / 4)) * 4 : tid % COLS;
+  const int wo_col = wo_vec ? (tid % (COLS / 4)) * 4 : tid % COLS;   // (NTHR is a multiple of COLS / 4 and of COLS)
   const int wo_tb = MAINT ? (wo_col & 7) : 0, wo_tcl = MAINT ? ((wo_col >> 3) % LC) : 0, wo_tg = MAINT ? wo_col / (8 * LC) : 0;
   bool wo_in;
   uint32_t wo_pword = 0;
@@ -406,8 +409,8 @@ __device__ __forceinline__ void gradw_direct_tile(const DirectArgs& A, float* re
     }
   };
 
-  // wave w takes steps w, w+4, ... of the workgroup's token range; two steps of loads are in flight
-  constexpr int64_t WS = 4 * DK;
+  // wave w takes steps w, w+NW, ... of the workgroup's token range; two steps of loads are in flight
+  constexpr int64_t WS = NW * DK;
   DirectRegs<SPT> R0, R1;
   uint32_t a0[NT][8], a1[NT][8];
   int64_t m0 = m_begin + (int64_t)wave * DK;
@@ -421,12 +424,14 @@ __device__ __forceinline__ void gradw_direct_tile(const DirectArgs& A, float* re
       if (m0 + 3 * WS < m_end) fetch(m0 + 3 * WS, R1, a1);
     }
   }
-  // ---- the four waves add up in LDS: (wave 0 + wave 2) in one half of `red`, (wave 1 + wave 3) in the other, the
-  // two halves are added by the write-out; layout of a half [row n][tile b][lane] with a padded pitch ----
+  // ---- the waves add up in LDS: the first half of them write their accumulators to a buffer each, the second half
+  // add theirs on top (wave w onto wave w - NW/2), and the write-out adds the NW/2 buffers; layout of a buffer
+  // [row n][tile b][lane] with a padded pitch ----
   // lane holds column (lane mod 16) and rows 4*(lane/16) + v of each 16x16 tile
-  constexpr int HALF = 16 * NT * NB * RP;
-  float* mine = red + (wave & 1) * HALF;
-  if (wave < 2) {
+  constexpr int NBUF = NW / 2;
+  constexpr int HALF = 16 * NT * NB * RP;                                        // floats of one buffer
+  float* mine = red + (wave % NBUF) * HALF;
+  if (wave < NBUF) {
 #pragma unroll
     for (int a = 0; a < NT; ++a)
 #pragma unroll
@@ -435,7 +440,7 @@ __device__ __forceinline__ void gradw_direct_tile(const DirectArgs& A, float* re
         for (int v = 0; v < 4; ++v) mine[((16 * a + 4 * kq + v) * NB + b) * RP + l16] = acc[a][b][v];
   }
   __syncthreads();
-  if (wave >= 2) {
+  if (wave >= NBUF) {
     // all reads first, then the adds and writes: written as read-add-write per element the compiler keeps them in
     // program order (it cannot see that the addresses differ) and every element waits out the LDS latency
 #pragma unroll
@@ -453,12 +458,19 @@ __device__ __forceinline__ void gradw_direct_tile(const DirectArgs& A, float* re
         for (int v = 0; v < 4; ++v) mine[((16 * a + 4 * kq + v) * NB + b) * RP + l16] = acc[a][b][v];
   }
   __syncthreads();
+  // sum of the buffers at one place, in buffer order
+  auto reduced = [&](int at) __attribute__((always_inline)) {
+    float v = red[at];
+#pragma unroll
+    for (int u = 1; u < NBUF; ++u) v += red[u * HALF + at];
+    return v;
+  };
   // ---- write-out by all threads, neighbouring threads = neighbouring channels ----
   const float alpha = A.alpha, beta = A.beta;
   if (!wo_in) return;
   // channel = (segment tg of the tile, chunk tcl of the tile, byte tb of the packed word): MFMA tile 8*tg + tb, lane tcl
   if (wo_vec) {                                        // partial sums of a main tile: 16-byte stores, 4 channels per thread
-    constexpr int NSTEP4 = 256 / (COLS / 4);
+    constexpr int NSTEP4 = NTHR / (COLS / 4);
     int ro[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) ro[i] = (wo_tg * NJ + wo_tb + i) * RP + wo_tcl;
@@ -466,7 +478,7 @@ __device__ __forceinline__ void gradw_direct_tile(const DirectArgs& A, float* re
     for (int nl = tid / (COLS / 4); nl < 16 * NT && n0 + nl < N_out; nl += NSTEP4) {
       float v[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) v[i] = red[nl * NB * RP + ro[i]] + red[HALF + nl * NB * RP + ro[i]];
+      for (int i = 0; i < 4; ++i) v[i] = reduced(nl * NB * RP + ro[i]);
       float* o = A.partial + ((int64_t)blockIdx.z * N_out + n0 + nl) * H + wo_h;
       if (m4 == 0) {
         *reinterpret_cast<float4*>(o) = make_float4(v[0], v[1], v[2], v[3]);
@@ -479,8 +491,8 @@ __device__ __forceinline__ void gradw_direct_tile(const DirectArgs& A, float* re
   }
   if (MAINT && ((wo_pword >> wo_tb) & 1u)) return;
   const int rb = MAINT ? wo_tg * NJ + wo_tb : 0, rl = MAINT ? wo_tcl : tid % COLS;
-  for (int nl = tid / COLS; nl < 16 * NT && n0 + nl < N_out; nl += 256 / COLS) {
-    const float val = red[(nl * NB + rb) * RP + rl] + red[HALF + (nl * NB + rb) * RP + rl];
+  for (int nl = tid / COLS; nl < 16 * NT && n0 + nl < N_out; nl += NTHR / COLS) {
+    const float val = reduced((nl * NB + rb) * RP + rl);
     const int64_t n = n0 + nl;
     if (mode == 0) {
       A.partial[((int64_t)blockIdx.z * N_out + n) * H + wo_h] = val;
@@ -496,15 +508,15 @@ __device__ __forceinline__ void gradw_direct_tile(const DirectArgs& A, float* re
 
 // one launch: blockIdx.y < (NSEG / SPT) * c_tiles are the tiles of quantised channels, the rest the outlier tiles
 // (two waves per SIMD at least: with 256 registers or fewer the accumulators stay in ordinary vector registers)
-template <int BITS, int NT, int SPT>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) k_gradw_direct(DirectArgs A) {
+template <int BITS, int NT, int SPT, int NW>
+__global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) k_gradw_direct(DirectArgs A) {
   static_assert(Q<BITS>::NSEG % SPT == 0, "segments per tile must divide the segments of a packed word");
   constexpr int NB = 8 * SPT;
-  __shared__ float red[2 * 16 * NT * NB * 17];
+  __shared__ float red[(NW / 2) * 16 * NT * NB * 17];
   const int main_tiles = (Q<BITS>::NSEG / SPT) * A.c_tiles;
   const int64_t n0 = (int64_t)blockIdx.x * (16 * NT);                            // first feature of the workgroup
-  if ((int)blockIdx.y < main_tiles) gradw_direct_tile<BITS, NT, true, SPT>(A, red, (int)blockIdx.y, n0);
-  else gradw_direct_tile<BITS, NT, false, 1>(A, red, (int)blockIdx.y - main_tiles, n0);
+  if ((int)blockIdx.y < main_tiles) gradw_direct_tile<BITS, NT, true, SPT, NW>(A, red, (int)blockIdx.y, n0);
+  else gradw_direct_tile<BITS, NT, false, 1, NW>(A, red, (int)blockIdx.y - main_tiles, n0);
 }
 
 // How a shape is laid on the kernel: SPT segments of a packed word per tile (two with one feature tile, so that every
@@ -519,25 +531,40 @@ static DirectPlan direct_plan(int bits, int64_t N_out) {
   return p;
 }
 
-// The streaming kernel serves N_out <= DIRECT_MAX_N.  Token splits: as many as keep the whole grid resident at once
-// (256 CUs x the plan's workgroups per CU).  The kernel is bound by its decode work, so a grid a little over that
+// The streaming kernel serves N_out <= DIRECT_MAX_N.  The token splits keep the whole grid resident at once
+// (256 CUs x the workgroups a CU holds): the kernel is bound by its decode work, so a grid a little over that
 // leaves most of the chip idle during a second round (65 536 x 4096 INT4, two per CU: 560 workgroups 88 us, 490
 // workgroups 65 us).
 // More than 32 features run as blockIdx.x tiles of 32 that decode the packed words again: up to four such tiles
 // that still beats staging the tile in LDS for a product this thin.
 constexpr int64_t DIRECT_MAX_N = 128;
 static int64_t direct_x_tiles(int64_t N_out) { return N_out <= 32 ? 1 : (N_out + 31) / 32; }
-static int direct_splits(int64_t M, int64_t yx_tiles, int per_cu) {
+// Token splits for workgroups of nw waves: as many as keep the whole grid resident at once (two workgroups of four
+// waves per CU, or one of eight), and no more than leave every wave two steps of 32 tokens (four for four waves from
+// 4096 tokens on: a split more is a partial result more for the second launch to add - 4096 x 16 x 4096: 16 splits
+// 12.1 us, 8 splits 11.3; 2048 tokens: 8 splits 9.3 us, 6 splits 11.6).
+static int direct_splits(int64_t M, int64_t yx_tiles, int nw, int per_cu4) {
+  const int per_cu = nw == 8 ? 1 : per_cu4;               // (per_cu4: workgroups of four waves a CU holds, see direct_plan)
   int64_t s = (int64_t)256 * per_cu / (yx_tiles > 0 ? yx_tiles : 1);
-  // at least two steps per wave, four from 4096 tokens on: a split more is a partial result more for the second
-  // launch to add (4096 x 16 x 4096: 16 splits 12.1 us, 8 splits 11.3; 32 features: 15.0 -> 13.1; 2048 tokens: 8 splits
-  // 9.3 us, 6 splits 11.6)
-  const int64_t per_wave = M >= 4096 ? 4 : M >= 3072 ? 3 : 2;
-  const int64_t max_by_tokens = (M + 4 * per_wave * DK - 1) / (4 * per_wave * DK);
+  const int64_t per_wave = nw == 8 ? 2 : M >= 4096 ? 4 : M >= 3072 ? 3 : 2;
+  const int64_t max_by_tokens = (M + nw * per_wave * DK - 1) / (nw * per_wave * DK);
   if (s > max_by_tokens) s = max_by_tokens;
   if (s < 1) s = 1;
   if (s > 64) s = 64;
   return (int)s;
+}
+// Waves per workgroup.  Eight waves walk a token range in half the steps and need half the splits (fewer partial
+// results to add): better wherever the kernel is short (4096 x 16 x 4096 4-bit: 10.6 us against 11.3, r = 64: 14.7
+// against 16.3, 11008 channels: 14.4 against 15.6).  With many steps per wave what counts is how much of the chip the
+// grid fills, and the two forms fill it in different grains (65 536 x 64 x 4096: 210 workgroups of eight waves, 109 us,
+// against 490 of four, 95 us); below 4096 tokens the larger reduction through LDS costs more than the steps saved
+// (2048 tokens: 11.2 against 9.3 us).
+static int direct_waves(int64_t M, int64_t yx_tiles, int per_cu4) {
+  if (M < 4096) return 4;
+  const int s8 = direct_splits(M, yx_tiles, 8, per_cu4), s4 = direct_splits(M, yx_tiles, 4, per_cu4);
+  const int64_t steps8 = (M + (int64_t)s8 * 8 * DK - 1) / ((int64_t)s8 * 8 * DK);
+  if (steps8 <= 8) return 8;
+  return yx_tiles * s8 * 8 >= yx_tiles * s4 * 4 ? 8 : 4;      // waves in flight
 }
 static int64_t direct_y_tiles(int64_t H, int bits, int k, int64_t N_out) {
   const DirectPlan p = direct_plan(bits, N_out);
@@ -548,7 +575,7 @@ static int64_t direct_y_tiles(int64_t H, int bits, int k, int64_t N_out) {
 static int direct_splits_max(int64_t M, int64_t N_out, int64_t H) {
   int best = 1;
   for (int bits = 1; bits <= 8; bits *= 2) {
-    const int sp = direct_splits(M, direct_y_tiles(H, bits, 0, N_out) * direct_x_tiles(N_out), direct_plan(bits, N_out).per_cu);
+    const int sp = direct_splits(M, direct_y_tiles(H, bits, 0, N_out) * direct_x_tiles(N_out), 4, direct_plan(bits, N_out).per_cu);   // (four waves: the form with more splits)
     if (sp > best) best = sp;
   }
   return best;
@@ -1263,7 +1290,8 @@ int hyc_gradw_gemm(const void* dy, int64_t ldy, const void* stored, const void* 
     const int c_tiles = (g.cps + 15) / 16, o_tiles = (d->k + 15) / 16;
     const int y_tiles = (g.nseg / pl.spt) * c_tiles + o_tiles;
     const int x_tiles = (int)direct_x_tiles(N_out);
-    const int splits = M > 0 ? direct_splits(M, (int64_t)y_tiles * x_tiles, pl.per_cu) : 1;
+    const int nw = direct_waves(M, (int64_t)y_tiles * x_tiles, pl.per_cu);
+    const int splits = M > 0 ? direct_splits(M, (int64_t)y_tiles * x_tiles, nw, pl.per_cu) : 1;
     if (splits > 1 && !workspace) return fail(HYC_EFAULT, "hyc_gradw_gemm: workspace of hyc_gradw_workspace_bytes() bytes required");
     if (splits > 1 && !aligned16(workspace)) return fail(HYC_EINVAL, "hyc_gradw_gemm: workspace must be 16-byte aligned");
     int64_t tps = (M + splits - 1) / splits;
@@ -1276,7 +1304,11 @@ int hyc_gradw_gemm(const void* dy, int64_t ldy, const void* stored, const void* 
     DirectArgs da = {static_cast<const uint16_t*>(dy), ldy, M, N_out, H, static_cast<const uint8_t*>(stored),
                      static_cast<const uint16_t*>(vals), static_cast<const uint16_t*>(scales), ca, g.cps, c_tiles, tps,
                      alpha, beta, out, of32, partial};
-#define HYC_DIRECT_K(B_, N_, S_) hipLaunchKernelGGL((k_gradw_direct<B_, N_, S_>), grid, dim3(256), 0, st, da)
+#define HYC_DIRECT_K(B_, N_, S_)                                                                               \
+  do {                                                                                                         \
+    if (nw == 8) hipLaunchKernelGGL((k_gradw_direct<B_, N_, S_, 8>), grid, dim3(512), 0, st, da);              \
+    else hipLaunchKernelGGL((k_gradw_direct<B_, N_, S_, 4>), grid, dim3(256), 0, st, da);                      \
+  } while (0)
 #define HYC_DIRECT(B_) do { if (nt == 1) HYC_DIRECT_K(B_, 1, (B_ < 8 ? 2 : 1)); else HYC_DIRECT_K(B_, 2, 1); } while (0)   /* direct_plan() */
     switch (d->bits) {
       case 1: HYC_DIRECT(1); break;
