@@ -199,6 +199,10 @@ typedef float floatx4_t __attribute__((ext_vector_type(4)));
 
 // Buffer loads with a scalar offset on top of the lane's: the hardware checks the SUM of both offsets against the
 // size of the resource, so a row selected through the scalar offset is dropped (reads zeros) when it lies past the end.
+__device__ __forceinline__ uint4 load_b128(BufferRsrc r, uint32_t off, uint32_t scalar_off) {
+  const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, (int)scalar_off, 0);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
 __device__ __forceinline__ uint2 load_b64(BufferRsrc r, uint32_t off, uint32_t scalar_off) {
   const u32x2_t v = __builtin_amdgcn_raw_buffer_load_b64(r, (int)off, (int)scalar_off, 0);
   return make_uint2(v.x, v.y);
@@ -900,54 +904,45 @@ k_gradw_big(const uint16_t* __restrict__ dy, int64_t ldy, int64_t M, int64_t N_o
   const bool slow_any = __ballot(slow) != 0;
   const BufferRsrc rs_x = make_rsrc(SRC == 0 && ca.k ? vals + m_begin * (int64_t)ca.k : nullptr,
                                     __builtin_amdgcn_readfirstlane((uint32_t)(m_end - m_begin) * kk2));
-  // the resources of the next stage to request
-  const char* pa = reinterpret_cast<const char*>(dy + m_begin * ldy);
-  const char* pb = reinterpret_cast<const char*>(stored) + m_begin * (int64_t)b_pitch;
-  const char* ps = reinterpret_cast<const char*>(scales + m_begin * (int64_t)gpr);
-  const char* po = reinterpret_cast<const char*>(vals + m_begin * (int64_t)ca.k);
-  int left = (int)(m_end - m_begin);                                                // tokens from that stage to the end
-  BufferRsrc rs_a = make_rsrc(pa, (uint32_t)left * a_pitch), rs_b = make_rsrc(pb, __builtin_amdgcn_readfirstlane((uint32_t)left * b_pitch));
-  BufferRsrc rs_s = make_rsrc(ps, (uint32_t)left * 2u * gpr), rs_o = make_rsrc(po, __builtin_amdgcn_readfirstlane((uint32_t)left * kk2));
-  // (the empty asm statements keep the scalar arithmetic in the slot it is written in, and in scalar registers)
-  auto renew = [&](BufferRsrc& rs, const char*& ptr, uint32_t step, uint32_t pitch) __attribute__((always_inline)) {
-    const uint64_t next = reinterpret_cast<uint64_t>(ptr) + step;
-    uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)next), hi = __builtin_amdgcn_readfirstlane((uint32_t)(next >> 32));
-    uint32_t bytes = __builtin_amdgcn_readfirstlane((uint32_t)left * pitch);
-    asm volatile("" : "+s"(lo), "+s"(hi), "+s"(bytes));
-    ptr = reinterpret_cast<const char*>(((uint64_t)hi << 32) | lo);
-    rs = make_rsrc(ptr, bytes);
-  };
-  auto advance = [&](int part) __attribute__((always_inline)) {                     // four parts, one resource each
-    if (part == 0) {
-      left = left > WK ? left - WK : 0;
-      renew(rs_a, pa, WK * a_pitch, a_pitch);
-    } else if (part == 1) {
-      renew(rs_b, pb, WK * b_pitch, b_pitch);
-    } else if (part == 2 && SRC == 0) {
-      renew(rs_s, ps, WK * 2u * gpr, 2u * gpr);
-    } else if (part == 3 && SRC == 0) {
-      renew(rs_o, po, WK * kk2, kk2);
-    }
+  // One resource per operand, from the workgroup's first token to the end of its token range; the stage being
+  // requested is selected through the scalar offset of the load (the hardware checks the sum of the lane's offset and
+  // the scalar one against the size, so a stage past the end reads zeros), which advances by one scalar add per
+  // operand and stage.  (Renewing the four resources every stage - a 64-bit add, the remaining length times the pitch
+  // and three moves into scalar registers each - was a twelfth of the stage's issue time.)
+  const int left0 = (int)(m_end - m_begin);
+  const BufferRsrc rs_a = make_rsrc(dy + m_begin * ldy, (uint32_t)left0 * a_pitch);
+  const BufferRsrc rs_b = make_rsrc(reinterpret_cast<const char*>(stored) + m_begin * (int64_t)b_pitch,
+                                    __builtin_amdgcn_readfirstlane((uint32_t)left0 * b_pitch));
+  const BufferRsrc rs_s = make_rsrc(SRC == 0 ? scales + m_begin * (int64_t)gpr : nullptr, SRC == 0 ? (uint32_t)left0 * 2u * gpr : 0u);
+  const BufferRsrc rs_o = make_rsrc(SRC == 0 && ca.k ? vals + m_begin * (int64_t)ca.k : nullptr,
+                                    __builtin_amdgcn_readfirstlane((uint32_t)left0 * kk2));
+  uint32_t so_a = 0, so_b = 0, so_s = 0, so_o = 0;                                  // byte offsets of the stage to request next
+  auto advance = [&](int part) __attribute__((always_inline)) {                     // four parts, one operand each
+    if (part == 0) so_a += WK * a_pitch;
+    else if (part == 1) so_b += WK * b_pitch;
+    else if (part == 2 && SRC == 0) so_s += WK * 2u * gpr;
+    else if (part == 3 && SRC == 0) so_o += WK * kk2;
+    asm volatile("" : "+s"(so_a), "+s"(so_b), "+s"(so_s), "+s"(so_o));              // (in the slot it is written in, in scalar registers)
   };
   // The requests of a stage, numbered: codes and scales (decoded first) before dY and the outlier values.
   constexpr int NLOAD = A_PER + (SRC == 0 ? B_PER * (1 + 3 * NST) : B_PER);
   auto request = [&](Regs& R, int j) __attribute__((always_inline)) {
     if (SRC != 0) {
-      if (j < B_PER) R.b[j] = load_b128(rs_b, vb[j]);
-      else R.a[j - B_PER] = load_b128(rs_a, va[j - B_PER]);
+      if (j < B_PER) R.b[j] = load_b128(rs_b, vb[j], so_b);
+      else R.a[j - B_PER] = load_b128(rs_a, va[j - B_PER], so_a);
     } else if (j < B_PER) {
-      const uint2 pk = load_b64(rs_b, vb[j]);
+      const uint2 pk = load_b64(rs_b, vb[j], so_b);
       R.b[j] = make_uint4(pk.x, pk.y, 0, 0);
     } else if (j < B_PER + NCH) {
       const int c = j - B_PER;
-      R.s[c / NST][c % NST] = load_b16(rs_s, vs[c / NST][c % NST]);
+      R.s[c / NST][c % NST] = load_b16(rs_s, vs[c / NST][c % NST], so_s);
     } else if (j < B_PER + NCH + A_PER) {
       const int u = j - B_PER - NCH;
-      R.a[u] = load_b128(rs_a, va[u]);
+      R.a[u] = load_b128(rs_a, va[u], so_a);
     } else {
       const int q = j - B_PER - NCH - A_PER, c = q >> 1;
-      if (q & 1) R.o1[c / NST][c % NST] = load_b16(rs_o, vo1[c / NST][c % NST]);
-      else R.o0[c / NST][c % NST] = load_b16(rs_o, vo0[c / NST][c % NST]);
+      if (q & 1) R.o1[c / NST][c % NST] = load_b16(rs_o, vo1[c / NST][c % NST], so_o);
+      else R.o0[c / NST][c % NST] = load_b16(rs_o, vo0[c / NST][c % NST], so_o);
     }
   };
   auto request_all = [&](Regs& R) __attribute__((always_inline)) {
