@@ -154,6 +154,35 @@ __device__ __forceinline__ void group_maxmin(float& mx, float& mn) {
   if (LPG >= 32) { mx = __builtin_elementwise_maximum(mx, xor_lane(mx, 16)); mn = __builtin_elementwise_minimum(mn, xor_lane(mn, 16)); }
   if (LPG >= 64) { mx = __builtin_elementwise_maximum(mx, xor_lane(mx, 32)); mn = __builtin_elementwise_minimum(mn, xor_lane(mn, 32)); }
 }
+// Maximum of a NON-NEGATIVE value over LPG consecutive lanes.  Non-negative floats order like their bit patterns, and
+// an integer maximum takes the other lane's value as a DPP operand (one v_max_u32_dpp per step); the float maximum
+// needs a v_mov_b32_dpp in front of every v_max_f32, because its operands have to be canonicalised first.
+template <int CTRL>
+__device__ __forceinline__ uint32_t umax_dpp(uint32_t v) {
+  const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, true);   // (every lane has a source; 0 is max's identity)
+  return v > o ? v : o;
+}
+template <int LPG>
+__device__ __forceinline__ float group_max_nonneg(float v) {
+  uint32_t b = __float_as_uint(v);
+  if (LPG >= 2) b = umax_dpp<0xB1>(b);     // quad_perm [1,0,3,2]
+  if (LPG >= 4) b = umax_dpp<0x4E>(b);     // quad_perm [2,3,0,1]
+  if (LPG >= 8) b = umax_dpp<0x141>(b);    // row_half_mirror
+  if (LPG >= 16) b = umax_dpp<0x140>(b);   // row_mirror
+  if (LPG >= 32) { const uint32_t o = (uint32_t)__shfl_xor((int)b, 16, 64); b = b > o ? b : o; }
+  if (LPG >= 64) { const uint32_t o = (uint32_t)__shfl_xor((int)b, 32, 64); b = b > o ? b : o; }
+  return __uint_as_float(b);
+}
+__device__ __forceinline__ float group_max_nonneg_rt(float v, int lpg) {
+  uint32_t b = __float_as_uint(v);
+  b = umax_dpp<0xB1>(b);
+  b = umax_dpp<0x4E>(b);
+  if (lpg >= 8) b = umax_dpp<0x141>(b);
+  if (lpg >= 16) b = umax_dpp<0x140>(b);
+  if (lpg >= 32) { const uint32_t o = (uint32_t)__shfl_xor((int)b, 16, 64); b = b > o ? b : o; }
+  if (lpg >= 64) { const uint32_t o = (uint32_t)__shfl_xor((int)b, 32, 64); b = b > o ? b : o; }
+  return __uint_as_float(b);
+}
 // runtime-width variant (lpg in {4, 8, 16, 32, 64}; the branches are uniform)
 template <typename Op>
 __device__ __forceinline__ float group_reduce_rt(float v, int lpg, Op op) {

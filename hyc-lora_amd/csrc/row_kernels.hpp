@@ -57,8 +57,8 @@ __device__ __forceinline__ float quant_seg(float (&v)[8], int lpg, uint32_t& cl,
     am = __builtin_elementwise_maximum(__builtin_elementwise_maximum(am, __builtin_fabsf(v[3])), __builtin_fabsf(v[4]));
     am = __builtin_elementwise_maximum(__builtin_elementwise_maximum(am, __builtin_fabsf(v[5])), __builtin_fabsf(v[6]));
     am = __builtin_elementwise_maximum(am, __builtin_fabsf(v[7]));
-    if (LPGT > 0) am = group_reduce<LPGT>(am, OpMax());
-    else am = group_reduce_rt(am, lpg, OpMax());
+    if (LPGT > 0) am = group_max_nonneg<LPGT>(am);
+    else am = group_max_nonneg_rt(am, lpg);
     s = BITS == 1 ? am : bfr((am + am) * Q<BITS>::INV_LEVELS);
   } else {
     float mx = __builtin_elementwise_maximum(__builtin_elementwise_maximum(v[0], v[1]), v[2]);
