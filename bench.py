@@ -364,6 +364,18 @@ def kernel_tour(pkg, torch, reps=5):
             K.gradw_gemm(dyN, cs[0], staged=True)         # x_hat restored once, then the dense form of the kernel
         torch.cuda.synchronize()
         del x, up, a, g, cs
+    # the trained shape of the weight gradient (LoRA-A, 16 features) at 16x config 2's tokens, INT4 and INT2 / group 64
+    M, H = 65536, 4096
+    x = mk(M, H, 20)
+    plan = K.select_channels(K.channel_absmax(x), 41)
+    dy16 = (0.01 * torch.randn(M, 16, generator=gen, device="cuda")).bfloat16()
+    for bits, G in ((4, 128), (2, 64)):
+        c = K.compress_channel(x, plan, bits, G)
+        for _ in range(reps):
+            K.gradw_gemm(dy16, c)
+        torch.cuda.synchronize()
+        del c
+    del x, dy16
     # the reference snapshot's own scheme (element threshold, static scale) at config 2's shape: 1 % outlier
     # elements, INT4, per-token and per-channel scales; consumers take the restored activation
     M, H, S = 4096, 4096, 1024
@@ -479,7 +491,38 @@ def cpu_baseline(torch, wl, rows, seconds):
     fwd_b, bwd_b, _ = algorithmic_bytes(rows, H, bits, group, wl.k)
     return {"value": round((fwd_b + bwd_b) / dt / 1e9, 4), "unit": "GB/s", "cores": threads, "kind": "port",
             "sample": "oracle rmsnorm_fwd + hyc_compress + hyc_decompress + rmsnorm_bwd on the first %d of %d tokens "
-                      "(H=%d), mean of %d passes, %.3f s per pass" % (rows, wl.M, H, reps, dt)}
+                      "(H=%d), mean of %d passes, %.3f s per pass" % (rows, wl.M, H, reps, dt),
+            "round_trip": cpu_round_trip(torch, O, threads)}
+
+
+def cpu_round_trip(torch, O, threads):
+    """the standalone compress -> decompress round trip of the oracle at configs[0]'s size (2048 x 4096, 41 channels
+    x50) and at configs[1]'s (4096 x 4096): 3 warm-ups, median of 10, algorithmic GB/s (20 772 B per token)"""
+    out = {}
+    for tag, M, gain in (("config1_2048x4096", 2048, 50.0), ("config2_size_4096x4096", 4096, 50.0)):
+        H, bits, group, k = 4096, 4, 128, 41
+        gen = torch.Generator().manual_seed(0)
+        x = torch.randn(M, H, generator=gen)
+        x[:, torch.randperm(H, generator=gen)[:k]] *= gain
+        x = x.bfloat16()
+        idx = O.hyc_select_channels(O.hyc_channel_scores(x), k)
+
+        def trip():
+            vals, stored, scales = O.hyc_compress(x, idx, bits, group)
+            return O.hyc_decompress(vals, stored, idx, scales, bits, group)
+
+        for _ in range(3):
+            trip()
+        times = []
+        for _ in range(10):
+            t0 = time.perf_counter()
+            trip()
+            times.append(time.perf_counter() - t0)
+        times.sort()
+        med = 0.5 * (times[4] + times[5])
+        nbytes = 2 * M * (2 * H + side_bytes(H, bits, group, k))
+        out[tag] = {"ms": round(med * 1e3, 2), "GBps": round(nbytes / med / 1e9, 3), "bytes": nbytes, "cores": threads}
+    return out
 
 
 def main():
