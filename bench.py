@@ -25,10 +25,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # (profiles/rmsnorm_fwd_bwd_config2.md).  The figures belong to one state of the kernel sources: TRAFFIC_SOURCES_SHA
 # is the digest of those files when the counters were taken, and `roofline.traffic` is null whenever the files on
 # disk differ (a changed kernel needs new counter runs, not an old number).
-TRAFFIC_FWD = int((16508.01 * 1.99840 + 41793.60) * 1024)    # FETCH_SIZE KiB x copy factor + WRITE_SIZE KiB
-TRAFFIC_BWD = int((21030.97 * 1.99840 + 36872.97) * 1024)
+TRAFFIC_FWD = int((16507.71 * 1.99841 + 41792.96) * 1024)    # FETCH_SIZE KiB x copy factor + WRITE_SIZE KiB
+TRAFFIC_BWD = int((21030.41 * 1.99841 + 36866.62) * 1024)
 TRAFFIC_SOURCES = ("norm.hip", "row_kernels.hpp", "row_codec.hpp")
-TRAFFIC_SOURCES_SHA = "daffe8c4f087f928"
+TRAFFIC_SOURCES_SHA = "fc680345caa21d65"
 
 
 def sources_sha():
