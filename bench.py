@@ -234,7 +234,7 @@ def gradw_extra(pkg, torch, c, sustained=False, shapes=(("full_w", 4096, 100, 30
                         "staged_frac_of_bf16_mfma_peak": round(flop / ms_staged / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
                         "dense_operand_ms": round(ms_dense, 5), "dense_operand_TFLOPs": round(flop / ms_dense / 1e9, 1),
                         "dense_operand_frac_of_bf16_mfma_peak": round(flop / ms_dense / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
-                        "default_route": "staged" if N >= K.STAGED_GRADW_MIN_FEATURES else "fused"})
+                        "default_route": "staged" if K.gradw_staged_by_default(N, H) else "fused"})
             if sustained:
                 # the same launches after 2.5 s without a pause: the GPU at its power limit
                 ms_s = time_sustained(torch, fn, ms)

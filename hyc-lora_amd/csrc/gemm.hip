@@ -1328,8 +1328,9 @@ int hyc_gradw_gemm(const void* dy, int64_t ldy, const void* stored, const void* 
   // wide tiles (256 columns) when the output is large and the tile grid fits the packing
   // (the channel scheme has the 256-feature form only)
   const bool wide = chan ? (N_out >= 2 * WN && g.seg % (WH / g.nseg) == 0) : (N_out >= WN && H % WH == 0);
-  // 256 features per workgroup (four waves of 128 x 128) when the tile grid fills the chip, else 128 (dense only)
-  const int wnt = !wide ? 0 : chan || (N_out >= 2 * WN && ((N_out + 2 * WN - 1) / (2 * WN)) * (H / WH) >= 128) ? 2 * WN : WN;
+  // 256 features per workgroup (four waves of 128 x 128) from 256 output features on, else 128 (dense only); a tile
+  // grid below the CU count is made up with token splits
+  const int wnt = !wide ? 0 : chan || N_out >= 2 * WN ? 2 * WN : WN;
   const int splits = M <= 0 ? 1 : wnt == 2 * WN ? choose_splits_big(M, ((N_out + 2 * WN - 1) / (2 * WN)) * (H / WH))
                                                 : choose_splits(M, n_tiles * h_tiles);   // (128 x 256 tiles: same value)
   if (chan && M > 0 && (!scales || (d->k > 0 && !vals))) return fail(HYC_EFAULT, "hyc_gradw_gemm: null vals/scales");

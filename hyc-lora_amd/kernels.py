@@ -738,22 +738,29 @@ def gated_act_fwd(act, gate2d, up2d, plan_act, plan_up, plan_gate, bits, group):
 # ----------------------------------------------------------------------------------------------------
 # weight gradient
 # ----------------------------------------------------------------------------------------------------
-STAGED_GRADW_MIN_FEATURES = 2048
+STAGED_GRADW_MIN_TILES = 96
+
+
+def gradw_staged_by_default(N_out, H):
+    """whether dW [N_out, H] from a channel-compressed activation restores x_hat first.  Every 256 output features
+    decode the same activation tile again (about a fifth on top of the dense product's time), against one pass that
+    writes x_hat and its second read.  Measured at 4096 and 16 384 tokens, H = 4096 and 11008, N_out = 256 ... 4096:
+    the staged route wins from 96 output tiles of 256 x 256 on (N_out >= 1536 at H = 4096, >= 768 at H = 11008)."""
+    return -(-N_out // 256) * (H // 256) >= STAGED_GRADW_MIN_TILES
 
 
 def gradw_gemm(dy2d, src, out_dtype=BF16, alpha=1.0, out=None, beta=0.0, staged=None):
     """dW [N_out, H] = alpha * dy^T @ x_hat (+ beta * out); src as for rmsnorm_bwd.
 
-    A compressed src is decoded inside the GEMM.  Every 256 output features decode the same activation tile again, so
-    for wide outputs (N_out >= 2048; not a shape LoRA training has) it is cheaper to restore x_hat once into a
-    transient matrix and run the same kernel on the dense operand (`staged`; None = by that rule)."""
+    A compressed src is decoded inside the GEMM, or (`staged`; None = by `gradw_staged_by_default`, never for the
+    few output features LoRA training has) restored once into a transient matrix for the same kernel's dense form."""
     _need_rows(dy2d, "grad_output")                # rows may be a column slice of a wider matrix (pitch = stride(0))
     M, N_out = dy2d.shape
+    H = src.H if isinstance(src, (ChannelCompressed, ThresholdCompressed)) else src.shape[-1]
     if staged is None:
-        staged = N_out >= STAGED_GRADW_MIN_FEATURES
+        staged = gradw_staged_by_default(N_out, H)
     if staged and isinstance(src, ChannelCompressed):
         src = decompress_channel(src)
-    H = src.H if isinstance(src, (ChannelCompressed, ThresholdCompressed)) else src.shape[-1]
     stored, vals, scales, d = _source(src, M, H)
     lib = _abi.load()
     if out is None:
