@@ -60,8 +60,9 @@ k_channel_absmax(const uint16_t* __restrict__ x, int64_t M, int64_t H, unsigned 
 
 // ---- selection: one workgroup of 1024 threads ---------------------------------------------------------------------
 // selected(c) <=> #{c' : s[c'] > s[c] or (s[c'] == s[c] and c' < c)} < k.  The k-th largest score T is found by a
-// radix select over order-preserving 32-bit keys (four passes of 8 bits, most significant first: a histogram of the
-// digit of every key that matches the prefix found so far, then the bin that holds rank k); the channels above T are
+// radix select over order-preserving 32-bit keys (four passes of 8 bits, most significant first, two when no key has
+// bits in its low half: a histogram of the digit of every key that matches the prefix found so far, then the bin that
+// holds rank k); the channels above T are
 // selected, and of those equal to T the first `need` by index.  Two prefix sums over the workgroup then give the rank of
 // every tie and the position of every selected channel, from which the plan words and the ascending list follow.
 constexpr int SEL_THREADS = 1024, SEL_LDS_KEYS = 16384;
@@ -108,12 +109,17 @@ k_select(const float* __restrict__ amax, int H, int k, uint32_t* __restrict__ pl
   const int tid = threadIdx.x;
   const bool cached = H <= SEL_LDS_KEYS;
   auto key_at = [&](int i) __attribute__((always_inline)) { return cached ? keys[i] : score_key(amax[i]); };
-  if (cached) for (int i = tid; i < H; i += SEL_THREADS) keys[i] = score_key(amax[i]);
+  uint32_t low = 0;                                         // scores that came from bf16 data have no low half:
+  for (int i = tid; i < H; i += SEL_THREADS) {              // the two passes over it are then skipped
+    const uint32_t key = score_key(amax[i]);
+    if (cached) keys[i] = key;
+    low |= key & 0xFFFFu;
+  }
   if (tid == 0) { s_prefix = 0; s_need = (uint32_t)k; }
-  __syncthreads();
+  const int last_shift = __syncthreads_or((int)low) ? 0 : 16;
   uint32_t mask = 0;
   const int trips = (H + SEL_THREADS - 1) / SEL_THREADS;    // the same for every lane: sel_tally votes wave-wide
-  for (int shift = 24; shift >= 0 && k > 0; shift -= 8) {
+  for (int shift = 24; shift >= last_shift && k > 0; shift -= 8) {
     if (tid < 256) hist[tid] = 0;
     __syncthreads();
     const uint32_t prefix = s_prefix;

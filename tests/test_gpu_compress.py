@@ -48,6 +48,16 @@ def test_selection_ties_go_to_lower_index(K):
     assert torch.equal(plan.idx.cpu(), O.hyc_select_channels(s, 10))
 
 
+@pytest.mark.parametrize("H,k", [(4096, 41), (512, 100), (20000, 7)])
+def test_selection_of_general_scores(K, H, k):
+    # fp32 scores with bits in their low half (the selection's two low radix passes run) and of both signs, with ties
+    gen = torch.Generator().manual_seed(H + k)
+    s = torch.randn(H, generator=gen)
+    s[torch.randperm(H, generator=gen)[:H // 4]] = float(s[0])
+    plan = K.select_channels(s.cuda(), k)
+    assert torch.equal(plan.idx.cpu(), O.hyc_select_channels(s, k))
+
+
 def test_absmax_accumulates(K):
     x1, _ = make_x(1, 40, 128, 2, 9.0)
     x2, _ = make_x(2, 24, 128, 2, 30.0)
