@@ -451,9 +451,24 @@ def layer_report(pkg, torch, steps=6, attentions=("eager", "flash"), quiet=False
                     peak = max(peak, torch.cuda.max_memory_allocated() - base)
                 del y, xg
             times.sort()
+            # the same steps issued back to back, as a training loop issues them (no synchronisation between steps, so
+            # the host's launch latency after an idle GPU is paid once, not per step)
+            xg = x.clone().requires_grad_(True)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            e0.record()
+            for it in range(steps):
+                for p in layer.parameters():
+                    p.grad = None
+                xg.grad = None
+                layer(xg).backward(g)
+            e1.record()
+            torch.cuda.synchronize()
             rec = {"layer_report": True, "compress": compress, "attention": attention, "batch": B, "seq": S,
                    "saved_for_backward_bytes": int(held), "peak_above_weights_bytes": int(peak),
-                   "step_ms": round(times[len(times) // 2], 3)}
+                   "step_ms": round(times[len(times) // 2], 3),
+                   "step_ms_back_to_back": round(e0.elapsed_time(e1) / steps, 3)}
+            del xg
             if compress:
                 rec["saved_analytic_bytes"] = int(layer.saved_activation_bytes(B, S))
             out.append(rec)
