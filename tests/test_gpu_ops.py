@@ -182,6 +182,38 @@ def test_softmax_kernels(K, shape):
     assert (dx.float() == want.float()).float().mean() > 0.995
 
 
+@pytest.mark.parametrize("rows", [0, 1, 5, 4095, 4096, 32768, 32771, 70001])
+@pytest.mark.parametrize("aligned", [True, False])
+def test_csr_offsets_against_a_cumulative_sum(hyc, K, rows, aligned):
+    """hyc_csr_offsets through the C ABI: row offsets = the exclusive prefix sums of the counts, clamped to the capacity;
+    the device word holds the unclamped total.  Sizes on both sides of its 4096-count tiles and 32 768-count rounds,
+    counts and offsets on 16-byte boundaries and off them (the scalar path), capacities that never bind, that cut a
+    row in the middle, and zero."""
+    import ctypes
+    abi = hyc._abi
+    lib = abi.load()
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    gen = torch.Generator().manual_seed(rows + int(aligned))
+    pad = 0 if aligned else 1
+    counts_buf = torch.zeros(rows + pad + 4, dtype=torch.int32)
+    counts_buf[pad:pad + rows] = torch.randint(0, 2049, (rows,), generator=gen, dtype=torch.int32)
+    counts_buf = counts_buf.cuda()
+    counts = counts_buf[pad:pad + rows]
+    exact = torch.zeros(rows + 1, dtype=torch.int64)
+    exact[1:] = torch.cumsum(counts.cpu().long(), 0)
+    true_total = int(exact[-1])
+    for capacity in (-1, true_total, true_total // 2 + 3, 0):
+        ptr_buf = torch.full((rows + 1 + pad + 4,), -7, dtype=torch.int32, device="cuda")
+        row_ptr = ptr_buf[pad:pad + rows + 1]
+        total = torch.full((1,), -1, dtype=torch.int64, device="cuda")
+        abi.check(lib.hyc_csr_offsets(p(counts) if rows else None, rows, capacity, p(row_ptr), p(total), None))
+        torch.cuda.synchronize()
+        cap = capacity if capacity >= 0 else 2 ** 31 - 1
+        assert int(total) == true_total
+        assert torch.equal(row_ptr.cpu().long(), exact.clamp(max=cap))
+        assert int((ptr_buf[:pad] != -7).sum()) == 0 and int((ptr_buf[pad + rows + 1:] != -7).sum()) == 0
+
+
 def test_softmax_kept_entries_sized_ahead_of_time(K):
     """A site's second call with the same threshold tensor sizes the kept entries from its budget and never reads the
     total back: same offsets, same entries, same gradient as the exact call, and the true total in a device word.
